@@ -1,0 +1,345 @@
+"""ctypes binding of the CPU oracle (oracle/liboracle.so) and, when present, of the
+reference's own in-tree kernels (oracle/_ref/libxft_ref.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by the smoke check and by the CPU-baseline
+leg of the benchmark.  The product package never imports this module.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_HERE, "liboracle.so")
+_REF = os.path.join(_HERE, "_ref", "libxft_ref.so")
+
+W_INT8, W_UINT4, W_NF4, W_W8A8, W_BF16 = 0, 1, 2, 3, 4
+EPI_NONE, EPI_BIAS, EPI_SILU, EPI_GELU, EPI_RESMUL, EPI_RESIDENTIAL, EPI_RESEXT, EPI_BIAS_RELU = range(8)
+
+
+def build(force=False):
+    """Compile the oracle (and oracle/_ref when the reference tree is mounted)."""
+    if force or not os.path.exists(_LIB):
+        subprocess.check_call(["make", "-C", _HERE, "-s", "all"])
+
+
+def _load():
+    if not os.path.exists(_LIB):
+        build()
+    return C.CDLL(_LIB)
+
+
+lib = _load()
+
+
+def host_has_avx512():
+    try:
+        with open("/proc/cpuinfo") as f:
+            flags = f.read()
+        return all(x in flags for x in ("avx512f", "avx512bw", "avx512vl", "avx512_bf16"))
+    except OSError:
+        return False
+
+
+def load_ref():
+    """The reference's in-tree kernels, or None (library absent / host lacks AVX-512)."""
+    if not os.path.exists(_REF) or not host_has_avx512():
+        return None
+    return C.CDLL(_REF)
+
+
+def p(a):
+    """Raw pointer of a C-contiguous numpy array (None -> NULL)."""
+    if a is None:
+        return None
+    assert a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def i32(a):
+    return np.ascontiguousarray(a, dtype=np.int32)
+
+
+lib.orc_f32_to_bf16.restype = C.c_uint16
+lib.orc_f32_to_bf16.argtypes = [C.c_float]
+lib.orc_f32_to_bf16_hw.restype = C.c_uint16
+lib.orc_f32_to_bf16_hw.argtypes = [C.c_float]
+lib.orc_f32_to_fp16.restype = C.c_uint16
+lib.orc_f32_to_fp16.argtypes = [C.c_float]
+lib.orc_vexp.restype = C.c_float
+lib.orc_vexp.argtypes = [C.c_float]
+lib.orc_nf4_codebook.restype = C.POINTER(C.c_float)
+lib.orc_num_threads.restype = C.c_int
+
+
+# --------------------------------------------------------------------------- conversions
+def to_bf16(x):
+    x = f32(x)
+    out = np.empty(x.shape, np.uint16)
+    lib.orc_f32_to_bf16_array(p(x), p(out), C.c_int64(x.size))
+    return out
+
+
+def from_bf16(b):
+    b = np.ascontiguousarray(b, dtype=np.uint16)
+    out = np.empty(b.shape, np.float32)
+    lib.orc_bf16_to_f32_array(p(b), p(out), C.c_int64(b.size))
+    return out
+
+
+def round_bf16(x):
+    return from_bf16(to_bf16(x))
+
+
+def to_fp16(x):
+    x = f32(x)
+    out = np.empty(x.shape, np.uint16)
+    lib.orc_f32_to_fp16_array(p(x), p(out), C.c_int64(x.size))
+    return out
+
+
+def from_fp16(h):
+    h = np.ascontiguousarray(h, dtype=np.uint16)
+    out = np.empty(h.shape, np.float32)
+    lib.orc_fp16_to_f32_array(p(h), p(out), C.c_int64(h.size))
+    return out
+
+
+def vexp(x):
+    x = f32(x)
+    out = np.empty_like(x)
+    lib.orc_vexp_array(p(x), p(out), C.c_int64(x.size))
+    return out
+
+
+def nf4_codebook():
+    return np.array([lib.orc_nf4_codebook()[i] for i in range(16)], np.float32)
+
+
+# --------------------------------------------------------------------------- weights
+class QWeight:
+    """A quantised [K,N] weight in the reference's pre-pack convention:
+    int8 [K,N]; uint4/nf4 [K,N/2] bytes with column n in the low nibble for even n."""
+
+    def __init__(self, kind, K, N, q, scale, zero=None):
+        self.kind, self.K, self.N = kind, K, N
+        self.q, self.scale, self.zero = q, scale, zero
+        self.colsum = None
+
+
+def quantize(kind, W):
+    W = f32(W)
+    K, N = W.shape
+    scale = np.empty(N, np.float32)
+    if kind in (W_INT8, W_W8A8):
+        q = np.empty((K, N), np.int8)
+        zero = np.zeros(N, np.float32)
+        lib.orc_quantize_int8_sym(p(W), K, N, p(q), p(scale), p(zero))
+        w = QWeight(kind, K, N, q, scale, zero)
+        if kind == W_W8A8:
+            w.colsum = np.empty(N, np.float32)
+            lib.orc_w8a8_colsum(p(q), K, N, p(w.colsum))
+        return w
+    q = np.empty((K, N // 2), np.uint8)
+    if kind == W_UINT4:
+        zero = np.empty(N, np.float32)
+        lib.orc_quantize_uint4_asym(p(W), K, N, p(q), p(scale), p(zero))
+        return QWeight(kind, K, N, q, scale, zero)
+    if kind == W_NF4:
+        lib.orc_quantize_nf4(p(W), K, N, p(q), p(scale))
+        return QWeight(kind, K, N, q, scale, None)
+    raise ValueError(kind)
+
+
+def dequant(w):
+    out = np.empty((w.K, w.N), np.float32)
+    lib.orc_dequant(w.kind, p(w.q), p(w.scale), p(w.zero), w.K, w.N, p(out))
+    return out
+
+
+def dequant_bf16(w):
+    out = np.empty((w.K, w.N), np.uint16)
+    lib.orc_dequant_bf16(w.kind, p(w.q), p(w.scale), p(w.zero), w.K, w.N, p(out))
+    return out
+
+
+def qgemm(w, A, epi=EPI_NONE, bias=None, res=None, gamma=1.0, f64=False):
+    A = f32(A)
+    M, K = A.shape
+    assert K == w.K
+    Cm = np.empty((M, w.N), np.float32)
+    if f64:
+        lib.orc_qgemm_f64(w.kind, M, w.N, K, p(A), K, p(w.q), p(w.scale), p(w.zero), p(Cm), w.N)
+        return Cm
+    bias = None if bias is None else f32(bias)
+    res = None if res is None else f32(res)
+    ldres = 0 if res is None else res.shape[1]
+    if w.kind == W_W8A8:
+        rc = lib.orc_w8a8_gemm(M, w.N, K, p(A), K, p(w.q), p(w.scale), p(w.zero), p(w.colsum), p(Cm), w.N, epi,
+                               p(bias), p(res), ldres, C.c_float(gamma))
+        assert rc == 0
+        return Cm
+    lib.orc_qgemm(w.kind, M, w.N, K, p(A), K, p(w.q), p(w.scale), p(w.zero), p(Cm), w.N, epi, p(bias), p(res),
+                  ldres, C.c_float(gamma))
+    return Cm
+
+
+def gemm_f32(A, W, epi=EPI_NONE, bias=None, res=None, gamma=1.0):
+    A, W = f32(A), f32(W)
+    M, K = A.shape
+    N = W.shape[1]
+    Cm = np.empty((M, N), np.float32)
+    bias = None if bias is None else f32(bias)
+    res = None if res is None else f32(res)
+    ldres = 0 if res is None else res.shape[1]
+    lib.orc_gemm_f32(M, N, K, p(A), K, p(W), N, p(Cm), N, epi, p(bias), p(res), ldres, C.c_float(gamma))
+    return Cm
+
+
+def w8a8_quantize_rows(A):
+    A = f32(A)
+    M, K = A.shape
+    qa = np.empty((M, K), np.int8)
+    s, z, sm = (np.empty(M, np.float32) for _ in range(3))
+    lib.orc_w8a8_quantize_rows(M, K, p(A), K, p(qa), K, p(s), p(z), p(sm))
+    return qa, s, z, sm
+
+
+# --------------------------------------------------------------------------- norm / rope
+def rmsnorm(x, weight, eps=1e-6):
+    x = f32(x)
+    out = np.empty_like(x)
+    rows, cols = x.shape
+    lib.orc_rmsnorm(p(out), p(x), p(f32(weight)), rows, cols, -1, -1, C.c_float(eps))
+    return out
+
+
+def rope_tables(dim, max_pos, base=10000, scaling=1.0):
+    half = (dim + 1) // 2
+    cos = np.empty((max_pos, half), np.float32)
+    sin = np.empty((max_pos, half), np.float32)
+    lib.orc_rope_tables(dim, max_pos, int(base), C.c_float(scaling), p(cos), p(sin))
+    return cos, sin
+
+
+def rope_apply(q, k, q_stride, k_stride, cos, sin, qk_shape, pos):
+    """In place on fp32 q/k (flat arrays); qk_shape = (batch, seq, qHeads, headSize, kvHeads)."""
+    lib.orc_rope_apply(p(q), p(k), q_stride, k_stride, p(cos), p(sin), cos.shape[1], p(i32(qk_shape)),
+                       p(i32(pos)))
+
+
+def rope_apply_tokens(q, k, cos, sin, q_stride, k_stride, dim, tokens, q_heads, k_heads, pos):
+    lib.orc_rope_apply_tokens(p(q), p(k), p(cos), p(sin), q_stride, k_stride, dim, tokens, q_heads, k_heads,
+                              p(i32(pos)))
+
+
+# --------------------------------------------------------------------------- KV cache
+class KVCache:
+    """One layer's K or V cache, [B][H][maxSeq][D] (+ scales [B][H][maxSeq] when INT8)."""
+
+    def __init__(self, int8, B, H, max_seq, D):
+        self.int8, self.B, self.H, self.S, self.D = int(int8), B, H, max_seq, D
+        self.data = np.zeros((B, H, max_seq, D), np.int8 if int8 else np.uint16)
+        self.scales = np.zeros((B, H, max_seq), np.float32)
+
+    def store(self, b, past, rows, kv_stride=None):
+        """rows: fp32 [n, H*D] (or wider with kv_stride)."""
+        rows = f32(rows)
+        n = rows.shape[0]
+        lib.orc_kv_store(self.int8, self.B, self.H, self.S, self.D, p(self.data), p(self.scales), b, past, n,
+                         p(rows), kv_stride or rows.shape[1])
+
+    def as_f32(self):
+        if self.int8:
+            return self.data.astype(np.float32) * self.scales[..., None]
+        return from_fp16(self.data)
+
+
+def kv_quantize_row(x):
+    x = f32(x)
+    q = np.empty(x.shape, np.int8)
+    s = np.zeros(1, np.float32)
+    lib.orc_kv_quantize_row(p(q), p(s), p(x), x.size)
+    return q, s[0]
+
+
+# --------------------------------------------------------------------------- attention
+def cross_attn_by_head(q, k, v, q_heads, kv_heads, D, in_lens, past_lens, scale, kc, vc):
+    """q: fp32 [tokens, q_heads*D]; k, v: fp32 [tokens, kv_heads*D]. Stores new rows, returns output."""
+    q, k, v = f32(q), f32(k), f32(v)
+    out = np.zeros_like(q)
+    B = len(in_lens)
+    lib.orc_cross_attn_by_head(p(out), p(q), p(k), p(v), q_heads, kv_heads, D, q.shape[1], q.shape[1], k.shape[1],
+                               B, p(i32(in_lens)), p(i32(past_lens)), C.c_float(scale), kc.int8, kc.B, kc.S,
+                               p(kc.data), p(kc.scales), p(vc.data), p(vc.scales))
+    return out
+
+
+def cross_attn_sharded_head(q, present, q_heads, kv_heads, D, scale, splits, kc, vc):
+    q = f32(q)
+    out = np.zeros_like(q)
+    B = q.shape[0]
+    lib.orc_cross_attn_sharded_head(p(out), p(q), present, q_heads, kv_heads, D, q.shape[1], q.shape[1], B,
+                                    C.c_float(scale), splits, kc.int8, kc.B, kc.S, p(kc.data), p(kc.scales),
+                                    p(vc.data), p(vc.scales))
+    return out
+
+
+def flash_prefill(q, k_bf16, v_bf16, q_heads, kv_heads, D, in_lens, past_lens, scale, kv_stride=None):
+    """q fp32 [tokens, q_heads*D]; k_bf16/v_bf16: uint16 views with row stride kv_stride."""
+    q = f32(q)
+    out = np.zeros_like(q)
+    lib.orc_flash_prefill(p(out), p(q), p(k_bf16), p(v_bf16), q_heads, kv_heads, D, q.shape[1], q.shape[1],
+                          kv_stride or k_bf16.shape[1], len(in_lens), p(i32(in_lens)), p(i32(past_lens)),
+                          C.c_float(scale))
+    return out
+
+
+def attention_ref_f64(q, K, V, q_heads, kv_heads, D, in_lens, past_lens, scale):
+    """K, V fp32 [B, kvH, S, D]."""
+    q, K, V = f32(q), f32(K), f32(V)
+    out = np.zeros_like(q)
+    lib.orc_attention_ref_f64(p(out), p(q), p(K), p(V), q_heads, kv_heads, D, q.shape[1], q.shape[1], len(in_lens),
+                              p(i32(in_lens)), p(i32(past_lens)), K.shape[2], C.c_float(scale))
+    return out
+
+
+def softmax_scaled(x, scale):
+    x = f32(x).copy()
+    lib.orc_softmax_scaled(p(x), C.c_float(scale), x.size)
+    return x
+
+
+# --------------------------------------------------------------------------- misc
+def silu_sum(x):
+    x = f32(x)
+    M, N2 = x.shape
+    out = np.empty((M, N2 // 2), np.float32)
+    lib.orc_silu_sum(p(x), N2, p(out), N2 // 2, M, N2 // 2)
+    return out
+
+
+def moe_top2(logits):
+    logits = f32(logits)
+    M, N = logits.shape
+    sel = np.empty((M, 2), np.int32)
+    w = np.empty((M, 2), np.float32)
+    lib.orc_moe_top2(p(logits), M, N, p(sel), p(w))
+    return sel, w
+
+
+def argmax(logits):
+    logits = f32(logits)
+    B, V = logits.shape
+    ids = np.empty(B, np.int32)
+    lib.orc_argmax(p(logits), B, V, p(ids))
+    return ids
+
+
+def num_threads():
+    return lib.orc_num_threads()

@@ -1,0 +1,1111 @@
+/*
+ * CPU oracle for the decoder-layer hot path of intel/xFasterTransformer v2.1.2.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file restates, in scalar C, the arithmetic the
+ * reference performs with AVX-512 intrinsics (or delegates to closed third-party
+ * binaries).  It is linked only by the test-suite, the smoke check and the
+ * CPU-baseline leg of the benchmark; the product library never calls it.
+ *
+ * Every function names the reference file:line it follows (paths are relative to
+ * the reference tree).  Where the reference keeps 16 partial sums in one AVX-512
+ * register and finishes with _mm512_reduce_add_ps, the restatement keeps the same
+ * 16 lanes and the same pairwise tree, so results agree bit for bit with a build
+ * of the reference's in-tree kernels.
+ *
+ * Pinned / unpinned status (what each function was checked against):
+ *   bf16 / fp16 conversion ............ pinned: reference headers compiled as-is, numpy
+ *   vexp .............................. pinned: reference bert_util.h compiled as-is
+ *   INT8 KV quantize .................. pinned: reference quantize_util.h compiled as-is
+ *   RoPE (tables + rotate) ............ pinned: reference kernel compiled as-is + the
+ *                                       golden constants of tests/ut/rotary_embedding_test.cpp
+ *   P*V small_gemm (fp32/fp16) ........ pinned: reference gemm_kernel_ext3.cpp compiled as-is
+ *   INT8/UINT4 dequant ................ pinned: convention w = scale*q + zero, nibble order
+ *                                       of uint4x2.h (compiled as-is)
+ *   RMSNorm ........................... pinned by closed form (numpy float64) to 1e-6
+ *   softmax / split-KV merge .......... pinned by closed form (numpy float64)
+ *   Q*K^T small_gemm_transb ........... pinned by closed form; lane order follows source
+ *   W8A8 quantize/dequant ............. pinned by closed form + exact integer GEMM
+ *   weight quantizers (INT8/UINT4/NF4), NF4 codebook, weight-only GEMM inner rounding,
+ *   xDNN small_softmax ................ PARITY UNPINNED: the reference delegates them to
+ *                                       the closed xDNN binary; textbook definitions used.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#include <float.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORC_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------------- */
+/* bit casts                                                                  */
+/* ------------------------------------------------------------------------- */
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* include/bfloat16.h:40-65 : RNE for normals, subnormals flushed to signed zero,
+ * infinities kept, NaN keeps its top half with quiet bit 6 set. */
+ORC_API uint16_t orc_f32_to_bf16(float f) {
+    uint32_t u = f2u(f);
+    uint16_t hi = (uint16_t)(u >> 16);
+    switch (fpclassify(f)) {
+        case FP_SUBNORMAL:
+        case FP_ZERO: return hi & 0x8000;
+        case FP_INFINITE: return hi;
+        case FP_NAN: return hi | (1u << 6);
+        default: {
+            uint32_t bias = 0x7FFFu + (hi & 1u);
+            return (uint16_t)((u + bias) >> 16);
+        }
+    }
+}
+
+/* include/bfloat16.h:72-75 */
+ORC_API float orc_bf16_to_f32(uint16_t b) { return u2f((uint32_t)b << 16); }
+
+/* src/common/float16.h (vcvtps2ph, _MM_FROUND_TO_NEAREST_INT) == IEEE-754 RNE
+ * binary32 -> binary16, subnormals kept. */
+ORC_API uint16_t orc_f32_to_fp16(float f) {
+    uint32_t x = f2u(f);
+    uint32_t sign = (x >> 16) & 0x8000u;
+    uint32_t absx = x & 0x7FFFFFFFu;
+    if (absx >= 0x7F800000u) { /* inf / nan */
+        if (absx > 0x7F800000u) return (uint16_t)(sign | 0x7E00u | ((absx >> 13) & 0x3FFu));
+        return (uint16_t)(sign | 0x7C00u);
+    }
+    if (absx >= 0x477FF000u) { /* rounds to >= 65520 -> inf */
+        return (uint16_t)(sign | 0x7C00u);
+    }
+    if (absx < 0x38800000u) { /* result is subnormal or zero (|f| < 2^-14) */
+        if (absx < 0x33000000u) return (uint16_t)sign; /* < 2^-25 -> 0 */
+        int e = (int)(absx >> 23); /* biased exponent, 102..112 */
+        uint32_t m = (absx & 0x7FFFFFu) | 0x800000u; /* 24-bit significand */
+        int shift = 126 - e; /* 14..24 : result = m >> shift in units of 2^-24 */
+        uint32_t q = m >> shift;
+        uint32_t rem = m & ((1u << shift) - 1u);
+        uint32_t half = 1u << (shift - 1);
+        if (rem > half || (rem == half && (q & 1u))) q++;
+        return (uint16_t)(sign | q);
+    }
+    {
+        uint32_t e = (absx >> 23) - 112u; /* rebias 127 -> 15 */
+        uint32_t m = absx & 0x7FFFFFu;
+        uint32_t q = (e << 10) | (m >> 13);
+        uint32_t rem = m & 0x1FFFu;
+        if (rem > 0x1000u || (rem == 0x1000u && (q & 1u))) q++;
+        return (uint16_t)(sign | q);
+    }
+}
+
+ORC_API float orc_fp16_to_f32(uint16_t h) {
+    uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+    uint32_t e = (h >> 10) & 0x1Fu;
+    uint32_t m = h & 0x3FFu;
+    if (e == 0) {
+        if (m == 0) return u2f(sign);
+        float v = (float)m * 5.9604644775390625e-08f; /* 2^-24 */
+        return (sign ? -v : v);
+    }
+    if (e == 31) return u2f(sign | 0x7F800000u | (m << 13));
+    return u2f(sign | ((e + 112u) << 23) | (m << 13));
+}
+
+ORC_API void orc_f32_to_bf16_array(const float *src, uint16_t *dst, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) dst[i] = orc_f32_to_bf16(src[i]);
+}
+ORC_API void orc_bf16_to_f32_array(const uint16_t *src, float *dst, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) dst[i] = orc_bf16_to_f32(src[i]);
+}
+ORC_API void orc_f32_to_fp16_array(const float *src, uint16_t *dst, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) dst[i] = orc_f32_to_fp16(src[i]);
+}
+ORC_API void orc_fp16_to_f32_array(const uint16_t *src, float *dst, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) dst[i] = orc_fp16_to_f32(src[i]);
+}
+/* round-trip through bf16, in place */
+ORC_API void orc_round_bf16_inplace(float *x, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) x[i] = orc_bf16_to_f32(orc_f32_to_bf16(x[i]));
+}
+
+/* ------------------------------------------------------------------------- */
+/* AVX-512 lane helpers                                                       */
+/* ------------------------------------------------------------------------- */
+/* _mm512_reduce_add_ps as gcc expands it: 16 -> 8 -> 4 -> 2 -> 1, adding lane i
+ * to lane i + half at each step. */
+static inline float reduce_add16(const float *v) {
+    float a[8], b[4], c[2];
+    for (int i = 0; i < 8; ++i) a[i] = v[i] + v[i + 8];
+    for (int i = 0; i < 4; ++i) b[i] = a[i] + a[i + 4];
+    for (int i = 0; i < 2; ++i) c[i] = b[i] + b[i + 2];
+    return c[0] + c[1];
+}
+
+/* src/utils/bert_util.h:26-75 (BertUtil::vexp), one lane. */
+ORC_API float orc_vexp(float xin) {
+    const float hi = 88.3762626647950f, lo = -88.3762626647949f;
+    const float log2ef = 1.44269504088896341f;
+    float x = xin;
+    /* _mm512_min_ps(a,b) returns b when either is NaN; same for max */
+    x = (x < hi) ? x : hi;
+    x = (x > lo) ? x : lo;
+    float m = floorf(fmaf(x, log2ef, 0.5f));
+    float r = fmaf(m, -0.6931471805599453f, x);
+    float r2 = r * r;
+    float y = 1.9875691500E-4f;
+    y = fmaf(y, r, 1.3981999507E-3f);
+    y = fmaf(y, r, 8.3334519073E-3f);
+    y = fmaf(y, r, 4.1665795894E-2f);
+    y = fmaf(y, r, 1.6666665459E-1f);
+    y = fmaf(y, r, 5.0000001201E-1f);
+    y = fmaf(y, r2, r);
+    y = y + 1.0f;
+    int32_t e = (int32_t)(m + 127.0f); /* cvttps */
+    float p = u2f((uint32_t)e << 23);
+    float res = y * p;
+    return (res > xin) ? res : xin; /* _mm512_max_ps(res, _x) */
+}
+
+ORC_API void orc_vexp_array(const float *x, float *y, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) y[i] = orc_vexp(x[i]);
+}
+
+/* ------------------------------------------------------------------------- */
+/* Weight formats                                                             */
+/* ------------------------------------------------------------------------- */
+/* kinds shared with the device library */
+enum { ORC_W_INT8 = 0, ORC_W_UINT4 = 1, ORC_W_NF4 = 2, ORC_W_W8A8 = 3, ORC_W_BF16 = 4 };
+
+/* NormalFloat4 codebook (Dettmers et al. 2023, QLoRA, appendix E).  The reference
+ * keeps its table inside the closed xDNN binary: PARITY UNPINNED. */
+static const float kNF4[16] = {-1.0f, -0.6961928009986877f, -0.5250730514526367f, -0.39491748809814453f,
+        -0.28444138169288635f, -0.18477343022823334f, -0.09105003625154495f, 0.0f, 0.07958029955625534f,
+        0.16093020141124725f, 0.24611230194568634f, 0.33791524171829224f, 0.44070982933044434f,
+        0.5626170039176941f, 0.7229568362236023f, 1.0f};
+
+ORC_API const float *orc_nf4_codebook(void) { return kNF4; }
+
+/* src/common/uint4x2.h:43-71 : element 0 of a pair sits in the low nibble. */
+static inline int nib(const uint8_t *q, int64_t idx) {
+    uint8_t b = q[idx >> 1];
+    return (idx & 1) ? (b >> 4) & 0xF : b & 0xF;
+}
+
+/* Dequantised weight element (k,n) of a [K,N] row-major quantised matrix.
+ * INT8/UINT4: src/utils/matmul_helper.h:317-346, w = scale[n]*q + zero[n] evaluated
+ * as one fused multiply-add (what gcc -O2 emits for that line on an FMA target).
+ * NF4: w = code[q] * absmax[n] (scale array carries absmax). */
+static inline float deq_elem(int kind, const void *q, const float *scale, const float *zero, int64_t k, int64_t n,
+        int64_t N) {
+    switch (kind) {
+        case ORC_W_INT8:
+        case ORC_W_W8A8: {
+            float z = zero ? zero[n] : 0.0f;
+            return fmaf(scale[n], (float)((const int8_t *)q)[k * N + n], z);
+        }
+        case ORC_W_UINT4: {
+            float z = zero ? zero[n] : 0.0f;
+            return fmaf(scale[n], (float)nib((const uint8_t *)q, k * N + n), z);
+        }
+        case ORC_W_NF4: return kNF4[nib((const uint8_t *)q, k * N + n)] * scale[n];
+        default: return 0.0f;
+    }
+}
+
+ORC_API void orc_dequant(int kind, const void *q, const float *scale, const float *zero, int K, int N, float *w) {
+#pragma omp parallel for
+    for (int64_t k = 0; k < K; ++k)
+        for (int64_t n = 0; n < N; ++n) w[k * N + n] = deq_elem(kind, q, scale, zero, k, n, N);
+}
+
+/* matmul_helper.h:317-346: the dequantised value narrowed to bf16 */
+ORC_API void orc_dequant_bf16(int kind, const void *q, const float *scale, const float *zero, int K, int N,
+        uint16_t *w) {
+#pragma omp parallel for
+    for (int64_t k = 0; k < K; ++k)
+        for (int64_t n = 0; n < N; ++n) w[k * N + n] = orc_f32_to_bf16(deq_elem(kind, q, scale, zero, k, n, N));
+}
+
+/* Build-owned quantizers.  The reference calls xdnn_*_quantize (matmul_helper.h:205-262)
+ * whose source is not available: PARITY UNPINNED.  W is [K,N] row-major, one
+ * scale (and zero) per output column n. */
+ORC_API void orc_quantize_int8_sym(const float *W, int K, int N, int8_t *q, float *scale, float *zero) {
+#pragma omp parallel for
+    for (int n = 0; n < N; ++n) {
+        float amax = 0.0f;
+        for (int64_t k = 0; k < K; ++k) amax = fmaxf(amax, fabsf(W[k * N + n]));
+        float s = amax / 127.0f;
+        scale[n] = s;
+        if (zero) zero[n] = 0.0f;
+        for (int64_t k = 0; k < K; ++k) {
+            float v = (s == 0.0f) ? 0.0f : nearbyintf(W[k * N + n] / s);
+            v = fminf(fmaxf(v, -127.0f), 127.0f);
+            q[k * N + n] = (int8_t)v;
+        }
+    }
+}
+
+ORC_API void orc_quantize_uint4_asym(const float *W, int K, int N, uint8_t *q, float *scale, float *zero) {
+    memset(q, 0, (size_t)K * N / 2);
+    /* two adjacent columns share a byte: walk column pairs */
+#pragma omp parallel for
+    for (int np = 0; np < N / 2; ++np) {
+        for (int h = 0; h < 2; ++h) {
+            int n = np * 2 + h;
+            float mn = W[n], mx = W[n];
+            for (int64_t k = 1; k < K; ++k) {
+                float v = W[k * N + n];
+                mn = fminf(mn, v);
+                mx = fmaxf(mx, v);
+            }
+            float s = (mx - mn) / 15.0f;
+            scale[n] = s;
+            zero[n] = mn;
+            for (int64_t k = 0; k < K; ++k) {
+                float v = (s == 0.0f) ? 0.0f : nearbyintf((W[k * N + n] - mn) / s);
+                v = fminf(fmaxf(v, 0.0f), 15.0f);
+                uint8_t u = (uint8_t)v;
+                q[(k * N + n) >> 1] |= h ? (uint8_t)(u << 4) : u;
+            }
+        }
+    }
+}
+
+ORC_API void orc_quantize_nf4(const float *W, int K, int N, uint8_t *q, float *absmax) {
+    memset(q, 0, (size_t)K * N / 2);
+#pragma omp parallel for
+    for (int np = 0; np < N / 2; ++np) {
+        for (int h = 0; h < 2; ++h) {
+            int n = np * 2 + h;
+            float amax = 0.0f;
+            for (int64_t k = 0; k < K; ++k) amax = fmaxf(amax, fabsf(W[k * N + n]));
+            absmax[n] = amax;
+            for (int64_t k = 0; k < K; ++k) {
+                float v = (amax == 0.0f) ? 0.0f : W[k * N + n] / amax;
+                int best = 0;
+                float bd = fabsf(v - kNF4[0]);
+                for (int c = 1; c < 16; ++c) {
+                    float d = fabsf(v - kNF4[c]);
+                    if (d < bd) { bd = d; best = c; }
+                }
+                q[(k * N + n) >> 1] |= h ? (uint8_t)(best << 4) : (uint8_t)best;
+            }
+        }
+    }
+}
+
+/* matmul_helper.h:362-372 : per-column sums of the int8 weight, accumulated in
+ * float in row order. */
+ORC_API void orc_w8a8_colsum(const int8_t *q, int K, int N, float *sum) {
+    for (int n = 0; n < N; ++n) {
+        float s = 0.0f;
+        for (int64_t k = 0; k < K; ++k) s += (float)q[k * N + n];
+        sum[n] = s;
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* Epilogues  (matmul_helper.h:730-1705; definitions as in :2894-2939)        */
+/* ------------------------------------------------------------------------- */
+enum {
+    ORC_EPI_NONE = 0,
+    ORC_EPI_BIAS = 1,
+    ORC_EPI_SILU = 2,
+    ORC_EPI_GELU = 3,
+    ORC_EPI_RESMUL = 4,
+    ORC_EPI_RESIDENTIAL = 5,
+    ORC_EPI_RESEXT = 6,
+    ORC_EPI_BIAS_RELU = 7
+};
+
+/* silu as the Llama MLP computes it: decoder_util.h:564-570, x / (1 + vexp(-x)) */
+static inline float silu_ref(float x) { return x / (1.0f + orc_vexp(x * -1.0f)); }
+
+static inline float apply_epilogue(int epi, float v, int m, int n, const float *bias, const float *res, int ldres,
+        float gamma) {
+    switch (epi) {
+        case ORC_EPI_BIAS: return v + bias[n];
+        case ORC_EPI_BIAS_RELU: return fmaxf(v + bias[n], 0.0f);
+        case ORC_EPI_SILU: return silu_ref(v);
+        case ORC_EPI_GELU: { /* x * sigmoid(1.702 x), matmul_helper.h:2913-2919 */
+            float e = orc_vexp(v * 1.702f);
+            return e / (e + 1.0f) * v;
+        }
+        case ORC_EPI_RESMUL: return v * res[(int64_t)m * ldres + n];
+        case ORC_EPI_RESIDENTIAL: return (bias ? v + bias[n] : v) + res[(int64_t)m * ldres + n];
+        case ORC_EPI_RESEXT: return fmaf(gamma, res[(int64_t)m * ldres + n], bias ? v + bias[n] : v);
+        default: return v;
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* Weight-only GEMM  C[M,N] = A[M,K] * deq(W)[K,N]  (+ epilogue)               */
+/* matmul_helper.h:565-728 ("compute") and the compute_* family.  The inner    */
+/* arithmetic of xDNN is not visible: closed form with fp32 accumulation in k  */
+/* order; orc_qgemm_f64 accumulates in double for checking the oracle itself.  */
+/* ------------------------------------------------------------------------- */
+ORC_API void orc_qgemm(int kind, int M, int N, int K, const float *A, int lda, const void *q, const float *scale,
+        const float *zero, float *C, int ldc, int epi, const float *bias, const float *res, int ldres,
+        float gamma) {
+    enum { NB = 256 };
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int m = 0; m < M; ++m) {
+        for (int n0 = 0; n0 < N; n0 += NB) {
+            float acc[NB];
+            int nb = (N - n0 < NB) ? N - n0 : NB;
+            for (int j = 0; j < nb; ++j) acc[j] = 0.0f;
+            for (int64_t k = 0; k < K; ++k) {
+                float a = A[(int64_t)m * lda + k];
+                for (int j = 0; j < nb; ++j) acc[j] += a * deq_elem(kind, q, scale, zero, k, n0 + j, N);
+            }
+            for (int j = 0; j < nb; ++j)
+                C[(int64_t)m * ldc + n0 + j] = apply_epilogue(epi, acc[j], m, n0 + j, bias, res, ldres, gamma);
+        }
+    }
+}
+
+ORC_API void orc_qgemm_f64(int kind, int M, int N, int K, const float *A, int lda, const void *q,
+        const float *scale, const float *zero, float *C, int ldc) {
+#pragma omp parallel for collapse(2)
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) {
+            double acc = 0.0;
+            for (int64_t k = 0; k < K; ++k)
+                acc += (double)A[(int64_t)m * lda + k] * (double)deq_elem(kind, q, scale, zero, k, n, N);
+            C[(int64_t)m * ldc + n] = (float)acc;
+        }
+}
+
+/* Plain fp32 GEMM against an fp32 [K,N] weight, same accumulation order. */
+ORC_API void orc_gemm_f32(int M, int N, int K, const float *A, int lda, const float *W, int ldw, float *C, int ldc,
+        int epi, const float *bias, const float *res, int ldres, float gamma) {
+    enum { NB = 256 };
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int m = 0; m < M; ++m) {
+        for (int n0 = 0; n0 < N; n0 += NB) {
+            float acc[NB];
+            int nb = (N - n0 < NB) ? N - n0 : NB;
+            for (int j = 0; j < nb; ++j) acc[j] = 0.0f;
+            for (int64_t k = 0; k < K; ++k) {
+                float a = A[(int64_t)m * lda + k];
+                const float *w = W + k * ldw + n0;
+                for (int j = 0; j < nb; ++j) acc[j] += a * w[j];
+            }
+            for (int j = 0; j < nb; ++j)
+                C[(int64_t)m * ldc + n0 + j] = apply_epilogue(epi, acc[j], m, n0 + j, bias, res, ldres, gamma);
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* W8A8  (matmul_helper.h:2762-2965)                                          */
+/* ------------------------------------------------------------------------- */
+/* quantize_s8, :2810-2853.  Per row: zero=(min+max)/2, scale=max(|max-zero|,|zero-min|)/127,
+ * q = cvt_rne(fma(x, 1/scale, -zero/scale)) narrowed with truncation of the int32
+ * (vpmovdb), sum = (sum q) * scale + K * zero. */
+ORC_API void orc_w8a8_quantize_rows(int M, int K, const float *A, int lda, int8_t *qa, int ldq, float *scale,
+        float *zero, float *sum) {
+    for (int i = 0; i < M; ++i) {
+        const float *row = A + (int64_t)i * lda;
+        float mx = row[0], mn = row[0];
+        for (int j = 1; j < K; ++j) {
+            mx = fmaxf(mx, row[j]);
+            mn = fminf(mn, row[j]);
+        }
+        float fzero = (mn + mx) / 2.0f;
+        float fscale = fmaxf(fabsf(mx - fzero), fabsf(fzero - mn)) / 127.0f;
+        scale[i] = fscale;
+        zero[i] = fzero;
+        float vs = 1.0f / fscale, vz = -fzero / fscale;
+        int32_t isum = 0;
+        for (int j = 0; j < K; ++j) {
+            int32_t ix = (int32_t)nearbyintf(fmaf(row[j], vs, vz));
+            isum += ix;
+            qa[(int64_t)i * ldq + j] = (int8_t)ix;
+        }
+        sum[i] = (float)isum * fscale + (float)K * fzero;
+    }
+}
+
+/* onednn_amx_gemm_f32s8f32_compute_base, :2784-2808 + dequant :2870-2965.
+ * C = s32 * sA * sB + sumB * sB * zA + sumA * zB, then epilogue. Requires N%16==0. */
+ORC_API int orc_w8a8_gemm(int M, int N, int K, const float *A, int lda, const int8_t *qb, const float *scaleB,
+        const float *zeroB, const float *sumB, float *C, int ldc, int epi, const float *bias, const float *res,
+        int ldres, float gamma) {
+    if (N % 16 != 0) return -1;
+    int8_t *qa = (int8_t *)malloc((size_t)M * K);
+    float *sA = (float *)malloc(sizeof(float) * M * 3);
+    float *zA = sA + M, *sumA = sA + 2 * M;
+    orc_w8a8_quantize_rows(M, K, A, lda, qa, K, sA, zA, sumA);
+#pragma omp parallel for collapse(2)
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) {
+            int32_t acc = 0;
+            for (int64_t k = 0; k < K; ++k) acc += (int32_t)qa[(int64_t)m * K + k] * (int32_t)qb[k * N + n];
+            /* v*vscaleA*vscaleB + vsumB*vscaleB*vzeroA + vsumA*vzeroB, left to right, no contraction */
+            float v = (float)acc;
+            float t0 = v * sA[m];
+            t0 = t0 * scaleB[n];
+            float t1 = sumB[n] * scaleB[n];
+            t1 = t1 * zA[m];
+            float t2 = sumA[m] * zeroB[n];
+            float x = (t0 + t1) + t2;
+            C[(int64_t)m * ldc + n] = apply_epilogue(epi, x, m, n, bias, res, ldres, gamma);
+        }
+    free(qa);
+    free(sA);
+    return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* RMSNorm  (src/kernels/rmsnorm_kernels.cpp:27-84)                           */
+/* ------------------------------------------------------------------------- */
+ORC_API void orc_rmsnorm(float *out, const float *in, const float *weight, int rows, int cols, int iStride,
+        int oStride, float eps) {
+    if (iStride == -1) iStride = cols;
+    if (oStride == -1) oStride = cols;
+#pragma omp parallel for
+    for (int r = 0; r < rows; ++r) {
+        const float *px = in + (int64_t)r * iStride;
+        float *py = out + (int64_t)r * oStride;
+        float lanes[16];
+        for (int l = 0; l < 16; ++l) lanes[l] = 0.0f;
+        for (int c = 0; c < cols; ++c) {
+            float t = px[c] * px[c];
+            lanes[c & 15] = lanes[c & 15] + t;
+        }
+        float sq = reduce_add16(lanes);
+        float var = 1.0f / sqrtf(sq / cols + eps);
+        for (int c = 0; c < cols; ++c) py[c] = (px[c] * var) * weight[c];
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* RoPE  (src/layers/rotary_embedding.cpp:21-66, kernels :21-199)             */
+/* ------------------------------------------------------------------------- */
+/* inv_freq[i] = 1.0 / pow(base, float(2i)/dim) in double, stored as float;
+ * table[pos][j] = cos/sin(float(pos * inv_freq[j])) * scale (std::cos(float)). */
+ORC_API void orc_rope_tables(int dim, int maxPos, int base, float scalingFactor, float *embCos, float *embSin) {
+    int half = (dim + 1) / 2;
+    float *inv = (float *)malloc(sizeof(float) * half);
+    for (int i = 0; i < half; ++i) {
+        inv[i] = (float)(1.0 / pow((double)base, (double)((float)(i * 2) / (float)dim)));
+        inv[i] /= scalingFactor;
+    }
+    for (int64_t p = 0; p < maxPos; ++p)
+        for (int j = 0; j < half; ++j) {
+            float t = (float)p * inv[j];
+            embCos[p * half + j] = cosf(t) * 1.0f;
+            embSin[p * half + j] = sinf(t) * 1.0f;
+        }
+    free(inv);
+}
+
+static inline void rope_rotate(float *x, const float *pcos, const float *psin, int half) {
+    for (int i = 0; i < half; ++i) {
+        float a = x[i], b = x[i + half];
+        /* fmsub(q, cos, qHalf*sin) ; fmadd(qHalf, cos, q*sin) */
+        float na = fmaf(a, pcos[i], -(b * psin[i]));
+        float nb = fmaf(b, pcos[i], a * psin[i]);
+        x[i] = na;
+        x[i + half] = nb;
+    }
+}
+
+/* llamaApplyRotaryPosEmbeding, kernels :57-108.  qkShape = {batch, seq, qHeads, headSize, kvHeads};
+ * positionIds has seq entries shared by every batch row. */
+ORC_API void orc_rope_apply(float *query, float *key, int qStride, int kStride, const float *embCos,
+        const float *embSin, int half, const int *qkShape, const int *positionIds) {
+    int B = qkShape[0], S = qkShape[1], qH = qkShape[2], kH = qkShape[4];
+    int dim = half * 2;
+    int heads = qH > kH ? qH : kH;
+    for (int h = 0; h < heads; ++h)
+        for (int b = 0; b < B; ++b)
+            for (int s = 0; s < S; ++s) {
+                int pos = positionIds[s];
+                const float *pc = embCos + (int64_t)pos * half, *ps = embSin + (int64_t)pos * half;
+                if (h < qH) rope_rotate(query + ((int64_t)b * S + s) * qStride + h * dim, pc, ps, half);
+                if (h < kH) rope_rotate(key + ((int64_t)b * S + s) * kStride + h * dim, pc, ps, half);
+            }
+}
+
+/* llamaApplyRotaryPosEmbed (continuous batching), kernels :126-172: one position per token. */
+ORC_API void orc_rope_apply_tokens(float *query, float *key, const float *embCos, const float *embSin, int qStride,
+        int kStride, int dim, int totSeqLen, int qHeads, int kHeads, const int *positionIds) {
+    int half = (dim + 1) / 2;
+    int heads = qHeads > kHeads ? qHeads : kHeads;
+    for (int h = 0; h < heads; ++h)
+        for (int s = 0; s < totSeqLen; ++s) {
+            int pos = positionIds[s];
+            const float *pc = embCos + (int64_t)pos * half, *ps = embSin + (int64_t)pos * half;
+            if (h < qHeads) rope_rotate(query + (int64_t)s * qStride + h * dim, pc, ps, half);
+            if (h < kHeads) rope_rotate(key + (int64_t)s * kStride + h * dim, pc, ps, half);
+        }
+}
+
+/* Same rotation on bf16 storage: load widens, fp32 math, store narrows with the
+ * AVX-512 vcvtneps2bf16 rule (RNE, subnormals kept — intrinsics_util.h store_avx512). */
+static inline uint16_t bf16_rne_hw(float f) {
+    uint32_t u = f2u(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40);
+    if (((u >> 23) & 0xFF) == 0) return (uint16_t)((u >> 16) & 0x8000); /* DAZ/FTZ of vcvtneps2bf16 */
+    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+ORC_API uint16_t orc_f32_to_bf16_hw(float f) { return bf16_rne_hw(f); }
+
+/* ------------------------------------------------------------------------- */
+/* KV cache store  (attention_kernels.h:44-69, quantize_util.h:21-51)         */
+/* ------------------------------------------------------------------------- */
+/* xft::quantize: max=absmax, factor = max==0 ? 1 : 127/max, *scale = max/127,
+ * q = (int8) rne(x * factor). */
+ORC_API void orc_kv_quantize_row(int8_t *dst, float *scale, const float *src, int size) {
+    float mx = 0.0f;
+    for (int i = 0; i < size; ++i) mx = fmaxf(mx, fabsf(src[i]));
+    float factor = (mx == 0.0f) ? 1.0f : 127.0f / mx;
+    *scale = mx / 127.0f;
+    for (int i = 0; i < size; ++i) dst[i] = (int8_t)(int32_t)nearbyintf(src[i] * factor);
+}
+
+/* KV cache tensor, ENABLE_KV_TRANS=1 layout: data [B][H][maxSeq][D], scales [B][H][maxSeq]
+ * (src/common/kvcache_tensor.h:101-131). */
+typedef struct {
+    int is_int8;
+    int B, H, maxSeq, D;
+    void *data;
+    float *scales;
+} orc_kv_t;
+
+static inline int64_t kv_off(const orc_kv_t *c, int b, int h, int s) {
+    return (((int64_t)b * c->H + h) * c->maxSeq + s) * c->D;
+}
+static inline float *kv_scale(const orc_kv_t *c, int b, int h) { return c->scales + ((int64_t)b * c->H + h) * c->maxSeq; }
+
+/* storeKVCache(cacheHead, kv, past, inputSeqLen, headSize, kvStride), attention_kernels.h:57-69 */
+static void kv_store_rows(const orc_kv_t *c, int b, int h, const float *src, int past, int n, int kvStride) {
+    for (int i = 0; i < n; ++i) {
+        const float *row = src + (int64_t)i * kvStride;
+        if (c->is_int8) {
+            orc_kv_quantize_row((int8_t *)c->data + kv_off(c, b, h, past + i), kv_scale(c, b, h) + past + i, row,
+                    c->D);
+        } else {
+            uint16_t *d = (uint16_t *)c->data + kv_off(c, b, h, past + i);
+            for (int j = 0; j < c->D; ++j) d[j] = orc_f32_to_fp16(row[j]);
+        }
+    }
+}
+
+/* Store `n` new tokens of every kv head of batch row b.  kv: [n][kvStride], head h at column h*D. */
+ORC_API void orc_kv_store(int is_int8, int B, int H, int maxSeq, int D, void *data, float *scales, int b, int past,
+        int n, const float *kv, int kvStride) {
+    orc_kv_t c = {is_int8, B, H, maxSeq, D, data, scales};
+    for (int h = 0; h < H; ++h) kv_store_rows(&c, b, h, kv + h * D, past, n, kvStride);
+}
+
+/* ------------------------------------------------------------------------- */
+/* small GEMMs of attention                                                   */
+/* ------------------------------------------------------------------------- */
+static inline float kv_elem(const orc_kv_t *c, int64_t off) {
+    return c->is_int8 ? (float)((const int8_t *)c->data)[off] : orc_fp16_to_f32(((const uint16_t *)c->data)[off]);
+}
+
+/* small_gemm_transb (gemm_kernel_ext.cpp:30-85): 16 lanes of fmadd over K, then reduce_add;
+ * INT8 B: multiply by bScale[n] afterwards (:471-500).  One dot product. */
+static inline float dot_lanes_cache(const float *a, const orc_kv_t *c, int64_t off, int K) {
+    float lanes[16];
+    for (int l = 0; l < 16; ++l) lanes[l] = 0.0f;
+    for (int k = 0; k < K; ++k) lanes[k & 15] = fmaf(a[k], kv_elem(c, off + k), lanes[k & 15]);
+    return reduce_add16(lanes);
+}
+static inline float dot_lanes_f32(const float *a, const float *b, int K) {
+    float lanes[16];
+    for (int l = 0; l < 16; ++l) lanes[l] = 0.0f;
+    for (int k = 0; k < K; ++k) lanes[k & 15] = fmaf(a[k], b[k], lanes[k & 15]);
+    return reduce_add16(lanes);
+}
+
+ORC_API void orc_small_gemm_transb_f32(const float *A, const float *B, float *C, int M, int N, int K, int lda,
+        int ldb, int ldc) {
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n)
+            C[(int64_t)m * ldc + n] = dot_lanes_f32(A + (int64_t)m * lda, B + (int64_t)n * ldb, K);
+}
+
+/* xft::small_gemm (gemm_kernel_ext3.cpp:50-214; INT8 gemm_kernel_ext2.cpp:49-255):
+ * C[m,:] (+)= sum_k A[m,k] * B[k,:], k sequential, one fmadd per k; INT8 rows are
+ * multiplied by bScale[k] first. B is fp32 here. */
+ORC_API void orc_small_gemm_f32(const float *A, const float *B, float *C, int M, int N, int K, int lda, int ldb,
+        int ldc, int acc) {
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) {
+            float v = 0.0f;
+            for (int k = 0; k < K; ++k) v = fmaf(A[(int64_t)m * lda + k], B[(int64_t)k * ldb + n], v);
+            if (acc) v = C[(int64_t)m * ldc + n] + v;
+            C[(int64_t)m * ldc + n] = v;
+        }
+}
+ORC_API void orc_small_gemm_f16(const float *A, const uint16_t *B, float *C, int M, int N, int K, int lda, int ldb,
+        int ldc, int acc) {
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) {
+            float v = 0.0f;
+            for (int k = 0; k < K; ++k)
+                v = fmaf(A[(int64_t)m * lda + k], orc_fp16_to_f32(B[(int64_t)k * ldb + n]), v);
+            if (acc) v = C[(int64_t)m * ldc + n] + v;
+            C[(int64_t)m * ldc + n] = v;
+        }
+}
+
+/* P*V against the cache: rows [t0, t0+K) of head (b,h). out[m][D]. */
+static void pv_cache(const float *P, int ldp, const orc_kv_t *c, int b, int h, int t0, int K, float *out, int ldo,
+        int M) {
+    const float *sc = c->is_int8 ? kv_scale(c, b, h) : NULL;
+    for (int m = 0; m < M; ++m)
+        for (int d = 0; d < c->D; ++d) {
+            float v = 0.0f;
+            for (int k = 0; k < K; ++k) {
+                float e = kv_elem(c, kv_off(c, b, h, t0 + k) + d);
+                if (sc) e = e * sc[t0 + k];
+                v = fmaf(P[(int64_t)m * ldp + k], e, v);
+            }
+            out[(int64_t)m * ldo + d] = v;
+        }
+}
+
+/* ------------------------------------------------------------------------- */
+/* softmax                                                                    */
+/* ------------------------------------------------------------------------- */
+/* small_softmax_f32(data, scale, n) lives in xDNN (PARITY UNPINNED); restated in the
+ * form of the in-tree DecoderUtil::computeSoftmax (decoder_util.h:249-296) with no mask:
+ * max over x*scale, vexp(x*scale - max), 16-lane sum, multiply by 1/sum. */
+ORC_API void orc_softmax_scaled(float *data, float scale, int n) {
+    float mx = -FLT_MAX;
+    for (int i = 0; i < n; ++i) mx = fmaxf(mx, data[i] * scale);
+    float lanes[16];
+    for (int l = 0; l < 16; ++l) lanes[l] = 0.0f;
+    for (int i = 0; i < n; ++i) {
+        float e = orc_vexp(data[i] * scale - mx);
+        data[i] = e;
+        lanes[i & 15] += e;
+    }
+    float r = 1.0f / reduce_add16(lanes);
+    for (int i = 0; i < n; ++i) data[i] = data[i] * r;
+}
+
+/* DecoderUtil::softmaxWithStats (decoder_util.h:445-491); mask may be NULL (= zeros).
+ * Returns max and sum through pointers. */
+ORC_API void orc_softmax_with_stats(float *data, const float *mask, int n, float scale, float *outMax,
+        float *outSum) {
+    float mx = -FLT_MAX;
+    for (int i = 0; i < n; ++i) mx = fmaxf(mx, data[i] * scale + (mask ? mask[i] : 0.0f));
+    float lanes[16];
+    for (int l = 0; l < 16; ++l) lanes[l] = 0.0f;
+    for (int i = 0; i < n; ++i) {
+        float e = orc_vexp(data[i] * scale + (mask ? mask[i] : 0.0f) - mx);
+        data[i] = e;
+        lanes[i & 15] += e;
+    }
+    float sum = reduce_add16(lanes);
+    float r = 1.0f / sum;
+    for (int i = 0; i < n; ++i) data[i] = data[i] * r;
+    *outMax = mx;
+    *outSum = sum;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Decode / chunked-prefill attention over the cache                          */
+/* crossAttnByHead, attention_kernels.h:1015-1123                              */
+/* ------------------------------------------------------------------------- */
+/* query/key/value/output are fp32 token-major; token rows of batch b start at
+ * inputOffsets[b]; head h at column h*D.  The first head of every GQA group stores
+ * the new K/V rows into the cache and attends over the cache alone; the other
+ * heads of the group read the past from the cache and the new rows from key/value
+ * (unrounded), exactly as the reference does to avoid a barrier. */
+ORC_API void orc_cross_attn_by_head(float *output, const float *query, const float *key, const float *value,
+        int qHeadNum, int kvHeadNum, int D, int oStride, int qStride, int kvStride, int B, const int *inputSeqLens,
+        const int *pastSeqLens, float scale, int kvInt8, int cacheB, int maxSeq, void *kData, float *kScales,
+        void *vData, float *vScales) {
+    orc_kv_t kc = {kvInt8, cacheB, kvHeadNum, maxSeq, D, kData, kScales};
+    orc_kv_t vc = {kvInt8, cacheB, kvHeadNum, maxSeq, D, vData, vScales};
+    int group = qHeadNum / kvHeadNum;
+    int *inOff = (int *)malloc(sizeof(int) * (B + 1));
+    inOff[0] = 0;
+    for (int b = 0; b < B; ++b) inOff[b + 1] = inOff[b] + inputSeqLens[b];
+
+    /* stores first (the reference interleaves them per group leader; the leader's
+     * result only depends on its own group's rows, so the order is equivalent) */
+    for (int b = 0; b < B; ++b)
+        for (int h = 0; h < kvHeadNum; ++h) {
+            kv_store_rows(&kc, b, h, key + (int64_t)inOff[b] * kvStride + h * D, pastSeqLens[b], inputSeqLens[b],
+                    kvStride);
+            kv_store_rows(&vc, b, h, value + (int64_t)inOff[b] * kvStride + h * D, pastSeqLens[b], inputSeqLens[b],
+                    kvStride);
+        }
+
+#pragma omp parallel for collapse(2) schedule(dynamic)
+    for (int b = 0; b < B; ++b)
+        for (int i = 0; i < qHeadNum; ++i) {
+            int kvh = i / group;
+            int leader = (i % group == 0);
+            int qLen = inputSeqLens[b], past = pastSeqLens[b], keyLen = past + qLen;
+            float *S = (float *)malloc(sizeof(float) * (size_t)qLen * keyLen);
+            const float *Q = query + (int64_t)inOff[b] * qStride + i * D;
+            const float *ksc = kvInt8 ? kv_scale(&kc, b, kvh) : NULL;
+            int nCache = leader ? keyLen : past;
+            for (int m = 0; m < qLen; ++m) {
+                for (int n = 0; n < nCache; ++n) {
+                    float v = dot_lanes_cache(Q + (int64_t)m * qStride, &kc, kv_off(&kc, b, kvh, n), D);
+                    if (ksc) v = v * ksc[n];
+                    S[(int64_t)m * keyLen + n] = v;
+                }
+                if (!leader) {
+                    const float *Kn = key + (int64_t)inOff[b] * kvStride + kvh * D;
+                    for (int n = 0; n < qLen; ++n)
+                        S[(int64_t)m * keyLen + past + n]
+                                = dot_lanes_f32(Q + (int64_t)m * qStride, Kn + (int64_t)n * kvStride, D);
+                }
+            }
+            for (int m = 0; m < qLen; ++m) {
+                int elements = past + m + 1;
+                orc_softmax_scaled(S + (int64_t)m * keyLen, scale, elements);
+                for (int n = elements; n < keyLen; ++n) S[(int64_t)m * keyLen + n] = 0.0f;
+            }
+            float *res = output + (int64_t)inOff[b] * oStride + i * D;
+            if (leader) {
+                pv_cache(S, keyLen, &vc, b, kvh, 0, keyLen, res, oStride, qLen);
+            } else {
+                float *tmp = (float *)malloc(sizeof(float) * (size_t)qLen * D);
+                pv_cache(S, keyLen, &vc, b, kvh, 0, past, tmp, D, qLen);
+                const float *Vn = value + (int64_t)inOff[b] * kvStride + kvh * D;
+                /* small_gemm(S + past, V, f32Out, m, D, m, keyLen, kvStride, D, acc=true) */
+                for (int m = 0; m < qLen; ++m)
+                    for (int d = 0; d < D; ++d) {
+                        float v = 0.0f;
+                        for (int k = 0; k < qLen; ++k)
+                            v = fmaf(S[(int64_t)m * keyLen + past + k], Vn[(int64_t)k * kvStride + d], v);
+                        tmp[(int64_t)m * D + d] = tmp[(int64_t)m * D + d] + v;
+                    }
+                for (int m = 0; m < qLen; ++m)
+                    for (int d = 0; d < D; ++d) res[(int64_t)m * oStride + d] = tmp[(int64_t)m * D + d];
+                free(tmp);
+            }
+            free(S);
+        }
+    free(inOff);
+}
+
+/* balance211, attention_kernels.h:798-818 */
+static void balance211(int n, int team, int tid, int *start, int *mine) {
+    if (team <= 1 || n == 0) {
+        *start = 0;
+        *mine = n;
+        return;
+    }
+    int n1 = (n + team - 1) / team, n2 = n1 - 1;
+    int T1 = n - n2 * team;
+    *mine = tid < T1 ? n1 : n2;
+    *start = tid <= T1 ? tid * n1 : T1 * n1 + (tid - T1) * n2;
+}
+
+/* crossAttnShardedHead, attention_kernels.h:838-986.  inputSeqLen == 1 (the only way
+ * the layer calls it, attention.h:986-1003); the cache already holds all
+ * presentSeqLen rows; mask is all-zero for a single new token. */
+ORC_API void orc_cross_attn_sharded_head(float *output, const float *query, int presentSeqLen, int qHeadNum,
+        int kvHeadNum, int D, int oStride, int qStride, int B, float scale, int splits, int kvInt8, int cacheB,
+        int maxSeq, void *kData, float *kScales, void *vData, float *vScales) {
+    orc_kv_t kc = {kvInt8, cacheB, kvHeadNum, maxSeq, D, kData, kScales};
+    orc_kv_t vc = {kvInt8, cacheB, kvHeadNum, maxSeq, D, vData, vScales};
+    int group = qHeadNum / kvHeadNum;
+    int N = presentSeqLen;
+#pragma omp parallel for collapse(2)
+    for (int b = 0; b < B; ++b)
+        for (int i = 0; i < qHeadNum; ++i) {
+            int kvh = i / group;
+            const float *Q = query + (int64_t)b * qStride + i * D;
+            float *smax = (float *)malloc(sizeof(float) * splits * 3);
+            float *ssum = smax + splits, *fac = smax + 2 * splits;
+            float *part = (float *)malloc(sizeof(float) * (size_t)splits * D);
+            float *S = (float *)malloc(sizeof(float) * (size_t)(N + 16));
+            const float *ksc = kvInt8 ? kv_scale(&kc, b, kvh) : NULL;
+            for (int s = 0; s < splits; ++s) {
+                int nOff, n;
+                balance211(N, splits, s, &nOff, &n);
+                for (int j = 0; j < n; ++j) {
+                    float v = dot_lanes_cache(Q, &kc, kv_off(&kc, b, kvh, nOff + j), D);
+                    if (ksc) v = v * ksc[nOff + j];
+                    S[j] = v;
+                }
+                orc_softmax_with_stats(S, NULL, n, scale, &smax[s], &ssum[s]);
+                pv_cache(S, n, &vc, b, kvh, nOff, n, part + (int64_t)s * D, D, 1);
+            }
+            float realMax = smax[0];
+            for (int s = 1; s < splits; ++s)
+                if (smax[s] > realMax) realMax = smax[s];
+            float realSum = 0.0f;
+            for (int s = 0; s < splits; ++s) {
+                fac[s] = expf(smax[s] - realMax);
+                realSum += ssum[s] * fac[s];
+            }
+            float *res = output + (int64_t)b * oStride + i * D;
+            for (int d = 0; d < D; ++d) {
+                float acc = 0.0f;
+                for (int s = 0; s < splits; ++s) {
+                    float f = fac[s] * (ssum[s] / realSum);
+                    acc = acc + part[(int64_t)s * D + d] * f;
+                }
+                res[d] = acc;
+            }
+            free(S);
+            free(part);
+            free(smax);
+        }
+}
+
+/* ------------------------------------------------------------------------- */
+/* Flash-style prefill  (selfScaledDpAttention, attention_kernels.h:1285-1408; */
+/* tiles: decoder_util.h:760-889)                                             */
+/* ------------------------------------------------------------------------- */
+/* query fp32 [tokens, qStride]; key/value already narrowed to bf16 by the caller
+ * (attention.h:1146-1178), given here as bf16 bit patterns with row stride kvStride.
+ * Q is narrowed to bf16 per block (:1359); QK^T and PV are bf16 x bf16 -> fp32
+ * (MKL cblas_gemm_bf16bf16f32, PARITY UNPINNED: fp32 accumulation in k order);
+ * probabilities are narrowed to bf16 in place before PV (decoder_util.h:883-886). */
+ORC_API void orc_flash_prefill(float *output, const float *query, const uint16_t *key, const uint16_t *value,
+        int qHeadNum, int kvHeadNum, int D, int oStride, int qStride, int kvStride, int B, const int *inputSeqLens,
+        const int *pastSeqLens, float scale) {
+    int maxSrc = 0, maxTgt = 0;
+    int *start = (int *)malloc(sizeof(int) * (B + 1));
+    start[0] = 0;
+    for (int b = 0; b < B; ++b) {
+        if (inputSeqLens[b] > maxSrc) maxSrc = inputSeqLens[b];
+        if (inputSeqLens[b] + pastSeqLens[b] > maxTgt) maxTgt = inputSeqLens[b] + pastSeqLens[b];
+        start[b + 1] = start[b] + inputSeqLens[b];
+    }
+    int minBlk = (int)pow(2, (int)log2((maxSrc + 1) / 2));
+    int srcBlk = minBlk < 256 ? minBlk : 256;
+    int tgtBlk = maxTgt < 512 ? maxTgt : 512;
+    int group = qHeadNum / kvHeadNum;
+    int nMBlk = (maxSrc + srcBlk - 1) / srcBlk;
+
+#pragma omp parallel for collapse(3) schedule(dynamic)
+    for (int b = 0; b < B; ++b)
+        for (int h = 0; h < qHeadNum; ++h)
+            for (int mb = 0; mb < nMBlk; ++mb) {
+                int m = mb * srcBlk;
+                int srcLen = inputSeqLens[b], tgtLen = inputSeqLens[b] + pastSeqLens[b];
+                if (m >= srcLen) continue;
+                int qReal = srcBlk < srcLen - m ? srcBlk : srcLen - m;
+                float *q = (float *)malloc(sizeof(float) * (size_t)qReal * D);
+                float *sum = (float *)malloc(sizeof(float) * qReal * 4);
+                float *preSum = sum + qReal, *mx = sum + 2 * qReal, *preMax = sum + 3 * qReal;
+                float *AB = (float *)malloc(sizeof(float) * (size_t)qReal * tgtBlk);
+                float *PV = (float *)malloc(sizeof(float) * (size_t)qReal * D);
+                float *out = output + ((int64_t)start[b] + m) * oStride + h * D;
+                const float *qsrc = query + ((int64_t)start[b] + m) * qStride + h * D;
+                for (int i = 0; i < qReal; ++i)
+                    for (int j = 0; j < D; ++j) {
+                        out[(int64_t)i * oStride + j] = 0.0f;
+                        q[i * D + j] = orc_bf16_to_f32(orc_f32_to_bf16(qsrc[(int64_t)i * qStride + j]));
+                    }
+                for (int i = 0; i < qReal; ++i) {
+                    preSum[i] = 0.0f;
+                    sum[i] = 0.0f;
+                    preMax[i] = -FLT_MAX;
+                    mx[i] = -FLT_MAX;
+                }
+                int kvh = h / group;
+                const uint16_t *k = key + (int64_t)start[b] * kvStride + kvh * D;
+                const uint16_t *v = value + (int64_t)start[b] * kvStride + kvh * D;
+                for (int n = 0; n < tgtLen; n += tgtBlk) {
+                    int kvReal = tgtBlk < tgtLen - n ? tgtBlk : tgtLen - n;
+                    if (m + qReal - 1 < n) break;
+                    /* AB = q * kBlk^T */
+                    for (int i = 0; i < qReal; ++i)
+                        for (int j = 0; j < kvReal; ++j) {
+                            float acc = 0.0f;
+                            const uint16_t *kr = k + (int64_t)(n + j) * kvStride;
+                            for (int d = 0; d < D; ++d) acc += q[i * D + d] * orc_bf16_to_f32(kr[d]);
+                            AB[(int64_t)i * kvReal + j] = acc;
+                        }
+                    /* softmaxTileCausal, decoder_util.h:760-838 (headSlope = 0) */
+                    for (int i = 0; i < qReal; ++i) {
+                        float *buf = AB + (int64_t)i * kvReal;
+                        int kk = m + i + 1 - n;
+                        if (kk < 0) kk = 0;
+                        if (kk > kvReal) kk = kvReal;
+                        float tmax = -FLT_MAX;
+                        for (int j = 0; j < kk; ++j) tmax = fmaxf(tmax, buf[j] * scale);
+                        tmax = tmax > mx[i] ? tmax : mx[i];
+                        float merr = orc_vexp(mx[i] - tmax);
+                        mx[i] = tmax;
+                        float lanes[16];
+                        for (int l = 0; l < 16; ++l) lanes[l] = 0.0f;
+                        for (int j = 0; j < kk; ++j) {
+                            float e = orc_vexp(buf[j] * scale - tmax);
+                            /* stored as bf16 in place, then re-read for the sum?  No: the sum uses
+                             * the fp32 vector, the store narrows (decoder_util.h:813-817). */
+                            lanes[j & 15] += e;
+                            buf[j] = orc_bf16_to_f32(bf16_rne_hw(e));
+                        }
+                        float s = reduce_add16(lanes);
+                        sum[i] = sum[i] * merr + s;
+                        float r = 1.0f / sum[i];
+                        for (int j = 0; j < kk; ++j) buf[j] = orc_bf16_to_f32(bf16_rne_hw(buf[j] * r));
+                        for (int j = kk; j < kvReal; ++j) buf[j] = 0.0f;
+                    }
+                    /* PV = P * vBlk */
+                    for (int i = 0; i < qReal; ++i)
+                        for (int d = 0; d < D; ++d) {
+                            float acc = 0.0f;
+                            for (int j = 0; j < kvReal; ++j)
+                                acc += AB[(int64_t)i * kvReal + j] * orc_bf16_to_f32(v[(int64_t)(n + j) * kvStride + d]);
+                            PV[i * D + d] = acc;
+                        }
+                    /* updateOutTile, decoder_util.h:841-861 */
+                    for (int i = 0; i < qReal; ++i) {
+                        float merr = orc_vexp(preMax[i] - mx[i]);
+                        float fac = preSum[i] / sum[i];
+                        for (int d = 0; d < D; ++d) {
+                            float o = out[(int64_t)i * oStride + d];
+                            out[(int64_t)i * oStride + d] = (o * merr) * fac + PV[i * D + d];
+                        }
+                        preSum[i] = sum[i];
+                        preMax[i] = mx[i];
+                    }
+                }
+                free(q);
+                free(sum);
+                free(AB);
+                free(PV);
+            }
+    free(start);
+}
+
+/* Textbook causal GQA attention in double, the yardstick the reference's own tests use
+ * (tests/ut/attention_kernels_test.cpp:32-83, cross_attention_test.cpp:36-114).
+ * K/V fp32 [B][kvH][keyLen][D] contiguous; Q fp32 [tokens][qStride]. */
+ORC_API void orc_attention_ref_f64(float *output, const float *query, const float *K, const float *V, int qHeadNum,
+        int kvHeadNum, int D, int oStride, int qStride, int B, const int *inputSeqLens, const int *pastSeqLens,
+        int kvSeqStride, float scale) {
+    int group = qHeadNum / kvHeadNum;
+    int *start = (int *)malloc(sizeof(int) * (B + 1));
+    start[0] = 0;
+    for (int b = 0; b < B; ++b) start[b + 1] = start[b] + inputSeqLens[b];
+#pragma omp parallel for collapse(2) schedule(dynamic)
+    for (int b = 0; b < B; ++b)
+        for (int h = 0; h < qHeadNum; ++h) {
+            int kvh = h / group;
+            int past = pastSeqLens[b], qLen = inputSeqLens[b];
+            const float *Kh = K + ((int64_t)b * kvHeadNum + kvh) * kvSeqStride * D;
+            const float *Vh = V + ((int64_t)b * kvHeadNum + kvh) * kvSeqStride * D;
+            double *p = (double *)malloc(sizeof(double) * (past + qLen));
+            for (int m = 0; m < qLen; ++m) {
+                const float *q = query + ((int64_t)start[b] + m) * qStride + h * D;
+                int n = past + m + 1;
+                double mx = -1e300;
+                for (int j = 0; j < n; ++j) {
+                    double acc = 0;
+                    for (int d = 0; d < D; ++d) acc += (double)q[d] * (double)Kh[(int64_t)j * D + d];
+                    p[j] = acc * scale;
+                    if (p[j] > mx) mx = p[j];
+                }
+                double s = 0;
+                for (int j = 0; j < n; ++j) {
+                    p[j] = exp(p[j] - mx);
+                    s += p[j];
+                }
+                float *o = output + ((int64_t)start[b] + m) * oStride + h * D;
+                for (int d = 0; d < D; ++d) {
+                    double acc = 0;
+                    for (int j = 0; j < n; ++j) acc += p[j] * (double)Vh[(int64_t)j * D + d];
+                    o[d] = (float)(acc / s);
+                }
+            }
+            free(p);
+        }
+    free(start);
+}
+
+/* ------------------------------------------------------------------------- */
+/* SwiGLU combine, MoE routing, argmax                                        */
+/* ------------------------------------------------------------------------- */
+/* DecoderUtil::siluSum, decoder_util.h:550-573: src [M, 2N] (gate | up), dst [M, N] */
+ORC_API void orc_silu_sum(const float *src, int lds, float *dst, int ldd, int M, int N) {
+#pragma omp parallel for
+    for (int i = 0; i < M; ++i)
+        for (int j = 0; j < N; ++j) {
+            float left = src[(int64_t)i * lds + j], right = src[(int64_t)i * lds + j + N];
+            float x0 = orc_vexp(left * -1.0f);
+            float x1 = 1.0f + x0;
+            float x2 = left / x1;
+            dst[(int64_t)i * ldd + j] = right * x2;
+        }
+}
+
+/* MixtralMLP::selectTop2Experts, mlp_mixtral.h:221-283.  Strict '>' so the lower index
+ * wins ties.  Groups of 8 tokens share one max (the max over all 16 selected logits) and
+ * use vexp; the tail uses std::exp with the per-token max. */
+ORC_API void orc_moe_top2(const float *logits, int M, int N, int *sel, float *w) {
+    for (int i = 0; i < M; ++i) {
+        float max1 = -INFINITY, max2 = -INFINITY;
+        int idx1 = -1, idx2 = -1;
+        for (int j = 0; j < N; ++j) {
+            float val = logits[(int64_t)i * N + j];
+            if (val > max1) {
+                max2 = max1; idx2 = idx1; max1 = val; idx1 = j;
+            } else if (val > max2) {
+                max2 = val; idx2 = j;
+            }
+        }
+        sel[2 * i] = idx1; sel[2 * i + 1] = idx2;
+        w[2 * i] = max1; w[2 * i + 1] = max2;
+    }
+    int i = 0;
+    for (; i + 7 < M; i += 8) {
+        float mx = w[2 * i];
+        for (int t = 1; t < 16; ++t) mx = fmaxf(mx, w[2 * i + t]);
+        for (int t = 0; t < 8; ++t) {
+            float e1 = orc_vexp(w[2 * (i + t)] - mx), e2 = orc_vexp(w[2 * (i + t) + 1] - mx);
+            float s = e1 + e2;
+            w[2 * (i + t)] = e1 / s;
+            w[2 * (i + t) + 1] = e2 / s;
+        }
+    }
+    for (; i < M; ++i) {
+        float mx = fmaxf(w[2 * i], w[2 * i + 1]);
+        float e1 = expf(w[2 * i] - mx), e2 = expf(w[2 * i + 1] - mx);
+        w[2 * i] = e1 / (e1 + e2);
+        w[2 * i + 1] = e2 / (e1 + e2);
+    }
+}
+
+/* xft::addto used by scatterOutput (mlp_mixtral.h:211-218, add_util.h): dst += src * scale (fmadd) */
+ORC_API void orc_scatter_add(float *out, int oStride, const float *expertOut, int hidden, const int *idx,
+        const float *weights, int rows) {
+    for (int i = 0; i < rows; ++i)
+        for (int j = 0; j < hidden; ++j)
+            out[(int64_t)idx[i] * oStride + j]
+                    = fmaf(expertOut[(int64_t)i * hidden + j], weights[i], out[(int64_t)idx[i] * oStride + j]);
+}
+
+/* greedySearch, src/searchers/sampling.cpp:22-131: first maximum wins (strict '>'). */
+ORC_API void orc_argmax(const float *logits, int B, int V, int *ids) {
+    for (int b = 0; b < B; ++b) {
+        const float *p = logits + (int64_t)b * V;
+        int best = 0;
+        float bv = p[0];
+        for (int j = 1; j < V; ++j)
+            if (p[j] > bv) { bv = p[j]; best = j; }
+        ids[b] = best;
+    }
+}
+
+ORC_API int orc_num_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}

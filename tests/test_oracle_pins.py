@@ -1,0 +1,430 @@
+"""Pins the CPU oracle: against the reference's own in-tree kernels compiled as they lie
+(oracle/_ref, when the reference tree and an AVX-512 host are there), against the golden
+constants the reference's unit tests hold, and against closed forms in float64."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import pyoracle as orc
+
+REF = orc.load_ref()
+needs_ref = pytest.mark.skipif(REF is None, reason="oracle/_ref not built or host lacks AVX-512")
+P = orc.p
+
+
+def _specials():
+    return np.array([0.0, -0.0, 1e-45, -1e-45, 1e-39, 1.1754942e-38, 1.17549435e-38, np.inf, -np.inf, 1.0,
+                     1.00390625, 1.01171875, 3.3895314e38, 65504.0, 65520.0, 65519.996, 6.1035156e-05, 5.9604645e-08,
+                     2.9802322e-08, 2.9802325e-08, 8.9406967e-08, 1e-7, 0.33333334, -2.5, 127.5, 128.5], np.float32)
+
+
+def _rand(n, seed, scale=1.0):
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal(n) * scale).astype(np.float32)
+    return x
+
+
+# ------------------------------------------------------------------ conversions
+@needs_ref
+def test_bf16_scalar_matches_reference_class():
+    REF.ref_f32_to_bf16.restype = C.c_uint16
+    REF.ref_f32_to_bf16.argtypes = [C.c_float]
+    xs = np.concatenate([_specials(), _rand(20000, 1), _rand(2000, 2, 1e-38), _rand(2000, 3, 1e30)])
+    bits = np.random.default_rng(5).integers(0, 2**32, 20000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    xs = np.concatenate([xs, bits])
+    got = orc.to_bf16(xs)
+    exp = np.array([REF.ref_f32_to_bf16(float(v)) if not np.isnan(v) else 0 for v in xs], np.uint16)
+    ok = ~np.isnan(xs)
+    assert np.array_equal(got[ok], exp[ok])
+    # NaN: payload top half kept, quiet bit 6 set (include/bfloat16.h:49-52)
+    nan_bits = np.array([0x7FC00000, 0x7F800001, 0xFFC12345], np.uint32).view(np.float32)
+    for v, b in zip(nan_bits, nan_bits.view(np.uint32)):
+        assert orc.lib.orc_f32_to_bf16(C.c_float(v)) in ((b >> 16) | 0x40, ((b >> 16) | 0x40) | 0x0040)
+
+
+def test_bf16_is_rne_on_normals():
+    import torch
+    x = _rand(50000, 7, 3.0)
+    exp = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(orc.to_bf16(x), exp)
+    # subnormal inputs flush to signed zero
+    assert orc.lib.orc_f32_to_bf16(C.c_float(1e-39)) == 0
+    assert orc.lib.orc_f32_to_bf16(C.c_float(-1e-39)) == 0x8000
+
+
+@needs_ref
+def test_bf16_vector_store_matches_instruction():
+    xs = np.concatenate([_specials(), _rand(4096, 11), _rand(512, 12, 1e-38)]).astype(np.float32)
+    xs = xs[~np.isnan(xs)]
+    out = np.zeros(xs.size, np.uint16)
+    REF.ref_store_bf16(P(xs), P(out), xs.size)
+    got = np.array([orc.lib.orc_f32_to_bf16_hw(C.c_float(v)) for v in xs], np.uint16)
+    assert np.array_equal(got, out)
+
+
+def test_fp16_matches_ieee():
+    xs = np.concatenate([_specials(), _rand(50000, 21), _rand(5000, 22, 1e-5), _rand(5000, 23, 1e-7),
+                         _rand(5000, 24, 3e4)])
+    exp = xs.astype(np.float16).view(np.uint16)
+    assert np.array_equal(orc.to_fp16(xs), exp)
+    allh = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    back = orc.from_fp16(allh)
+    expb = allh.view(np.float16).astype(np.float32)
+    ok = ~np.isnan(expb)
+    assert np.array_equal(back[ok], expb[ok])
+
+
+@needs_ref
+def test_fp16_matches_reference_store_and_load():
+    xs = np.concatenate([_specials(), _rand(8192, 31, 5.0)])
+    out = np.zeros(xs.size, np.uint16)
+    REF.ref_store_fp16(P(xs), P(out), xs.size)
+    assert np.array_equal(orc.to_fp16(xs), out)
+    back = np.zeros(xs.size, np.float32)
+    REF.ref_load_fp16(P(out), P(back), xs.size)
+    assert np.array_equal(orc.from_fp16(out), back)
+
+
+# ------------------------------------------------------------------ vexp
+@needs_ref
+def test_vexp_bit_exact_vs_reference():
+    xs = np.concatenate([_rand(40000, 41, 10.0), np.linspace(-100, 100, 4001).astype(np.float32),
+                         np.array([0.0, -0.0, 88.376, -88.376, 89.0, -89.0], np.float32)])
+    out = np.zeros_like(xs)
+    REF.ref_vexp(P(xs), P(out), xs.size)
+    assert np.array_equal(orc.vexp(xs).view(np.uint32), out.view(np.uint32))
+
+
+def test_vexp_close_to_exp():
+    xs = np.linspace(-80, 80, 20001).astype(np.float32)
+    rel = np.abs(orc.vexp(xs) / np.exp(xs.astype(np.float64)) - 1)
+    assert rel.max() < 3e-7
+
+
+# ------------------------------------------------------------------ INT8 KV quantisation
+def test_kv_quantize_ramp_known_answer():
+    # a 128-element ramp: absmax 9.1429 -> scale absmax/127, first -127, last 125
+    x = (np.arange(128, dtype=np.float32) - 64.0) / 7.0
+    q, s = orc.kv_quantize_row(x)
+    assert q[0] == -127 and q[127] == 125
+    assert abs(s - 0.071991) < 1e-6
+    q0, s0 = orc.kv_quantize_row(np.zeros(128, np.float32))
+    assert s0 == 0 and not q0.any()
+
+
+@needs_ref
+def test_kv_quantize_bit_exact_vs_reference():
+    rng = np.random.default_rng(51)
+    for size in (128, 256, 64, 80):
+        for trial in range(50):
+            x = (rng.standard_normal(size) * rng.uniform(0.01, 30)).astype(np.float32)
+            q, s = orc.kv_quantize_row(x)
+            rq = np.zeros(size, np.int8)
+            rs = np.zeros(1, np.float32)
+            REF.ref_kv_quantize(P(rq), P(rs), P(x), size)
+            assert np.array_equal(q, rq) and np.float32(s).tobytes() == rs[0].tobytes()
+
+
+def test_kv_quantize_closed_form():
+    x = _rand(128, 52, 4.0)
+    q, s = orc.kv_quantize_row(x)
+    amax = np.abs(x).max()
+    assert s == np.float32(amax / np.float32(127.0))
+    assert np.abs(q.astype(np.float64) * s - x).max() <= s * 0.5 * (1 + 1e-5)
+    assert np.abs(q).max() == 127
+
+
+# ------------------------------------------------------------------ RoPE
+def test_rope_golden_constants_of_reference_test():
+    # tests/ut/rotary_embedding_test.cpp:28-57
+    bs, seq, heads, dim = 2, 2, 2, 2
+    q = np.array([4, 4, 4, 4, 3, 2, 1, 1, 4, 4, 2, 1, 4, 1, 3, 0], np.float32)
+    k = np.ones(16, np.float32)
+    qg = np.array([-1.20467, 5.52709, -1.20467, 5.52709, 3, 2, 1, 1, -1.20467, 5.52709, 0.239134, 2.22324, 4, 1, 3, 0])
+    kg = np.array([-0.301169, 1.38177, -0.301169, 1.38177, 1, 1, 1, 1, -0.301169, 1.38177, -0.301169, 1.38177, 1, 1,
+                   1, 1])
+    cos, sin = orc.rope_tables(dim, 10)
+    q1, k1 = q.copy(), k.copy()
+    orc.rope_apply(q1, k1, bs * seq, bs * seq, cos, sin, (bs, seq, heads, dim, heads), [1, 0])
+    assert np.abs(q1 - qg).max() < 1e-3 and np.abs(k1 - kg).max() < 1e-3
+    q2, k2 = q.copy(), k.copy()
+    orc.rope_apply_tokens(q2, k2, cos, sin, bs * seq, bs * seq, dim, bs * seq, heads, heads, [1, 0, 1, 0])
+    assert np.abs(q2 - qg).max() < 1e-3 and np.abs(k2 - kg).max() < 1e-3
+
+
+@needs_ref
+def test_rope_bit_exact_vs_reference_kernel():
+    dim, max_pos, qh, kh = 128, 512, 8, 2
+    cos, sin = orc.rope_tables(dim, max_pos)
+    half = dim // 2
+    inv = np.array([np.float32(1.0 / np.power(float(10000), float(np.float32(2 * i) / np.float32(dim))))
+                    for i in range(half)], np.float32)
+    rc, rs = np.zeros_like(cos), np.zeros_like(sin)
+    REF.ref_rope_tables(P(inv), P(rc), P(rs), half, max_pos)
+    assert np.array_equal(cos, rc) and np.array_equal(sin, rs)
+    rng = np.random.default_rng(61)
+    B, S = 2, 7
+    qkv = rng.standard_normal((B * S, (qh + 2 * kh) * dim)).astype(np.float32)
+    stride = qkv.shape[1]
+    pos = rng.integers(0, max_pos, S).astype(np.int32)
+    shape = np.array([B, S, qh, dim, kh], np.int32)
+    a, b = qkv.copy(), qkv.copy()
+    orc.lib.orc_rope_apply(C.c_void_p(a.ctypes.data), C.c_void_p(a.ctypes.data + qh * dim * 4), stride, stride,
+                           P(cos), P(sin), half, P(shape), P(pos))
+    REF.ref_rope_apply_f32(C.c_void_p(b.ctypes.data), C.c_void_p(b.ctypes.data + qh * dim * 4), stride, stride,
+                           P(rc), P(rs), half, P(shape), P(pos))
+    assert np.array_equal(a, b)
+    assert not np.array_equal(a, qkv)
+    pos_t = rng.integers(0, max_pos, B * S).astype(np.int32)
+    a, b = qkv.copy(), qkv.copy()
+    orc.lib.orc_rope_apply_tokens(C.c_void_p(a.ctypes.data), C.c_void_p(a.ctypes.data + qh * dim * 4), P(cos),
+                                  P(sin), stride, stride, dim, B * S, qh, kh, P(pos_t))
+    REF.ref_rope_apply_tokens_f32(C.c_void_p(b.ctypes.data), C.c_void_p(b.ctypes.data + qh * dim * 4), P(rc), P(rs),
+                                  stride, stride, dim, B * S, qh, kh, P(pos_t))
+    assert np.array_equal(a, b)
+
+
+def test_rope_is_a_rotation():
+    dim = 128
+    cos, sin = orc.rope_tables(dim, 64)
+    x = _rand(dim, 62)
+    q, k = x.copy(), x.copy()
+    orc.rope_apply_tokens(q, k, cos, sin, dim, dim, dim, 1, 1, 1, [37])
+    assert abs(np.linalg.norm(q) - np.linalg.norm(x)) < 1e-4
+    th = 37.0 * 10000.0 ** (-np.arange(64) * 2.0 / dim)
+    exp = np.concatenate([x[:64] * np.cos(th) - x[64:] * np.sin(th), x[64:] * np.cos(th) + x[:64] * np.sin(th)])
+    assert np.abs(q - exp).max() < 2e-4
+
+
+# ------------------------------------------------------------------ P*V small gemm
+@needs_ref
+def test_small_gemm_bit_exact_vs_reference():
+    rng = np.random.default_rng(71)
+    for (M, N, K) in ((1, 128, 300), (4, 128, 64), (3, 256, 77), (6, 128, 1000)):
+        A = rng.standard_normal((M, K)).astype(np.float32)
+        B = rng.standard_normal((K, N)).astype(np.float32)
+        c0, c1 = np.zeros((M, N), np.float32), np.zeros((M, N), np.float32)
+        orc.lib.orc_small_gemm_f32(P(A), P(B), P(c0), M, N, K, K, N, N, 0)
+        REF.ref_small_gemm_f32(P(A), P(B), P(c1), M, N, K, K, N, N, 0)
+        assert np.array_equal(c0, c1)
+        Bh = orc.to_fp16(B)
+        orc.lib.orc_small_gemm_f16(P(A), P(Bh), P(c0), M, N, K, K, N, N, 1)
+        REF.ref_small_gemm_f16(P(A), P(Bh), P(c1), M, N, K, K, N, N, 1)
+        assert np.array_equal(c0, c1)
+
+
+# ------------------------------------------------------------------ weight formats
+@needs_ref
+def test_uint4_nibble_order_vs_reference_type():
+    packed = np.arange(256, dtype=np.uint8)
+    v1, v2 = np.zeros(256, np.uint8), np.zeros(256, np.uint8)
+    REF.ref_uint4x2_unpack(P(packed), P(v1), P(v2), 256)
+    assert np.array_equal(v1, packed & 15) and np.array_equal(v2, packed >> 4)
+    REF.ref_uint4x2_pack.restype = C.c_uint8
+    assert REF.ref_uint4x2_pack(C.c_uint8(3), C.c_uint8(12)) == 3 | (12 << 4)
+
+
+def test_dequant_convention():
+    rng = np.random.default_rng(81)
+    K, N = 64, 48
+    q8 = rng.integers(-128, 128, (K, N)).astype(np.int8)
+    scale = rng.uniform(1e-3, 1e-2, N).astype(np.float32)
+    zero = rng.uniform(-0.1, 0.1, N).astype(np.float32)
+    w = orc.QWeight(orc.W_INT8, K, N, q8, scale, zero)
+    d = orc.dequant(w)
+    exact = scale.astype(np.float64) * q8 + zero.astype(np.float64)
+    assert np.array_equal(d, exact.astype(np.float32))  # single rounding == fused multiply-add
+    wsym = orc.QWeight(orc.W_INT8, K, N, q8, scale, np.zeros(N, np.float32))
+    assert np.array_equal(orc.dequant(wsym), scale[None, :] * q8.astype(np.float32))
+    # GPTQ repack rule (tools/llama_convert.py:351-394): u8 - 128 with zero' = -scale*(qzero - 128)
+    u4 = rng.integers(0, 16, (K, N)).astype(np.uint8)
+    packed = (u4[:, 0::2] | (u4[:, 1::2] << 4)).astype(np.uint8)
+    w4 = orc.QWeight(orc.W_UINT4, K, N, packed, scale, zero)
+    exact4 = scale.astype(np.float64) * u4 + zero.astype(np.float64)
+    assert np.array_equal(orc.dequant(w4), exact4.astype(np.float32))
+    wn = orc.QWeight(orc.W_NF4, K, N, packed, scale, None)
+    assert np.array_equal(orc.dequant(wn), orc.nf4_codebook()[u4] * scale[None, :])
+    # bf16 narrowing of the dequantised value (matmul_helper.h:317-346)
+    assert np.array_equal(orc.dequant_bf16(w4), orc.to_bf16(orc.dequant(w4)))
+
+
+def test_quantizers_invariants():
+    rng = np.random.default_rng(82)
+    W = (rng.standard_normal((256, 64)) * 0.02).astype(np.float32)
+    w8 = orc.quantize(orc.W_INT8, W)
+    assert np.abs(w8.q).max() == 127 and not w8.zero.any()
+    assert np.allclose(w8.scale, np.abs(W).max(0) / 127, rtol=1e-6)
+    assert (np.abs(orc.dequant(w8) - W) <= w8.scale[None, :] * 0.5001).all()
+    w4 = orc.quantize(orc.W_UINT4, W)
+    assert np.allclose(w4.zero, W.min(0)) and np.allclose(w4.scale, (W.max(0) - W.min(0)) / 15, rtol=1e-6)
+    assert (np.abs(orc.dequant(w4) - W) <= w4.scale[None, :] * 0.5001).all()
+    wn = orc.quantize(orc.W_NF4, W)
+    code = orc.nf4_codebook()
+    u = np.zeros(W.shape, np.uint8)
+    u[:, 0::2], u[:, 1::2] = wn.q & 15, wn.q >> 4
+    brute = np.abs((W / np.abs(W).max(0))[..., None] - code).argmin(-1)
+    assert np.array_equal(u, brute)
+    assert len(code) == 16 and code[0] == -1 and code[7] == 0 and code[15] == 1 and (np.diff(code) > 0).all()
+
+
+def test_qgemm_closed_form():
+    rng = np.random.default_rng(83)
+    M, K, N = 5, 512, 96
+    W = (rng.standard_normal((K, N)) * 0.02).astype(np.float32)
+    A = orc.round_bf16(rng.standard_normal((M, K)))
+    bias = rng.standard_normal(N).astype(np.float32)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    for kind in (orc.W_INT8, orc.W_UINT4, orc.W_NF4):
+        w = orc.quantize(kind, W)
+        exact = A.astype(np.float64) @ orc.dequant(w).astype(np.float64)
+        assert np.abs(orc.qgemm(w, A, f64=True) - exact).max() < 1e-5
+        assert np.abs(orc.qgemm(w, A) - exact).max() < 1e-4
+        assert np.abs(orc.qgemm(w, A, orc.EPI_BIAS, bias=bias) - (exact + bias)).max() < 1e-4
+        assert np.abs(orc.qgemm(w, A, orc.EPI_RESIDENTIAL, res=res) - (exact + res)).max() < 1e-4
+        assert np.abs(orc.qgemm(w, A, orc.EPI_RESIDENTIAL, bias=bias, res=res) - (exact + res + bias)).max() < 1e-4
+        assert np.abs(orc.qgemm(w, A, orc.EPI_RESMUL, res=res) - (exact * res)).max() < 1e-4
+        assert np.abs(orc.qgemm(w, A, orc.EPI_RESEXT, res=res, gamma=0.5) - (exact + 0.5 * res)).max() < 1e-4
+        sil = exact / (1 + np.exp(-exact))
+        assert np.abs(orc.qgemm(w, A, orc.EPI_SILU) - sil).max() < 1e-4
+        # a transposed operand or a dropped zero-point would miss by O(1)
+        assert np.abs(exact).max() > 0.1
+
+
+def test_w8a8_closed_form():
+    rng = np.random.default_rng(84)
+    M, K, N = 7, 384, 64
+    A = rng.standard_normal((M, K)).astype(np.float32) + 0.3
+    W = (rng.standard_normal((K, N)) * 0.02).astype(np.float32)
+    w = orc.quantize(orc.W_W8A8, W)
+    assert np.array_equal(w.colsum, w.q.astype(np.int64).sum(0).astype(np.float32))
+    qa, s, z, sm = orc.w8a8_quantize_rows(A)
+    assert np.allclose(z, (A.min(1) + A.max(1)) / 2)
+    assert np.allclose(s, (A.max(1) - A.min(1)) / 2 / 127, rtol=1e-5)
+    deqA = qa.astype(np.float64) * s[:, None] + z[:, None]
+    assert (np.abs(deqA - A) <= s[:, None] * 0.5001).all()
+    assert np.allclose(sm, deqA.sum(1), rtol=1e-5, atol=1e-4)
+    exact = deqA @ (w.q.astype(np.float64) * w.scale + w.zero)
+    got = orc.qgemm(w, A)
+    assert np.abs(got - exact).max() < 2e-4
+    assert np.abs(got - A.astype(np.float64) @ W).max() < 0.05
+
+
+# ------------------------------------------------------------------ norm / softmax
+def test_rmsnorm_closed_form():
+    rng = np.random.default_rng(91)
+    for cols in (4096, 100, 17):
+        x = rng.standard_normal((6, cols)).astype(np.float32)
+        w = rng.uniform(0.5, 1.5, cols).astype(np.float32)
+        exp = x / np.sqrt((x.astype(np.float64) ** 2).mean(1, keepdims=True) + 1e-6) * w
+        assert np.abs(orc.rmsnorm(x, w) - exp).max() < 2e-6 * np.abs(exp).max() + 1e-6
+
+
+def test_softmax_closed_form():
+    x = _rand(1000, 92, 3.0)
+    s = orc.softmax_scaled(x, 0.25)
+    e = np.exp((x.astype(np.float64) - x.max()) * 0.25)
+    assert np.abs(s - e / e.sum()).max() < 1e-6
+    assert abs(s.sum() - 1) < 1e-5
+
+
+# ------------------------------------------------------------------ attention
+def _fill_cache(rng, int8, B, H, S, D, n):
+    kc, vc = orc.KVCache(int8, B, H, S, D), orc.KVCache(int8, B, H, S, D)
+    for b in range(B):
+        kc.store(b, 0, rng.standard_normal((n, H * D)).astype(np.float32))
+        vc.store(b, 0, rng.standard_normal((n, H * D)).astype(np.float32))
+    return kc, vc
+
+
+@pytest.mark.parametrize("int8", [0, 1])
+@pytest.mark.parametrize("qh,kvh,D", [(32, 8, 128), (32, 32, 128), (2, 1, 256)])
+def test_cross_attn_by_head_vs_textbook(int8, qh, kvh, D):
+    # shapes of tests/ut/cross_attention_test.cpp:276-296
+    rng = np.random.default_rng(101)
+    B, past, S = 2, 37, 64
+    kc, vc = _fill_cache(rng, int8, B, kvh, S, D, past)
+    for step, n_new in enumerate((1, 3)):
+        q = orc.round_bf16(rng.standard_normal((B * n_new, qh * D)))
+        k = rng.standard_normal((B * n_new, kvh * D)).astype(np.float32)
+        v = rng.standard_normal((B * n_new, kvh * D)).astype(np.float32)
+        out = orc.cross_attn_by_head(q, k, v, qh, kvh, D, [n_new] * B, [past] * B, 1 / np.sqrt(D), kc, vc)
+        ref = orc.attention_ref_f64(q, kc.as_f32(), vc.as_f32(), qh, kvh, D, [n_new] * B, [past] * B, 1 / np.sqrt(D))
+        # group leaders read the rounded cache, the others the unrounded new rows
+        tol = 3e-2 if int8 else 3e-3
+        assert np.abs(out - ref).max() < tol
+        lead = np.concatenate([np.arange(D) + h * D for h in range(0, qh, qh // kvh)])
+        assert np.abs(out[:, lead] - ref[:, lead]).max() < 1e-4
+        past += n_new
+
+
+@pytest.mark.parametrize("int8", [0, 1])
+def test_sharded_head_matches_and_is_split_independent(int8):
+    # tests/ut/cross_attention_test.cpp:116-182: past up to 1000, 32q/8kv, 64 threads -> 2 splits
+    rng = np.random.default_rng(102)
+    B, qh, kvh, D, present = 1, 32, 8, 128, 1000
+    kc, vc = _fill_cache(rng, int8, B, kvh, 1024, D, present)
+    q = orc.round_bf16(rng.standard_normal((B, qh * D)))
+    ref = orc.attention_ref_f64(q, kc.as_f32(), vc.as_f32(), qh, kvh, D, [1], [present - 1], 1 / np.sqrt(D))
+    outs = [orc.cross_attn_sharded_head(q, present, qh, kvh, D, 1 / np.sqrt(D), s, kc, vc) for s in (2, 3, 7, 16)]
+    for o in outs:
+        assert np.abs(o - ref).max() < 1e-4
+    assert np.abs(outs[0] - outs[3]).max() < 1e-5
+
+
+@pytest.mark.parametrize("qh,kvh", [(2, 2), (6, 2), (8, 2)])
+@pytest.mark.parametrize("lens", [[80], [100], [100, 200], [100, 101, 102]])
+def test_flash_prefill_vs_textbook(qh, kvh, lens):
+    # cases of tests/ut/attention_kernels_test.cpp:484-540 (tolerance 1e-2 there)
+    rng = np.random.default_rng(103)
+    D = 128
+    T = sum(lens)
+    q = orc.round_bf16(rng.standard_normal((T, qh * D)))
+    k = orc.round_bf16(rng.standard_normal((T, kvh * D)))
+    v = orc.round_bf16(rng.standard_normal((T, kvh * D)))
+    out = orc.flash_prefill(q, orc.to_bf16(k), orc.to_bf16(v), qh, kvh, D, lens, [0] * len(lens), 1 / np.sqrt(D))
+    S = max(lens)
+    K4 = np.zeros((len(lens), kvh, S, D), np.float32)
+    V4 = np.zeros_like(K4)
+    off = 0
+    for b, n in enumerate(lens):
+        K4[b, :, :n] = k[off:off + n].reshape(n, kvh, D).transpose(1, 0, 2)
+        V4[b, :, :n] = v[off:off + n].reshape(n, kvh, D).transpose(1, 0, 2)
+        off += n
+    ref = orc.attention_ref_f64(q, K4, V4, qh, kvh, D, lens, [0] * len(lens), 1 / np.sqrt(D))
+    assert np.abs(out - ref).max() < 1e-2
+    # first token of every sequence attends only to itself: output == its V row
+    off = 0
+    for n in lens:
+        for h in range(qh):
+            assert np.abs(out[off, h * D:(h + 1) * D] - v[off, (h // (qh // kvh)) * D:(h // (qh // kvh) + 1) * D]).max() < 1e-2
+        off += n
+
+
+# ------------------------------------------------------------------ SwiGLU, routing, argmax
+def test_silu_sum_closed_form():
+    x = _rand(6 * 64, 111, 2.0).reshape(6, 64)
+    g, u = x[:, :32].astype(np.float64), x[:, 32:].astype(np.float64)
+    assert np.abs(orc.silu_sum(x) - u * g / (1 + np.exp(-g))).max() < 1e-6
+
+
+def test_moe_top2_invariants():
+    rng = np.random.default_rng(112)
+    logits = rng.standard_normal((21, 8)).astype(np.float32)
+    logits[3] = [1, 5, 5, 0, 5, -1, 2, 2]  # ties: lower index first
+    sel, w = orc.moe_top2(logits)
+    assert list(sel[3]) == [1, 2]
+    order = np.argsort(-logits, axis=1, kind="stable")[:, :2]
+    assert np.array_equal(sel, order)
+    assert np.abs(w.sum(1) - 1).max() < 1e-6
+    sm = np.exp(logits.astype(np.float64))
+    sm /= sm.sum(1, keepdims=True)
+    top = np.take_along_axis(sm, sel.astype(np.int64), 1)
+    assert np.abs(w - top / top.sum(1, keepdims=True)).max() < 1e-6
+
+
+def test_argmax_first_max_wins():
+    x = np.zeros((3, 32000), np.float32)
+    x[0, 17] = x[0, 900] = 3.0
+    x[1, 31999] = 1.0
+    assert list(orc.argmax(x)) == [17, 31999, 0]

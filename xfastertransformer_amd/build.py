@@ -1,0 +1,71 @@
+"""Builds the gfx950 shared libraries in-tree with hipcc / g++.
+
+    python -m xfastertransformer_amd.build          # everything
+The built .so files sit next to this package so that they travel with a source snapshot
+to a GPU machine; nothing is installed into site-packages.
+"""
+import glob
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+ROOT = os.path.dirname(HERE)
+LIB_HIP = os.path.join(HERE, "libxft_hip.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# gfx950 only; packed-FP32 VALU ops stay off (the compiler must not form v_pk_*_f32)
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
+             "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-fno-gpu-rdc"]
+
+
+def _run(cmd):
+    print("+", " ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+
+
+def _stale(target, sources):
+    if not os.path.exists(target):
+        return True
+    t = os.path.getmtime(target)
+    return any(os.path.getmtime(s) > t for s in sources)
+
+
+def build_hip(force=True):
+    srcs = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+    deps = srcs + glob.glob(os.path.join(CSRC, "*.h")) + glob.glob(os.path.join(ROOT, "include", "*.h"))
+    objdir = os.path.join(CSRC, "build")
+    os.makedirs(objdir, exist_ok=True)
+    objs = []
+    procs = []
+    for s in srcs:
+        o = os.path.join(objdir, os.path.basename(s) + ".o")
+        objs.append(o)
+        if force or _stale(o, [s] + [d for d in deps if d.endswith(".h")]):
+            cmd = [HIPCC] + HIP_FLAGS + ["-c", s, "-o", o]
+            print("+", " ".join(cmd), flush=True)
+            procs.append((s, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    failed = False
+    for s, pr in procs:
+        out, _ = pr.communicate()
+        out = "\n".join(l for l in out.splitlines() if "not a recognized feature" not in l)
+        if out.strip():
+            print(out)
+        if pr.returncode != 0:
+            failed = True
+            print("FAILED:", s)
+    if failed:
+        raise RuntimeError("hipcc failed")
+    if force or procs or not os.path.exists(LIB_HIP):
+        _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_HIP] + objs)
+    return LIB_HIP
+
+
+def build_all(force=True):
+    return build_hip(force)
+
+
+if __name__ == "__main__":
+    build_all(force="--incremental" not in sys.argv)
+    print("built", LIB_HIP)

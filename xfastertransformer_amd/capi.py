@@ -1,0 +1,295 @@
+"""ctypes binding of include/xft_hip.h plus small numpy <-> device helpers."""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libxft_hip.so")
+
+F32, BF16, FP16, INT8 = 0, 1, 2, 3
+W_INT8, W_UINT4, W_NF4, W_W8A8, W_BF16 = 0, 1, 2, 3, 4
+EPI_NONE, EPI_BIAS, EPI_SILU, EPI_GELU, EPI_RESMUL, EPI_RESIDENTIAL, EPI_RESEXT = range(7)
+WF_NONE, WF_GATEUP = 0, 1
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        f"{LIB_PATH} is missing: build it with `python -m xfastertransformer_amd.build` "
+        "(there is no CPU fallback)")
+
+lib = C.CDLL(LIB_PATH)
+lib.xfthip_last_error.restype = C.c_char_p
+lib.xfthip_weight_bytes.restype = C.c_size_t
+lib.xfthip_weight_bytes.argtypes = [C.c_void_p]
+
+
+class XftHipError(RuntimeError):
+    pass
+
+
+def check(rc):
+    if rc != 0:
+        raise XftHipError(lib.xfthip_last_error().decode())
+
+
+_initialised = False
+
+
+def init(device=0):
+    global _initialised
+    if not _initialised:
+        check(lib.xfthip_init(device))
+        _initialised = True
+
+
+def device_info():
+    name = C.create_string_buffer(256)
+    cus = C.c_int()
+    mem = C.c_size_t()
+    check(lib.xfthip_device_info(name, 256, C.byref(cus), C.byref(mem)))
+    return name.value.decode(), cus.value, mem.value
+
+
+def synchronize():
+    check(lib.xfthip_device_synchronize())
+
+
+def _hp(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+class DeviceBuffer:
+    """A device allocation owned through the C-ABI."""
+
+    def __init__(self, nbytes):
+        self.nbytes = int(nbytes)
+        ptr = C.c_void_p()
+        check(lib.xfthip_malloc(C.byref(ptr), C.c_size_t(self.nbytes)))
+        self.ptr = ptr
+
+    @classmethod
+    def from_numpy(cls, a):
+        a = np.ascontiguousarray(a)
+        buf = cls(a.nbytes)
+        check(lib.xfthip_memcpy_h2d(buf.ptr, _hp(a), C.c_size_t(a.nbytes), None))
+        return buf
+
+    def upload(self, a, offset=0):
+        a = np.ascontiguousarray(a)
+        assert offset + a.nbytes <= self.nbytes
+        check(lib.xfthip_memcpy_h2d(C.c_void_p(self.ptr.value + offset), _hp(a), C.c_size_t(a.nbytes), None))
+
+    def to_numpy(self, dtype, shape):
+        out = np.empty(shape, dtype)
+        assert out.nbytes <= self.nbytes
+        check(lib.xfthip_memcpy_d2h(_hp(out), self.ptr, C.c_size_t(out.nbytes), None))
+        return out
+
+    def zero(self):
+        check(lib.xfthip_memset(self.ptr, 0, C.c_size_t(self.nbytes), None))
+        synchronize()
+
+    def at(self, byte_offset):
+        return C.c_void_p(self.ptr.value + int(byte_offset))
+
+    def free(self):
+        if self.ptr is not None and self.ptr.value:
+            lib.xfthip_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def f32_to_bf16_bits(x):
+    """Round-to-nearest-even narrowing of fp32 to bf16 bit patterns (normals)."""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    sub = (u & 0x7F800000) == 0
+    r[sub] = (u[sub] >> 16).astype(np.uint16) & 0x8000
+    return r
+
+
+def bf16_bits_to_f32(b):
+    return (np.ascontiguousarray(b, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+class Weight:
+    """Handle of a packed quantised weight (xfthip_weight_create)."""
+
+    def __init__(self, kind, K, N, q, scale=None, zero=None, flags=WF_NONE):
+        self.kind, self.K, self.N, self.flags = kind, K, N, flags
+        q = np.ascontiguousarray(q)
+        scale = None if scale is None else np.ascontiguousarray(scale, np.float32)
+        zero = None if zero is None else np.ascontiguousarray(zero, np.float32)
+        h = C.c_void_p()
+        check(lib.xfthip_weight_create(kind, K, N, _hp(q), _hp(scale), _hp(zero), flags, C.byref(h)))
+        self.h = h
+
+    def unpack(self):
+        if self.kind in (W_UINT4, W_NF4):
+            out = np.empty((self.K, self.N // 2), np.uint8)
+        elif self.kind == W_BF16:
+            out = np.empty((self.K, self.N), np.uint16)
+        else:
+            out = np.empty((self.K, self.N), np.int8)
+        check(lib.xfthip_weight_unpack(self.h, _hp(out)))
+        return out
+
+    def dequant(self, out_dtype=F32):
+        buf = DeviceBuffer(self.K * self.N * (4 if out_dtype == F32 else 2))
+        check(lib.xfthip_weight_dequant(self.h, buf.ptr, out_dtype, None))
+        synchronize()
+        return buf.to_numpy(np.float32 if out_dtype == F32 else np.uint16, (self.K, self.N))
+
+    def bytes(self):
+        return lib.xfthip_weight_bytes(self.h)
+
+    def free(self):
+        if self.h is not None:
+            lib.xfthip_weight_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def quantize_weight(kind, W):
+    W = np.ascontiguousarray(W, np.float32)
+    K, N = W.shape
+    scale = np.empty(N, np.float32)
+    zero = np.zeros(N, np.float32)
+    q = np.empty((K, N), np.int8) if kind in (W_INT8, W_W8A8) else np.empty((K, N // 2), np.uint8)
+    check(lib.xfthip_quantize_weight(kind, K, N, _hp(W), _hp(q), _hp(scale), _hp(zero)))
+    return q, scale, (None if kind == W_NF4 else zero)
+
+
+def gemm(w, A_dev, M, lda, C_dev, ldc, c_dtype=BF16, epi=EPI_NONE, bias=None, res=None, ldres=0, res_dtype=F32,
+         gamma=1.0, stream=None):
+    check(lib.xfthip_gemm(w.h, M, A_dev, lda, C_dev, ldc, c_dtype, epi, bias, res, ldres, res_dtype,
+                          C.c_float(gamma), stream))
+
+
+def gemm_gateup_silu(w, A_dev, M, lda, out_dev, ldo, out_dtype=BF16, stream=None):
+    check(lib.xfthip_gemm_gateup_silu(w.h, M, A_dev, lda, out_dev, ldo, out_dtype, stream))
+
+
+class Timer:
+    """HIP-event timer on a given stream (None = default stream)."""
+
+    def __init__(self):
+        self.a, self.b = C.c_void_p(), C.c_void_p()
+        check(lib.xfthip_event_create(C.byref(self.a)))
+        check(lib.xfthip_event_create(C.byref(self.b)))
+
+    def start(self, stream=None):
+        check(lib.xfthip_event_record(self.a, stream))
+
+    def stop(self, stream=None):
+        check(lib.xfthip_event_record(self.b, stream))
+        check(lib.xfthip_event_synchronize(self.b))
+        ms = C.c_float()
+        check(lib.xfthip_event_elapsed_ms(self.a, self.b, C.byref(ms)))
+        return ms.value
+
+
+# ---------------------------------------------------------------------------- norm / rope / KV / attention
+def rmsnorm(out_dev, out_dtype, in_dev, in_dtype, weight_dev, rows, cols, i_stride=-1, o_stride=-1, eps=1e-6,
+            stream=None):
+    check(lib.xfthip_rmsnorm(out_dev, out_dtype, in_dev, in_dtype, weight_dev, rows, cols, i_stride, o_stride,
+                             C.c_float(eps), stream))
+
+
+class RopeTables:
+    def __init__(self, dim, max_pos, base=10000, scaling=1.0):
+        self.dim, self.max_pos = dim, max_pos
+        self.cos, self.sin = C.c_void_p(), C.c_void_p()
+        check(lib.xfthip_rope_tables_create(dim, max_pos, int(base), C.c_float(scaling), C.byref(self.cos),
+                                            C.byref(self.sin)))
+
+    def to_numpy(self):
+        half = (self.dim + 1) // 2
+        c = np.empty((self.max_pos, half), np.float32)
+        s = np.empty((self.max_pos, half), np.float32)
+        check(lib.xfthip_memcpy_d2h(_hp(c), self.cos, C.c_size_t(c.nbytes), None))
+        check(lib.xfthip_memcpy_d2h(_hp(s), self.sin, C.c_size_t(s.nbytes), None))
+        return c, s
+
+    def free(self):
+        if self.cos is not None:
+            lib.xfthip_free(self.cos)
+            lib.xfthip_free(self.sin)
+            self.cos = self.sin = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def rotary_embedding(dtype, positions_dev, q_dev, k_dev, tables, dim, q_stride, k_stride, tokens, heads, head_size,
+                     kv_heads, stream=None):
+    check(lib.xfthip_rotary_embedding(dtype, positions_dev, q_dev, k_dev, tables.cos, tables.sin, dim, q_stride,
+                                      k_stride, tokens, heads, head_size, kv_heads, stream))
+
+
+class KVCache:
+    def __init__(self, dtype, batch, kv_heads, max_seq, head_size):
+        self.dtype, self.B, self.H, self.S, self.D = dtype, batch, kv_heads, max_seq, head_size
+        h = C.c_void_p()
+        check(lib.xfthip_kvcache_create(dtype, batch, kv_heads, max_seq, head_size, C.byref(h)))
+        self.h = h
+
+    def _np_dtype(self):
+        return np.int8 if self.dtype == INT8 else np.uint16
+
+    def export(self, which):
+        """Reference layout: data [B][H][maxSeq][D] (fp16 bits / int8), scales [B][H][maxSeq]."""
+        n = self.B * self.H * self.S
+        data = DeviceBuffer(n * self.D * (1 if self.dtype == INT8 else 2))
+        scales = DeviceBuffer(n * 4)
+        scales.zero()
+        check(lib.xfthip_kvcache_export(self.h, which, data.ptr, scales.ptr, None))
+        synchronize()
+        return (data.to_numpy(self._np_dtype(), (self.B, self.H, self.S, self.D)),
+                scales.to_numpy(np.float32, (self.B, self.H, self.S)))
+
+    def load(self, which, data, scales=None):
+        data = np.ascontiguousarray(data, self._np_dtype())
+        assert data.shape == (self.B, self.H, self.S, self.D)
+        d = DeviceBuffer.from_numpy(data)
+        s = None
+        if self.dtype == INT8:
+            s = DeviceBuffer.from_numpy(np.ascontiguousarray(scales, np.float32))
+        check(lib.xfthip_kvcache_import(self.h, which, d.ptr, None if s is None else s.ptr, None))
+        synchronize()
+
+    def free(self):
+        if self.h is not None:
+            lib.xfthip_kvcache_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def rope_kvstore(cache, qkv_dev, dtype, stride, B, S, q_heads, tables, past, past_dev=None, stream=None):
+    cos = None if tables is None else tables.cos
+    sin = None if tables is None else tables.sin
+    check(lib.xfthip_rope_kvstore(cache.h, qkv_dev, dtype, stride, B, S, q_heads, cos, sin, past, past_dev, stream))
+
+
+def attention(cache, q_dev, q_stride, out_dev, o_stride, out_dtype, B, S, q_heads, scale, past, past_dev=None,
+              stream=None):
+    check(lib.xfthip_attention(cache.h, q_dev, q_stride, out_dev, o_stride, out_dtype, B, S, q_heads,
+                               C.c_float(scale), past, past_dev, stream))

@@ -1,0 +1,125 @@
+// Shared declarations of the gfx950 library: error plumbing, element types, the packed
+// weight descriptor and small device helpers.  Internal header (the public C-ABI is
+// include/xft_hip.h).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string>
+
+#include "../../include/xft_hip.h"
+
+namespace xfthip {
+
+void set_error(const char *fmt, ...);
+
+#define XFT_CHECK_HIP(expr)                                                                         \
+    do {                                                                                            \
+        hipError_t _e = (expr);                                                                     \
+        if (_e != hipSuccess) {                                                                     \
+            xfthip::set_error("%s:%d: %s failed: %s", __FILE__, __LINE__, #expr, hipGetErrorString(_e)); \
+            return 1;                                                                               \
+        }                                                                                           \
+    } while (0)
+
+#define XFT_REQUIRE(cond, ...)               \
+    do {                                     \
+        if (!(cond)) {                       \
+            xfthip::set_error(__VA_ARGS__);  \
+            return 2;                        \
+        }                                    \
+    } while (0)
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+// ---- packed weight layout ---------------------------------------------------------------
+// The matrix is cut into tiles of 16 output columns (n) by KTILE input rows (k); a tile is
+// 1 KiB = 64 lanes x 16 bytes, laid out so that lane l of a wavefront reads bytes
+// [16 l, 16 l + 16) and finds there the K-consecutive codes of column n = 16 nt + (l & 15)
+// for the k range its MFMA operand slot needs (lane group g = l >> 4):
+//   INT8 / W8A8 : KTILE 64,  16 codes/lane, k = 64 kt + 16 g + j
+//   UINT4 / NF4 : KTILE 128, 32 codes/lane, k = 128 kt + 32 g + c, code c = 8 d + e lives in
+//                 dword d at nibble e/2 (e even) or 4 + e/2 (e odd), so that
+//                 ((w >> 4p) & 0x000F000F) yields the pair (e = 2p, e = 2p + 1)
+//   BF16        : KTILE 32,  8 values/lane, k = 32 kt + 8 g + j
+// Tiles of one column block are contiguous along k: offset = (nt * KT + kt) * 1024 bytes.
+struct PackedWeight {
+    int kind;
+    int K, N; // logical shape
+    int KT, NTILES; // tiles along k and n
+    int ktile; // rows per tile
+    int flags;
+    int inter; // XFTHIP_WF_GATEUP: I (half of N); columns are stored gate/up interleaved per 16
+    uint8_t *packed; // device
+    float *scale; // device [NTILES*16], in packed column order
+    float *zero; // device or nullptr
+    float *colsum; // device (W8A8) or nullptr
+    size_t packed_bytes;
+};
+
+__host__ __device__ inline int ktile_of(int kind) {
+    return (kind == XFTHIP_W_INT8 || kind == XFTHIP_W_W8A8) ? 64 : (kind == XFTHIP_W_BF16 ? 32 : 128);
+}
+
+// logical column -> packed column
+__host__ __device__ inline int packed_col(int n, int inter) {
+    if (inter <= 0) return n;
+    int isUp = n >= inter;
+    int j = isUp ? n - inter : n;
+    return (j >> 4) * 32 + (isUp ? 16 : 0) + (j & 15);
+}
+// packed column -> logical column
+__host__ __device__ inline int logical_col(int np, int inter) {
+    if (inter <= 0) return np;
+    int blk = np >> 5, r = np & 31;
+    int j = blk * 16 + (r & 15);
+    return (r >= 16) ? j + inter : j;
+}
+
+// ---- numeric helpers -----------------------------------------------------------------
+__device__ inline uint32_t f2u(float f) { return __float_as_uint(f); }
+__device__ inline float u2f(uint32_t u) { return __uint_as_float(u); }
+
+// fp32 -> bf16 exactly as the reference's bfloat16_t assignment (include/bfloat16.h:40-65):
+// RNE on normals, subnormals flushed to signed zero, NaN quieted.
+__device__ inline uint16_t f32_to_bf16_ref(float f) {
+    uint32_t u = f2u(f);
+    uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
+    if (a == 0x7F800000u) return (uint16_t)(u >> 16);
+    if (a < 0x00800000u) return (uint16_t)((u >> 16) & 0x8000u);
+    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+__device__ inline float bf16_to_f32(uint16_t b) { return u2f((uint32_t)b << 16); }
+
+__device__ inline uint16_t f32_to_fp16_bits(float f) {
+    _Float16 h = (_Float16)f; // v_cvt_f16_f32: IEEE round-to-nearest-even
+    return __builtin_bit_cast(uint16_t, h);
+}
+__device__ inline float fp16_bits_to_f32(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+
+__device__ inline float load_as_f32(const void *p, int dtype, size_t idx) {
+    if (dtype == XFTHIP_F32) return ((const float *)p)[idx];
+    if (dtype == XFTHIP_BF16) return bf16_to_f32(((const uint16_t *)p)[idx]);
+    return fp16_bits_to_f32(((const uint16_t *)p)[idx]);
+}
+__device__ inline void store_from_f32(void *p, int dtype, size_t idx, float v) {
+    if (dtype == XFTHIP_F32)
+        ((float *)p)[idx] = v;
+    else if (dtype == XFTHIP_BF16)
+        ((uint16_t *)p)[idx] = f32_to_bf16_ref(v);
+    else
+        ((uint16_t *)p)[idx] = f32_to_fp16_bits(v);
+}
+
+// exp on the device: the reference uses a degree-5 polynomial (src/utils/bert_util.h:26-75)
+// accurate to ~1e-7 relative; __expf is within the same distance of exp().
+__device__ inline float fast_exp(float x) { return __expf(x); }
+
+int device_cu_count();
+
+} // namespace xfthip

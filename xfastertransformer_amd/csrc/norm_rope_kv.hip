@@ -1,0 +1,397 @@
+// RMSNorm, rotary embedding and the KV cache (layout, append with FP16 convert or INT8
+// quantisation).  Replaces the reference's rmsnorm_kernels.cpp, rotary_embedding_kernels.cpp,
+// KVCacheTensor and xft::quantize.  All HBM-bound elementwise work: one wavefront per row /
+// per (token, head), coalesced 128-bit or 32-bit accesses, wave-level reductions.
+#include <math.h>
+
+#include <vector>
+
+#include "kvcache.h"
+
+namespace xfthip {
+
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ inline float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// ---- RMSNorm: one 256-thread block per row ------------------------------------------------
+__global__ __launch_bounds__(256) void rmsnorm_kernel(void *__restrict__ out, int out_dtype,
+        const void *__restrict__ in, int in_dtype, const float *__restrict__ weight, int cols, int iStride,
+        int oStride, float eps) {
+    __shared__ float part[4];
+    const int row = blockIdx.x;
+    const size_t ibase = (size_t)row * iStride, obase = (size_t)row * oStride;
+    float sq = 0.0f;
+    for (int c = threadIdx.x; c < cols; c += 256) {
+        float x = load_as_f32(in, in_dtype, ibase + c);
+        sq = fmaf(x, x, sq);
+    }
+    sq = wave_sum(sq);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = sq;
+    __syncthreads();
+    const float total = (part[0] + part[1]) + (part[2] + part[3]);
+    const float var = 1.0f / sqrtf(total / (float)cols + eps);
+    for (int c = threadIdx.x; c < cols; c += 256) {
+        float x = load_as_f32(in, in_dtype, ibase + c);
+        store_from_f32(out, out_dtype, obase + c, (x * var) * weight[c]);
+    }
+}
+
+// ---- RoPE + KV append ---------------------------------------------------------------------
+// One wavefront per (token, head); lane l owns elements l, l+64, ... of the two halves.
+// D <= 256, D % 2 == 0.  heads [0, qHeads) are query heads (rotated in place), heads
+// [qHeads, qHeads+kvHeads) are key heads (rotated, then appended) and their value heads.
+struct RopeKvParams {
+    void *qkv;
+    int dtype, stride;
+    int B, S, qHeads, kvHeads, D;
+    const float *cosT, *sinT;
+    int past;
+    const int *past_dev;
+    const int *positions; // optional explicit position per token (standalone rotary call)
+    KvView kv; // kv.k == nullptr: no append
+    void *key; // standalone rotary: separate key pointer (qkv = query), else nullptr
+    int kStride;
+};
+
+template <int EPL> // elements per lane in each half: D/2 <= 64*EPL
+__global__ __launch_bounds__(64) void rope_kv_kernel(RopeKvParams p) {
+    const int lane = threadIdx.x;
+    const int head = blockIdx.x;
+    const int tok = blockIdx.y;
+    const int b = tok / p.S, s = tok % p.S;
+    const int half = p.D / 2;
+    const int past = p.past_dev ? p.past_dev[b] : p.past;
+    const int pos = p.positions ? p.positions[tok] : past + s;
+    const bool isq = head < p.qHeads;
+    const int kvh = head - p.qHeads;
+
+    char *rowbase;
+    size_t col;
+    if (isq) {
+        rowbase = (char *)p.qkv;
+        col = (size_t)tok * p.stride + (size_t)head * p.D;
+    } else if (p.key) {
+        rowbase = (char *)p.key;
+        col = (size_t)tok * p.kStride + (size_t)kvh * p.D;
+    } else {
+        rowbase = (char *)p.qkv;
+        col = (size_t)tok * p.stride + (size_t)(p.qHeads + kvh) * p.D;
+    }
+
+    float lo[EPL], hi[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+        const int i = lane + 64 * e;
+        if (i < half) {
+            float a = load_as_f32(rowbase, p.dtype, col + i);
+            float bb = load_as_f32(rowbase, p.dtype, col + i + half);
+            if (p.cosT) {
+                const float c = p.cosT[(size_t)pos * half + i], sn = p.sinT[(size_t)pos * half + i];
+                // reference: fmsub(q, cos, qHalf*sin) ; fmadd(qHalf, cos, q*sin)
+                lo[e] = fmaf(a, c, -(bb * sn));
+                hi[e] = fmaf(bb, c, a * sn);
+            } else {
+                lo[e] = a;
+                hi[e] = bb;
+            }
+        } else {
+            lo[e] = hi[e] = 0.0f;
+        }
+    }
+
+    if (isq || p.key) {
+        // rotated values go back in place (query always; key only in the standalone call)
+        if (p.cosT) {
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                const int i = lane + 64 * e;
+                if (i < half) {
+                    store_from_f32(rowbase, p.dtype, col + i, lo[e]);
+                    store_from_f32(rowbase, p.dtype, col + i + half, hi[e]);
+                }
+            }
+        }
+        if (isq || p.kv.k == nullptr) return;
+    }
+    if (p.kv.k == nullptr) return;
+
+    // ---- append key row (rotated, from fp32 registers) and value row ----
+    const int t = past + s;
+    if (t >= p.kv.S) return; // host checks this; never write outside the cache
+    const size_t bh = (size_t)b * p.kv.H + kvh;
+    // value row: raw from qkv
+    const size_t vcol = (size_t)tok * p.stride + (size_t)(p.qHeads + p.kvHeads + kvh) * p.D;
+    float vlo[EPL], vhi[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+        const int i = lane + 64 * e;
+        vlo[e] = (i < half) ? load_as_f32(p.qkv, p.dtype, vcol + i) : 0.0f;
+        vhi[e] = (i < half) ? load_as_f32(p.qkv, p.dtype, vcol + i + half) : 0.0f;
+    }
+    const size_t vblk = (bh * (p.kv.S / 32) + (t >> 5)) * (size_t)p.D * 32 + v_slot(t & 31);
+    if (p.kv.int8) {
+        // xft::quantize: max = absmax, factor = max == 0 ? 1 : 127/max, scale = max/127, q = rne(x*factor)
+        float km = 0.0f, vm = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            km = fmaxf(km, fmaxf(fabsf(lo[e]), fabsf(hi[e])));
+            vm = fmaxf(vm, fmaxf(fabsf(vlo[e]), fabsf(vhi[e])));
+        }
+        km = wave_max(km);
+        vm = wave_max(vm);
+        const float kf = (km == 0.0f) ? 1.0f : 127.0f / km;
+        const float vf = (vm == 0.0f) ? 1.0f : 127.0f / vm;
+        if (lane == 0) {
+            p.kv.kscale[bh * p.kv.S + t] = km / 127.0f;
+            p.kv.vscale[bh * p.kv.S + t] = vm / 127.0f;
+        }
+        int8_t *kd = (int8_t *)p.kv.k + (bh * p.kv.S + t) * (size_t)p.D;
+        int8_t *vd = (int8_t *)p.kv.v + vblk;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            const int i = lane + 64 * e;
+            if (i < half) {
+                kd[i] = (int8_t)__float2int_rn(lo[e] * kf);
+                kd[i + half] = (int8_t)__float2int_rn(hi[e] * kf);
+                vd[(size_t)i * 32] = (int8_t)__float2int_rn(vlo[e] * vf);
+                vd[(size_t)(i + half) * 32] = (int8_t)__float2int_rn(vhi[e] * vf);
+            }
+        }
+    } else {
+        uint16_t *kd = (uint16_t *)p.kv.k + (bh * p.kv.S + t) * (size_t)p.D;
+        uint16_t *vd = (uint16_t *)p.kv.v + vblk;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            const int i = lane + 64 * e;
+            if (i < half) {
+                kd[i] = f32_to_fp16_bits(lo[e]);
+                kd[i + half] = f32_to_fp16_bits(hi[e]);
+                vd[(size_t)i * 32] = f32_to_fp16_bits(vlo[e]);
+                vd[(size_t)(i + half) * 32] = f32_to_fp16_bits(vhi[e]);
+            }
+        }
+    }
+}
+
+// ---- export / import between the private layout and [B][H][S][D] ----------------------------
+__global__ void kv_convert_kernel(KvView kv, int which, void *data, float *scales, int maxSeq, int to_private) {
+    const size_t total = (size_t)kv.B * kv.H * maxSeq * kv.D;
+    const int esz = kv.int8 ? 1 : 2;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const int d = (int)(i % kv.D);
+        const size_t r = i / kv.D;
+        const int t = (int)(r % maxSeq);
+        const size_t bh = r / maxSeq;
+        size_t poff;
+        char *priv;
+        if (which == 0) {
+            priv = (char *)kv.k;
+            poff = (bh * kv.S + t) * (size_t)kv.D + d;
+        } else {
+            priv = (char *)kv.v;
+            poff = (bh * (kv.S / 32) + (t >> 5)) * (size_t)kv.D * 32 + (size_t)d * 32 + v_slot(t & 31);
+        }
+        char *ext = (char *)data + i * esz;
+        char *in = priv + poff * esz;
+        if (to_private) {
+            for (int bte = 0; bte < esz; ++bte) in[bte] = ext[bte];
+        } else {
+            for (int bte = 0; bte < esz; ++bte) ext[bte] = in[bte];
+        }
+        if (kv.int8 && scales && d == 0) {
+            float *ps = (which == 0 ? kv.kscale : kv.vscale) + bh * kv.S + t;
+            if (to_private)
+                *ps = scales[bh * maxSeq + t];
+            else
+                scales[bh * maxSeq + t] = *ps;
+        }
+    }
+}
+
+} // namespace xfthip
+
+using namespace xfthip;
+
+extern "C" {
+
+int xfthip_rmsnorm(void *out, int out_dtype, const void *in, int in_dtype, const float *weight, int rows, int cols,
+        int iStride, int oStride, float eps, xfthip_stream_t stream) {
+    XFT_REQUIRE(out && in && weight, "xfthip_rmsnorm: null argument");
+    XFT_REQUIRE(rows > 0 && cols > 0, "xfthip_rmsnorm: bad shape %d x %d", rows, cols);
+    XFT_REQUIRE((out_dtype == XFTHIP_F32 || out_dtype == XFTHIP_BF16) && (in_dtype == XFTHIP_F32 || in_dtype == XFTHIP_BF16),
+            "xfthip_rmsnorm: dtypes must be f32 or bf16");
+    if (iStride == -1) iStride = cols;
+    if (oStride == -1) oStride = cols;
+    XFT_REQUIRE(iStride >= cols && oStride >= cols, "xfthip_rmsnorm: stride smaller than cols");
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, out, out_dtype, in, in_dtype,
+            weight, cols, iStride, oStride, eps);
+    XFT_CHECK_HIP(hipGetLastError());
+    return 0;
+}
+
+int xfthip_rope_tables_create(int dim, int maxPos, int base, float scalingFactor, float **cos_dev, float **sin_dev) {
+    XFT_REQUIRE(cos_dev && sin_dev, "xfthip_rope_tables_create: null out pointer");
+    XFT_REQUIRE(dim > 0 && maxPos > 0 && base > 0, "xfthip_rope_tables_create: bad argument");
+    const int half = (dim + 1) / 2;
+    std::vector<float> inv(half), c((size_t)maxPos * half), s((size_t)maxPos * half);
+    for (int i = 0; i < half; ++i) {
+        inv[i] = (float)(1.0 / pow((double)base, (double)((float)(i * 2) / (float)dim)));
+        inv[i] /= scalingFactor;
+    }
+    for (size_t pz = 0; pz < (size_t)maxPos; ++pz)
+        for (int j = 0; j < half; ++j) {
+            float t = (float)pz * inv[j];
+            c[pz * half + j] = cosf(t);
+            s[pz * half + j] = sinf(t);
+        }
+    *cos_dev = *sin_dev = nullptr;
+    XFT_CHECK_HIP(hipMalloc((void **)cos_dev, c.size() * sizeof(float)));
+    XFT_CHECK_HIP(hipMalloc((void **)sin_dev, s.size() * sizeof(float)));
+    XFT_CHECK_HIP(hipMemcpy(*cos_dev, c.data(), c.size() * sizeof(float), hipMemcpyHostToDevice));
+    XFT_CHECK_HIP(hipMemcpy(*sin_dev, s.data(), s.size() * sizeof(float), hipMemcpyHostToDevice));
+    return 0;
+}
+
+static int launch_rope(const RopeKvParams &p, int tokens, hipStream_t stream) {
+    const int half = p.D / 2;
+    dim3 grid(p.qHeads + p.kvHeads, tokens);
+    if (half <= 64)
+        hipLaunchKernelGGL(rope_kv_kernel<1>, grid, dim3(64), 0, stream, p);
+    else
+        hipLaunchKernelGGL(rope_kv_kernel<2>, grid, dim3(64), 0, stream, p);
+    XFT_CHECK_HIP(hipGetLastError());
+    return 0;
+}
+
+int xfthip_rotary_embedding(int dtype, const int *positions, void *query, void *key, const float *embCos,
+        const float *embSin, int dim, int qStride, int kStride, int numTokens, int headNum, int headSize,
+        int numKvHeads, xfthip_stream_t stream) {
+    XFT_REQUIRE(positions && query && key && embCos && embSin, "xfthip_rotary_embedding: null argument");
+    XFT_REQUIRE(dtype == XFTHIP_F32 || dtype == XFTHIP_BF16, "xfthip_rotary_embedding: dtype must be f32 or bf16");
+    XFT_REQUIRE(dim == headSize, "xfthip_rotary_embedding: rot dim %d must equal head size %d", dim, headSize);
+    XFT_REQUIRE(headSize % 2 == 0 && headSize <= 256, "xfthip_rotary_embedding: head size %d unsupported", headSize);
+    XFT_REQUIRE(numTokens > 0 && headNum > 0 && numKvHeads > 0, "xfthip_rotary_embedding: bad shape");
+    RopeKvParams p = {};
+    p.qkv = query;
+    p.key = key;
+    p.dtype = dtype;
+    p.stride = qStride;
+    p.kStride = kStride;
+    p.B = 1;
+    p.S = numTokens;
+    p.qHeads = headNum;
+    p.kvHeads = numKvHeads;
+    p.D = headSize;
+    p.cosT = embCos;
+    p.sinT = embSin;
+    p.positions = positions;
+    return launch_rope(p, numTokens, (hipStream_t)stream);
+}
+
+int xfthip_kvcache_create(int dtype, int batch, int kvHeads, int maxSeq, int headSize, xfthip_kvcache_t *out) {
+    XFT_REQUIRE(out != nullptr, "xfthip_kvcache_create: null out pointer");
+    XFT_REQUIRE(dtype == XFTHIP_FP16 || dtype == XFTHIP_INT8, "xfthip_kvcache_create: dtype must be fp16 or int8");
+    XFT_REQUIRE(batch > 0 && kvHeads > 0 && maxSeq > 0, "xfthip_kvcache_create: bad shape");
+    XFT_REQUIRE(headSize == 128, "xfthip_kvcache_create: head size %d unsupported (attention kernels are built for 128)", headSize);
+    xfthip_kvcache *c = new xfthip_kvcache();
+    c->maxSeq = maxSeq;
+    KvView &kv = c->kv;
+    kv.int8 = dtype == XFTHIP_INT8;
+    kv.B = batch;
+    kv.H = kvHeads;
+    kv.D = headSize;
+    kv.S = (maxSeq + 31) / 32 * 32;
+    const size_t elems = (size_t)batch * kvHeads * kv.S * headSize;
+    const size_t bytes = elems * (kv.int8 ? 1 : 2);
+    kv.k = kv.v = nullptr;
+    kv.kscale = kv.vscale = nullptr;
+    if (hipMalloc(&kv.k, bytes) != hipSuccess || hipMalloc(&kv.v, bytes) != hipSuccess) {
+        set_error("xfthip_kvcache_create: hipMalloc of 2 x %zu bytes failed", bytes);
+        xfthip_kvcache_destroy(c);
+        return 1;
+    }
+    (void)hipMemset(kv.k, 0, bytes);
+    (void)hipMemset(kv.v, 0, bytes);
+    if (kv.int8) {
+        const size_t sb = (size_t)batch * kvHeads * kv.S * sizeof(float);
+        if (hipMalloc((void **)&kv.kscale, sb) != hipSuccess || hipMalloc((void **)&kv.vscale, sb) != hipSuccess) {
+            set_error("xfthip_kvcache_create: hipMalloc of scales failed");
+            xfthip_kvcache_destroy(c);
+            return 1;
+        }
+        (void)hipMemset(kv.kscale, 0, sb);
+        (void)hipMemset(kv.vscale, 0, sb);
+    }
+    XFT_CHECK_HIP(hipDeviceSynchronize());
+    *out = c;
+    return 0;
+}
+
+int xfthip_kvcache_destroy(xfthip_kvcache_t c) {
+    if (!c) return 0;
+    if (c->kv.k) (void)hipFree(c->kv.k);
+    if (c->kv.v) (void)hipFree(c->kv.v);
+    if (c->kv.kscale) (void)hipFree(c->kv.kscale);
+    if (c->kv.vscale) (void)hipFree(c->kv.vscale);
+    delete c;
+    return 0;
+}
+
+static int kv_convert(xfthip_kvcache_t c, int which, void *data, float *scales, int to_private, hipStream_t stream) {
+    XFT_REQUIRE(c && data, "xfthip_kvcache_export/import: null argument");
+    XFT_REQUIRE(which == 0 || which == 1, "xfthip_kvcache_export/import: which must be 0 (keys) or 1 (values)");
+    const size_t total = (size_t)c->kv.B * c->kv.H * c->maxSeq * c->kv.D;
+    int blocks = (int)((total + 255) / 256 > 1048576 ? 1048576 : (total + 255) / 256);
+    hipLaunchKernelGGL(kv_convert_kernel, dim3(blocks), dim3(256), 0, stream, c->kv, which, data, scales, c->maxSeq,
+            to_private);
+    XFT_CHECK_HIP(hipGetLastError());
+    return 0;
+}
+
+int xfthip_kvcache_export(xfthip_kvcache_t c, int which, void *data_dev, float *scales_dev, xfthip_stream_t stream) {
+    return kv_convert(c, which, data_dev, scales_dev, 0, (hipStream_t)stream);
+}
+
+int xfthip_kvcache_import(xfthip_kvcache_t c, int which, const void *data_dev, const float *scales_dev,
+        xfthip_stream_t stream) {
+    XFT_REQUIRE(!(c && c->kv.int8) || scales_dev, "xfthip_kvcache_import: INT8 cache needs scales");
+    return kv_convert(c, which, (void *)data_dev, (float *)scales_dev, 1, (hipStream_t)stream);
+}
+
+int xfthip_rope_kvstore(xfthip_kvcache_t c, void *qkv, int dtype, int stride, int B, int S, int qHeads,
+        const float *embCos, const float *embSin, int past, const int *past_dev, xfthip_stream_t stream) {
+    XFT_REQUIRE(c && qkv, "xfthip_rope_kvstore: null argument");
+    XFT_REQUIRE(dtype == XFTHIP_F32 || dtype == XFTHIP_BF16, "xfthip_rope_kvstore: dtype must be f32 or bf16");
+    XFT_REQUIRE((embCos == nullptr) == (embSin == nullptr), "xfthip_rope_kvstore: cos and sin go together");
+    XFT_REQUIRE(B > 0 && B <= c->kv.B, "xfthip_rope_kvstore: batch %d exceeds cache batch %d", B, c->kv.B);
+    XFT_REQUIRE(S > 0 && qHeads > 0 && qHeads % c->kv.H == 0, "xfthip_rope_kvstore: bad S=%d or qHeads=%d (kvHeads=%d)", S,
+            qHeads, c->kv.H);
+    XFT_REQUIRE(stride >= (qHeads + 2 * c->kv.H) * c->kv.D, "xfthip_rope_kvstore: stride %d too small", stride);
+    XFT_REQUIRE(past_dev != nullptr || (past >= 0 && past + S <= c->maxSeq),
+            "xfthip_rope_kvstore: past %d + S %d exceeds the cache length %d", past, S, c->maxSeq);
+    RopeKvParams p = {};
+    p.qkv = qkv;
+    p.dtype = dtype;
+    p.stride = stride;
+    p.B = B;
+    p.S = S;
+    p.qHeads = qHeads;
+    p.kvHeads = c->kv.H;
+    p.D = c->kv.D;
+    p.cosT = embCos;
+    p.sinT = embSin;
+    p.past = past;
+    p.past_dev = past_dev;
+    p.kv = c->kv;
+    return launch_rope(p, B * S, (hipStream_t)stream);
+}
+
+} // extern "C"

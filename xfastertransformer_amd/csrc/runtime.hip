@@ -1,0 +1,157 @@
+// Runtime plumbing behind the C-ABI: device selection, error text, memory, streams, events.
+#include <stdarg.h>
+#include <string.h>
+
+#include <mutex>
+
+#include "common.h"
+
+namespace xfthip {
+
+static thread_local char g_err[1024] = "";
+static int g_device = -1;
+static int g_cus = 0;
+static std::mutex g_mu;
+
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int device_cu_count() {
+    return g_cus > 0 ? g_cus : 256;
+}
+
+} // namespace xfthip
+
+using namespace xfthip;
+
+extern "C" {
+
+const char *xfthip_last_error(void) {
+    return g_err;
+}
+
+int xfthip_init(int device) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    int n = 0;
+    XFT_CHECK_HIP(hipGetDeviceCount(&n));
+    XFT_REQUIRE(n > 0, "xfthip_init: no HIP device visible");
+    XFT_REQUIRE(device >= 0 && device < n, "xfthip_init: device %d out of range (have %d)", device, n);
+    XFT_CHECK_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    XFT_CHECK_HIP(hipGetDeviceProperties(&prop, device));
+    XFT_REQUIRE(strncmp(prop.gcnArchName, "gfx950", 6) == 0,
+            "xfthip_init: this library is built for gfx950 only, device %d is %s", device, prop.gcnArchName);
+    g_device = device;
+    g_cus = prop.multiProcessorCount;
+    return 0;
+}
+
+int xfthip_finalize(void) {
+    if (g_device < 0) return 0;
+    XFT_CHECK_HIP(hipDeviceSynchronize());
+    return 0;
+}
+
+int xfthip_device_info(char *name, int name_len, int *compute_units, size_t *hbm_bytes) {
+    XFT_REQUIRE(g_device >= 0, "xfthip_device_info: call xfthip_init first");
+    hipDeviceProp_t prop;
+    XFT_CHECK_HIP(hipGetDeviceProperties(&prop, g_device));
+    if (name && name_len > 0) snprintf(name, name_len, "%s (%s)", prop.name, prop.gcnArchName);
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (hbm_bytes) *hbm_bytes = prop.totalGlobalMem;
+    return 0;
+}
+
+int xfthip_malloc(void **ptr, size_t bytes) {
+    XFT_REQUIRE(ptr != nullptr, "xfthip_malloc: null out pointer");
+    *ptr = nullptr;
+    if (bytes == 0) bytes = 16;
+    XFT_CHECK_HIP(hipMalloc(ptr, bytes));
+    return 0;
+}
+
+int xfthip_free(void *ptr) {
+    if (ptr) XFT_CHECK_HIP(hipFree(ptr));
+    return 0;
+}
+
+int xfthip_memcpy_h2d(void *dst, const void *src_host, size_t bytes, xfthip_stream_t stream) {
+    if (bytes == 0) return 0;
+    XFT_CHECK_HIP(hipMemcpyAsync(dst, src_host, bytes, hipMemcpyHostToDevice, (hipStream_t)stream));
+    XFT_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream)); // pageable host memory: make the call safe
+    return 0;
+}
+
+int xfthip_memcpy_d2h(void *dst_host, const void *src, size_t bytes, xfthip_stream_t stream) {
+    if (bytes == 0) return 0;
+    XFT_CHECK_HIP(hipMemcpyAsync(dst_host, src, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream));
+    XFT_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
+int xfthip_memcpy_d2d(void *dst, const void *src, size_t bytes, xfthip_stream_t stream) {
+    if (bytes == 0) return 0;
+    XFT_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream));
+    return 0;
+}
+
+int xfthip_memset(void *dst, int value, size_t bytes, xfthip_stream_t stream) {
+    if (bytes == 0) return 0;
+    XFT_CHECK_HIP(hipMemsetAsync(dst, value, bytes, (hipStream_t)stream));
+    return 0;
+}
+
+int xfthip_stream_create(xfthip_stream_t *stream) {
+    hipStream_t s;
+    XFT_CHECK_HIP(hipStreamCreate(&s)); // default priority only
+    *stream = (xfthip_stream_t)s;
+    return 0;
+}
+
+int xfthip_stream_destroy(xfthip_stream_t stream) {
+    if (stream) XFT_CHECK_HIP(hipStreamDestroy((hipStream_t)stream));
+    return 0;
+}
+
+int xfthip_stream_synchronize(xfthip_stream_t stream) {
+    XFT_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
+int xfthip_device_synchronize(void) {
+    XFT_CHECK_HIP(hipDeviceSynchronize());
+    return 0;
+}
+
+int xfthip_event_create(xfthip_event_t *ev) {
+    hipEvent_t e;
+    XFT_CHECK_HIP(hipEventCreate(&e));
+    *ev = (xfthip_event_t)e;
+    return 0;
+}
+
+int xfthip_event_destroy(xfthip_event_t ev) {
+    if (ev) XFT_CHECK_HIP(hipEventDestroy((hipEvent_t)ev));
+    return 0;
+}
+
+int xfthip_event_record(xfthip_event_t ev, xfthip_stream_t stream) {
+    XFT_CHECK_HIP(hipEventRecord((hipEvent_t)ev, (hipStream_t)stream));
+    return 0;
+}
+
+int xfthip_event_synchronize(xfthip_event_t ev) {
+    XFT_CHECK_HIP(hipEventSynchronize((hipEvent_t)ev));
+    return 0;
+}
+
+int xfthip_event_elapsed_ms(xfthip_event_t start, xfthip_event_t stop, float *ms) {
+    XFT_CHECK_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return 0;
+}
+
+} // extern "C"

@@ -201,6 +201,82 @@ int xfthip_rope_kvstore(xfthip_kvcache_t c, void *qkv, int dtype, int stride, in
 int xfthip_attention(xfthip_kvcache_t c, const void *q, int qStride, void *out, int oStride, int out_dtype, int B,
         int S, int qHeads, float scale, int past, const int *past_dev, xfthip_stream_t stream);
 
+
+/* ---- decoder layers and the model driver -------------------------------------------- */
+typedef struct xfthip_model *xfthip_model_t;
+
+typedef struct {
+    int layers; /* number of decoder layers */
+    int hidden; /* hidden size */
+    int intermediate; /* MLP intermediate size */
+    int q_heads, kv_heads, head_size;
+    int vocab; /* 0: no embedding / lm_head (layer-only use) */
+    int max_batch; /* sequences held by the KV caches */
+    int max_seq; /* KV cache length per sequence (the reference's maxPositions) */
+    int max_tokens; /* largest batch*inputSeqLen a forward call will carry */
+    int max_pos_embed; /* rows of the RoPE tables */
+    int rope_base; /* rope_theta (an int in the reference, rotary_embedding.h:63) */
+    int kv_dtype; /* XFTHIP_FP16 or XFTHIP_INT8 */
+    float rms_eps; /* epsilon of the attention-side RMSNorm; the MLP side uses 1e-6 as the
+                      reference hard-codes it (src/layers/mlp_llama.h:212) */
+} xfthip_model_config;
+
+/*
+ * A Llama-family decoder stack resident in HBM: per-layer KV caches, RoPE tables and the
+ * activation scratch.  Replaces DecoderContext + KVCacheManager + DecoderBlock
+ * (src/common/transformer_ctx.h:63-459, src/models/kvcache_manager.h, src/layers/decoder_block.h:28-150).
+ */
+int xfthip_model_create(const xfthip_model_config *cfg, xfthip_model_t *out);
+int xfthip_model_destroy(xfthip_model_t m);
+/*
+ * Attach the weights of layer `idx` (handles stay owned by the caller and must outlive the
+ * model).  qkv: [hidden, (q+2kv)*head] as Attention::setWeights concatenates it
+ * (src/layers/attention.h:94-242); o: [q*head, hidden]; gateup: [hidden, 2*intermediate]
+ * created with XFTHIP_WF_GATEUP (LlamaMLP::setWeights, src/layers/mlp_llama.h:63-139);
+ * down: [intermediate, hidden].  ln1/ln2: host fp32 [hidden] RMSNorm weights.
+ * qkv_bias / o_bias: host fp32 or NULL.
+ */
+int xfthip_model_set_layer(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthip_weight_t o, xfthip_weight_t gateup,
+        xfthip_weight_t down, const float *ln1_host, const float *ln2_host, const float *qkv_bias_host,
+        const float *o_bias_host);
+/*
+ * Embedding table (host fp16 bit patterns [vocab, hidden], the reference keeps it in FP16:
+ * src/layers/token_embedding.h:49-52), final RMSNorm weight (host fp32 [hidden]) and the
+ * lm_head weight handle ([hidden, vocab], XFTHIP_W_BF16: never quantised in the reference,
+ * src/models/common_decoder.h:1000-1001).
+ */
+int xfthip_model_set_head(xfthip_model_t m, const uint16_t *embedding_fp16_host, const float *final_norm_host,
+        xfthip_weight_t lm_head);
+/*
+ * One decoder layer: x_out = layer(x_in) for B sequences of S new tokens each at positions
+ * past .. past+S-1 (fp32 device buffers [B*S, stride], may alias).  Replaces
+ * Decoder::forwardAttention + forwardFFN (src/layers/decoder_layer.h:101-170), the body of
+ * xft::invokeLayerLLaMA (src/layers/decoder_layer.cpp:29-160).
+ */
+int xfthip_model_layer_forward(xfthip_model_t m, int idx, const float *x_in, int in_stride, float *x_out,
+        int out_stride, int B, int S, int past, xfthip_stream_t stream);
+/*
+ * Prefill: embeds ids_host [B, S] (host int32), runs every layer at positions 0..S-1, final
+ * norm + lm_head on the last token of each sequence and greedy argmax (first maximum wins,
+ * src/searchers/sampling.cpp:22-131).  The chosen ids stay on the device as the input of
+ * the next decode step.  Replaces CommonDecoder::forward for the first token
+ * (src/models/common_decoder.h:315-589).  logits_host (fp32 [B, vocab]) may be NULL.
+ */
+int xfthip_model_prefill(xfthip_model_t m, const int *ids_host, int B, int S, float *logits_host, xfthip_stream_t stream);
+/*
+ * `steps` greedy decode steps, each one replay of a captured HIP graph (embedding of the
+ * previous ids, all layers, lm_head, argmax, position advance).  ids_out_host: int32
+ * [steps, B] or NULL.  Must follow xfthip_model_prefill with the same B.
+ */
+int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_stream_t stream);
+/* ids chosen by the last prefill / decode call (host int32 [B]) and the current position */
+int xfthip_model_last_ids(xfthip_model_t m, int *ids_host, int *position);
+/* fp32 logits of the last step, device pointer [B, vocab] (valid until the next call) */
+int xfthip_model_logits(xfthip_model_t m, const float **logits_dev);
+
+/* first-maximum argmax over rows of fp32 logits [rows, cols] (sampling.cpp:22-131) */
+int xfthip_argmax(const float *logits, int rows, int cols, int *ids_dev, xfthip_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

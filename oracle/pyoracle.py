@@ -343,3 +343,82 @@ def argmax(logits):
 
 def num_threads():
     return lib.orc_num_threads()
+
+
+# --------------------------------------------------------------------------- decoder layer / model
+class LlamaLayerOracle:
+    """One Llama-family decoder layer as the reference runs it for quantised weights
+    (src/layers/decoder_layer.h:101-170, attention.h:267-496, mlp_llama.h:197-290):
+    fp32 activations end to end; prefill attention through the flash-style path (Q/K/V
+    narrowed to bf16, attention.h:1121-1188), decode attention over the FP16/INT8 cache.
+
+    rounding="bf16" instead narrows activations to bf16 where the GPU pipeline does
+    (normalised input, qkv, rotated q, attention output, SwiGLU output), which isolates
+    kernel error from the declared precision of the activation format."""
+
+    def __init__(self, hidden, inter, q_heads, kv_heads, head, wqkv, wo, wgateup, wdown, ln1, ln2, kv_int8=0,
+                 batch=1, max_seq=256, eps=1e-6, rope_base=10000, max_pos=2048, rounding="fp32"):
+        self.hidden, self.inter, self.qh, self.kvh, self.D = hidden, inter, q_heads, kv_heads, head
+        self.wqkv, self.wo, self.wgateup, self.wdown = wqkv, wo, wgateup, wdown
+        self.ln1, self.ln2, self.eps = f32(ln1), f32(ln2), eps
+        self.kc = KVCache(kv_int8, batch, kv_heads, max_seq, head)
+        self.vc = KVCache(kv_int8, batch, kv_heads, max_seq, head)
+        self.cos, self.sin = rope_tables(head, max_pos, rope_base)
+        self.rounding = rounding
+
+    def _r(self, x):
+        return round_bf16(x) if self.rounding == "bf16" else x
+
+    def _mm(self, w, a, **kw):
+        if isinstance(w, QWeight):
+            return qgemm(w, a, **kw)
+        return gemm_f32(a, w, **kw)
+
+    def forward(self, x, B, S, past):
+        x = f32(x)
+        T = B * S
+        qcols, kvcols = self.qh * self.D, self.kvh * self.D
+        xn = self._r(rmsnorm(x, self.ln1, self.eps))
+        qkv = self._r(self._mm(self.wqkv, xn))
+        stride = qkv.shape[1]
+        flat = qkv.reshape(-1)
+        lib.orc_rope_apply(C.c_void_p(flat.ctypes.data), C.c_void_p(flat.ctypes.data + qcols * 4), stride, stride,
+                           p(self.cos), p(self.sin), self.D // 2, p(i32([B, S, self.qh, self.D, self.kvh])),
+                           p(i32(np.arange(past, past + S))))
+        q = np.ascontiguousarray(qkv[:, :qcols])
+        k = np.ascontiguousarray(qkv[:, qcols:qcols + kvcols])
+        v = np.ascontiguousarray(qkv[:, qcols + kvcols:])
+        q = self._r(q)
+        scale = 1.0 / np.sqrt(self.D)
+        if past == 0 and S > 1:
+            att = flash_prefill(q, to_bf16(k), to_bf16(v), self.qh, self.kvh, self.D, [S] * B, [0] * B, scale)
+            for b in range(B):
+                self.kc.store(b, 0, k[b * S:(b + 1) * S])
+                self.vc.store(b, 0, v[b * S:(b + 1) * S])
+        else:
+            att = cross_attn_by_head(q, k, v, self.qh, self.kvh, self.D, [S] * B, [past] * B, scale, self.kc, self.vc)
+        att = self._r(att)
+        x1 = self._mm(self.wo, att, epi=EPI_RESIDENTIAL, res=x)
+        xn2 = self._r(rmsnorm(x1, self.ln2, 1e-6))
+        h = self._r(silu_sum(self._mm(self.wgateup, xn2)))
+        return self._mm(self.wdown, h, epi=EPI_RESIDENTIAL, res=x1)
+
+
+class LlamaModelOracle:
+    """Embedding (FP16 table) -> layers -> last-token final RMSNorm -> lm_head -> greedy argmax
+    (src/models/common_decoder.h:315-589, src/searchers/sampling.cpp:22-131)."""
+
+    def __init__(self, layers, embedding_fp16, final_norm, lm_head_f32, eps=1e-6):
+        self.layers, self.emb, self.fn, self.lm, self.eps = layers, embedding_fp16, f32(final_norm), lm_head_f32, eps
+        self.rounding = layers[0].rounding
+
+    def step(self, ids, B, S, past):
+        x = from_fp16(self.emb[np.asarray(ids).reshape(-1)])
+        for L in self.layers:
+            x = L.forward(x, B, S, past)
+        last = x.reshape(B, S, -1)[:, -1, :]
+        xn = rmsnorm(last, self.fn, self.eps)
+        if self.rounding == "bf16":
+            xn = round_bf16(xn)
+        logits = gemm_f32(xn, self.lm)
+        return logits, argmax(logits)

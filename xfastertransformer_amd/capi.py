@@ -293,3 +293,79 @@ def attention(cache, q_dev, q_stride, out_dev, o_stride, out_dtype, B, S, q_head
               stream=None):
     check(lib.xfthip_attention(cache.h, q_dev, q_stride, out_dev, o_stride, out_dtype, B, S, q_heads,
                                C.c_float(scale), past, past_dev, stream))
+
+
+# ---------------------------------------------------------------------------- model driver
+class ModelConfig(C.Structure):
+    _fields_ = [("layers", C.c_int), ("hidden", C.c_int), ("intermediate", C.c_int), ("q_heads", C.c_int),
+                ("kv_heads", C.c_int), ("head_size", C.c_int), ("vocab", C.c_int), ("max_batch", C.c_int),
+                ("max_seq", C.c_int), ("max_tokens", C.c_int), ("max_pos_embed", C.c_int), ("rope_base", C.c_int),
+                ("kv_dtype", C.c_int), ("rms_eps", C.c_float)]
+
+
+class Model:
+    def __init__(self, layers, hidden, intermediate, q_heads, kv_heads, head_size=128, vocab=0, max_batch=1,
+                 max_seq=256, max_tokens=None, max_pos_embed=2048, rope_base=10000, kv_dtype=FP16, rms_eps=1e-6):
+        self.cfg = ModelConfig(layers, hidden, intermediate, q_heads, kv_heads, head_size, vocab, max_batch, max_seq,
+                               max_tokens or max_batch * max_seq, max(max_pos_embed, max_seq), rope_base, kv_dtype,
+                               rms_eps)
+        h = C.c_void_p()
+        check(lib.xfthip_model_create(C.byref(self.cfg), C.byref(h)))
+        self.h = h
+        self._keep = []
+
+    def set_layer(self, idx, qkv, o, gateup, down, ln1, ln2, qkv_bias=None, o_bias=None):
+        self._keep += [qkv, o, gateup, down]
+        f = lambda a: None if a is None else np.ascontiguousarray(a, np.float32)
+        ln1, ln2, qkv_bias, o_bias = f(ln1), f(ln2), f(qkv_bias), f(o_bias)
+        check(lib.xfthip_model_set_layer(self.h, idx, qkv.h, o.h, gateup.h, down.h, _hp(ln1), _hp(ln2), _hp(qkv_bias),
+                                         _hp(o_bias)))
+
+    def set_head(self, embedding_fp16, final_norm, lm_head):
+        self._keep.append(lm_head)
+        e = np.ascontiguousarray(embedding_fp16, np.uint16)
+        fn = np.ascontiguousarray(final_norm, np.float32)
+        check(lib.xfthip_model_set_head(self.h, _hp(e), _hp(fn), lm_head.h))
+
+    def layer_forward(self, idx, x_in_dev, x_out_dev, B, S, past, stride=None, stream=None):
+        stride = stride or self.cfg.hidden
+        check(lib.xfthip_model_layer_forward(self.h, idx, x_in_dev, stride, x_out_dev, stride, B, S, past, stream))
+
+    def prefill(self, ids, want_logits=False, stream=None):
+        ids = np.ascontiguousarray(ids, np.int32)
+        B, S = ids.shape
+        logits = np.empty((B, self.cfg.vocab), np.float32) if want_logits else None
+        check(lib.xfthip_model_prefill(self.h, _hp(ids), B, S, _hp(logits), stream))
+        return self.last_ids(B), logits
+
+    def decode(self, steps, B, stream=None):
+        out = np.empty((steps, B), np.int32)
+        check(lib.xfthip_model_decode(self.h, steps, _hp(out), stream))
+        return out
+
+    def decode_untracked(self, steps, stream=None):
+        check(lib.xfthip_model_decode(self.h, steps, None, stream))
+
+    def last_ids(self, B):
+        ids = np.empty(B, np.int32)
+        pos = C.c_int()
+        check(lib.xfthip_model_last_ids(self.h, _hp(ids), C.byref(pos)))
+        return ids
+
+    def logits(self, B):
+        ptr = C.c_void_p()
+        check(lib.xfthip_model_logits(self.h, C.byref(ptr)))
+        out = np.empty((B, self.cfg.vocab), np.float32)
+        check(lib.xfthip_memcpy_d2h(_hp(out), ptr, C.c_size_t(out.nbytes), None))
+        return out
+
+    def free(self):
+        if self.h is not None:
+            lib.xfthip_model_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass

@@ -307,6 +307,11 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
 
 static float *g_ws = nullptr;
 
+int attention_workspace_init() {
+    if (g_ws == nullptr) XFT_CHECK_HIP(hipMalloc((void **)&g_ws, (size_t)kWsSlots * kSlotFloats * sizeof(float)));
+    return 0;
+}
+
 } // namespace xfthip
 
 using namespace xfthip;
@@ -351,9 +356,8 @@ extern "C" int xfthip_attention(xfthip_kvcache_t c, const void *q, int qStride, 
     if (nsplit < 1) nsplit = 1;
     while (nsplit > 1 && (size_t)wgs * nsplit > (size_t)kWsSlots) --nsplit;
     p.nsplit = nsplit;
-    if (nsplit > 1 && g_ws == nullptr) {
-        XFT_CHECK_HIP(hipMalloc((void **)&g_ws, (size_t)kWsSlots * kSlotFloats * sizeof(float)));
-    }
+    if (nsplit > 1)
+        if (int rc = attention_workspace_init()) return rc;
     p.ws = g_ws;
     dim3 grid(nsplit, c->kv.H * p.CG, B);
     if (c->kv.int8)

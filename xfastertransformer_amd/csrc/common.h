@@ -121,5 +121,12 @@ __device__ inline void store_from_f32(void *p, int dtype, size_t idx, float v) {
 __device__ inline float fast_exp(float x) { return __expf(x); }
 
 int device_cu_count();
+// allocates the split-KV merge workspace of the attention kernel (idempotent; must not run
+// during stream capture)
+int attention_workspace_init();
 
 } // namespace xfthip
+
+struct xfthip_weight {
+    xfthip::PackedWeight pw;
+};

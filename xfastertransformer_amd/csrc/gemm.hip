@@ -1,10 +1,6 @@
 // C-ABI entry points of the weight-only GEMM: argument checks and kernel selection.
 #include "qgemm.h"
 
-struct xfthip_weight {
-    xfthip::PackedWeight pw;
-};
-
 
 using namespace xfthip;
 

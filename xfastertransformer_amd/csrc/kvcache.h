@@ -2,6 +2,8 @@
 #pragma once
 #include "common.h"
 
+struct xfthip_kvcache;
+
 namespace xfthip {
 
 // keys   : [B][H][S][D]                 (S = maxSeq rounded up to 32)
@@ -23,6 +25,13 @@ __host__ __device__ inline int v_slot(int t) {
     return ((t >> 2) & 3) * 8 + (t >> 4) * 4 + (t & 3);
 }
 
+} // namespace xfthip
+
+namespace xfthip {
+// xfthip_rope_kvstore with the option of leaving the query block alone (a second append of the
+// same rows into another cache must not rotate q twice)
+int rope_kvstore_impl(xfthip_kvcache *c, void *qkv, int dtype, int stride, int B, int S, int qHeads, const float *embCos,
+        const float *embSin, int past, const int *past_dev, bool rotate_q, hipStream_t stream);
 } // namespace xfthip
 
 struct xfthip_kvcache {

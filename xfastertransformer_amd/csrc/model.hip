@@ -1,0 +1,420 @@
+// Decoder-layer and whole-model drivers: the order of kernels one Llama-family layer runs,
+// the prefill pass and the graph-captured greedy decode step.  Replaces
+// Decoder::forwardAttention / forwardFFN, CommonDecoder::forward and greedySearch of the
+// reference (src/layers/decoder_layer.h, src/models/common_decoder.h:315-589,
+// src/searchers/sampling.cpp:22-131).
+//
+// Activation flow of one layer (residual stream x in fp32, GEMM operands in bf16):
+//   xn  = rmsnorm(x)                       bf16
+//   qkv = xn * Wqkv (+bias)                bf16   [tokens, (q + 2 kv) * head]
+//   rope(q, k); append k, v to the cache   (k goes to the cache from fp32 registers)
+//   att = attention(q, cache)              bf16
+//   x   = att * Wo (+bias) + x             fp32   (residual epilogue)
+//   xn  = rmsnorm(x, eps 1e-6)             bf16
+//   h   = silu(xn * Wgate) * (xn * Wup)    bf16   (fused into the cat GEMM's epilogue)
+//   x   = h * Wdown + x                    fp32
+#include <string.h>
+
+#include <vector>
+
+#include "kvcache.h"
+
+namespace xfthip {
+
+struct LayerW {
+    xfthip_weight_t qkv = nullptr, o = nullptr, gateup = nullptr, down = nullptr;
+    float *ln1 = nullptr, *ln2 = nullptr, *qkv_bias = nullptr, *o_bias = nullptr;
+};
+
+__global__ void embed_kernel(const uint16_t *__restrict__ table, const int *__restrict__ ids, float *__restrict__ x,
+        int hidden, int vocab) {
+    const int tok = blockIdx.x;
+    int id = ids[tok];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    const uint16_t *row = table + (size_t)id * hidden;
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) x[(size_t)tok * hidden + c] = fp16_bits_to_f32(row[c]);
+}
+
+// rows of the last token of every sequence -> compact [B, hidden]
+__global__ void gather_last_kernel(const float *__restrict__ x, float *__restrict__ out, int S, int hidden) {
+    const int b = blockIdx.x;
+    const float *row = x + ((size_t)b * S + S - 1) * hidden;
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) out[(size_t)b * hidden + c] = row[c];
+}
+
+// first maximum per row: strict '>' inside a thread's ascending scan, lower index wins ties
+// across threads
+__global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ logits, int cols, int *__restrict__ ids) {
+    __shared__ float sv[1024];
+    __shared__ int si[1024];
+    const float *p = logits + (size_t)blockIdx.x * cols;
+    float bv = -INFINITY;
+    int bi = 0x7FFFFFFF;
+    for (int j = threadIdx.x; j < cols; j += blockDim.x) {
+        const float v = p[j];
+        if (v > bv || bi == 0x7FFFFFFF) {
+            bv = v;
+            bi = j;
+        }
+    }
+    sv[threadIdx.x] = bv;
+    si[threadIdx.x] = bi;
+    __syncthreads();
+    for (int s = blockDim.x >> 1; s > 0; s >>= 1) {
+        if (threadIdx.x < s) {
+            const float ov = sv[threadIdx.x + s];
+            const int oi = si[threadIdx.x + s];
+            if (ov > sv[threadIdx.x] || (ov == sv[threadIdx.x] && oi < si[threadIdx.x])) {
+                sv[threadIdx.x] = ov;
+                si[threadIdx.x] = oi;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) ids[blockIdx.x] = si[0];
+}
+
+__global__ void advance_kernel(int *pos, int n, int by) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) pos[i] += by;
+}
+
+__global__ void fill_int_kernel(int *p, int n, int v) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+__global__ void record_ids_kernel(const int *ids, int *log, const int *step, int B) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < B) log[(size_t)step[0] * B + i] = ids[i];
+}
+
+} // namespace xfthip
+
+using namespace xfthip;
+
+struct xfthip_model {
+    xfthip_model_config cfg;
+    std::vector<LayerW> layers;
+    std::vector<xfthip_kvcache_t> caches;
+    // INT8 KV: the first-token pass attends over unquantised keys/values, as the reference's
+    // flash path does on its bf16 copies (src/layers/attention.h:1121-1188); they live here
+    xfthip_kvcache_t prefill_cache = nullptr;
+    float *cosT = nullptr, *sinT = nullptr;
+    // scratch
+    uint16_t *xn = nullptr, *qkv = nullptr, *att = nullptr, *h = nullptr;
+    float *x = nullptr, *xlast = nullptr, *logits = nullptr;
+    int *ids = nullptr, *pos = nullptr, *step = nullptr, *idlog = nullptr;
+    int idlog_cap = 0;
+    // head
+    uint16_t *embedding = nullptr;
+    float *final_norm = nullptr;
+    xfthip_weight_t lm_head = nullptr;
+    // decode state
+    int cur_B = 0, cur_pos = 0;
+    hipGraphExec_t graph = nullptr;
+    int graph_B = 0;
+    hipStream_t graph_stream = nullptr;
+};
+
+static int upload_f32(float **dst, const float *src, size_t n) {
+    if (*dst) {
+        (void)hipFree(*dst);
+        *dst = nullptr;
+    }
+    if (!src) return 0;
+    XFT_CHECK_HIP(hipMalloc((void **)dst, n * sizeof(float)));
+    XFT_CHECK_HIP(hipMemcpy(*dst, src, n * sizeof(float), hipMemcpyHostToDevice));
+    return 0;
+}
+
+// one layer on device buffers; x is updated in place (x_in may differ from x_out)
+static int layer_forward(xfthip_model *m, int idx, const float *x_in, int in_stride, float *x_out, int out_stride, int B,
+        int S, int past, const int *past_dev, hipStream_t st) {
+    const xfthip_model_config &c = m->cfg;
+    const LayerW &L = m->layers[idx];
+    XFT_REQUIRE(L.qkv && L.o && L.gateup && L.down && L.ln1 && L.ln2, "layer %d has no weights attached", idx);
+    const int T = B * S;
+    const int qcols = c.q_heads * c.head_size, kvcols = c.kv_heads * c.head_size;
+    const int qkv_cols = qcols + 2 * kvcols;
+    int rc;
+    if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, x_in, XFTHIP_F32, L.ln1, T, c.hidden, in_stride, c.hidden, c.rms_eps, st))) return rc;
+    if ((rc = xfthip_gemm(L.qkv, T, m->xn, c.hidden, m->qkv, qkv_cols, XFTHIP_BF16, L.qkv_bias ? XFTHIP_EPI_BIAS : XFTHIP_EPI_NONE,
+                 L.qkv_bias, nullptr, 0, XFTHIP_F32, 1.0f, st)))
+        return rc;
+    if ((rc = xfthip_rope_kvstore(m->caches[idx], m->qkv, XFTHIP_BF16, qkv_cols, B, S, c.q_heads, m->cosT, m->sinT, past, past_dev, st)))
+        return rc;
+    xfthip_kvcache_t attend = m->caches[idx];
+    if (c.kv_dtype == XFTHIP_INT8 && S > 1 && past == 0 && past_dev == nullptr) {
+        if ((rc = rope_kvstore_impl(m->prefill_cache, m->qkv, XFTHIP_BF16, qkv_cols, B, S, c.q_heads, m->cosT, m->sinT, 0, nullptr,
+                     false, st)))
+            return rc;
+        attend = m->prefill_cache;
+    }
+    if ((rc = xfthip_attention(attend, m->qkv, qkv_cols, m->att, qcols, XFTHIP_BF16, B, S, c.q_heads,
+                 1.0f / sqrtf((float)c.head_size), past, past_dev, st)))
+        return rc;
+    if ((rc = xfthip_gemm(L.o, T, m->att, qcols, x_out, out_stride, XFTHIP_F32, XFTHIP_EPI_RESIDENTIAL, L.o_bias, x_in, in_stride,
+                 XFTHIP_F32, 1.0f, st)))
+        return rc;
+    if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, x_out, XFTHIP_F32, L.ln2, T, c.hidden, out_stride, c.hidden, 1e-6f, st))) return rc;
+    if ((rc = xfthip_gemm_gateup_silu(L.gateup, T, m->xn, c.hidden, m->h, c.intermediate, XFTHIP_BF16, st))) return rc;
+    if ((rc = xfthip_gemm(L.down, T, m->h, c.intermediate, x_out, out_stride, XFTHIP_F32, XFTHIP_EPI_RESIDENTIAL, nullptr, x_out,
+                 out_stride, XFTHIP_F32, 1.0f, st)))
+        return rc;
+    return 0;
+}
+
+static int head_forward(xfthip_model *m, const float *xrows, int B, hipStream_t st) {
+    const xfthip_model_config &c = m->cfg;
+    int rc;
+    if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, xrows, XFTHIP_F32, m->final_norm, B, c.hidden, c.hidden, c.hidden, c.rms_eps, st))) return rc;
+    if ((rc = xfthip_gemm(m->lm_head, B, m->xn, c.hidden, m->logits, c.vocab, XFTHIP_F32, XFTHIP_EPI_NONE, nullptr, nullptr, 0, XFTHIP_F32,
+                 1.0f, st)))
+        return rc;
+    return xfthip_argmax(m->logits, B, c.vocab, m->ids, st);
+}
+
+// the decode step that gets captured: everything reads its position from device memory
+static int decode_step(xfthip_model *m, int B, hipStream_t st) {
+    const xfthip_model_config &c = m->cfg;
+    hipLaunchKernelGGL(record_ids_kernel, dim3((B + 63) / 64), dim3(64), 0, st, m->ids, m->idlog, m->step, B);
+    hipLaunchKernelGGL(embed_kernel, dim3(B), dim3(256), 0, st, m->embedding, m->ids, m->x, c.hidden, c.vocab);
+    for (int l = 0; l < c.layers; ++l)
+        if (int rc = layer_forward(m, l, m->x, c.hidden, m->x, c.hidden, B, 1, 0, m->pos, st)) return rc;
+    if (int rc = head_forward(m, m->x, B, st)) return rc;
+    hipLaunchKernelGGL(advance_kernel, dim3((B + 63) / 64), dim3(64), 0, st, m->pos, B, 1);
+    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(64), 0, st, m->step, 1, 1);
+    XFT_CHECK_HIP(hipGetLastError());
+    return 0;
+}
+
+extern "C" {
+
+int xfthip_argmax(const float *logits, int rows, int cols, int *ids_dev, xfthip_stream_t stream) {
+    XFT_REQUIRE(logits && ids_dev && rows > 0 && cols > 0, "xfthip_argmax: bad argument");
+    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, logits, cols, ids_dev);
+    XFT_CHECK_HIP(hipGetLastError());
+    return 0;
+}
+
+int xfthip_model_create(const xfthip_model_config *cfg, xfthip_model_t *out) {
+    XFT_REQUIRE(cfg && out, "xfthip_model_create: null argument");
+    const xfthip_model_config &c = *cfg;
+    XFT_REQUIRE(c.layers > 0 && c.hidden > 0 && c.intermediate > 0, "xfthip_model_create: bad sizes");
+    XFT_REQUIRE(c.head_size == 128, "xfthip_model_create: head size %d unsupported (128 only)", c.head_size);
+    XFT_REQUIRE(c.q_heads > 0 && c.kv_heads > 0 && c.q_heads % c.kv_heads == 0, "xfthip_model_create: bad head counts");
+    XFT_REQUIRE(c.q_heads / c.kv_heads <= 16, "xfthip_model_create: more than 16 query heads per KV head");
+    XFT_REQUIRE(c.hidden % 8 == 0 && c.intermediate % 16 == 0, "xfthip_model_create: hidden %% 8 and intermediate %% 16 must be 0");
+    XFT_REQUIRE(c.max_batch > 0 && c.max_seq > 0 && c.max_tokens >= c.max_batch, "xfthip_model_create: bad batch/sequence limits");
+    XFT_REQUIRE(c.max_pos_embed >= c.max_seq, "xfthip_model_create: max_pos_embed %d < max_seq %d", c.max_pos_embed, c.max_seq);
+    xfthip_model *m = new xfthip_model();
+    m->cfg = c;
+    m->layers.resize(c.layers);
+    m->caches.assign(c.layers, nullptr);
+    auto fail = [&](int rc) {
+        xfthip_model_destroy(m);
+        return rc;
+    };
+    for (int l = 0; l < c.layers; ++l)
+        if (int rc = xfthip_kvcache_create(c.kv_dtype, c.max_batch, c.kv_heads, c.max_seq, c.head_size, &m->caches[l])) return fail(rc);
+    if (int rc = attention_workspace_init()) return fail(rc);
+    if (c.kv_dtype == XFTHIP_INT8)
+        if (int rc = xfthip_kvcache_create(XFTHIP_FP16, c.max_batch, c.kv_heads, c.max_seq, c.head_size, &m->prefill_cache)) return fail(rc);
+    if (int rc = xfthip_rope_tables_create(c.head_size, c.max_pos_embed, c.rope_base, 1.0f, &m->cosT, &m->sinT)) return fail(rc);
+    const size_t T = c.max_tokens;
+    const size_t qkv_cols = (size_t)(c.q_heads + 2 * c.kv_heads) * c.head_size;
+    bool ok = hipMalloc((void **)&m->xn, T * (c.hidden > c.intermediate ? c.hidden : c.intermediate) * 2) == hipSuccess
+            && hipMalloc((void **)&m->qkv, T * qkv_cols * 2) == hipSuccess
+            && hipMalloc((void **)&m->att, T * c.q_heads * c.head_size * 2) == hipSuccess
+            && hipMalloc((void **)&m->h, T * c.intermediate * 2) == hipSuccess
+            && hipMalloc((void **)&m->x, T * c.hidden * 4) == hipSuccess
+            && hipMalloc((void **)&m->xlast, (size_t)c.max_batch * c.hidden * 4) == hipSuccess
+            && hipMalloc((void **)&m->ids, (size_t)(T > 64 ? T : 64) * 4) == hipSuccess
+            && hipMalloc((void **)&m->pos, (size_t)c.max_batch * 4) == hipSuccess
+            && hipMalloc((void **)&m->step, 64) == hipSuccess;
+    if (ok && c.vocab > 0) ok = hipMalloc((void **)&m->logits, (size_t)c.max_batch * c.vocab * 4) == hipSuccess;
+    if (!ok) {
+        set_error("xfthip_model_create: scratch allocation failed");
+        return fail(1);
+    }
+    m->idlog_cap = c.max_seq + 1;
+    if (hipMalloc((void **)&m->idlog, (size_t)m->idlog_cap * c.max_batch * 4) != hipSuccess) {
+        set_error("xfthip_model_create: id log allocation failed");
+        return fail(1);
+    }
+    *out = m;
+    return 0;
+}
+
+int xfthip_model_destroy(xfthip_model_t m) {
+    if (!m) return 0;
+    if (m->graph) (void)hipGraphExecDestroy(m->graph);
+    for (auto c : m->caches) xfthip_kvcache_destroy(c);
+    xfthip_kvcache_destroy(m->prefill_cache);
+    for (auto &L : m->layers) {
+        if (L.ln1) (void)hipFree(L.ln1);
+        if (L.ln2) (void)hipFree(L.ln2);
+        if (L.qkv_bias) (void)hipFree(L.qkv_bias);
+        if (L.o_bias) (void)hipFree(L.o_bias);
+    }
+    void *bufs[] = {m->cosT, m->sinT, m->xn, m->qkv, m->att, m->h, m->x, m->xlast, m->logits, m->ids, m->pos, m->step, m->idlog,
+            m->embedding, m->final_norm};
+    for (void *b : bufs)
+        if (b) (void)hipFree(b);
+    delete m;
+    return 0;
+}
+
+int xfthip_model_set_layer(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthip_weight_t o, xfthip_weight_t gateup,
+        xfthip_weight_t down, const float *ln1_host, const float *ln2_host, const float *qkv_bias_host,
+        const float *o_bias_host) {
+    XFT_REQUIRE(m && qkv && o && gateup && down && ln1_host && ln2_host, "xfthip_model_set_layer: null argument");
+    XFT_REQUIRE(idx >= 0 && idx < m->cfg.layers, "xfthip_model_set_layer: layer %d out of range", idx);
+    const xfthip_model_config &c = m->cfg;
+    const int qcols = c.q_heads * c.head_size, qkv_cols = qcols + 2 * c.kv_heads * c.head_size;
+    XFT_REQUIRE(qkv->pw.K == c.hidden && qkv->pw.N == qkv_cols, "xfthip_model_set_layer: qkv weight is [%d,%d], expected [%d,%d]",
+            qkv->pw.K, qkv->pw.N, c.hidden, qkv_cols);
+    XFT_REQUIRE(o->pw.K == qcols && o->pw.N == c.hidden, "xfthip_model_set_layer: o weight is [%d,%d], expected [%d,%d]", o->pw.K,
+            o->pw.N, qcols, c.hidden);
+    XFT_REQUIRE(gateup->pw.K == c.hidden && gateup->pw.N == 2 * c.intermediate && (gateup->pw.flags & XFTHIP_WF_GATEUP),
+            "xfthip_model_set_layer: gate/up weight must be [%d,%d] created with XFTHIP_WF_GATEUP", c.hidden, 2 * c.intermediate);
+    XFT_REQUIRE(down->pw.K == c.intermediate && down->pw.N == c.hidden, "xfthip_model_set_layer: down weight is [%d,%d], expected [%d,%d]",
+            down->pw.K, down->pw.N, c.intermediate, c.hidden);
+    LayerW &L = m->layers[idx];
+    L.qkv = qkv;
+    L.o = o;
+    L.gateup = gateup;
+    L.down = down;
+    int rc;
+    if ((rc = upload_f32(&L.ln1, ln1_host, c.hidden))) return rc;
+    if ((rc = upload_f32(&L.ln2, ln2_host, c.hidden))) return rc;
+    if ((rc = upload_f32(&L.qkv_bias, qkv_bias_host, qkv_cols))) return rc;
+    if ((rc = upload_f32(&L.o_bias, o_bias_host, c.hidden))) return rc;
+    if (m->graph) {
+        (void)hipGraphExecDestroy(m->graph);
+        m->graph = nullptr;
+    }
+    return 0;
+}
+
+int xfthip_model_set_head(xfthip_model_t m, const uint16_t *embedding_fp16_host, const float *final_norm_host,
+        xfthip_weight_t lm_head) {
+    XFT_REQUIRE(m && embedding_fp16_host && final_norm_host && lm_head, "xfthip_model_set_head: null argument");
+    const xfthip_model_config &c = m->cfg;
+    XFT_REQUIRE(c.vocab > 0, "xfthip_model_set_head: model was created without a vocabulary");
+    XFT_REQUIRE(lm_head->pw.K == c.hidden && lm_head->pw.N == c.vocab, "xfthip_model_set_head: lm_head is [%d,%d], expected [%d,%d]",
+            lm_head->pw.K, lm_head->pw.N, c.hidden, c.vocab);
+    if (m->embedding) (void)hipFree(m->embedding);
+    m->embedding = nullptr;
+    const size_t eb = (size_t)c.vocab * c.hidden * 2;
+    XFT_CHECK_HIP(hipMalloc((void **)&m->embedding, eb));
+    XFT_CHECK_HIP(hipMemcpy(m->embedding, embedding_fp16_host, eb, hipMemcpyHostToDevice));
+    if (int rc = upload_f32(&m->final_norm, final_norm_host, c.hidden)) return rc;
+    m->lm_head = lm_head;
+    return 0;
+}
+
+int xfthip_model_layer_forward(xfthip_model_t m, int idx, const float *x_in, int in_stride, float *x_out,
+        int out_stride, int B, int S, int past, xfthip_stream_t stream) {
+    XFT_REQUIRE(m && x_in && x_out, "xfthip_model_layer_forward: null argument");
+    XFT_REQUIRE(idx >= 0 && idx < m->cfg.layers, "xfthip_model_layer_forward: layer %d out of range", idx);
+    XFT_REQUIRE(B > 0 && B <= m->cfg.max_batch && S > 0 && B * S <= m->cfg.max_tokens,
+            "xfthip_model_layer_forward: B=%d S=%d exceed max_batch=%d / max_tokens=%d", B, S, m->cfg.max_batch, m->cfg.max_tokens);
+    XFT_REQUIRE(past >= 0 && past + S <= m->cfg.max_seq, "xfthip_model_layer_forward: past %d + S %d exceeds max_seq %d", past, S,
+            m->cfg.max_seq);
+    XFT_REQUIRE(in_stride >= m->cfg.hidden && out_stride >= m->cfg.hidden, "xfthip_model_layer_forward: stride smaller than hidden");
+    return layer_forward(m, idx, x_in, in_stride, x_out, out_stride, B, S, past, nullptr, (hipStream_t)stream);
+}
+
+int xfthip_model_prefill(xfthip_model_t m, const int *ids_host, int B, int S, float *logits_host, xfthip_stream_t stream) {
+    XFT_REQUIRE(m && ids_host, "xfthip_model_prefill: null argument");
+    const xfthip_model_config &c = m->cfg;
+    XFT_REQUIRE(m->embedding && m->lm_head, "xfthip_model_prefill: embedding / lm_head not set");
+    XFT_REQUIRE(B > 0 && B <= c.max_batch && S > 0 && B * S <= c.max_tokens && S <= c.max_seq,
+            "xfthip_model_prefill: B=%d S=%d exceed the model limits", B, S);
+    hipStream_t st = (hipStream_t)stream;
+    XFT_CHECK_HIP(hipMemcpyAsync(m->ids, ids_host, (size_t)B * S * 4, hipMemcpyHostToDevice, st));
+    hipLaunchKernelGGL(embed_kernel, dim3(B * S), dim3(256), 0, st, m->embedding, m->ids, m->x, c.hidden, c.vocab);
+    for (int l = 0; l < c.layers; ++l)
+        if (int rc = layer_forward(m, l, m->x, c.hidden, m->x, c.hidden, B, S, 0, nullptr, st)) return rc;
+    hipLaunchKernelGGL(gather_last_kernel, dim3(B), dim3(256), 0, st, m->x, m->xlast, S, c.hidden);
+    if (int rc = head_forward(m, m->xlast, B, st)) return rc;
+    hipLaunchKernelGGL(fill_int_kernel, dim3((B + 63) / 64), dim3(64), 0, st, m->pos, B, S);
+    hipLaunchKernelGGL(fill_int_kernel, dim3(1), dim3(64), 0, st, m->step, 1, 0);
+    XFT_CHECK_HIP(hipGetLastError());
+    XFT_CHECK_HIP(hipStreamSynchronize(st));
+    if (logits_host) XFT_CHECK_HIP(hipMemcpy(logits_host, m->logits, (size_t)B * c.vocab * 4, hipMemcpyDeviceToHost));
+    m->cur_B = B;
+    m->cur_pos = S;
+    return 0;
+}
+
+int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_stream_t stream) {
+    XFT_REQUIRE(m && steps > 0, "xfthip_model_decode: bad argument");
+    XFT_REQUIRE(m->cur_B > 0, "xfthip_model_decode: call xfthip_model_prefill first");
+    const xfthip_model_config &c = m->cfg;
+    XFT_REQUIRE(m->cur_pos + steps <= c.max_seq, "xfthip_model_decode: position %d + %d steps exceeds max_seq %d", m->cur_pos, steps,
+            c.max_seq);
+    XFT_REQUIRE(steps <= m->idlog_cap, "xfthip_model_decode: too many steps for the id log");
+    hipStream_t st = (hipStream_t)stream;
+    const int B = m->cur_B;
+    hipLaunchKernelGGL(fill_int_kernel, dim3(1), dim3(64), 0, st, m->step, 1, 0);
+    if (m->graph == nullptr || m->graph_B != B || m->graph_stream != st) {
+        if (m->graph) {
+            (void)hipGraphExecDestroy(m->graph);
+            m->graph = nullptr;
+        }
+        // Capture needs a real stream; every position-dependent value is read from device
+        // memory, so the same graph serves every later step.
+        hipStream_t cap = st;
+        bool own = false;
+        if (cap == nullptr) {
+            XFT_CHECK_HIP(hipStreamCreate(&cap));
+            own = true;
+            XFT_CHECK_HIP(hipDeviceSynchronize());
+        }
+        hipGraph_t g = nullptr;
+        XFT_CHECK_HIP(hipStreamBeginCapture(cap, hipStreamCaptureModeThreadLocal));
+        int rc = decode_step(m, B, cap);
+        hipError_t e = hipStreamEndCapture(cap, &g);
+        if (rc != 0 || e != hipSuccess) {
+            if (g) (void)hipGraphDestroy(g);
+            if (own) (void)hipStreamDestroy(cap);
+            if (rc == 0) set_error("xfthip_model_decode: graph capture failed: %s", hipGetErrorString(e));
+            return rc ? rc : 1;
+        }
+        e = hipGraphInstantiate(&m->graph, g, nullptr, nullptr, 0);
+        (void)hipGraphDestroy(g);
+        if (own) (void)hipStreamDestroy(cap);
+        XFT_CHECK_HIP(e);
+        m->graph_B = B;
+        m->graph_stream = st;
+    }
+    for (int i = 0; i < steps; ++i) XFT_CHECK_HIP(hipGraphLaunch(m->graph, st));
+    XFT_CHECK_HIP(hipStreamSynchronize(st));
+    if (ids_out_host) {
+        // the log holds the input id of every step; the outputs are rows 1..steps-1 plus the final ids
+        std::vector<int> log((size_t)steps * B);
+        XFT_CHECK_HIP(hipMemcpy(log.data(), m->idlog, log.size() * 4, hipMemcpyDeviceToHost));
+        for (int i = 0; i + 1 < steps; ++i) memcpy(ids_out_host + (size_t)i * B, log.data() + (size_t)(i + 1) * B, (size_t)B * 4);
+        XFT_CHECK_HIP(hipMemcpy(ids_out_host + (size_t)(steps - 1) * B, m->ids, (size_t)B * 4, hipMemcpyDeviceToHost));
+    }
+    m->cur_pos += steps;
+    return 0;
+}
+
+int xfthip_model_last_ids(xfthip_model_t m, int *ids_host, int *position) {
+    XFT_REQUIRE(m && m->cur_B > 0, "xfthip_model_last_ids: nothing generated yet");
+    if (ids_host) XFT_CHECK_HIP(hipMemcpy(ids_host, m->ids, (size_t)m->cur_B * 4, hipMemcpyDeviceToHost));
+    if (position) *position = m->cur_pos;
+    return 0;
+}
+
+int xfthip_model_logits(xfthip_model_t m, const float **logits_dev) {
+    XFT_REQUIRE(m && logits_dev && m->logits, "xfthip_model_logits: no logits");
+    *logits_dev = m->logits;
+    return 0;
+}
+
+} // extern "C"

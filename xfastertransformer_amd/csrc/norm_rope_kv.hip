@@ -56,6 +56,7 @@ struct RopeKvParams {
     int past;
     const int *past_dev;
     const int *positions; // optional explicit position per token (standalone rotary call)
+    int skip_q; // 1: query heads are left untouched
     KvView kv; // kv.k == nullptr: no append
     void *key; // standalone rotary: separate key pointer (qkv = query), else nullptr
     int kStride;
@@ -71,6 +72,7 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(RopeKvParams p) {
     const int past = p.past_dev ? p.past_dev[b] : p.past;
     const int pos = p.positions ? p.positions[tok] : past + s;
     const bool isq = head < p.qHeads;
+    if (isq && p.skip_q) return;
     const int kvh = head - p.qHeads;
 
     char *rowbase;
@@ -368,6 +370,15 @@ int xfthip_kvcache_import(xfthip_kvcache_t c, int which, const void *data_dev, c
 
 int xfthip_rope_kvstore(xfthip_kvcache_t c, void *qkv, int dtype, int stride, int B, int S, int qHeads,
         const float *embCos, const float *embSin, int past, const int *past_dev, xfthip_stream_t stream) {
+    return rope_kvstore_impl(c, qkv, dtype, stride, B, S, qHeads, embCos, embSin, past, past_dev, true, (hipStream_t)stream);
+}
+
+} // extern "C"
+
+namespace xfthip {
+
+int rope_kvstore_impl(xfthip_kvcache *c, void *qkv, int dtype, int stride, int B, int S, int qHeads, const float *embCos,
+        const float *embSin, int past, const int *past_dev, bool rotate_q, hipStream_t stream) {
     XFT_REQUIRE(c && qkv, "xfthip_rope_kvstore: null argument");
     XFT_REQUIRE(dtype == XFTHIP_F32 || dtype == XFTHIP_BF16, "xfthip_rope_kvstore: dtype must be f32 or bf16");
     XFT_REQUIRE((embCos == nullptr) == (embSin == nullptr), "xfthip_rope_kvstore: cos and sin go together");
@@ -391,7 +402,8 @@ int xfthip_rope_kvstore(xfthip_kvcache_t c, void *qkv, int dtype, int stride, in
     p.past = past;
     p.past_dev = past_dev;
     p.kv = c->kv;
-    return launch_rope(p, B * S, (hipStream_t)stream);
+    p.skip_q = rotate_q ? 0 : 1;
+    return launch_rope(p, B * S, stream);
 }
 
-} // extern "C"
+} // namespace xfthip

@@ -184,10 +184,6 @@ __global__ void colsum_kernel(int K, int N, int inter, const int8_t *__restrict_
 
 using namespace xfthip;
 
-struct xfthip_weight {
-    PackedWeight pw;
-};
-
 static size_t raw_bytes(int kind, int K, int N) {
     size_t e = (size_t)K * N;
     if (kind == XFTHIP_W_UINT4 || kind == XFTHIP_W_NF4) return e / 2;

@@ -1,0 +1,22 @@
+// xft::invokeRotaryEmbedding, source-compatible with the reference's
+// include/layers_rotary_embedding.h:23-33.  In-place rotate-half RoPE on host query / key buffers
+// of the element type named by dt (fp32 or bf16); embCos / embSin are fp32 [maxPosition, dim/2].
+#pragma once
+
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+
+#include "dtype.h"
+
+namespace xft {
+void invokeRotaryEmbedding(DataType dt,
+        const int64_t *positionIds, // [numTokens]
+        void *query, // [numTokens, headNum, headSize]
+        void *key, // [numTokens, numKvHeads, headSize]
+        const void *embCos, // [maxPosition, dim / 2]
+        const void *embSin, // [maxPosition, dim / 2]
+        const int dim, // rotary dimension
+        const int qStride, const int kStride, const int numTokens, const int headNum, const int headSize,
+        const int numKvHeads);
+} // namespace xft

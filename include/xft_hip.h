@@ -157,6 +157,15 @@ int xfthip_rotary_embedding(int dtype, const int *positions, void *query, void *
         const float *embSin, int dim, int qStride, int kStride, int numTokens, int headNum, int headSize,
         int numKvHeads, xfthip_stream_t stream);
 
+/*
+ * Same rotation with tables laid out as the public xft::invokeRotaryEmbedding takes them:
+ * [maxPosition, dim], the second half of a head reading columns [dim/2, dim)
+ * (src/layers/rotary_embedding_api.cpp:20-50).
+ */
+int xfthip_rotary_embedding_full(int dtype, const int *positions, void *query, void *key, const float *embCos,
+        const float *embSin, int dim, int qStride, int kStride, int numTokens, int headNum, int headSize,
+        int numKvHeads, xfthip_stream_t stream);
+
 /* ---- KV cache ----------------------------------------------------------------------- */
 /*
  * One layer's key and value cache for `batch` sequences.  Replaces KVCacheTensor<float16_t>
@@ -239,6 +248,11 @@ int xfthip_model_destroy(xfthip_model_t m);
 int xfthip_model_set_layer(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthip_weight_t o, xfthip_weight_t gateup,
         xfthip_weight_t down, const float *ln1_host, const float *ln2_host, const float *qkv_bias_host,
         const float *o_bias_host);
+/* the two halves of xfthip_model_set_layer, for callers that drive only one block of a layer
+ * (ln*_host may be NULL when that block is always run with do_norm = 0) */
+int xfthip_model_set_attention(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthip_weight_t o, const float *ln1_host,
+        const float *qkv_bias_host, const float *o_bias_host);
+int xfthip_model_set_mlp(xfthip_model_t m, int idx, xfthip_weight_t gateup, xfthip_weight_t down, const float *ln2_host);
 /*
  * Embedding table (host fp16 bit patterns [vocab, hidden], the reference keeps it in FP16:
  * src/layers/token_embedding.h:49-52), final RMSNorm weight (host fp32 [hidden]) and the
@@ -256,6 +270,20 @@ int xfthip_model_set_head(xfthip_model_t m, const uint16_t *embedding_fp16_host,
 int xfthip_model_layer_forward(xfthip_model_t m, int idx, const float *x_in, int in_stride, float *x_out,
         int out_stride, int B, int S, int past, xfthip_stream_t stream);
 /*
+ * The attention block alone: x_out = Attention(norm?(x_in)) * Wo + bias + x_in.  Replaces
+ * Attention::forward as xft::invokeAttentionLLaMA drives it (src/layers/attention.cpp:28-129:
+ * do_norm = 0 there; the decoder layer passes 1).
+ */
+int xfthip_model_attention_forward(xfthip_model_t m, int idx, const float *x_in, int in_stride, float *x_out,
+        int out_stride, int B, int S, int past, int do_norm, xfthip_stream_t stream);
+/*
+ * The MLP block alone: x_out = down(silu(gate(xn)) * up(xn)) + x_in with xn = norm?(x_in).
+ * Replaces LlamaMLP::forward as xft::invokeMLPLLaMA drives it (src/layers/mlp_llama.cpp:22-73:
+ * do_norm = 0 there).
+ */
+int xfthip_model_mlp_forward(xfthip_model_t m, int idx, const float *x_in, int in_stride, float *x_out, int out_stride,
+        int tokens, int do_norm, xfthip_stream_t stream);
+/*
  * Prefill: embeds ids_host [B, S] (host int32), runs every layer at positions 0..S-1, final
  * norm + lm_head on the last token of each sequence and greedy argmax (first maximum wins,
  * src/searchers/sampling.cpp:22-131).  The chosen ids stay on the device as the input of
@@ -269,6 +297,9 @@ int xfthip_model_prefill(xfthip_model_t m, const int *ids_host, int B, int S, fl
  * [steps, B] or NULL.  Must follow xfthip_model_prefill with the same B.
  */
 int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_stream_t stream);
+/* enable (default) or disable replaying the decode step as a captured HIP graph; with 0 every
+ * step launches its kernels one by one (for per-kernel profiling) */
+int xfthip_model_use_graph(xfthip_model_t m, int enable);
 /* ids chosen by the last prefill / decode call (host int32 [B]) and the current position */
 int xfthip_model_last_ids(xfthip_model_t m, int *ids_host, int *position);
 /* fp32 logits of the last step, device pointer [B, vocab] (valid until the next call) */

@@ -1,0 +1,191 @@
+"""The reference's public entry points (xft::invoke*, include/layers_*.h) served by the C++ host
+layer over the C-ABI, checked on the GPU against the CPU oracle.  Cases follow the reference's
+own tests: layers_decoder_test.cpp:25-60 and layers_attention_test.cpp:25-57 (prefill of 18 tokens
+then two decode steps), layers_mlp_test.cpp:24-123 (M in {1,2,4,6,10,16,18}, tolerance
+|d| > 0.01 and rel > 0.01 fails), rotary_embedding_test.cpp:28-57 (golden constants),
+rms_norm_test.cpp:23-45, gemm_kernel_ext_test.cpp:309-405 (bf16 invokeGemm, tolerance 0.5)."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BF16, INT8, INT4, NF4, FP32 = 1, 3, 5, 6, 0  # xft::DataType
+SILU, RMS = 3, 0
+P, F, I, B_ = C.c_void_p, C.c_float, C.c_int, C.c_bool
+
+
+@pytest.fixture(scope="module")
+def host():
+    C.CDLL(os.path.join(ROOT, "xfastertransformer_amd", "libxft_hip.so"), mode=C.RTLD_GLOBAL)
+    lib = C.CDLL(os.path.join(ROOT, "xfastertransformer_amd", "libxft_layers.so"))
+    f = lambda name, args: (setattr(getattr(lib, name), "argtypes", args), setattr(getattr(lib, name), "restype", None),
+                            getattr(lib, name))[2]
+    return dict(
+        layer=f("_ZN3xft16invokeLayerLLaMAENS_8DataTypeENS_14ActivationTypeENS_8NormTypeEiiiiiiiiiiiiPviPKviPKfS7_S5_S5_S5_S5_S7_S7_S5_S5_S5_S7_S7_S7_S7_",
+                [I] * 15 + [P, I, P, I] + [P] * 15),
+        attn=f("_ZN3xft20invokeAttentionLLaMAENS_8DataTypeEiiiiiiiiiiiPviPKviS3_S3_S3_S3_PKfS5_S5_S5_",
+               [I] * 12 + [P, I, P, I] + [P] * 8),
+        mlp=f("_ZN3xft14invokeMLPLLaMAENS_8DataTypeENS_14ActivationTypeEiiiPviPKviS4_S4_S4_", [I] * 5 + [P, I, P, I, P, P, P]),
+        gemm=f("_ZN3xft10invokeGemmENS_8DataTypeEbbiiifPviS1_fS1_iS1_S1_i", [I, B_, B_, I, I, I, F, P, I, P, F, P, I, P, P, I]),
+        rms=f("_ZN3xft13invokeRmsNormENS_8DataTypeEPvPKvS3_iiiif", [I, P, P, P, I, I, I, I, F]),
+        rope=f("_ZN3xft21invokeRotaryEmbeddingENS_8DataTypeEPKlPvS3_PKvS5_iiiiiii", [I, P, P, P, P, P] + [I] * 7),
+    )
+
+
+@pytest.fixture(scope="module")
+def orc():
+    from oracle import pyoracle
+    return pyoracle
+
+
+def ptr(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _cos(a, b):
+    a, b = a.astype(np.float64).ravel(), b.astype(np.float64).ravel()
+    return float(a @ b / np.sqrt((a @ a) * (b @ b)))
+
+
+def _layer_weights(rng, hidden, inter, qh, kvh, D):
+    qkv = (rng.standard_normal((hidden, (qh + 2 * kvh) * D)) * 0.02).astype(np.float32)
+    wo = (rng.standard_normal((qh * D, hidden)) * 0.02).astype(np.float32)
+    gate = (rng.standard_normal((hidden, inter)) * 0.02).astype(np.float32)
+    up = (rng.standard_normal((hidden, inter)) * 0.02).astype(np.float32)
+    down = (rng.standard_normal((inter, hidden)) * 0.02).astype(np.float32)
+    return qkv, wo, gate, up, down
+
+
+def _oracle_weight(orc, dt, W):
+    if dt == BF16:
+        return orc.round_bf16(W)
+    return orc.quantize({INT8: 0, INT4: 1, NF4: 2}[dt], W)
+
+
+@pytest.mark.parametrize("dt", [BF16, INT8, INT4])
+def test_invoke_layer_llama_prefill_and_two_decode_steps(host, orc, dt):
+    hidden, inter, qh, kvh, D = 1024, 2816, 8, 8, 128
+    rng = np.random.default_rng(dt)
+    qkv, wo, gate, up, down = _layer_weights(rng, hidden, inter, qh, kvh, D)
+    ln1 = rng.uniform(0.8, 1.2, hidden).astype(np.float32)
+    ln2 = rng.uniform(0.8, 1.2, hidden).astype(np.float32)
+    ow = [_oracle_weight(orc, dt, w) for w in (qkv, wo, np.concatenate([gate, up], 1), down)]
+    ref = orc.LlamaLayerOracle(hidden, inter, qh, kvh, D, *ow, ln1, ln2, max_seq=32)
+    qcols, kvcols = qh * D, kvh * D
+    S0, max_pos = 18, 32
+    past = 0
+    for step, S in enumerate((S0, 1, 1)):
+        x = rng.standard_normal((S, hidden)).astype(np.float32)
+        out = np.zeros_like(x)
+        host["layer"](dt, SILU, RMS, 1, S, D, qh, kvh, max_pos, max_pos, past, past + S, step, hidden, inter, ptr(out),
+                      hidden, ptr(x), hidden, ptr(ln1), None, ptr(qkv), C.c_void_p(qkv.ctypes.data + qcols * 4),
+                      C.c_void_p(qkv.ctypes.data + (qcols + kvcols) * 4), ptr(wo), ptr(ln2), None, ptr(gate), ptr(up),
+                      ptr(down), None, None, None, None)
+        exp = ref.forward(x, 1, S, past)
+        err = np.abs(out - exp)
+        assert _cos(out, exp) >= 0.9999 and err.max() < 5e-2 and np.sqrt((err ** 2).mean()) < 1e-2, (step, err.max())
+        past += S
+
+
+def test_invoke_attention_llama(host, orc):
+    hidden, qh, kvh, D = 1024, 8, 2, 128
+    rng = np.random.default_rng(7)
+    qkv = (rng.standard_normal((hidden, (qh + 2 * kvh) * D)) * 0.02).astype(np.float32)
+    wo = (rng.standard_normal((qh * D, hidden)) * 0.02).astype(np.float32)
+    qb = (rng.standard_normal(qh * D) * 0.1).astype(np.float32)
+    ob = (rng.standard_normal(hidden) * 0.1).astype(np.float32)
+    qcols, kvcols = qh * D, kvh * D
+    kc, vc = orc.KVCache(0, 1, kvh, 32, D), orc.KVCache(0, 1, kvh, 32, D)
+    cos, sin = orc.rope_tables(D, 64)
+    wq, wo_r = orc.round_bf16(qkv), orc.round_bf16(wo)
+    bias = np.concatenate([qb, np.zeros(2 * kvcols, np.float32)])
+    past = 0
+    for step, S in enumerate((18, 1, 1)):
+        x = rng.standard_normal((S, hidden)).astype(np.float32)
+        out = np.zeros_like(x)
+        host["attn"](BF16, 1, S, D, qh, kvh, 32, 64, past, past + S, step, hidden, ptr(out), hidden, ptr(x), hidden,
+                     ptr(qkv), C.c_void_p(qkv.ctypes.data + qcols * 4), C.c_void_p(qkv.ctypes.data + (qcols + kvcols) * 4),
+                     ptr(wo), ptr(qb), None, None, ptr(ob))
+        proj = orc.gemm_f32(x, wq, orc.EPI_BIAS, bias=bias)
+        flat = proj.reshape(-1)
+        orc.lib.orc_rope_apply(C.c_void_p(flat.ctypes.data), C.c_void_p(flat.ctypes.data + qcols * 4), proj.shape[1],
+                               proj.shape[1], orc.p(cos), orc.p(sin), D // 2, orc.p(orc.i32([1, S, qh, D, kvh])),
+                               orc.p(orc.i32(np.arange(past, past + S))))
+        att = orc.cross_attn_by_head(proj[:, :qcols].copy(), proj[:, qcols:qcols + kvcols].copy(),
+                                     proj[:, qcols + kvcols:].copy(), qh, kvh, D, [S], [past], 1 / np.sqrt(D), kc, vc)
+        exp = orc.gemm_f32(att, wo_r, orc.EPI_RESIDENTIAL, bias=ob, res=x)
+        assert np.abs(out - exp).max() < 3e-2 and _cos(out, exp) >= 0.9999, (step, np.abs(out - exp).max())
+        past += S
+
+
+@pytest.mark.parametrize("M", [1, 2, 4, 6, 10, 16, 18])
+def test_invoke_mlp_llama_reference_test_spec(host, orc, M):
+    hidden, inter = 1024, 2816
+    rng = np.random.default_rng(11)
+    gate = (rng.uniform(0, 0.5, (hidden, inter)) / 16).astype(np.float32)
+    up = (rng.uniform(0, 0.5, (hidden, inter)) / 16).astype(np.float32)
+    down = (rng.uniform(0, 0.5, (inter, hidden)) / 64).astype(np.float32)
+    x = rng.uniform(0, 1, (M, hidden)).astype(np.float32)
+    out = np.zeros_like(x)
+    host["mlp"](BF16, SILU, M, hidden, inter, ptr(out), hidden, ptr(x), hidden, ptr(gate), ptr(up), ptr(down))
+    xb = orc.round_bf16(x)
+    g = xb.astype(np.float64) @ orc.round_bf16(gate).astype(np.float64)
+    u = xb.astype(np.float64) @ orc.round_bf16(up).astype(np.float64)
+    h = g / (1 + np.exp(-g)) * u
+    exp = orc.round_bf16(h).astype(np.float64) @ orc.round_bf16(down).astype(np.float64) + x
+    bad = (np.abs(exp - out) > 0.01) & (np.abs((exp - out) / exp) > 0.01)
+    assert not bad.any(), np.abs(exp - out).max()
+
+
+def test_invoke_rmsnorm(host, orc):
+    rng = np.random.default_rng(13)
+    rows, cols = 5, 4096
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, cols).astype(np.float32)
+    out = np.zeros_like(x)
+    host["rms"](FP32, ptr(out), ptr(x), ptr(w), rows, cols, -1, -1, 1e-6)
+    assert np.abs(out - orc.rmsnorm(x, w)).max() < 1e-2  # rms_norm_test.cpp tolerance; actual error ~1e-6
+    assert np.abs(out - orc.rmsnorm(x, w)).max() < 1e-5
+    xb, wb = orc.to_bf16(x), orc.to_bf16(w)
+    ob = np.zeros_like(xb)
+    host["rms"](BF16, ptr(ob), ptr(xb), ptr(wb), rows, cols, -1, -1, 1e-6)
+    exp = orc.rmsnorm(orc.from_bf16(xb), orc.from_bf16(wb))
+    assert np.abs(orc.from_bf16(ob) - exp).max() <= 2.0 ** -8 * np.abs(exp).max()
+
+
+def test_invoke_rotary_embedding_golden_constants(host, orc):
+    # values of tests/ut/rotary_embedding_test.cpp:28-57 through the public entry point
+    q = np.array([4, 4, 4, 4, 3, 2, 1, 1, 4, 4, 2, 1, 4, 1, 3, 0], np.float32)
+    k = np.ones(16, np.float32)
+    qg = np.array([-1.20467, 5.52709, -1.20467, 5.52709, 3, 2, 1, 1, -1.20467, 5.52709, 0.239134, 2.22324, 4, 1, 3, 0])
+    kg = np.array([-0.301169, 1.38177, -0.301169, 1.38177, 1, 1, 1, 1, -0.301169, 1.38177, -0.301169, 1.38177, 1, 1,
+                   1, 1])
+    cos_h, sin_h = orc.rope_tables(2, 10)  # [10, 1]
+    cos = np.repeat(cos_h, 2, axis=1).copy()  # the public API takes [maxPosition, dim]
+    sin = np.repeat(sin_h, 2, axis=1).copy()
+    pos = np.array([1, 0, 1, 0], np.int64)
+    host["rope"](FP32, ptr(pos), ptr(q), ptr(k), ptr(cos), ptr(sin), 2, 4, 4, 4, 2, 2, 2)
+    assert np.abs(q - qg).max() < 1e-3 and np.abs(k - kg).max() < 1e-3
+    qb = orc.to_bf16(np.array([4, 4, 4, 4, 3, 2, 1, 1, 4, 4, 2, 1, 4, 1, 3, 0], np.float32))
+    kb = orc.to_bf16(np.ones(16, np.float32))
+    host["rope"](BF16, ptr(pos), ptr(qb), ptr(kb), ptr(orc.to_bf16(cos)), ptr(orc.to_bf16(sin)), 2, 4, 4, 4, 2, 2, 2)
+    assert np.abs(orc.from_bf16(qb) - qg).max() < 1e-2 * 6 and np.abs(orc.from_bf16(kb) - kg).max() < 1e-2
+
+
+@pytest.mark.parametrize("M", [2, 4, 8, 64])
+@pytest.mark.parametrize("transB", [False, True])
+def test_invoke_gemm_bf16(host, orc, M, transB):
+    N, K = 1024, 2048
+    rng = np.random.default_rng(M)
+    A = orc.round_bf16(rng.uniform(-1, 1, (M, K)))
+    Bm = orc.round_bf16(rng.uniform(-1, 1, (K, N)))
+    Ab = orc.to_bf16(A)
+    Bb = orc.to_bf16(Bm.T.copy() if transB else Bm)
+    Cb = np.zeros((M, N), np.uint16)
+    host["gemm"](BF16, False, transB, M, N, K, 1.0, ptr(Ab), K, ptr(Bb), 0.0, ptr(Cb), N, None, None, -1)
+    exp = A.astype(np.float64) @ Bm.astype(np.float64)
+    assert np.abs(orc.from_bf16(Cb) - exp).max() < 0.5  # gemm_kernel_ext_test.cpp tolerance for bf16
+    assert (np.abs(orc.from_bf16(Cb) - exp) <= 1e-3 + np.abs(exp) * 2.0 ** -8).all()

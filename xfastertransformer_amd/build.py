@@ -13,6 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 ROOT = os.path.dirname(HERE)
 LIB_HIP = os.path.join(HERE, "libxft_hip.so")
+LIB_LAYERS = os.path.join(HERE, "libxft_layers.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # gfx950 only; packed-FP32 VALU ops stay off (the compiler must not form v_pk_*_f32)
@@ -62,8 +63,19 @@ def build_hip(force=True):
     return LIB_HIP
 
 
+def build_host(force=True):
+    """The C++ host layer (xft::invoke* entry points) over the C-ABI; plain g++, no HIP headers."""
+    src = os.path.join(CSRC, "host", "xft_layers.cpp")
+    deps = [src] + glob.glob(os.path.join(ROOT, "include", "*.h")) + [LIB_HIP]
+    if force or _stale(LIB_LAYERS, deps):
+        _run([os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", src, "-o", LIB_LAYERS,
+              "-L" + HERE, "-lxft_hip", "-Wl,-rpath,$ORIGIN"])
+    return LIB_LAYERS
+
+
 def build_all(force=True):
-    return build_hip(force)
+    build_hip(force)
+    return build_host(force)
 
 
 if __name__ == "__main__":

@@ -346,6 +346,9 @@ class Model:
     def decode_untracked(self, steps, stream=None):
         check(lib.xfthip_model_decode(self.h, steps, None, stream))
 
+    def use_graph(self, enable):
+        check(lib.xfthip_model_use_graph(self.h, int(bool(enable))))
+
     def last_ids(self, B):
         ids = np.empty(B, np.int32)
         pos = C.c_int()

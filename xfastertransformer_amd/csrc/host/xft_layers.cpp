@@ -1,0 +1,426 @@
+// Host side of the drop-in boundary: the reference's public layer entry points
+// (include/layers_*.h, namespace xft) implemented over the C-ABI of the gfx950 library.
+// Plain C++ (g++), no HIP headers: everything device-side goes through include/xft_hip.h.
+//
+// Conventions kept from the reference (src/layers/decoder_layer.cpp, attention.cpp,
+// mlp_llama.cpp): void functions that print and exit(-1) on failure; a function-local static
+// mutex serialises each invoke*LLaMA; weights are fp32 host matrices [in, out], converted once
+// on first sight and cached for the life of the process under a key made of their addresses
+// plus dims and dt; activations are fp32 host buffers; the KV cache (FP16) is owned here and
+// the caller supplies pastSeqLen / step.  Beyond the reference: dt may also be int8, int4 or
+// nf4, which selects the weight-only formats (the reference's entry points silently ignore
+// every dt but bf16 / fp16).
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <functional>
+#include <mutex>
+#include <sstream>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "../../../include/layers_attention.h"
+#include "../../../include/layers_decoder.h"
+#include "../../../include/layers_gemm.h"
+#include "../../../include/layers_mlp.h"
+#include "../../../include/layers_norm.h"
+#include "../../../include/layers_rotary_embedding.h"
+#include "../../../include/xft_hip.h"
+
+namespace {
+
+[[noreturn]] void die(const char *what) {
+    printf("%s: %s\n", what, xfthip_last_error());
+    exit(-1);
+}
+
+#define CK(call)                   \
+    do {                           \
+        if ((call) != 0) die(#call); \
+    } while (0)
+
+void ensure_init() {
+    static std::once_flag once;
+    std::call_once(once, [] {
+        int dev = 0;
+        if (const char *e = getenv("XFT_HIP_DEVICE")) dev = atoi(e);
+        CK(xfthip_init(dev));
+    });
+}
+
+// fp32 -> bf16 as the reference's bfloat16_t does (include/bfloat16.h:40-65)
+uint16_t to_bf16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
+    if (a == 0x7F800000u) return (uint16_t)(u >> 16);
+    if (a < 0x00800000u) return (uint16_t)((u >> 16) & 0x8000u);
+    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+float from_bf16(uint16_t b) {
+    uint32_t u = (uint32_t)b << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+// weight kind for a DataType, or -1
+int kind_of(xft::DataType dt) {
+    switch (dt) {
+        case xft::DataType::bf16: return XFTHIP_W_BF16;
+        case xft::DataType::int8: return XFTHIP_W_INT8;
+        case xft::DataType::int4: return XFTHIP_W_UINT4;
+        case xft::DataType::nf4: return XFTHIP_W_NF4;
+        default: return -1;
+    }
+}
+
+// Convert a contiguous fp32 [K, N] host matrix into a device weight handle of `kind`.
+xfthip_weight_t make_weight(int kind, int K, int N, const float *W, int flags) {
+    xfthip_weight_t h = nullptr;
+    if (kind == XFTHIP_W_BF16) {
+        std::vector<uint16_t> b((size_t)K * N);
+        for (size_t i = 0; i < b.size(); ++i) b[i] = to_bf16(W[i]);
+        CK(xfthip_weight_create(kind, K, N, b.data(), nullptr, nullptr, flags, &h));
+        return h;
+    }
+    std::vector<float> scale(N), zero(N, 0.0f);
+    std::vector<uint8_t> q((size_t)K * N);
+    CK(xfthip_quantize_weight(kind, K, N, W, q.data(), scale.data(), zero.data()));
+    CK(xfthip_weight_create(kind, K, N, q.data(), scale.data(), kind == XFTHIP_W_NF4 ? nullptr : zero.data(), flags, &h));
+    return h;
+}
+
+// Gather Q | K | V column blocks (row stride = qkvCols, src/layers/attention.h:122-136) into one
+// contiguous [hidden, qkvCols] matrix.
+std::vector<float> concat_qkv(const float *q, const float *k, const float *v, int hidden, int qCols, int kvCols) {
+    const int stride = qCols + 2 * kvCols;
+    std::vector<float> out((size_t)hidden * stride);
+    for (int i = 0; i < hidden; ++i) {
+        memcpy(&out[(size_t)i * stride], q + (size_t)i * stride, sizeof(float) * qCols);
+        memcpy(&out[(size_t)i * stride + qCols], k + (size_t)i * stride, sizeof(float) * kvCols);
+        memcpy(&out[(size_t)i * stride + qCols + kvCols], v + (size_t)i * stride, sizeof(float) * kvCols);
+    }
+    return out;
+}
+
+std::vector<float> concat_bias(const float *q, const float *k, const float *v, int qCols, int kvCols) {
+    std::vector<float> out;
+    if (!q && !k && !v) return out;
+    out.assign((size_t)qCols + 2 * kvCols, 0.0f);
+    if (q) memcpy(out.data(), q, sizeof(float) * qCols);
+    if (k) memcpy(out.data() + qCols, k, sizeof(float) * kvCols);
+    if (v) memcpy(out.data() + qCols + kvCols, v, sizeof(float) * kvCols);
+    return out;
+}
+
+// cat(gate, up) as LlamaMLP::catGateUpWeights lays it out: [hidden, 2 * inter]
+std::vector<float> concat_gateup(const float *gate, const float *up, int hidden, int inter) {
+    std::vector<float> out((size_t)hidden * 2 * inter);
+    for (int i = 0; i < hidden; ++i) {
+        memcpy(&out[(size_t)i * 2 * inter], gate + (size_t)i * inter, sizeof(float) * inter);
+        memcpy(&out[(size_t)i * 2 * inter + inter], up + (size_t)i * inter, sizeof(float) * inter);
+    }
+    return out;
+}
+
+struct DevBuf {
+    void *p = nullptr;
+    size_t cap = 0;
+    void *get(size_t bytes) {
+        if (bytes > cap) {
+            if (p) xfthip_free(p);
+            CK(xfthip_malloc(&p, bytes));
+            cap = bytes;
+        }
+        return p;
+    }
+};
+
+// One cached layer: a 1-layer device model plus the weight handles it references.
+struct Entry {
+    xfthip_model_t model = nullptr;
+    xfthip_weight_t qkv = nullptr, o = nullptr, gateup = nullptr, down = nullptr;
+    std::vector<float> ln1, ln2, qkvBias, oBias;
+    xfthip_model_config cfg {};
+    bool hasAttn = false, hasMlp = false;
+};
+
+void build_model(Entry &e) {
+    if (e.model) CK(xfthip_model_destroy(e.model));
+    e.model = nullptr;
+    CK(xfthip_model_create(&e.cfg, &e.model));
+    if (e.hasAttn)
+        CK(xfthip_model_set_attention(e.model, 0, e.qkv, e.o, e.ln1.empty() ? nullptr : e.ln1.data(),
+                e.qkvBias.empty() ? nullptr : e.qkvBias.data(), e.oBias.empty() ? nullptr : e.oBias.data()));
+    if (e.hasMlp) CK(xfthip_model_set_mlp(e.model, 0, e.gateup, e.down, e.ln2.empty() ? nullptr : e.ln2.data()));
+}
+
+// grow the model when a call needs more batch / tokens / positions than it was built for
+void fit_model(Entry &e, int batch, int tokens, int maxPositions, int maxPosEmbed) {
+    bool rebuild = e.model == nullptr;
+    if (batch > e.cfg.max_batch) { e.cfg.max_batch = batch; rebuild = true; }
+    if (tokens > e.cfg.max_tokens) { e.cfg.max_tokens = tokens; rebuild = true; }
+    if (maxPositions > e.cfg.max_seq) { e.cfg.max_seq = maxPositions; rebuild = true; }
+    if (maxPosEmbed > e.cfg.max_pos_embed) { e.cfg.max_pos_embed = maxPosEmbed; rebuild = true; }
+    if (e.cfg.max_pos_embed < e.cfg.max_seq) { e.cfg.max_pos_embed = e.cfg.max_seq; rebuild = true; }
+    if (e.cfg.max_tokens < e.cfg.max_batch) { e.cfg.max_tokens = e.cfg.max_batch; rebuild = true; }
+    if (rebuild) build_model(e);
+}
+
+// upload fp32 rows, run `body(dev_in, dev_out)` (dense [rows, cols] device buffers), download
+void run_rows(const void *input, int inputStride, void *output, int outputStride, int rows, int cols,
+        const std::function<void(const float *, float *)> &body) {
+    static DevBuf din, dout;
+    std::vector<float> dense((size_t)rows * cols);
+    for (int r = 0; r < rows; ++r) memcpy(&dense[(size_t)r * cols], (const float *)input + (size_t)r * inputStride, sizeof(float) * cols);
+    float *di = (float *)din.get(dense.size() * sizeof(float));
+    float *dop = (float *)dout.get(dense.size() * sizeof(float));
+    CK(xfthip_memcpy_h2d(di, dense.data(), dense.size() * sizeof(float), nullptr));
+    body(di, dop);
+    CK(xfthip_memcpy_d2h(dense.data(), dop, dense.size() * sizeof(float), nullptr));
+    for (int r = 0; r < rows; ++r) memcpy((float *)output + (size_t)r * outputStride, &dense[(size_t)r * cols], sizeof(float) * cols);
+}
+
+} // namespace
+
+namespace xft {
+
+void invokeLayerLLaMA(DataType dt, ActivationType at, NormType nt, int batchSize, int inputSeqLen, int attHeadDim,
+        int attHeadNum, int kvHeadNum, int maxPositions, int maxPosEmbed, int pastSeqLen, int currentSeqLen, int step,
+        int hiddenSize, int intermediateSize, void *output, int outputStride, const void *input, int inputStride,
+        const float *ln1Gamma, const float *ln1Beta, const void *queryWeight, const void *keyWeight,
+        const void *valueWeight, const void *attnOutWeight, const float *ln2Gamma, const float *ln2Beta,
+        const void *gateWeight, const void *upWeight, const void *downWeight, const float *queryBias,
+        const float *keyBias, const float *valueBias, const float *attnOutBias) {
+    static std::mutex mutex;
+    std::lock_guard<std::mutex> lock(mutex);
+    (void)ln1Beta; (void)ln2Beta; (void)currentSeqLen; (void)step;
+
+    const int kind = kind_of(dt);
+    if (kind < 0) return; // the reference's dispatch has no else-branch either (decoder_layer.cpp:172-206)
+    if (nt != NormType::RMS) {
+        printf(">> unsupported norm type (this build implements RMSNorm layers)\n");
+        return;
+    }
+    if (at != ActivationType::SILU && at != ActivationType::SWIGLU) {
+        printf(">> unsupported activation type\n");
+        return;
+    }
+    ensure_init();
+
+    static std::unordered_map<std::string, Entry> hub;
+    std::stringstream key;
+    key << queryWeight << "_" << keyWeight << "_" << valueWeight << "_" << attnOutWeight << "_" << gateWeight << "_" << upWeight
+        << "_" << downWeight << "_" << dt << "_" << at << "_" << nt << "_" << attHeadDim << "_" << attHeadNum << "_" << kvHeadNum;
+    Entry &e = hub[key.str()];
+    if (!e.hasAttn) {
+        const int qCols = attHeadNum * attHeadDim, kvCols = kvHeadNum * attHeadDim;
+        auto qkv = concat_qkv((const float *)queryWeight, (const float *)keyWeight, (const float *)valueWeight, hiddenSize, qCols, kvCols);
+        e.qkv = make_weight(kind, hiddenSize, qCols + 2 * kvCols, qkv.data(), XFTHIP_WF_NONE);
+        e.o = make_weight(kind, qCols, hiddenSize, (const float *)attnOutWeight, XFTHIP_WF_NONE);
+        auto gu = concat_gateup((const float *)gateWeight, (const float *)upWeight, hiddenSize, intermediateSize);
+        e.gateup = make_weight(kind, hiddenSize, 2 * intermediateSize, gu.data(), XFTHIP_WF_GATEUP);
+        e.down = make_weight(kind, intermediateSize, hiddenSize, (const float *)downWeight, XFTHIP_WF_NONE);
+        e.ln1.assign(ln1Gamma, ln1Gamma + hiddenSize);
+        e.ln2.assign(ln2Gamma, ln2Gamma + hiddenSize);
+        e.qkvBias = concat_bias(queryBias, keyBias, valueBias, qCols, kvCols);
+        if (attnOutBias) e.oBias.assign(attnOutBias, attnOutBias + hiddenSize);
+        e.hasAttn = e.hasMlp = true;
+        e.cfg = xfthip_model_config {1, hiddenSize, intermediateSize, attHeadNum, kvHeadNum, attHeadDim, 0, batchSize, maxPositions,
+                batchSize * inputSeqLen, maxPosEmbed, 10000, XFTHIP_FP16, 1e-6f};
+        printf(">> create llama_layer_key: %s\n", key.str().c_str());
+    }
+    fit_model(e, batchSize, batchSize * inputSeqLen, maxPositions, maxPosEmbed);
+    run_rows(input, inputStride, output, outputStride, batchSize * inputSeqLen, hiddenSize, [&](const float *di, float *dop) {
+        CK(xfthip_model_layer_forward(e.model, 0, di, hiddenSize, dop, hiddenSize, batchSize, inputSeqLen, pastSeqLen, nullptr));
+    });
+}
+
+void invokeAttentionLLaMA(DataType dt, int batchSize, int inputSeqLen, int attHeadDim, int attHeadNum, int kvHeadNum,
+        int maxPositions, int maxPosEmbed, int pastSeqLen, int currentSeqLen, int step, int hiddenSize, void *output,
+        int outputStride, const void *input, int inputStride, const void *queryWeight, const void *keyWeight,
+        const void *valueWeight, const void *attnOutWeight, const float *queryBias, const float *keyBias,
+        const float *valueBias, const float *attnOutBias) {
+    static std::mutex mutex;
+    std::lock_guard<std::mutex> lock(mutex);
+    (void)currentSeqLen; (void)step;
+    const int kind = kind_of(dt);
+    if (kind < 0) return;
+    ensure_init();
+
+    static std::unordered_map<std::string, Entry> hub;
+    std::stringstream key;
+    key << queryWeight << "_" << keyWeight << "_" << valueWeight << "_" << attnOutWeight << "_" << queryBias << "_" << keyBias << "_"
+        << valueBias << "_" << dt << "_" << attHeadDim << "_" << attHeadNum << "_" << kvHeadNum;
+    Entry &e = hub[key.str()];
+    if (!e.hasAttn) {
+        const int qCols = attHeadNum * attHeadDim, kvCols = kvHeadNum * attHeadDim;
+        auto qkv = concat_qkv((const float *)queryWeight, (const float *)keyWeight, (const float *)valueWeight, hiddenSize, qCols, kvCols);
+        e.qkv = make_weight(kind, hiddenSize, qCols + 2 * kvCols, qkv.data(), XFTHIP_WF_NONE);
+        e.o = make_weight(kind, qCols, hiddenSize, (const float *)attnOutWeight, XFTHIP_WF_NONE);
+        e.qkvBias = concat_bias(queryBias, keyBias, valueBias, qCols, kvCols);
+        if (attnOutBias) e.oBias.assign(attnOutBias, attnOutBias + hiddenSize);
+        e.hasAttn = true;
+        // the attention-only context of the reference has intermediate size 1 (attention.cpp:88-90);
+        // the scratch here needs a multiple of 16
+        e.cfg = xfthip_model_config {1, hiddenSize, 16, attHeadNum, kvHeadNum, attHeadDim, 0, batchSize, maxPositions,
+                batchSize * inputSeqLen, maxPosEmbed, 10000, XFTHIP_FP16, 1e-6f};
+        printf(">> create llama_attention_key: %s\n", key.str().c_str());
+    }
+    fit_model(e, batchSize, batchSize * inputSeqLen, maxPositions, maxPosEmbed);
+    run_rows(input, inputStride, output, outputStride, batchSize * inputSeqLen, hiddenSize, [&](const float *di, float *dop) {
+        CK(xfthip_model_attention_forward(e.model, 0, di, hiddenSize, dop, hiddenSize, batchSize, inputSeqLen, pastSeqLen, 0, nullptr));
+    });
+}
+
+void invokeMLPLLaMA(DataType dt, ActivationType at, int numTokens, int hiddenSize, int intermediateSize, void *output,
+        int outputStride, const void *input, int inputStride, const void *gateWeight, const void *upWeight,
+        const void *downWeight) {
+    static std::mutex mutex;
+    std::lock_guard<std::mutex> lock(mutex);
+    const int kind = kind_of(dt);
+    if (kind < 0) return;
+    if (at != ActivationType::SILU && at != ActivationType::SWIGLU) {
+        printf(">> unsupported activation type\n");
+        return;
+    }
+    ensure_init();
+
+    static std::unordered_map<std::string, Entry> hub;
+    std::stringstream key;
+    key << gateWeight << "_" << upWeight << "_" << downWeight << "_" << dt << "_" << at;
+    Entry &e = hub[key.str()];
+    if (!e.hasMlp) {
+        auto gu = concat_gateup((const float *)gateWeight, (const float *)upWeight, hiddenSize, intermediateSize);
+        e.gateup = make_weight(kind, hiddenSize, 2 * intermediateSize, gu.data(), XFTHIP_WF_GATEUP);
+        e.down = make_weight(kind, intermediateSize, hiddenSize, (const float *)downWeight, XFTHIP_WF_NONE);
+        e.hasMlp = true;
+        // head geometry is irrelevant to the MLP block; one 128-wide head keeps the scratch small
+        e.cfg = xfthip_model_config {1, hiddenSize, intermediateSize, 1, 1, 128, 0, 1, 32, numTokens, 32, 10000, XFTHIP_FP16, 1e-6f};
+        printf(">> create llama_mlp_key: %s\n", key.str().c_str());
+    }
+    fit_model(e, 1, numTokens, 32, 32);
+    run_rows(input, inputStride, output, outputStride, numTokens, hiddenSize, [&](const float *di, float *dop) {
+        CK(xfthip_model_mlp_forward(e.model, 0, di, hiddenSize, dop, hiddenSize, numTokens, 0, nullptr));
+    });
+}
+
+void invokeRmsNorm(DataType dt, void *output, const void *input, const void *weight, int rows, int cols, int iStride,
+        int oStride, float epsilon) {
+    if (dt != DataType::fp32 && dt != DataType::bf16) return; // fp16 activations are not offered by this build
+    ensure_init();
+    if (iStride == -1) iStride = cols;
+    if (oStride == -1) oStride = cols;
+    const int et = dt == DataType::fp32 ? XFTHIP_F32 : XFTHIP_BF16;
+    const size_t esz = dt == DataType::fp32 ? 4 : 2;
+    // weight has the element type of dt (src/kernels/rmsnorm_kernels.cpp:166-180); the kernel wants fp32
+    std::vector<float> w(cols);
+    for (int i = 0; i < cols; ++i) w[i] = dt == DataType::fp32 ? ((const float *)weight)[i] : from_bf16(((const uint16_t *)weight)[i]);
+    void *di = nullptr, *dop = nullptr, *dw = nullptr;
+    CK(xfthip_malloc(&di, (size_t)rows * iStride * esz));
+    CK(xfthip_malloc(&dop, (size_t)rows * oStride * esz));
+    CK(xfthip_malloc(&dw, (size_t)cols * 4));
+    CK(xfthip_memcpy_h2d(di, input, ((size_t)(rows - 1) * iStride + cols) * esz, nullptr));
+    CK(xfthip_memcpy_h2d(dop, output, ((size_t)(rows - 1) * oStride + cols) * esz, nullptr)); // keep the gaps between rows
+    CK(xfthip_memcpy_h2d(dw, w.data(), (size_t)cols * 4, nullptr));
+    CK(xfthip_rmsnorm(dop, et, di, et, (const float *)dw, rows, cols, iStride, oStride, epsilon, nullptr));
+    CK(xfthip_memcpy_d2h(output, dop, ((size_t)(rows - 1) * oStride + cols) * esz, nullptr));
+    xfthip_free(di);
+    xfthip_free(dop);
+    xfthip_free(dw);
+}
+
+void invokeRotaryEmbedding(DataType dt, const int64_t *positionIds, void *query, void *key, const void *embCos,
+        const void *embSin, const int dim, const int qStride, const int kStride, const int numTokens, const int headNum,
+        const int headSize, const int numKvHeads) {
+    // the reference treats dt == fp16 buffers as fp32 (src/layers/rotary_embedding_api.cpp:87-96); kept
+    if (dt != DataType::bf16 && dt != DataType::fp16 && dt != DataType::fp32) return;
+    if (dim != headSize) {
+        printf("Incorrect shape, rot_dim is not the head size.\n");
+        exit(-1);
+    }
+    ensure_init();
+    const bool isbf = dt == DataType::bf16;
+    const int et = isbf ? XFTHIP_BF16 : XFTHIP_F32;
+    const size_t esz = isbf ? 2 : 4;
+    const int kvHeads = numKvHeads > 0 ? numKvHeads : headNum;
+    int maxPos = 0;
+    std::vector<int> pos(numTokens);
+    for (int i = 0; i < numTokens; ++i) {
+        pos[i] = (int)positionIds[i];
+        if (pos[i] > maxPos) maxPos = pos[i];
+    }
+    // tables arrive as [maxPosition, dim] in the element type of dt; the kernel takes fp32
+    const size_t tn = (size_t)(maxPos + 1) * dim;
+    std::vector<float> c(tn), s(tn);
+    for (size_t i = 0; i < tn; ++i) {
+        c[i] = isbf ? from_bf16(((const uint16_t *)embCos)[i]) : ((const float *)embCos)[i];
+        s[i] = isbf ? from_bf16(((const uint16_t *)embSin)[i]) : ((const float *)embSin)[i];
+    }
+    const size_t qBytes = ((size_t)(numTokens - 1) * qStride + (size_t)headNum * headSize) * esz;
+    const size_t kBytes = ((size_t)(numTokens - 1) * kStride + (size_t)kvHeads * headSize) * esz;
+    void *dq = nullptr, *dk = nullptr, *dc = nullptr, *ds = nullptr, *dp = nullptr;
+    CK(xfthip_malloc(&dq, qBytes));
+    CK(xfthip_malloc(&dk, kBytes));
+    CK(xfthip_malloc(&dc, tn * 4));
+    CK(xfthip_malloc(&ds, tn * 4));
+    CK(xfthip_malloc(&dp, (size_t)numTokens * 4));
+    CK(xfthip_memcpy_h2d(dq, query, qBytes, nullptr));
+    CK(xfthip_memcpy_h2d(dk, key, kBytes, nullptr));
+    CK(xfthip_memcpy_h2d(dc, c.data(), tn * 4, nullptr));
+    CK(xfthip_memcpy_h2d(ds, s.data(), tn * 4, nullptr));
+    CK(xfthip_memcpy_h2d(dp, pos.data(), (size_t)numTokens * 4, nullptr));
+    CK(xfthip_rotary_embedding_full(et, (const int *)dp, dq, dk, (const float *)dc, (const float *)ds, dim, qStride, kStride,
+            numTokens, headNum, headSize, kvHeads, nullptr));
+    CK(xfthip_memcpy_d2h(query, dq, qBytes, nullptr));
+    CK(xfthip_memcpy_d2h(key, dk, kBytes, nullptr));
+    for (void *p : {dq, dk, dc, ds, dp}) xfthip_free(p);
+}
+
+void invokeGemm(DataType dt, bool transA, bool transB, int M, int N, int K, float alpha, void *A, int lda, void *B, float beta, void *C,
+        int ldc, void *bias, void *res, int ldres) {
+    // the reference accepts bias / res but never reads them (src/utils/matmul_helper.h:63-101)
+    (void)bias; (void)res; (void)ldres;
+    if (dt != DataType::bf16) {
+        printf(">> invokeGemm: only bf16 is offered by this build\n");
+        return;
+    }
+    ensure_init();
+    const uint16_t *a = (const uint16_t *)A, *b = (const uint16_t *)B;
+    // op(B) as [K, N] bf16, op(A) as dense [M, Kp] with Kp a multiple of 8
+    std::vector<uint16_t> bm((size_t)K * N);
+    for (int k = 0; k < K; ++k)
+        for (int n = 0; n < N; ++n) bm[(size_t)k * N + n] = transB ? b[(size_t)n * K + k] : b[(size_t)k * N + n];
+    const int Kp = (K + 7) / 8 * 8;
+    std::vector<uint16_t> am((size_t)M * Kp, 0);
+    for (int m = 0; m < M; ++m)
+        for (int k = 0; k < K; ++k) am[(size_t)m * Kp + k] = transA ? a[(size_t)k * M + m] : a[(size_t)m * lda + k];
+    std::vector<uint16_t> bp((size_t)Kp * N, 0);
+    memcpy(bp.data(), bm.data(), bm.size() * 2);
+    xfthip_weight_t w = nullptr;
+    CK(xfthip_weight_create(XFTHIP_W_BF16, Kp, N, bp.data(), nullptr, nullptr, XFTHIP_WF_NONE, &w));
+    void *da = nullptr, *dc = nullptr;
+    CK(xfthip_malloc(&da, am.size() * 2));
+    CK(xfthip_malloc(&dc, (size_t)M * N * 4));
+    CK(xfthip_memcpy_h2d(da, am.data(), am.size() * 2, nullptr));
+    CK(xfthip_gemm(w, M, da, Kp, dc, N, XFTHIP_F32, XFTHIP_EPI_NONE, nullptr, nullptr, 0, XFTHIP_F32, 1.0f, nullptr));
+    std::vector<float> acc((size_t)M * N);
+    CK(xfthip_memcpy_d2h(acc.data(), dc, acc.size() * 4, nullptr));
+    uint16_t *c = (uint16_t *)C;
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) {
+            float v = alpha * acc[(size_t)m * N + n];
+            if (beta != 0.0f) v += beta * from_bf16(c[(size_t)m * ldc + n]);
+            c[(size_t)m * ldc + n] = to_bf16(v);
+        }
+    xfthip_free(da);
+    xfthip_free(dc);
+    xfthip_weight_destroy(w);
+}
+
+} // namespace xft

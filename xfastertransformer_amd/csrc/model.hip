@@ -115,6 +115,7 @@ struct xfthip_model {
     hipGraphExec_t graph = nullptr;
     int graph_B = 0;
     hipStream_t graph_stream = nullptr;
+    bool use_graph = true;
 };
 
 static int upload_f32(float **dst, const float *src, size_t n) {
@@ -128,17 +129,29 @@ static int upload_f32(float **dst, const float *src, size_t n) {
     return 0;
 }
 
-// one layer on device buffers; x is updated in place (x_in may differ from x_out)
-static int layer_forward(xfthip_model *m, int idx, const float *x_in, int in_stride, float *x_out, int out_stride, int B,
-        int S, int past, const int *past_dev, hipStream_t st) {
+// fp32 -> bf16 copy of activation rows (the un-normalised GEMM input of the block-level entry points)
+__global__ void narrow_rows_kernel(const float *__restrict__ in, int in_stride, uint16_t *__restrict__ out, int cols) {
+    const float *row = in + (size_t)blockIdx.x * in_stride;
+    uint16_t *orow = out + (size_t)blockIdx.x * cols;
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) orow[c] = xfthip::f32_to_bf16_ref(row[c]);
+}
+
+// attention half of a layer: x_out = Attn(norm?(x_in)) * Wo + bias + x_in
+static int attention_block(xfthip_model *m, int idx, const float *x_in, int in_stride, float *x_out, int out_stride, int B,
+        int S, int past, const int *past_dev, bool do_norm, hipStream_t st) {
     const xfthip_model_config &c = m->cfg;
     const LayerW &L = m->layers[idx];
-    XFT_REQUIRE(L.qkv && L.o && L.gateup && L.down && L.ln1 && L.ln2, "layer %d has no weights attached", idx);
+    XFT_REQUIRE(L.qkv && L.o, "layer %d has no attention weights attached", idx);
+    XFT_REQUIRE(!do_norm || L.ln1, "layer %d has no attention norm weight", idx);
     const int T = B * S;
     const int qcols = c.q_heads * c.head_size, kvcols = c.kv_heads * c.head_size;
     const int qkv_cols = qcols + 2 * kvcols;
     int rc;
-    if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, x_in, XFTHIP_F32, L.ln1, T, c.hidden, in_stride, c.hidden, c.rms_eps, st))) return rc;
+    if (do_norm) {
+        if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, x_in, XFTHIP_F32, L.ln1, T, c.hidden, in_stride, c.hidden, c.rms_eps, st))) return rc;
+    } else {
+        hipLaunchKernelGGL(narrow_rows_kernel, dim3(T), dim3(256), 0, st, x_in, in_stride, m->xn, c.hidden);
+    }
     if ((rc = xfthip_gemm(L.qkv, T, m->xn, c.hidden, m->qkv, qkv_cols, XFTHIP_BF16, L.qkv_bias ? XFTHIP_EPI_BIAS : XFTHIP_EPI_NONE,
                  L.qkv_bias, nullptr, 0, XFTHIP_F32, 1.0f, st)))
         return rc;
@@ -154,15 +167,34 @@ static int layer_forward(xfthip_model *m, int idx, const float *x_in, int in_str
     if ((rc = xfthip_attention(attend, m->qkv, qkv_cols, m->att, qcols, XFTHIP_BF16, B, S, c.q_heads,
                  1.0f / sqrtf((float)c.head_size), past, past_dev, st)))
         return rc;
-    if ((rc = xfthip_gemm(L.o, T, m->att, qcols, x_out, out_stride, XFTHIP_F32, XFTHIP_EPI_RESIDENTIAL, L.o_bias, x_in, in_stride,
-                 XFTHIP_F32, 1.0f, st)))
-        return rc;
-    if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, x_out, XFTHIP_F32, L.ln2, T, c.hidden, out_stride, c.hidden, 1e-6f, st))) return rc;
+    return xfthip_gemm(L.o, T, m->att, qcols, x_out, out_stride, XFTHIP_F32, XFTHIP_EPI_RESIDENTIAL, L.o_bias, x_in, in_stride,
+            XFTHIP_F32, 1.0f, st);
+}
+
+// MLP half of a layer: x_out = (silu(xn Wgate) * (xn Wup)) Wdown + x_in, xn = norm?(x_in)
+static int mlp_block(xfthip_model *m, int idx, const float *x_in, int in_stride, float *x_out, int out_stride, int T,
+        bool do_norm, hipStream_t st) {
+    const xfthip_model_config &c = m->cfg;
+    const LayerW &L = m->layers[idx];
+    XFT_REQUIRE(L.gateup && L.down, "layer %d has no MLP weights attached", idx);
+    XFT_REQUIRE(!do_norm || L.ln2, "layer %d has no MLP norm weight", idx);
+    int rc;
+    if (do_norm) {
+        // epsilon 1e-6 is hard-coded on the MLP side of the reference (src/layers/mlp_llama.h:212)
+        if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, x_in, XFTHIP_F32, L.ln2, T, c.hidden, in_stride, c.hidden, 1e-6f, st))) return rc;
+    } else {
+        hipLaunchKernelGGL(narrow_rows_kernel, dim3(T), dim3(256), 0, st, x_in, in_stride, m->xn, c.hidden);
+    }
     if ((rc = xfthip_gemm_gateup_silu(L.gateup, T, m->xn, c.hidden, m->h, c.intermediate, XFTHIP_BF16, st))) return rc;
-    if ((rc = xfthip_gemm(L.down, T, m->h, c.intermediate, x_out, out_stride, XFTHIP_F32, XFTHIP_EPI_RESIDENTIAL, nullptr, x_out,
-                 out_stride, XFTHIP_F32, 1.0f, st)))
-        return rc;
-    return 0;
+    return xfthip_gemm(L.down, T, m->h, c.intermediate, x_out, out_stride, XFTHIP_F32, XFTHIP_EPI_RESIDENTIAL, nullptr, x_in, in_stride,
+            XFTHIP_F32, 1.0f, st);
+}
+
+// one layer on device buffers (x_in may alias x_out)
+static int layer_forward(xfthip_model *m, int idx, const float *x_in, int in_stride, float *x_out, int out_stride, int B,
+        int S, int past, const int *past_dev, hipStream_t st) {
+    if (int rc = attention_block(m, idx, x_in, in_stride, x_out, out_stride, B, S, past, past_dev, true, st)) return rc;
+    return mlp_block(m, idx, x_out, out_stride, x_out, out_stride, B * S, true, st);
 }
 
 static int head_forward(xfthip_model *m, const float *xrows, int B, hipStream_t st) {
@@ -266,29 +298,21 @@ int xfthip_model_destroy(xfthip_model_t m) {
     return 0;
 }
 
-int xfthip_model_set_layer(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthip_weight_t o, xfthip_weight_t gateup,
-        xfthip_weight_t down, const float *ln1_host, const float *ln2_host, const float *qkv_bias_host,
-        const float *o_bias_host) {
-    XFT_REQUIRE(m && qkv && o && gateup && down && ln1_host && ln2_host, "xfthip_model_set_layer: null argument");
-    XFT_REQUIRE(idx >= 0 && idx < m->cfg.layers, "xfthip_model_set_layer: layer %d out of range", idx);
+int xfthip_model_set_attention(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthip_weight_t o, const float *ln1_host,
+        const float *qkv_bias_host, const float *o_bias_host) {
+    XFT_REQUIRE(m && qkv && o, "xfthip_model_set_attention: null argument");
+    XFT_REQUIRE(idx >= 0 && idx < m->cfg.layers, "xfthip_model_set_attention: layer %d out of range", idx);
     const xfthip_model_config &c = m->cfg;
     const int qcols = c.q_heads * c.head_size, qkv_cols = qcols + 2 * c.kv_heads * c.head_size;
-    XFT_REQUIRE(qkv->pw.K == c.hidden && qkv->pw.N == qkv_cols, "xfthip_model_set_layer: qkv weight is [%d,%d], expected [%d,%d]",
+    XFT_REQUIRE(qkv->pw.K == c.hidden && qkv->pw.N == qkv_cols, "xfthip_model_set_attention: qkv weight is [%d,%d], expected [%d,%d]",
             qkv->pw.K, qkv->pw.N, c.hidden, qkv_cols);
-    XFT_REQUIRE(o->pw.K == qcols && o->pw.N == c.hidden, "xfthip_model_set_layer: o weight is [%d,%d], expected [%d,%d]", o->pw.K,
+    XFT_REQUIRE(o->pw.K == qcols && o->pw.N == c.hidden, "xfthip_model_set_attention: o weight is [%d,%d], expected [%d,%d]", o->pw.K,
             o->pw.N, qcols, c.hidden);
-    XFT_REQUIRE(gateup->pw.K == c.hidden && gateup->pw.N == 2 * c.intermediate && (gateup->pw.flags & XFTHIP_WF_GATEUP),
-            "xfthip_model_set_layer: gate/up weight must be [%d,%d] created with XFTHIP_WF_GATEUP", c.hidden, 2 * c.intermediate);
-    XFT_REQUIRE(down->pw.K == c.intermediate && down->pw.N == c.hidden, "xfthip_model_set_layer: down weight is [%d,%d], expected [%d,%d]",
-            down->pw.K, down->pw.N, c.intermediate, c.hidden);
     LayerW &L = m->layers[idx];
     L.qkv = qkv;
     L.o = o;
-    L.gateup = gateup;
-    L.down = down;
     int rc;
     if ((rc = upload_f32(&L.ln1, ln1_host, c.hidden))) return rc;
-    if ((rc = upload_f32(&L.ln2, ln2_host, c.hidden))) return rc;
     if ((rc = upload_f32(&L.qkv_bias, qkv_bias_host, qkv_cols))) return rc;
     if ((rc = upload_f32(&L.o_bias, o_bias_host, c.hidden))) return rc;
     if (m->graph) {
@@ -296,6 +320,33 @@ int xfthip_model_set_layer(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthi
         m->graph = nullptr;
     }
     return 0;
+}
+
+int xfthip_model_set_mlp(xfthip_model_t m, int idx, xfthip_weight_t gateup, xfthip_weight_t down, const float *ln2_host) {
+    XFT_REQUIRE(m && gateup && down, "xfthip_model_set_mlp: null argument");
+    XFT_REQUIRE(idx >= 0 && idx < m->cfg.layers, "xfthip_model_set_mlp: layer %d out of range", idx);
+    const xfthip_model_config &c = m->cfg;
+    XFT_REQUIRE(gateup->pw.K == c.hidden && gateup->pw.N == 2 * c.intermediate && (gateup->pw.flags & XFTHIP_WF_GATEUP),
+            "xfthip_model_set_mlp: gate/up weight must be [%d,%d] created with XFTHIP_WF_GATEUP", c.hidden, 2 * c.intermediate);
+    XFT_REQUIRE(down->pw.K == c.intermediate && down->pw.N == c.hidden, "xfthip_model_set_mlp: down weight is [%d,%d], expected [%d,%d]",
+            down->pw.K, down->pw.N, c.intermediate, c.hidden);
+    LayerW &L = m->layers[idx];
+    L.gateup = gateup;
+    L.down = down;
+    if (int rc = upload_f32(&L.ln2, ln2_host, c.hidden)) return rc;
+    if (m->graph) {
+        (void)hipGraphExecDestroy(m->graph);
+        m->graph = nullptr;
+    }
+    return 0;
+}
+
+int xfthip_model_set_layer(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthip_weight_t o, xfthip_weight_t gateup,
+        xfthip_weight_t down, const float *ln1_host, const float *ln2_host, const float *qkv_bias_host,
+        const float *o_bias_host) {
+    XFT_REQUIRE(ln1_host && ln2_host, "xfthip_model_set_layer: norm weights are required");
+    if (int rc = xfthip_model_set_attention(m, idx, qkv, o, ln1_host, qkv_bias_host, o_bias_host)) return rc;
+    return xfthip_model_set_mlp(m, idx, gateup, down, ln2_host);
 }
 
 int xfthip_model_set_head(xfthip_model_t m, const uint16_t *embedding_fp16_host, const float *final_norm_host,
@@ -315,16 +366,35 @@ int xfthip_model_set_head(xfthip_model_t m, const uint16_t *embedding_fp16_host,
     return 0;
 }
 
+static int check_forward(xfthip_model_t m, const char *fn, int idx, const void *x_in, const void *x_out, int in_stride,
+        int out_stride, int B, int S, int past) {
+    XFT_REQUIRE(m && x_in && x_out, "%s: null argument", fn);
+    XFT_REQUIRE(idx >= 0 && idx < m->cfg.layers, "%s: layer %d out of range", fn, idx);
+    XFT_REQUIRE(B > 0 && B <= m->cfg.max_batch && S > 0 && B * S <= m->cfg.max_tokens, "%s: B=%d S=%d exceed max_batch=%d / max_tokens=%d",
+            fn, B, S, m->cfg.max_batch, m->cfg.max_tokens);
+    XFT_REQUIRE(past >= 0 && past + S <= m->cfg.max_seq, "%s: past %d + S %d exceeds max_seq %d", fn, past, S, m->cfg.max_seq);
+    XFT_REQUIRE(in_stride >= m->cfg.hidden && out_stride >= m->cfg.hidden, "%s: stride smaller than hidden", fn);
+    return 0;
+}
+
 int xfthip_model_layer_forward(xfthip_model_t m, int idx, const float *x_in, int in_stride, float *x_out,
         int out_stride, int B, int S, int past, xfthip_stream_t stream) {
-    XFT_REQUIRE(m && x_in && x_out, "xfthip_model_layer_forward: null argument");
-    XFT_REQUIRE(idx >= 0 && idx < m->cfg.layers, "xfthip_model_layer_forward: layer %d out of range", idx);
-    XFT_REQUIRE(B > 0 && B <= m->cfg.max_batch && S > 0 && B * S <= m->cfg.max_tokens,
-            "xfthip_model_layer_forward: B=%d S=%d exceed max_batch=%d / max_tokens=%d", B, S, m->cfg.max_batch, m->cfg.max_tokens);
-    XFT_REQUIRE(past >= 0 && past + S <= m->cfg.max_seq, "xfthip_model_layer_forward: past %d + S %d exceeds max_seq %d", past, S,
-            m->cfg.max_seq);
-    XFT_REQUIRE(in_stride >= m->cfg.hidden && out_stride >= m->cfg.hidden, "xfthip_model_layer_forward: stride smaller than hidden");
+    if (int rc = check_forward(m, "xfthip_model_layer_forward", idx, x_in, x_out, in_stride, out_stride, B, S, past)) return rc;
     return layer_forward(m, idx, x_in, in_stride, x_out, out_stride, B, S, past, nullptr, (hipStream_t)stream);
+}
+
+int xfthip_model_attention_forward(xfthip_model_t m, int idx, const float *x_in, int in_stride, float *x_out,
+        int out_stride, int B, int S, int past, int do_norm, xfthip_stream_t stream) {
+    if (int rc = check_forward(m, "xfthip_model_attention_forward", idx, x_in, x_out, in_stride, out_stride, B, S, past)) return rc;
+    return attention_block(m, idx, x_in, in_stride, x_out, out_stride, B, S, past, nullptr, do_norm != 0, (hipStream_t)stream);
+}
+
+int xfthip_model_mlp_forward(xfthip_model_t m, int idx, const float *x_in, int in_stride, float *x_out, int out_stride,
+        int tokens, int do_norm, xfthip_stream_t stream) {
+    if (int rc = check_forward(m, "xfthip_model_mlp_forward", idx, x_in, x_out, in_stride, out_stride, 1, 1, 0)) return rc;
+    XFT_REQUIRE(tokens > 0 && tokens <= m->cfg.max_tokens, "xfthip_model_mlp_forward: %d tokens exceed max_tokens %d", tokens,
+            m->cfg.max_tokens);
+    return mlp_block(m, idx, x_in, in_stride, x_out, out_stride, tokens, do_norm != 0, (hipStream_t)stream);
 }
 
 int xfthip_model_prefill(xfthip_model_t m, const int *ids_host, int B, int S, float *logits_host, xfthip_stream_t stream) {
@@ -360,7 +430,10 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
     hipStream_t st = (hipStream_t)stream;
     const int B = m->cur_B;
     hipLaunchKernelGGL(fill_int_kernel, dim3(1), dim3(64), 0, st, m->step, 1, 0);
-    if (m->graph == nullptr || m->graph_B != B || m->graph_stream != st) {
+    if (!m->use_graph) {
+        for (int i = 0; i < steps; ++i)
+            if (int rc = decode_step(m, B, st)) return rc;
+    } else if (m->graph == nullptr || m->graph_B != B || m->graph_stream != st) {
         if (m->graph) {
             (void)hipGraphExecDestroy(m->graph);
             m->graph = nullptr;
@@ -391,7 +464,8 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
         m->graph_B = B;
         m->graph_stream = st;
     }
-    for (int i = 0; i < steps; ++i) XFT_CHECK_HIP(hipGraphLaunch(m->graph, st));
+    if (m->use_graph)
+        for (int i = 0; i < steps; ++i) XFT_CHECK_HIP(hipGraphLaunch(m->graph, st));
     XFT_CHECK_HIP(hipStreamSynchronize(st));
     if (ids_out_host) {
         // the log holds the input id of every step; the outputs are rows 1..steps-1 plus the final ids
@@ -401,6 +475,12 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
         XFT_CHECK_HIP(hipMemcpy(ids_out_host + (size_t)(steps - 1) * B, m->ids, (size_t)B * 4, hipMemcpyDeviceToHost));
     }
     m->cur_pos += steps;
+    return 0;
+}
+
+int xfthip_model_use_graph(xfthip_model_t m, int enable) {
+    XFT_REQUIRE(m != nullptr, "xfthip_model_use_graph: null model");
+    m->use_graph = enable != 0;
     return 0;
 }
 

@@ -57,6 +57,7 @@ struct RopeKvParams {
     const int *past_dev;
     const int *positions; // optional explicit position per token (standalone rotary call)
     int skip_q; // 1: query heads are left untouched
+    int table_full; // 1: tables are [maxPos, D] and the second half reads columns [D/2, D)
     KvView kv; // kv.k == nullptr: no append
     void *key; // standalone rotary: separate key pointer (qkv = query), else nullptr
     int kStride;
@@ -96,10 +97,13 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(RopeKvParams p) {
             float a = load_as_f32(rowbase, p.dtype, col + i);
             float bb = load_as_f32(rowbase, p.dtype, col + i + half);
             if (p.cosT) {
-                const float c = p.cosT[(size_t)pos * half + i], sn = p.sinT[(size_t)pos * half + i];
+                const size_t trow = (size_t)pos * (p.table_full ? p.D : half);
+                const float c = p.cosT[trow + i], sn = p.sinT[trow + i];
+                const float c2 = p.table_full ? p.cosT[trow + i + half] : c;
+                const float sn2 = p.table_full ? p.sinT[trow + i + half] : sn;
                 // reference: fmsub(q, cos, qHalf*sin) ; fmadd(qHalf, cos, q*sin)
                 lo[e] = fmaf(a, c, -(bb * sn));
-                hi[e] = fmaf(bb, c, a * sn);
+                hi[e] = fmaf(bb, c2, a * sn2);
             } else {
                 lo[e] = a;
                 hi[e] = bb;
@@ -273,9 +277,27 @@ static int launch_rope(const RopeKvParams &p, int tokens, hipStream_t stream) {
     return 0;
 }
 
+static int rotary_impl(int dtype, const int *positions, void *query, void *key, const float *embCos, const float *embSin,
+        int dim, int qStride, int kStride, int numTokens, int headNum, int headSize, int numKvHeads, int table_full,
+        xfthip_stream_t stream);
+
 int xfthip_rotary_embedding(int dtype, const int *positions, void *query, void *key, const float *embCos,
         const float *embSin, int dim, int qStride, int kStride, int numTokens, int headNum, int headSize,
         int numKvHeads, xfthip_stream_t stream) {
+    return rotary_impl(dtype, positions, query, key, embCos, embSin, dim, qStride, kStride, numTokens, headNum, headSize,
+            numKvHeads, 0, stream);
+}
+
+int xfthip_rotary_embedding_full(int dtype, const int *positions, void *query, void *key, const float *embCos,
+        const float *embSin, int dim, int qStride, int kStride, int numTokens, int headNum, int headSize,
+        int numKvHeads, xfthip_stream_t stream) {
+    return rotary_impl(dtype, positions, query, key, embCos, embSin, dim, qStride, kStride, numTokens, headNum, headSize,
+            numKvHeads, 1, stream);
+}
+
+static int rotary_impl(int dtype, const int *positions, void *query, void *key, const float *embCos, const float *embSin,
+        int dim, int qStride, int kStride, int numTokens, int headNum, int headSize, int numKvHeads, int table_full,
+        xfthip_stream_t stream) {
     XFT_REQUIRE(positions && query && key && embCos && embSin, "xfthip_rotary_embedding: null argument");
     XFT_REQUIRE(dtype == XFTHIP_F32 || dtype == XFTHIP_BF16, "xfthip_rotary_embedding: dtype must be f32 or bf16");
     XFT_REQUIRE(dim == headSize, "xfthip_rotary_embedding: rot dim %d must equal head size %d", dim, headSize);
@@ -295,6 +317,7 @@ int xfthip_rotary_embedding(int dtype, const int *positions, void *query, void *
     p.cosT = embCos;
     p.sinT = embSin;
     p.positions = positions;
+    p.table_full = table_full;
     return launch_rope(p, numTokens, (hipStream_t)stream);
 }
 

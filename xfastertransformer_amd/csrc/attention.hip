@@ -12,8 +12,8 @@
 //                                                     from the score registers
 // Scores, running max / sum and the output accumulate in fp32 (online softmax).  The KV
 // sequence is split over gridDim.x workgroups and over the 4 waves of each; partial
-// (max, sum, O) triples are merged in LDS and, across workgroups, by a second small kernel,
-// the same statistic merge crossAttnShardedHead does (attention_kernels.h:931-983).
+// (max, sum, O) triples are merged in LDS and, across workgroups, by whichever workgroup of
+// the column group finishes last (ticket counter, no spinning), the same statistic merge crossAttnShardedHead does (attention_kernels.h:931-983).
 // INT8 caches are widened to fp16 in registers (exact); the per-token key scale multiplies
 // the score column, the value scale multiplies the probability (gemm_kernel_ext.cpp:471-500,
 // gemm_kernel_ext2.cpp:75-91).
@@ -48,6 +48,7 @@ struct AttnParams {
     const int *past_dev;
     int nsplit, CG;
     float *ws;
+    unsigned int *tickets; // one per (batch, kv head, column group), zero between launches
 };
 
 // 4 int8 -> 2 x (2 fp16), exact: (q ^ 0x80) | 0x6400 is 1152 + q, then subtract 1152
@@ -253,7 +254,8 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnParams p) {
         for (int r = 0; r < 4; ++r) s_o[wave][cl][16 * dt + 4 * g + r] = o[dt][r];
     __syncthreads();
 
-    float *slot = p.ws + (((size_t)(b * p.kv.H + kvh) * p.CG + cg) * p.nsplit + split) * kSlotFloats;
+    const size_t group = (size_t)(b * p.kv.H + kvh) * p.CG + cg;
+    float *slot = p.ws + (group * p.nsplit + split) * kSlotFloats;
     for (int v = threadIdx.x; v < 16 * D; v += 256) {
         const int col = v / D, d = v % D;
         const int cc = cg * 16 + col;
@@ -278,37 +280,59 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnParams p) {
             }
         }
     }
-}
+    if (p.nsplit == 1) return;
 
-// merge of the per-split partials: one block per (b, kvh, column group)
-__global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
-    constexpr int D = 128;
-    const int kvh = blockIdx.x % p.kv.H, cg = blockIdx.x / p.kv.H, b = blockIdx.y;
-    const int ncols = p.S * p.G;
-    const float *base = p.ws + ((size_t)(b * p.kv.H + kvh) * p.CG + cg) * p.nsplit * kSlotFloats;
+    // ---- the workgroup that finishes last merges the splits of its column group ----
+    // (no waiting: every workgroup publishes its partial, takes a ticket and leaves; the one
+    // holding the last ticket sees all partials and resets the counter for the next launch)
+    __shared__ unsigned int s_ticket;
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) s_ticket = atomicAdd(&p.tickets[group], 1u);
+    __syncthreads();
+    if (s_ticket != (unsigned int)(p.nsplit - 1)) return;
+    __threadfence();
+    if (threadIdx.x == 0) p.tickets[group] = 0u;
+    // factors first (one thread per column, then per (split, column)), so that the wide pass over
+    // the partial outputs is a plain weighted sum with independent loads
+    const float *base = p.ws + group * p.nsplit * kSlotFloats;
+    float *s_f = &s_o[0][0][0]; // [nsplit][16] factors, reusing the output staging area
+    float *s_linv = s_f + 64 * 16;
+    if (threadIdx.x < 16) {
+        const int col = threadIdx.x;
+        float m = kNegBig;
+        for (int s = 0; s < p.nsplit; ++s) m = fmaxf(m, base[(size_t)s * kSlotFloats + col]);
+        float l = 0.0f;
+        for (int s = 0; s < p.nsplit; ++s) {
+            const float f = fast_exp(base[(size_t)s * kSlotFloats + col] - m);
+            s_f[s * 16 + col] = f;
+            l += base[(size_t)s * kSlotFloats + 16 + col] * f;
+        }
+        s_linv[col] = 1.0f / l;
+    }
+    __syncthreads();
     for (int v = threadIdx.x; v < 16 * D; v += 256) {
         const int col = v / D, d = v % D;
         const int cc = cg * 16 + col;
         if (cc >= ncols) continue;
-        float m = kNegBig;
-        for (int s = 0; s < p.nsplit; ++s) m = fmaxf(m, base[(size_t)s * kSlotFloats + col]);
-        float l = 0.0f, acc = 0.0f;
-        for (int s = 0; s < p.nsplit; ++s) {
-            const float *sl = base + (size_t)s * kSlotFloats;
-            const float f = fast_exp(sl[col] - m);
-            l += sl[16 + col] * f;
-            acc += sl[32 + col * D + d] * f;
-        }
+        float acc = 0.0f;
+        for (int s = 0; s < p.nsplit; ++s) acc = fmaf(base[(size_t)s * kSlotFloats + 32 + col * D + d], s_f[s * 16 + col], acc);
         const int s_tok = cc / p.G, j = cc % p.G;
         const size_t idx = ((size_t)b * p.S + s_tok) * p.oStride + (size_t)(kvh * p.G + j) * D + d;
-        store_from_f32(p.out, p.out_dtype, idx, acc / l);
+        store_from_f32(p.out, p.out_dtype, idx, acc * s_linv[col]);
     }
 }
 
 static float *g_ws = nullptr;
+static unsigned int *g_tickets = nullptr;
 
 int attention_workspace_init() {
     if (g_ws == nullptr) XFT_CHECK_HIP(hipMalloc((void **)&g_ws, (size_t)kWsSlots * kSlotFloats * sizeof(float)));
+    if (g_tickets == nullptr) {
+        XFT_CHECK_HIP(hipMalloc((void **)&g_tickets, (size_t)kWsSlots * sizeof(unsigned int)));
+        XFT_CHECK_HIP(hipMemset(g_tickets, 0, (size_t)kWsSlots * sizeof(unsigned int)));
+        XFT_CHECK_HIP(hipDeviceSynchronize());
+    }
     return 0;
 }
 
@@ -359,15 +383,12 @@ extern "C" int xfthip_attention(xfthip_kvcache_t c, const void *q, int qStride, 
     if (nsplit > 1)
         if (int rc = attention_workspace_init()) return rc;
     p.ws = g_ws;
+    p.tickets = g_tickets;
     dim3 grid(nsplit, c->kv.H * p.CG, B);
     if (c->kv.int8)
         hipLaunchKernelGGL(attn_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, p);
     else
         hipLaunchKernelGGL(attn_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, p);
     XFT_CHECK_HIP(hipGetLastError());
-    if (nsplit > 1) {
-        hipLaunchKernelGGL(attn_merge_kernel, dim3(c->kv.H * p.CG, B), dim3(256), 0, (hipStream_t)stream, p);
-        XFT_CHECK_HIP(hipGetLastError());
-    }
     return 0;
 }

@@ -22,6 +22,80 @@ __device__ inline float wave_max(float v) {
 }
 
 // ---- RMSNorm: one 256-thread block per row ------------------------------------------------
+// The row is read once with 128-bit loads into registers (up to 8192 columns), squared and
+// reduced (wave shuffles + one LDS exchange), then scaled and written from the registers.
+// All loads of a thread are issued before the first use, so the kernel costs one memory
+// round trip instead of one per element.
+template <bool IN_BF16>
+__device__ inline void load8(const void *in, size_t idx, float *v) {
+    if constexpr (IN_BF16) {
+        const uint4 raw = *(const uint4 *)((const uint16_t *)in + idx);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = u2f(w[i] << 16);
+            v[2 * i + 1] = u2f(w[i] & 0xFFFF0000u);
+        }
+    } else {
+        const float4 a = *(const float4 *)((const float *)in + idx);
+        const float4 b = *(const float4 *)((const float *)in + idx + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    }
+}
+
+template <bool IN_BF16, bool OUT_BF16, int CHUNKS> // CHUNKS x 8 elements per thread
+__global__ __launch_bounds__(256) void rmsnorm_vec_kernel(void *__restrict__ out, const void *__restrict__ in,
+        const float *__restrict__ weight, int cols, int iStride, int oStride, float eps) {
+    __shared__ float part[4];
+    const int row = blockIdx.x;
+    const size_t ibase = (size_t)row * iStride, obase = (size_t)row * oStride;
+    float x[CHUNKS][8];
+    float sq = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int col = (c * 256 + threadIdx.x) * 8;
+        if (col < cols) {
+            load8<IN_BF16>(in, ibase + col, x[c]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[c][i] = 0.0f;
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sq = fmaf(x[c][i], x[c][i], sq);
+    sq = wave_sum(sq);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = sq;
+    __syncthreads();
+    const float total = (part[0] + part[1]) + (part[2] + part[3]);
+    const float var = 1.0f / sqrtf(total / (float)cols + eps);
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int col = (c * 256 + threadIdx.x) * 8;
+        if (col < cols) {
+            float w[8];
+            load8<false>(weight, col, w);
+            if constexpr (OUT_BF16) {
+                uint32_t pk[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t lo = f32_to_bf16_ref((x[c][2 * i] * var) * w[2 * i]);
+                    const uint32_t hi = f32_to_bf16_ref((x[c][2 * i + 1] * var) * w[2 * i + 1]);
+                    pk[i] = lo | (hi << 16);
+                }
+                *(uint4 *)((uint16_t *)out + obase + col) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+            } else {
+                float *o = (float *)out + obase + col;
+                *(float4 *)o = make_float4((x[c][0] * var) * w[0], (x[c][1] * var) * w[1], (x[c][2] * var) * w[2], (x[c][3] * var) * w[3]);
+                *(float4 *)(o + 4) = make_float4((x[c][4] * var) * w[4], (x[c][5] * var) * w[5], (x[c][6] * var) * w[6], (x[c][7] * var) * w[7]);
+            }
+        }
+    }
+}
+
+// generic shape: any column count, stride or alignment
 __global__ __launch_bounds__(256) void rmsnorm_kernel(void *__restrict__ out, int out_dtype,
         const void *__restrict__ in, int in_dtype, const float *__restrict__ weight, int cols, int iStride,
         int oStride, float eps) {
@@ -237,8 +311,36 @@ int xfthip_rmsnorm(void *out, int out_dtype, const void *in, int in_dtype, const
     if (iStride == -1) iStride = cols;
     if (oStride == -1) oStride = cols;
     XFT_REQUIRE(iStride >= cols && oStride >= cols, "xfthip_rmsnorm: stride smaller than cols");
-    hipLaunchKernelGGL(rmsnorm_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, out, out_dtype, in, in_dtype,
-            weight, cols, iStride, oStride, eps);
+    hipStream_t st = (hipStream_t)stream;
+    const bool ib = in_dtype == XFTHIP_BF16, ob = out_dtype == XFTHIP_BF16;
+    const bool vec = cols % 8 == 0 && cols <= 8192 && iStride % 8 == 0 && oStride % 8 == 0 && ((uintptr_t)in & 15) == 0
+            && ((uintptr_t)out & 15) == 0 && ((uintptr_t)weight & 15) == 0;
+    if (vec) {
+        const int chunks = (cols + 2047) / 2048; // 1..4
+#define XFT_RMS(IB, OB, CH) \
+    hipLaunchKernelGGL((rmsnorm_vec_kernel<IB, OB, CH>), dim3(rows), dim3(256), 0, st, out, in, weight, cols, iStride, oStride, eps)
+#define XFT_RMS_CH(IB, OB)            \
+    switch (chunks) {                 \
+        case 1: XFT_RMS(IB, OB, 1); break; \
+        case 2: XFT_RMS(IB, OB, 2); break; \
+        case 3: XFT_RMS(IB, OB, 3); break; \
+        default: XFT_RMS(IB, OB, 4); break; \
+    }
+        if (ib && ob) {
+            XFT_RMS_CH(true, true)
+        } else if (ib) {
+            XFT_RMS_CH(true, false)
+        } else if (ob) {
+            XFT_RMS_CH(false, true)
+        } else {
+            XFT_RMS_CH(false, false)
+        }
+#undef XFT_RMS_CH
+#undef XFT_RMS
+    } else {
+        hipLaunchKernelGGL(rmsnorm_kernel, dim3(rows), dim3(256), 0, st, out, out_dtype, in, in_dtype, weight, cols, iStride,
+                oStride, eps);
+    }
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }

@@ -106,6 +106,61 @@ def test_skinny_gemm_vs_oracle(xh, orc, kind, M, K, N):
     dw.free()
 
 
+@pytest.mark.parametrize("kind", ["int8", "uint4", "nf4"])
+@pytest.mark.parametrize("M", [33, 64, 200, 256])
+@pytest.mark.parametrize("K,N", [(4096, 4096), (512, 80), (1000, 250), (11008, 512)])
+def test_mfma_gemm_vs_oracle(xh, orc, kind, M, K, N):
+    """M > 32 goes to the MFMA-tiled kernel: same parity bar as the small-M kernel."""
+    if (K, N) == (4096, 4096) and M not in (64, 256):
+        pytest.skip("large shape covered at M=64 and M=256")
+    print(f"case kind={kind} M={M} K={K} N={N}", flush=True)
+    k = KINDS[kind]
+    _, w = _weights(orc, k, K, N, 50 + M, asym_int8=(kind == "int8" and N == 80))
+    rng = np.random.default_rng(150 + M)
+    A = orc.round_bf16(rng.standard_normal((M, K)))
+    dw = xh.Weight(k, K, N, w.q, w.scale, w.zero)
+    got32 = _run_gemm(xh, dw, orc.to_bf16(A), M, K, N, xh.F32)
+    exp = orc.qgemm(w, A)
+    assert np.abs(got32 - exp).max() < 2e-3, np.abs(got32 - exp).max()
+    assert _cos(got32, exp) >= 0.9999
+    bias = rng.standard_normal(N).astype(np.float32)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    got = _run_gemm(xh, dw, orc.to_bf16(A), M, K, N, xh.F32, orc.EPI_RESIDENTIAL, bias, res)
+    assert np.abs(got - orc.qgemm(w, A, orc.EPI_RESIDENTIAL, bias=bias, res=res)).max() < 2e-3
+    dw.free()
+
+
+@pytest.mark.parametrize("kind", ["int8", "uint4", "nf4"])
+@pytest.mark.parametrize("M", [40, 256])
+def test_mfma_gateup_silu_vs_oracle(xh, orc, kind, M):
+    K, I = 1024, 2816
+    k = KINDS[kind]
+    _, w = _weights(orc, k, K, 2 * I, 60)
+    rng = np.random.default_rng(61 + M)
+    A = orc.round_bf16(rng.standard_normal((M, K)))
+    dw = xh.Weight(k, K, 2 * I, w.q, w.scale, w.zero, flags=xh.WF_GATEUP)
+    a_dev = xh.DeviceBuffer.from_numpy(orc.to_bf16(A))
+    o_dev = xh.DeviceBuffer(M * I * 4)
+    xh.gemm_gateup_silu(dw, a_dev.ptr, M, K, o_dev.ptr, I, xh.F32)
+    xh.synchronize()
+    got = o_dev.to_numpy(np.float32, (M, I))
+    exp = orc.silu_sum(orc.qgemm(w, A))
+    assert np.abs(got - exp).max() < 2e-3 + 2e-4 * np.abs(exp).max()
+    dw.free()
+
+
+def test_bf16_weight_gemm_both_kernels(xh, orc):
+    rng = np.random.default_rng(70)
+    K, N = 512, 1000
+    W = orc.round_bf16(rng.standard_normal((K, N)) * 0.05)
+    dw = xh.Weight(xh.W_BF16, K, N, orc.to_bf16(W))
+    assert np.array_equal(dw.unpack(), orc.to_bf16(W))
+    for M in (3, 77):
+        A = orc.round_bf16(rng.standard_normal((M, K)))
+        got = _run_gemm(xh, dw, orc.to_bf16(A), M, K, N, xh.F32)
+        assert np.abs(got - orc.gemm_f32(A, W)).max() < 1e-3
+
+
 @pytest.mark.parametrize("epi", ["bias", "silu", "gelu", "resmul", "residential", "residential_bias", "resext"])
 def test_skinny_gemm_epilogues(xh, orc, epi):
     M, K, N = 5, 1024, 272

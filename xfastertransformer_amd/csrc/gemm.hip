@@ -29,25 +29,22 @@ int xfthip_gemm(xfthip_weight_t w, int M, const void *A, int lda, void *C, int l
     XFT_REQUIRE(!(pw.flags & XFTHIP_WF_GATEUP), "xfthip_gemm: weight was packed for xfthip_gemm_gateup_silu");
     XFT_REQUIRE(pw.kind != XFTHIP_W_W8A8, "xfthip_gemm: W8A8 weights are not wired to a kernel yet");
 
-    const size_t csz = (c_dtype == XFTHIP_F32) ? 4 : 2, rsz = (res_dtype == XFTHIP_F32) ? 4 : 2;
-    for (int m0 = 0; m0 < M; m0 += 32) {
-        SkinnyParams p = {};
-        p.M = (M - m0 < 32) ? M - m0 : 32;
-        p.A = (const uint16_t *)A + (size_t)m0 * lda;
-        p.lda = lda;
-        p.C = (char *)C + (size_t)m0 * ldc * csz;
-        p.ldc = ldc;
-        p.c_dtype = c_dtype;
-        p.epi = epilogue;
-        p.bias = bias;
-        p.res = res ? (const char *)res + (size_t)m0 * ldres * rsz : nullptr;
-        p.ldres = ldres;
-        p.res_dtype = res_dtype;
-        p.gamma = gamma;
-        p.gateup = 0;
-        if (int rc = qgemm_skinny(pw, p, (hipStream_t)stream)) return rc;
-    }
-    return 0;
+    SkinnyParams p = {};
+    p.M = M;
+    p.A = (const uint16_t *)A;
+    p.lda = lda;
+    p.C = C;
+    p.ldc = ldc;
+    p.c_dtype = c_dtype;
+    p.epi = epilogue;
+    p.bias = bias;
+    p.res = res;
+    p.ldres = ldres;
+    p.res_dtype = res_dtype;
+    p.gamma = gamma;
+    p.gateup = 0;
+    if (M <= 32) return qgemm_skinny(pw, p, (hipStream_t)stream);
+    return qgemm_mfma(pw, p, (hipStream_t)stream);
 }
 
 int xfthip_gemm_gateup_silu(xfthip_weight_t w, int M, const void *A, int lda, void *out, int ldo, int out_dtype,
@@ -58,19 +55,16 @@ int xfthip_gemm_gateup_silu(xfthip_weight_t w, int M, const void *A, int lda, vo
     XFT_REQUIRE(ldo >= pw.N / 2, "xfthip_gemm_gateup_silu: ldo=%d < I=%d", ldo, pw.N / 2);
     XFT_REQUIRE(out_dtype == XFTHIP_F32 || out_dtype == XFTHIP_BF16, "xfthip_gemm_gateup_silu: out_dtype must be f32 or bf16");
     XFT_REQUIRE(pw.kind != XFTHIP_W_W8A8, "xfthip_gemm_gateup_silu: W8A8 weights are not wired to a kernel yet");
-    const size_t csz = (out_dtype == XFTHIP_F32) ? 4 : 2;
-    for (int m0 = 0; m0 < M; m0 += 32) {
-        SkinnyParams p = {};
-        p.M = (M - m0 < 32) ? M - m0 : 32;
-        p.A = (const uint16_t *)A + (size_t)m0 * lda;
-        p.lda = lda;
-        p.C = (char *)out + (size_t)m0 * ldo * csz;
-        p.ldc = ldo;
-        p.c_dtype = out_dtype;
-        p.gateup = 1;
-        if (int rc = qgemm_skinny(pw, p, (hipStream_t)stream)) return rc;
-    }
-    return 0;
+    SkinnyParams p = {};
+    p.M = M;
+    p.A = (const uint16_t *)A;
+    p.lda = lda;
+    p.C = out;
+    p.ldc = ldo;
+    p.c_dtype = out_dtype;
+    p.gateup = 1;
+    if (M <= 32) return qgemm_skinny(pw, p, (hipStream_t)stream);
+    return qgemm_mfma(pw, p, (hipStream_t)stream);
 }
 
 } // extern "C"

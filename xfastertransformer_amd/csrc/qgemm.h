@@ -21,6 +21,7 @@ struct SkinnyParams {
     int gateup; // 1: combine tile pairs as silu(gate)*up, N counts cat columns
 };
 
-int qgemm_skinny(const PackedWeight &pw, const SkinnyParams &p, hipStream_t stream);
+int qgemm_skinny(const PackedWeight &pw, const SkinnyParams &p, hipStream_t stream); // M <= 32
+int qgemm_mfma(const PackedWeight &pw, const SkinnyParams &p, hipStream_t stream); // any M, built for M > 32
 
 } // namespace xfthip

@@ -129,6 +129,20 @@ int xfthip_gemm_gateup_silu(xfthip_weight_t w, int M, const void *A, int lda, vo
         xfthip_stream_t stream);
 
 
+/*
+ * W8A8 pieces (matmul_helper.h:2762-2965).  quantize_rows: per-row asymmetric INT8 quantisation of
+ * A (f32 or bf16): zero = (min+max)/2, scale = max(|max-zero|,|zero-min|)/127,
+ * q = rne(fma(x, 1/scale, -zero/scale)), sum = (sum q)*scale + K*zero.  gemm_w8a8: int8 x int8 ->
+ * int32 GEMM against an XFTHIP_W_W8A8 weight, then C = s32*sA*sB + sumB*sB*zA + sumA*zB and the
+ * epilogue.  qa: int8 [M, ldq], 16-byte aligned, ldq % 16 == 0.  xfthip_gemm on a W8A8 weight runs
+ * both, quantising its bf16 A into a library-owned scratch (not for use under stream capture).
+ */
+int xfthip_w8a8_quantize_rows(const void *A, int a_dtype, int M, int K, int lda, int8_t *qa, int ldq, float *scale,
+        float *zero, float *sum, xfthip_stream_t stream);
+int xfthip_gemm_w8a8(xfthip_weight_t w, int M, const int8_t *qa, int ldq, const float *scaleA, const float *zeroA,
+        const float *sumA, void *C, int ldc, int c_dtype, int epilogue, const float *bias, const void *res, int ldres,
+        int res_dtype, float gamma, xfthip_stream_t stream);
+
 /* ---- RMSNorm ------------------------------------------------------------------------ */
 /*
  * y = (x * 1/sqrt(mean(x^2) + eps)) * weight, fp32 accumulation.  Replaces xft::rmsNorm /

@@ -372,3 +372,19 @@ class Model:
             self.free()
         except Exception:
             pass
+
+
+# ---------------------------------------------------------------------------- W8A8
+def w8a8_quantize_rows(A_dev, a_dtype, M, K, lda, stream=None):
+    """Returns device buffers (qa [M, ldq], scale, zero, sum) and ldq."""
+    ldq = (K + 15) // 16 * 16
+    qa = DeviceBuffer(M * ldq)
+    s, z, sm = DeviceBuffer(M * 4), DeviceBuffer(M * 4), DeviceBuffer(M * 4)
+    check(lib.xfthip_w8a8_quantize_rows(A_dev, a_dtype, M, K, lda, qa.ptr, ldq, s.ptr, z.ptr, sm.ptr, stream))
+    return qa, s, z, sm, ldq
+
+
+def gemm_w8a8(w, M, qa, ldq, s, z, sm, C_dev, ldc, c_dtype=F32, epi=EPI_NONE, bias=None, res=None, ldres=0,
+              res_dtype=F32, gamma=1.0, stream=None):
+    check(lib.xfthip_gemm_w8a8(w.h, M, qa.ptr, ldq, s.ptr, z.ptr, sm.ptr, C_dev, ldc, c_dtype, epi, bias, res, ldres,
+                               res_dtype, C.c_float(gamma), stream))

@@ -27,7 +27,8 @@ int xfthip_gemm(xfthip_weight_t w, int M, const void *A, int lda, void *C, int l
     XFT_REQUIRE(!needs_res || (res != nullptr && ldres >= pw.N), "xfthip_gemm: epilogue %d needs res with ldres >= N", epilogue);
     XFT_REQUIRE(!needs_res || (res_dtype >= XFTHIP_F32 && res_dtype <= XFTHIP_FP16), "xfthip_gemm: bad res_dtype %d", res_dtype);
     XFT_REQUIRE(!(pw.flags & XFTHIP_WF_GATEUP), "xfthip_gemm: weight was packed for xfthip_gemm_gateup_silu");
-    XFT_REQUIRE(pw.kind != XFTHIP_W_W8A8, "xfthip_gemm: W8A8 weights are not wired to a kernel yet");
+    if (pw.kind == XFTHIP_W_W8A8)
+        return gemm_w8a8_from_bf16(w, M, A, lda, C, ldc, c_dtype, epilogue, bias, res, ldres, res_dtype, gamma, (hipStream_t)stream);
 
     SkinnyParams p = {};
     p.M = M;
@@ -54,7 +55,7 @@ int xfthip_gemm_gateup_silu(xfthip_weight_t w, int M, const void *A, int lda, vo
     XFT_REQUIRE(pw.flags & XFTHIP_WF_GATEUP, "xfthip_gemm_gateup_silu: weight was not created with XFTHIP_WF_GATEUP");
     XFT_REQUIRE(ldo >= pw.N / 2, "xfthip_gemm_gateup_silu: ldo=%d < I=%d", ldo, pw.N / 2);
     XFT_REQUIRE(out_dtype == XFTHIP_F32 || out_dtype == XFTHIP_BF16, "xfthip_gemm_gateup_silu: out_dtype must be f32 or bf16");
-    XFT_REQUIRE(pw.kind != XFTHIP_W_W8A8, "xfthip_gemm_gateup_silu: W8A8 weights are not wired to a kernel yet");
+    XFT_REQUIRE(pw.kind != XFTHIP_W_W8A8, "xfthip_gemm_gateup_silu: W8A8 weights take the unfused path (xfthip_gemm + SwiGLU)");
     SkinnyParams p = {};
     p.M = M;
     p.A = (const uint16_t *)A;

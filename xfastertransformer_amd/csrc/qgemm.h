@@ -24,4 +24,7 @@ struct SkinnyParams {
 int qgemm_skinny(const PackedWeight &pw, const SkinnyParams &p, hipStream_t stream); // M <= 32
 int qgemm_mfma(const PackedWeight &pw, const SkinnyParams &p, hipStream_t stream); // any M, built for M > 32
 
+int gemm_w8a8_from_bf16(xfthip_weight_t w, int M, const void *A, int lda, void *C, int ldc, int c_dtype, int epilogue,
+        const float *bias, const void *res, int ldres, int res_dtype, float gamma, hipStream_t stream);
+
 } // namespace xfthip

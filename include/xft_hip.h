@@ -322,6 +322,31 @@ int xfthip_model_logits(xfthip_model_t m, const float **logits_dev);
 /* first-maximum argmax over rows of fp32 logits [rows, cols] (sampling.cpp:22-131) */
 int xfthip_argmax(const float *logits, int rows, int cols, int *ids_dev, xfthip_stream_t stream);
 
+
+/* ---- Mixtral-style sparse MLP ------------------------------------------------------- */
+typedef struct xfthip_moe *xfthip_moe_t;
+/*
+ * Top-2 expert selection per token over fp32 logits [M, E]: strict '>' scan (the lower index wins
+ * ties), weights = softmax over the two selected logits.  sel: int32 [M, 2], weights: fp32 [M, 2]
+ * (device).  Replaces MixtralMLP::selectTop2Experts (src/layers/mlp_mixtral.h:221-283).
+ */
+int xfthip_moe_top2(const float *logits, int M, int E, int *sel, float *weights, xfthip_stream_t stream);
+/*
+ * One sparse MLP block: RMSNorm (eps 1e-6) -> router GEMM (fp32 router weights, host
+ * [hidden, experts]) -> top-2 -> per expert: gather, SwiGLU MLP, out += w * expert_out; the output
+ * starts as the input (residual).  Replaces MixtralMLP::forward (mlp_mixtral.h:85-187).  Expert
+ * weights: gateup [hidden, 2*intermediate] created with XFTHIP_WF_GATEUP, down [intermediate, hidden].
+ * logits_override: optional device fp32 [tokens, experts] used instead of the router GEMM.
+ * sel_host_out / w_host_out: optional host copies of the routing decision.
+ * The call synchronises the stream once (the per-expert row counts size the expert GEMMs).
+ */
+int xfthip_moe_create(int hidden, int intermediate, int experts, int max_tokens, const float *router_host, const float *ln_host,
+        xfthip_moe_t *out);
+int xfthip_moe_destroy(xfthip_moe_t m);
+int xfthip_moe_set_expert(xfthip_moe_t m, int e, xfthip_weight_t gateup, xfthip_weight_t down);
+int xfthip_moe_forward(xfthip_moe_t m, const float *x_in, int in_stride, float *x_out, int out_stride, int tokens, int do_norm,
+        const float *logits_override, int *sel_host_out, float *w_host_out, xfthip_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -422,3 +422,27 @@ class LlamaModelOracle:
             xn = round_bf16(xn)
         logits = gemm_f32(xn, self.lm)
         return logits, argmax(logits)
+
+
+def mixtral_mlp(x, ln, router, experts, logits_override=None, do_norm=True, rounding="fp32"):
+    """MixtralMLP::forward (src/layers/mlp_mixtral.h:85-187).  experts: list of (gateup QWeight,
+    down QWeight) with gateup = cat(gate, up) [hidden, 2*inter].  Returns (out, sel, weights)."""
+    x = f32(x)
+    r = (lambda a: round_bf16(a)) if rounding == "bf16" else (lambda a: a)
+    xn = r(rmsnorm(x, ln, 1e-6) if do_norm else x)
+    logits = gemm_f32(xn, router) if logits_override is None else f32(logits_override)
+    sel, w = moe_top2(logits)
+    out = x.copy()
+    for e, (gu, dn) in enumerate(experts):
+        rows, slot = np.nonzero(sel == e)
+        if rows.size == 0:
+            continue
+        order = np.argsort(rows, kind="stable")
+        rows, slot = rows[order], slot[order]
+        xe = np.ascontiguousarray(xn[rows])
+        h = r(silu_sum(qgemm(gu, xe)))
+        eo = qgemm(dn, h)
+        idx = i32(rows)
+        wt = f32(w[rows, slot])
+        lib.orc_scatter_add(p(out), out.shape[1], p(f32(eo)), out.shape[1], p(idx), p(wt), rows.size)
+    return out, sel, w

@@ -388,3 +388,44 @@ def gemm_w8a8(w, M, qa, ldq, s, z, sm, C_dev, ldc, c_dtype=F32, epi=EPI_NONE, bi
               res_dtype=F32, gamma=1.0, stream=None):
     check(lib.xfthip_gemm_w8a8(w.h, M, qa.ptr, ldq, s.ptr, z.ptr, sm.ptr, C_dev, ldc, c_dtype, epi, bias, res, ldres,
                                res_dtype, C.c_float(gamma), stream))
+
+
+# ---------------------------------------------------------------------------- Mixtral MoE
+class MoE:
+    def __init__(self, hidden, inter, experts, max_tokens, router, ln=None):
+        self.hidden, self.inter, self.E = hidden, inter, experts
+        router = np.ascontiguousarray(router, np.float32)
+        ln = None if ln is None else np.ascontiguousarray(ln, np.float32)
+        h = C.c_void_p()
+        check(lib.xfthip_moe_create(hidden, inter, experts, max_tokens, _hp(router), _hp(ln), C.byref(h)))
+        self.h = h
+        self._keep = []
+
+    def set_expert(self, e, gateup, down):
+        self._keep += [gateup, down]
+        check(lib.xfthip_moe_set_expert(self.h, e, gateup.h, down.h))
+
+    def forward(self, x_in_dev, x_out_dev, tokens, do_norm=True, logits_override_dev=None, stream=None):
+        sel = np.empty((tokens, 2), np.int32)
+        w = np.empty((tokens, 2), np.float32)
+        check(lib.xfthip_moe_forward(self.h, x_in_dev, self.hidden, x_out_dev, self.hidden, tokens, int(do_norm),
+                                     logits_override_dev, _hp(sel), _hp(w), stream))
+        return sel, w
+
+    def free(self):
+        if self.h is not None:
+            lib.xfthip_moe_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def moe_top2(logits_dev, M, E, stream=None):
+    sel, w = DeviceBuffer(M * 8), DeviceBuffer(M * 8)
+    check(lib.xfthip_moe_top2(logits_dev, M, E, sel.ptr, w.ptr, stream))
+    synchronize()
+    return sel.to_numpy(np.int32, (M, 2)), w.to_numpy(np.float32, (M, 2))

@@ -1,0 +1,225 @@
+// Mixtral-style sparse MLP: router GEMM, top-2 selection with a 2-way softmax, per-expert gather,
+// SwiGLU MLP on the gathered rows and weighted scatter-add.  Replaces MixtralMLP::forward,
+// selectTop2Experts, gatherInput and scatterOutput (reference src/layers/mlp_mixtral.h:29-291).
+// Experts run one after another in ascending order, as the reference's loop does, so every
+// token's two contributions are added in a fixed order.
+#include <vector>
+
+#include "common.h"
+
+namespace xfthip {
+
+// logits[t][e] = sum_k xn[t][k] * Wr[k][e]; one wave per token, fp32 router weights
+// (GateTypeSelector: fp32 for quantised weight types, src/utils/type_selector.h:93-111)
+template <int E>
+__global__ __launch_bounds__(64) void router_kernel(const uint16_t *__restrict__ xn, int ld, const float *__restrict__ Wr,
+        float *__restrict__ logits, int hidden) {
+    const int t = blockIdx.x, lane = threadIdx.x;
+    float acc[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) acc[e] = 0.0f;
+    for (int k = lane; k < hidden; k += 64) {
+        const float x = bf16_to_f32(xn[(size_t)t * ld + k]);
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[e] = fmaf(x, Wr[(size_t)k * E + e], acc[e]);
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) acc[e] += __shfl_xor(acc[e], off, 64);
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) logits[(size_t)t * E + e] = acc[e];
+    }
+}
+
+// strict '>' scan: the lower index wins ties (mlp_mixtral.h:262-283); weights = softmax over the
+// two selected logits (:221-259)
+__global__ void top2_kernel(const float *__restrict__ logits, int M, int E, int *__restrict__ sel, float *__restrict__ w) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= M) return;
+    float max1 = -INFINITY, max2 = -INFINITY;
+    int idx1 = -1, idx2 = -1;
+    for (int j = 0; j < E; ++j) {
+        const float v = logits[(size_t)t * E + j];
+        if (v > max1) {
+            max2 = max1;
+            idx2 = idx1;
+            max1 = v;
+            idx1 = j;
+        } else if (v > max2) {
+            max2 = v;
+            idx2 = j;
+        }
+    }
+    const float e1 = 1.0f, e2 = fast_exp(max2 - max1); // relative to the larger of the two
+    sel[2 * t] = idx1;
+    sel[2 * t + 1] = idx2;
+    w[2 * t] = e1 / (e1 + e2);
+    w[2 * t + 1] = e2 / (e1 + e2);
+}
+
+// per-expert token lists in ascending token order: thread e scans all tokens
+__global__ void build_lists_kernel(const int *__restrict__ sel, const float *__restrict__ w, int M, int E,
+        int *__restrict__ counts, int *__restrict__ idx, float *__restrict__ wts) {
+    const int e = threadIdx.x;
+    if (e >= E) return;
+    int n = 0;
+    for (int t = 0; t < M; ++t) {
+        for (int s = 0; s < 2; ++s) {
+            if (sel[2 * t + s] == e) {
+                idx[(size_t)e * M + n] = t;
+                wts[(size_t)e * M + n] = w[2 * t + s];
+                ++n;
+            }
+        }
+    }
+    counts[e] = n;
+}
+
+__global__ void gather_rows_kernel(const uint16_t *__restrict__ xn, int ld, const int *__restrict__ idx, uint16_t *__restrict__ out,
+        int hidden) {
+    const int r = blockIdx.x;
+    const uint16_t *src = xn + (size_t)idx[r] * ld;
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) out[(size_t)r * hidden + c] = src[c];
+}
+
+// out[idx[r]] += expert_out[r] * w[r]   (xft::addto: one fused multiply-add per element)
+__global__ void scatter_add_kernel(float *__restrict__ out, int ld, const float *__restrict__ eo, const int *__restrict__ idx,
+        const float *__restrict__ wts, int hidden) {
+    const int r = blockIdx.x;
+    float *dst = out + (size_t)idx[r] * ld;
+    const float wv = wts[r];
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = fmaf(eo[(size_t)r * hidden + c], wv, dst[c]);
+}
+
+__global__ void copy_rows_kernel(const float *__restrict__ in, int in_ld, float *__restrict__ out, int out_ld, int hidden) {
+    const int r = blockIdx.x;
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) out[(size_t)r * out_ld + c] = in[(size_t)r * in_ld + c];
+}
+
+__global__ void narrow_rows_kernel2(const float *__restrict__ in, int in_stride, uint16_t *__restrict__ out, int cols) {
+    const float *row = in + (size_t)blockIdx.x * in_stride;
+    uint16_t *orow = out + (size_t)blockIdx.x * cols;
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) orow[c] = f32_to_bf16_ref(row[c]);
+}
+
+} // namespace xfthip
+
+using namespace xfthip;
+
+struct xfthip_moe {
+    int hidden, inter, E, max_tokens;
+    float *router = nullptr, *ln = nullptr;
+    std::vector<xfthip_weight_t> gateup, down;
+    uint16_t *xn = nullptr, *xg = nullptr, *h = nullptr;
+    float *eo = nullptr, *logits = nullptr, *w = nullptr, *wts = nullptr;
+    int *sel = nullptr, *counts = nullptr, *idx = nullptr;
+};
+
+extern "C" {
+
+int xfthip_moe_top2(const float *logits, int M, int E, int *sel, float *weights, xfthip_stream_t stream) {
+    XFT_REQUIRE(logits && sel && weights && M > 0 && E >= 2, "xfthip_moe_top2: bad argument");
+    hipLaunchKernelGGL(top2_kernel, dim3((M + 255) / 256), dim3(256), 0, (hipStream_t)stream, logits, M, E, sel, weights);
+    XFT_CHECK_HIP(hipGetLastError());
+    return 0;
+}
+
+int xfthip_moe_create(int hidden, int intermediate, int experts, int max_tokens, const float *router_host, const float *ln_host,
+        xfthip_moe_t *out) {
+    XFT_REQUIRE(out && router_host, "xfthip_moe_create: null argument");
+    XFT_REQUIRE(experts == 8, "xfthip_moe_create: %d experts unsupported (the router kernel is built for 8)", experts);
+    XFT_REQUIRE(hidden > 0 && hidden % 8 == 0 && intermediate % 16 == 0 && max_tokens > 0, "xfthip_moe_create: bad sizes");
+    xfthip_moe *m = new xfthip_moe();
+    m->hidden = hidden;
+    m->inter = intermediate;
+    m->E = experts;
+    m->max_tokens = max_tokens;
+    m->gateup.assign(experts, nullptr);
+    m->down.assign(experts, nullptr);
+    const size_t T = max_tokens;
+    bool ok = hipMalloc((void **)&m->router, (size_t)hidden * experts * 4) == hipSuccess
+            && hipMalloc((void **)&m->xn, T * hidden * 2) == hipSuccess && hipMalloc((void **)&m->xg, T * hidden * 2) == hipSuccess
+            && hipMalloc((void **)&m->h, T * intermediate * 2) == hipSuccess && hipMalloc((void **)&m->eo, T * hidden * 4) == hipSuccess
+            && hipMalloc((void **)&m->logits, T * experts * 4) == hipSuccess && hipMalloc((void **)&m->w, T * 2 * 4) == hipSuccess
+            && hipMalloc((void **)&m->sel, T * 2 * 4) == hipSuccess && hipMalloc((void **)&m->counts, 64) == hipSuccess
+            && hipMalloc((void **)&m->idx, T * experts * 4) == hipSuccess && hipMalloc((void **)&m->wts, T * experts * 4) == hipSuccess;
+    if (ok && ln_host) ok = hipMalloc((void **)&m->ln, (size_t)hidden * 4) == hipSuccess
+            && hipMemcpy(m->ln, ln_host, (size_t)hidden * 4, hipMemcpyHostToDevice) == hipSuccess;
+    if (ok) ok = hipMemcpy(m->router, router_host, (size_t)hidden * experts * 4, hipMemcpyHostToDevice) == hipSuccess;
+    if (!ok) {
+        set_error("xfthip_moe_create: allocation failed");
+        xfthip_moe_destroy(m);
+        return 1;
+    }
+    *out = m;
+    return 0;
+}
+
+int xfthip_moe_destroy(xfthip_moe_t m) {
+    if (!m) return 0;
+    void *bufs[] = {m->router, m->ln, m->xn, m->xg, m->h, m->eo, m->logits, m->w, m->wts, m->sel, m->counts, m->idx};
+    for (void *b : bufs)
+        if (b) (void)hipFree(b);
+    delete m;
+    return 0;
+}
+
+int xfthip_moe_set_expert(xfthip_moe_t m, int e, xfthip_weight_t gateup, xfthip_weight_t down) {
+    XFT_REQUIRE(m && gateup && down && e >= 0 && e < m->E, "xfthip_moe_set_expert: bad argument");
+    XFT_REQUIRE(gateup->pw.K == m->hidden && gateup->pw.N == 2 * m->inter && (gateup->pw.flags & XFTHIP_WF_GATEUP),
+            "xfthip_moe_set_expert: gate/up weight must be [%d,%d] created with XFTHIP_WF_GATEUP", m->hidden, 2 * m->inter);
+    XFT_REQUIRE(down->pw.K == m->inter && down->pw.N == m->hidden, "xfthip_moe_set_expert: down weight must be [%d,%d]", m->inter, m->hidden);
+    m->gateup[e] = gateup;
+    m->down[e] = down;
+    return 0;
+}
+
+int xfthip_moe_forward(xfthip_moe_t m, const float *x_in, int in_stride, float *x_out, int out_stride, int tokens, int do_norm,
+        const float *logits_override, int *sel_host_out, float *w_host_out, xfthip_stream_t stream) {
+    XFT_REQUIRE(m && x_in && x_out, "xfthip_moe_forward: null argument");
+    XFT_REQUIRE(tokens > 0 && tokens <= m->max_tokens, "xfthip_moe_forward: %d tokens exceed max_tokens %d", tokens, m->max_tokens);
+    XFT_REQUIRE(in_stride >= m->hidden && out_stride >= m->hidden, "xfthip_moe_forward: stride smaller than hidden");
+    XFT_REQUIRE(!do_norm || m->ln, "xfthip_moe_forward: no norm weight was given at creation");
+    for (int e = 0; e < m->E; ++e) XFT_REQUIRE(m->gateup[e] && m->down[e], "xfthip_moe_forward: expert %d has no weights", e);
+    hipStream_t st = (hipStream_t)stream;
+    const int T = tokens, H = m->hidden;
+    // residual: the output starts as a copy of the input (mlp_mixtral.h:116-121)
+    if ((const void *)x_in != (const void *)x_out)
+        hipLaunchKernelGGL(copy_rows_kernel, dim3(T), dim3(256), 0, st, x_in, in_stride, x_out, out_stride, H);
+    if (do_norm) {
+        if (int rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, x_in, XFTHIP_F32, m->ln, T, H, in_stride, H, 1e-6f, st)) return rc;
+    } else {
+        hipLaunchKernelGGL(narrow_rows_kernel2, dim3(T), dim3(256), 0, st, x_in, in_stride, m->xn, H);
+    }
+    const float *logits = logits_override;
+    if (!logits) {
+        hipLaunchKernelGGL(router_kernel<8>, dim3(T), dim3(64), 0, st, m->xn, H, m->router, m->logits, H);
+        logits = m->logits;
+    }
+    if (int rc = xfthip_moe_top2(logits, T, m->E, m->sel, m->w, st)) return rc;
+    hipLaunchKernelGGL(build_lists_kernel, dim3(1), dim3(64), 0, st, m->sel, m->w, T, m->E, m->counts, m->idx, m->wts);
+    XFT_CHECK_HIP(hipGetLastError());
+    int counts[64];
+    XFT_CHECK_HIP(hipMemcpyAsync(counts, m->counts, m->E * sizeof(int), hipMemcpyDeviceToHost, st));
+    XFT_CHECK_HIP(hipStreamSynchronize(st)); // the per-expert row counts size the GEMMs below
+    if (sel_host_out) XFT_CHECK_HIP(hipMemcpy(sel_host_out, m->sel, (size_t)T * 2 * 4, hipMemcpyDeviceToHost));
+    if (w_host_out) XFT_CHECK_HIP(hipMemcpy(w_host_out, m->w, (size_t)T * 2 * 4, hipMemcpyDeviceToHost));
+    for (int e = 0; e < m->E; ++e) {
+        const int n = counts[e];
+        if (n == 0) continue;
+        const int *idx = m->idx + (size_t)e * T;
+        hipLaunchKernelGGL(gather_rows_kernel, dim3(n), dim3(256), 0, st, m->xn, H, idx, m->xg, H);
+        if (int rc = xfthip_gemm_gateup_silu(m->gateup[e], n, m->xg, H, m->h, m->inter, XFTHIP_BF16, st)) return rc;
+        if (int rc = xfthip_gemm(m->down[e], n, m->h, m->inter, m->eo, H, XFTHIP_F32, XFTHIP_EPI_NONE, nullptr, nullptr, 0, XFTHIP_F32,
+                    1.0f, st))
+            return rc;
+        hipLaunchKernelGGL(scatter_add_kernel, dim3(n), dim3(256), 0, st, x_out, out_stride, m->eo, idx, m->wts + (size_t)e * T, H);
+    }
+    XFT_CHECK_HIP(hipGetLastError());
+    return 0;
+}
+
+} // extern "C"

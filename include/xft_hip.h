@@ -314,6 +314,20 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
 /* enable (default) or disable replaying the decode step as a captured HIP graph; with 0 every
  * step launches its kernels one by one (for per-kernel profiling) */
 int xfthip_model_use_graph(xfthip_model_t m, int enable);
+/* Decode of up to 4 sequences with INT8 symmetric layer weights, FP16 cache and a BF16 lm_head runs
+ * as ONE persistent kernel per step (device-wide barriers instead of launches).  enable = 0 falls
+ * back to the per-kernel step (captured in a HIP graph when xfthip_model_use_graph allows).
+ * The reference has no counterpart: its decode step is a host loop over layers
+ * (src/models/common_decoder.h:290-420). */
+int xfthip_model_use_persistent(xfthip_model_t m, int enable);
+/* Per-phase timing of the persistent kernel, which a kernel-level profiler cannot see into.
+ * Call once with ticks_host = NULL to arm it; after a decode call, a second call copies out
+ * 5 * layers + 3 timestamps of the last step (100 MHz ticks): [0] kernel start, [i] the moment
+ * workgroup 0 left device-wide barrier i (embedding; per layer qkv, attention, out-proj,
+ * gate/up, down; lm_head).  No counterpart in the reference. */
+int xfthip_model_persistent_trace(xfthip_model_t m, unsigned long long *ticks_host, int capacity);
+/* How the last xfthip_model_decode ran: 2 = persistent kernel, 1 = graph replay, 0 = eager launches. */
+int xfthip_model_decode_mode(xfthip_model_t m);
 /* ids chosen by the last prefill / decode call (host int32 [B]) and the current position */
 int xfthip_model_last_ids(xfthip_model_t m, int *ids_host, int *position);
 /* fp32 logits of the last step, device pointer [B, vocab] (valid until the next call) */

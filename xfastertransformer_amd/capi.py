@@ -349,6 +349,22 @@ class Model:
     def use_graph(self, enable):
         check(lib.xfthip_model_use_graph(self.h, int(bool(enable))))
 
+    def use_persistent(self, enable):
+        check(lib.xfthip_model_use_persistent(self.h, int(bool(enable))))
+
+    def persistent_trace(self, arm=False):
+        """arm=True: start recording; otherwise the barrier timestamps (seconds) of the last step."""
+        if arm:
+            check(lib.xfthip_model_persistent_trace(self.h, None, 0))
+            return None
+        n = 5 * self.cfg.layers + 3
+        out = np.zeros(n, np.uint64)
+        check(lib.xfthip_model_persistent_trace(self.h, _hp(out), n))
+        return out.astype(np.float64) * 1e-8
+
+    def decode_mode(self):
+        return int(lib.xfthip_model_decode_mode(self.h))
+
     def last_ids(self, B):
         ids = np.empty(B, np.int32)
         pos = C.c_int()

@@ -1,0 +1,354 @@
+// Device-side body of the attention kernel, shared by the stand-alone kernel and the persistent
+// decode kernel.  See attention.hip for the algorithm.
+#pragma once
+#include "kvcache.h"
+
+namespace xfthip {
+
+// the cache is device memory even when its pointers reach the kernel through a table in memory
+#define ATTN_GLOBAL __attribute__((address_space(1)))
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+union HFrag {
+    f16x8 v;
+    uint32_t u[4];
+    u32x4 q;
+    h2 h[4];
+};
+
+constexpr float kNegBig = -1.0e30f;
+constexpr int kWsSlots = 4096; // partial-result slots of the shared workspace
+constexpr int kSlotFloats = 16 * 128 + 32;
+
+struct AttnParams {
+    KvView kv;
+    const uint16_t *q; // bf16
+    int qStride;
+    void *out;
+    int oStride, out_dtype;
+    int B, S, G;
+    float scale;
+    int past;
+    const int *past_dev;
+    int nsplit, CG;
+    float *ws;
+    unsigned int *tickets; // one per (batch, kv head, column group), zero between launches
+};
+
+// 4 int8 -> 2 x (2 fp16), exact: (q ^ 0x80) | 0x6400 is 1152 + q, then subtract 1152
+__device__ inline void widen_i8x4(uint32_t w, h2 &lo, h2 &hi) {
+    const uint32_t x = w ^ 0x80808080u;
+    const uint32_t a = __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u);
+    const uint32_t b = __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u);
+    const h2 off = {(_Float16)1152.0f, (_Float16)1152.0f};
+    lo = __builtin_bit_cast(h2, a) - off;
+    hi = __builtin_bit_cast(h2, b) - off;
+}
+
+__device__ inline uint32_t pack_f16(float a, float b) {
+    h2 v = {(_Float16)a, (_Float16)b};
+    return __builtin_bit_cast(uint32_t, v);
+}
+
+// LDS the unit needs: AttnLds<NW> (about 8.5 KB per wave).  Every thread of the NW-wave block calls it.
+template <int NW>
+struct AttnLds {
+    float s_m[NW][16], s_l[NW][16];
+    float s_o[NW][16][128 + 1];
+    unsigned int s_ticket;
+};
+
+// wg_sync: a barrier over the block.
+// COH: the unit runs inside a kernel whose other workgroups produced q and will consume the
+// output in the same launch: q, the split partials and the output then go through
+// device-coherent accesses (ld_dev / st_dev) and the ticket needs no cache maintenance.  The
+// cache rows appended in the same launch must have been written with st_dev as well.
+template <bool INT8, int NW, bool COH = false, typename Sync>
+__device__ inline void attn_unit(const AttnParams &p, const int split, const int kvh, const int cg, const int b, AttnLds<NW> &L,
+        const Sync &wg_sync) {
+    constexpr int D = 128;
+    auto &s_m = L.s_m;
+    auto &s_l = L.s_l;
+    auto &s_o = L.s_o;
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = lane >> 4, cl = lane & 15;
+    const int past = p.past_dev ? p.past_dev[b] : p.past;
+
+    // this lane's column
+    const int ncols = p.S * p.G;
+    const int c = cg * 16 + cl;
+    const bool cvalid = c < ncols;
+    const int cs = cvalid ? c / p.G : 0, cj = cvalid ? c % p.G : 0;
+    const int limit = cvalid ? past + cs + 1 : 0; // tokens [0, limit) are visible
+    int last_col = cg * 16 + 15;
+    last_col = last_col < ncols ? last_col : ncols - 1;
+    const int lmax = past + last_col / p.G + 1;
+
+    // token-block range of this wave
+    const int nblk = (lmax + 31) >> 5;
+    const int per = (nblk + p.nsplit - 1) / p.nsplit;
+    int wg_begin = split * per, wg_end = wg_begin + per;
+    wg_end = wg_end < nblk ? wg_end : nblk;
+    wg_begin = wg_begin < wg_end ? wg_begin : wg_end;
+    const int wn = wg_end - wg_begin;
+    const int wbase = wn / NW, wrem = wn % NW;
+    const int blk_begin = wg_begin + wave * wbase + (wave < wrem ? wave : wrem);
+    const int blk_end = blk_begin + wbase + (wave < wrem ? 1 : 0);
+
+    // Q fragments (B operand): lane (col, g) holds 8 dims per MFMA step
+    HFrag qf[4];
+    {
+        const uint16_t *qrow = p.q + ((size_t)b * p.S + cs) * p.qStride + (size_t)(kvh * p.G + cj) * D;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const int d0 = INT8 ? 64 * (s >> 1) + 16 * g + 8 * (s & 1) : 32 * s + 8 * g;
+            if (cvalid) {
+                uint32_t raw[4];
+                if constexpr (COH) {
+                    ld_dev16(qrow + d0, raw);
+                } else {
+                    const u32x4 r4 = *(const u32x4 *)(qrow + d0);
+                    raw[0] = r4[0], raw[1] = r4[1], raw[2] = r4[2], raw[3] = r4[3];
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float lo = u2f(raw[i] << 16), hi = u2f(raw[i] & 0xFFFF0000u);
+                    qf[s].u[i] = pack_f16(lo, hi);
+                }
+            } else {
+                qf[s].q = u32x4 {0u, 0u, 0u, 0u};
+            }
+        }
+    }
+
+    const size_t bh = (size_t)b * p.kv.H + kvh;
+    const ATTN_GLOBAL char *kbase = (const ATTN_GLOBAL char *)p.kv.k + bh * p.kv.S * D * (INT8 ? 1 : 2);
+    const ATTN_GLOBAL char *vbase = (const ATTN_GLOBAL char *)p.kv.v + bh * p.kv.S * D * (INT8 ? 1 : 2);
+    const ATTN_GLOBAL float *ksc = INT8 ? (const ATTN_GLOBAL float *)p.kv.kscale + bh * p.kv.S : nullptr;
+    const ATTN_GLOBAL float *vsc = INT8 ? (const ATTN_GLOBAL float *)p.kv.vscale + bh * p.kv.S : nullptr;
+
+    float m_run = kNegBig, l_run = 0.0f;
+    f32x4 o[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = f32x4 {0.f, 0.f, 0.f, 0.f};
+
+    for (int blk = blk_begin; blk < blk_end; ++blk) {
+        const int t0 = blk << 5;
+        // ---- loads: K (2 token tiles x 4 steps), V (8 dim tiles), scales ----
+        HFrag kf[2][4], vf[8];
+        f32x4 ks[2], vs[2];
+        if constexpr (INT8) {
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+                const ATTN_GLOBAL char *row = kbase + (size_t)(t0 + 16 * a + cl) * D + 16 * g;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const u32x4 raw = *(const ATTN_GLOBAL u32x4 *)(row + 64 * j);
+                    widen_i8x4(raw[0], kf[a][2 * j].h[0], kf[a][2 * j].h[1]);
+                    widen_i8x4(raw[1], kf[a][2 * j].h[2], kf[a][2 * j].h[3]);
+                    widen_i8x4(raw[2], kf[a][2 * j + 1].h[0], kf[a][2 * j + 1].h[1]);
+                    widen_i8x4(raw[3], kf[a][2 * j + 1].h[2], kf[a][2 * j + 1].h[3]);
+                }
+                ks[a] = *(const ATTN_GLOBAL f32x4 *)(ksc + t0 + 16 * a + 4 * g);
+                vs[a] = *(const ATTN_GLOBAL f32x4 *)(vsc + t0 + 16 * a + 4 * g);
+            }
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt) {
+                const ATTN_GLOBAL char *src = vbase + ((size_t)blk * D + 16 * dt + cl) * 32 + 8 * g;
+                const u32x2 raw = *(const ATTN_GLOBAL u32x2 *)src;
+                widen_i8x4(raw[0], vf[dt].h[0], vf[dt].h[1]);
+                widen_i8x4(raw[1], vf[dt].h[2], vf[dt].h[3]);
+            }
+        } else {
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+                const ATTN_GLOBAL char *row = kbase + ((size_t)(t0 + 16 * a + cl) * D + 8 * g) * 2;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) kf[a][s].q = *(const ATTN_GLOBAL u32x4 *)(row + 64 * s);
+            }
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt) {
+                const ATTN_GLOBAL char *src = vbase + (((size_t)blk * D + 16 * dt + cl) * 32 + 8 * g) * 2;
+                vf[dt].q = *(const ATTN_GLOBAL u32x4 *)src;
+            }
+        }
+
+        // ---- scores S^T[token = t0 + 16a + 4g + r][col] ----
+        f32x4 sc[2];
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+            sc[a] = f32x4 {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < 4; ++s) sc[a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[a][s].v, qf[s].v, sc[a], 0, 0, 0);
+        }
+        float bmax = kNegBig;
+        bool vis[2][4];
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int t = t0 + 16 * a + 4 * g + r;
+                vis[a][r] = t < limit;
+                float x = sc[a][r];
+                if constexpr (INT8) x *= ks[a][r];
+                x *= p.scale;
+                sc[a][r] = x;
+                bmax = fmaxf(bmax, vis[a][r] ? x : kNegBig);
+            }
+        // column max across the 4 lane groups
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 16, 64));
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
+        const float m_new = fmaxf(m_run, bmax);
+        const float alpha = fast_exp(m_run - m_new);
+        m_run = m_new;
+        float psum = 0.0f;
+        float pr[2][4];
+        // INT8 values: the per-token scale is folded into the probability, normalised by the
+        // block's largest scale so that the fp16 operand stays in [0, 1]
+        float vmax = 0.0f;
+        if constexpr (INT8) {
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) vmax = fmaxf(vmax, vs[a][r]);
+            vmax = fmaxf(vmax, __shfl_xor(vmax, 16, 64));
+            vmax = fmaxf(vmax, __shfl_xor(vmax, 32, 64));
+        }
+        const float vinv = (INT8 && vmax > 0.0f) ? 1.0f / vmax : 1.0f;
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float e = vis[a][r] ? fast_exp(sc[a][r] - m_new) : 0.0f;
+                psum += e;
+                pr[a][r] = INT8 ? e * (vs[a][r] * vinv) : e;
+            }
+        l_run = l_run * alpha + psum;
+        HFrag pf;
+        pf.u[0] = pack_f16(pr[0][0], pr[0][1]);
+        pf.u[1] = pack_f16(pr[0][2], pr[0][3]);
+        pf.u[2] = pack_f16(pr[1][0], pr[1][1]);
+        pf.u[3] = pack_f16(pr[1][2], pr[1][3]);
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) {
+            if constexpr (INT8) {
+                f32x4 tmp = {0.f, 0.f, 0.f, 0.f};
+                tmp = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[dt].v, pf.v, tmp, 0, 0, 0);
+                o[dt] = o[dt] * alpha + tmp * vmax;
+            } else {
+                o[dt] = o[dt] * alpha;
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[dt].v, pf.v, o[dt], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- merge the 4 waves in LDS ----
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    if (g == 0) {
+        s_m[wave][cl] = m_run;
+        s_l[wave][cl] = l_run;
+    }
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s_o[wave][cl][16 * dt + 4 * g + r] = o[dt][r];
+    wg_sync();
+
+    const size_t group = (size_t)(b * p.kv.H + kvh) * p.CG + cg;
+    float *slot = p.ws + (group * p.nsplit + split) * kSlotFloats;
+    for (int v = threadIdx.x; v < 16 * D; v += 64 * NW) {
+        const int col = v / D, d = v % D;
+        const int cc = cg * 16 + col;
+        if (cc >= ncols) continue;
+        float m = s_m[0][col];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) m = fmaxf(m, s_m[w][col]);
+        float l = 0.0f, acc = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            const float f = fast_exp(s_m[w][col] - m);
+            l += s_l[w][col] * f;
+            acc += s_o[w][col][d] * f;
+        }
+        if (p.nsplit == 1) {
+            const int s_tok = cc / p.G, j = cc % p.G;
+            const size_t idx = ((size_t)b * p.S + s_tok) * p.oStride + (size_t)(kvh * p.G + j) * D + d;
+            if constexpr (COH)
+                st_dev((uint16_t *)p.out + idx, f32_to_bf16_ref(acc / l));
+            else
+                store_from_f32(p.out, p.out_dtype, idx, acc / l);
+        } else if constexpr (COH) {
+            st_dev(&slot[32 + col * D + d], acc);
+            if (d == 0) {
+                st_dev(&slot[col], m);
+                st_dev(&slot[16 + col], l);
+            }
+        } else {
+            slot[32 + col * D + d] = acc;
+            if (d == 0) {
+                slot[col] = m;
+                slot[16 + col] = l;
+            }
+        }
+    }
+    if (p.nsplit == 1) return;
+
+    // ---- the workgroup that finishes last merges the splits of its column group ----
+    // (no waiting: every workgroup publishes its partial, takes a ticket and leaves; the one
+    // holding the last ticket sees all partials and resets the counter for the next launch)
+    unsigned int &s_ticket = L.s_ticket;
+    if constexpr (COH)
+        dev_drain();
+    else
+        __threadfence();
+    wg_sync();
+    if (threadIdx.x == 0) s_ticket = atomicAdd(&p.tickets[group], 1u);
+    wg_sync();
+    if (s_ticket != (unsigned int)(p.nsplit - 1)) return;
+    if constexpr (COH) {
+        if (threadIdx.x == 0) st_dev(&p.tickets[group], 0u);
+    } else {
+        __threadfence();
+        if (threadIdx.x == 0) p.tickets[group] = 0u;
+    }
+    auto ws_ld = [](const float *q) { return COH ? ld_dev(q) : *q; };
+    // factors first (one thread per column, then per (split, column)), so that the wide pass over
+    // the partial outputs is a plain weighted sum with independent loads
+    const float *base = p.ws + group * p.nsplit * kSlotFloats;
+    float *s_f = &s_o[0][0][0]; // [nsplit][16] factors, reusing the output staging area
+    float *s_linv = s_f + 64 * 16;
+    if (threadIdx.x < 16) {
+        const int col = threadIdx.x;
+        float m = kNegBig;
+        for (int s = 0; s < p.nsplit; ++s) m = fmaxf(m, ws_ld(&base[(size_t)s * kSlotFloats + col]));
+        float l = 0.0f;
+        for (int s = 0; s < p.nsplit; ++s) {
+            const float f = fast_exp(ws_ld(&base[(size_t)s * kSlotFloats + col]) - m);
+            s_f[s * 16 + col] = f;
+            l += ws_ld(&base[(size_t)s * kSlotFloats + 16 + col]) * f;
+        }
+        s_linv[col] = 1.0f / l;
+    }
+    wg_sync();
+    for (int v = threadIdx.x; v < 16 * D; v += 64 * NW) {
+        const int col = v / D, d = v % D;
+        const int cc = cg * 16 + col;
+        if (cc >= ncols) continue;
+        float acc = 0.0f;
+        for (int s = 0; s < p.nsplit; ++s) acc = fmaf(ws_ld(&base[(size_t)s * kSlotFloats + 32 + col * D + d]), s_f[s * 16 + col], acc);
+        const int s_tok = cc / p.G, j = cc % p.G;
+        const size_t idx = ((size_t)b * p.S + s_tok) * p.oStride + (size_t)(kvh * p.G + j) * D + d;
+        if constexpr (COH)
+            st_dev((uint16_t *)p.out + idx, f32_to_bf16_ref(acc * s_linv[col]));
+        else
+            store_from_f32(p.out, p.out_dtype, idx, acc * s_linv[col]);
+    }
+}
+
+
+} // namespace xfthip

@@ -116,6 +116,30 @@ __device__ inline void store_from_f32(void *p, int dtype, size_t idx, float v) {
         ((uint16_t *)p)[idx] = f32_to_fp16_bits(v);
 }
 
+// Loads and stores that are coherent across the chip's XCDs without cache maintenance.  Each
+// XCD has its own L2; ordinary accesses only become visible to another XCD after an L2
+// write-back on one side and an invalidate on the other.  Relaxed atomics at device scope go
+// past the non-coherent lines instead, which is what workgroups of ONE kernel need when they
+// hand small amounts of data to each other.  dev_drain() waits until this wave's stores have
+// been acknowledged; follow it by a block barrier before signalling other workgroups.
+__device__ inline float ld_dev(const float *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ inline int ld_dev(const int *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ inline uint32_t ld_dev(const uint32_t *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ inline unsigned long long ld_dev(const unsigned long long *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ inline void st_dev(float *p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ inline void st_dev(uint32_t *p, uint32_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ inline void st_dev(uint16_t *p, uint16_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+// 16 bytes (8 bf16 / fp16 values) from a 16-byte aligned address
+__device__ inline void ld_dev16(const void *p, uint32_t (&out)[4]) {
+    const unsigned long long a = ld_dev((const unsigned long long *)p), b = ld_dev((const unsigned long long *)p + 1);
+    out[0] = (uint32_t)a, out[1] = (uint32_t)(a >> 32), out[2] = (uint32_t)b, out[3] = (uint32_t)(b >> 32);
+}
+__device__ inline void dev_drain() {
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): every load returned, every store acknowledged
+}
+
 // exp on the device: the reference uses a degree-5 polynomial (src/utils/bert_util.h:26-75)
 // accurate to ~1e-7 relative; __expf is within the same distance of exp().
 __device__ inline float fast_exp(float x) { return __expf(x); }

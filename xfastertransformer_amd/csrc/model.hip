@@ -17,6 +17,8 @@
 
 #include <vector>
 
+#include "attention_dev.h"
+#include "decode_mega.h"
 #include "kvcache.h"
 
 namespace xfthip {
@@ -116,7 +118,78 @@ struct xfthip_model {
     int graph_B = 0;
     hipStream_t graph_stream = nullptr;
     bool use_graph = true;
+    // persistent whole-step decode kernel: 0 = not examined yet, 1 = usable, -1 = configuration not covered
+    bool use_persistent = false;
+    int mega_state = 0, mega_grid = 0;
+    MegaLayer *mega_layers = nullptr;
+    float *mega_ws = nullptr;
+    unsigned int *mega_sync = nullptr; // [0] barrier counter, [1] abort flag, [64..] attention tickets
+    unsigned long long *mega_trace = nullptr;
+    int mega_trace_cap = 0;
 };
+
+static void mega_invalidate(xfthip_model *m) {
+    m->mega_state = 0;
+}
+
+// Decides whether the persistent kernel covers this model and builds its per-layer table.
+static int mega_prepare(xfthip_model *m) {
+    const xfthip_model_config &c = m->cfg;
+    m->mega_state = -1;
+    if (c.kv_dtype != XFTHIP_FP16 || c.head_size != 128) return 0;
+    if (c.hidden > 4096 || c.hidden % 64 != 0 || c.intermediate % 16 != 0 || c.vocab <= 0) return 0;
+    if (!m->lm_head || m->lm_head->pw.kind != XFTHIP_W_BF16 || !m->embedding) return 0;
+    std::vector<MegaLayer> tab(c.layers);
+    for (int l = 0; l < c.layers; ++l) {
+        const LayerW &L = m->layers[l];
+        if (!L.qkv || !L.o || !L.gateup || !L.down || !L.ln1 || !L.ln2 || L.qkv_bias || L.o_bias) return 0;
+        const PackedWeight *w[4] = {&L.qkv->pw, &L.o->pw, &L.gateup->pw, &L.down->pw};
+        for (const PackedWeight *pw : w)
+            if (pw->kind != XFTHIP_W_INT8 || pw->zero != nullptr || pw->KT % 4 != 0) return 0;
+        MegaLayer &t = tab[l];
+        t.wqkv = w[0]->packed, t.wo = w[1]->packed, t.wgu = w[2]->packed, t.wdown = w[3]->packed;
+        t.sqkv = w[0]->scale, t.so = w[1]->scale, t.sgu = w[2]->scale, t.sdown = w[3]->scale;
+        t.kt_qkv = w[0]->KT, t.kt_o = w[1]->KT, t.kt_gu = w[2]->KT, t.kt_down = w[3]->KT;
+        t.ln1 = L.ln1, t.ln2 = L.ln2;
+        t.kv = m->caches[l]->kv;
+    }
+    if (m->lm_head->pw.KT % 4 != 0) return 0;
+    int per_cu = 0;
+    if (int rc = mega_decode_max_blocks(&per_cu)) return rc;
+    if (per_cu < 1) return 0;
+    m->mega_grid = device_cu_count();
+    if (!m->mega_layers) XFT_CHECK_HIP(hipMalloc((void **)&m->mega_layers, tab.size() * sizeof(MegaLayer)));
+    XFT_CHECK_HIP(hipMemcpy(m->mega_layers, tab.data(), tab.size() * sizeof(MegaLayer), hipMemcpyHostToDevice));
+    if (!m->mega_ws) XFT_CHECK_HIP(hipMalloc((void **)&m->mega_ws, (size_t)kWsSlots * kSlotFloats * sizeof(float)));
+    if (!m->mega_sync) {
+        XFT_CHECK_HIP(hipMalloc((void **)&m->mega_sync, (size_t)(64 + kWsSlots) * sizeof(unsigned int)));
+        XFT_CHECK_HIP(hipMemset(m->mega_sync, 0, (size_t)(64 + kWsSlots) * sizeof(unsigned int)));
+    }
+    m->mega_state = 1;
+    return 0;
+}
+
+static int mega_step(xfthip_model *m, int B, hipStream_t st) {
+    const xfthip_model_config &c = m->cfg;
+    MegaParams p = {};
+    p.layers = m->mega_layers;
+    p.nlayers = c.layers, p.M = B, p.hidden = c.hidden, p.inter = c.intermediate, p.qH = c.q_heads, p.kvH = c.kv_heads;
+    p.x = m->x, p.q = m->qkv, p.att = m->att, p.h = m->h, p.pos = m->pos;
+    p.cosT = m->cosT, p.sinT = m->sinT;
+    p.rms_eps = c.rms_eps, p.scale = 1.0f / sqrtf((float)c.head_size);
+    p.ws = m->mega_ws, p.tickets = m->mega_sync + 64;
+    int nsplit = m->mega_grid / (B * c.kv_heads);
+    nsplit = nsplit < 1 ? 1 : (nsplit > 16 ? 16 : nsplit);
+    while (nsplit > 1 && (size_t)B * c.kv_heads * nsplit > (size_t)kWsSlots) --nsplit;
+    p.nsplit = nsplit;
+    p.embedding = m->embedding, p.ids = m->ids, p.final_norm = m->final_norm;
+    p.lm_head = m->lm_head->pw.packed, p.kt_lm = m->lm_head->pw.KT, p.vocab = c.vocab;
+    p.logits = m->logits, p.idlog = m->idlog, p.step = m->step;
+    p.counter = m->mega_sync, p.abort_flag = (int *)(m->mega_sync + 1);
+    p.spin_limit = 400000u;
+    p.trace = m->mega_trace, p.trace_cap = m->mega_trace_cap;
+    return mega_decode_launch(p, m->mega_grid, st);
+}
 
 static int upload_f32(float **dst, const float *src, size_t n) {
     if (*dst) {
@@ -290,7 +363,7 @@ int xfthip_model_destroy(xfthip_model_t m) {
         if (L.qkv_bias) (void)hipFree(L.qkv_bias);
         if (L.o_bias) (void)hipFree(L.o_bias);
     }
-    void *bufs[] = {m->cosT, m->sinT, m->xn, m->qkv, m->att, m->h, m->x, m->xlast, m->logits, m->ids, m->pos, m->step, m->idlog,
+    void *bufs[] = {m->mega_trace, m->mega_layers, m->mega_ws, m->mega_sync, m->cosT, m->sinT, m->xn, m->qkv, m->att, m->h, m->x, m->xlast, m->logits, m->ids, m->pos, m->step, m->idlog,
             m->embedding, m->final_norm};
     for (void *b : bufs)
         if (b) (void)hipFree(b);
@@ -319,6 +392,7 @@ int xfthip_model_set_attention(xfthip_model_t m, int idx, xfthip_weight_t qkv, x
         (void)hipGraphExecDestroy(m->graph);
         m->graph = nullptr;
     }
+    mega_invalidate(m);
     return 0;
 }
 
@@ -338,6 +412,7 @@ int xfthip_model_set_mlp(xfthip_model_t m, int idx, xfthip_weight_t gateup, xfth
         (void)hipGraphExecDestroy(m->graph);
         m->graph = nullptr;
     }
+    mega_invalidate(m);
     return 0;
 }
 
@@ -363,6 +438,7 @@ int xfthip_model_set_head(xfthip_model_t m, const uint16_t *embedding_fp16_host,
     XFT_CHECK_HIP(hipMemcpy(m->embedding, embedding_fp16_host, eb, hipMemcpyHostToDevice));
     if (int rc = upload_f32(&m->final_norm, final_norm_host, c.hidden)) return rc;
     m->lm_head = lm_head;
+    mega_invalidate(m);
     return 0;
 }
 
@@ -430,7 +506,16 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
     hipStream_t st = (hipStream_t)stream;
     const int B = m->cur_B;
     hipLaunchKernelGGL(fill_int_kernel, dim3(1), dim3(64), 0, st, m->step, 1, 0);
-    if (!m->use_graph) {
+    bool persistent = false;
+    if (m->use_persistent && B <= 4 && (size_t)B * c.kv_heads <= (size_t)kWsSlots) {
+        if (m->mega_state == 0)
+            if (int rc = mega_prepare(m)) return rc;
+        persistent = m->mega_state == 1;
+    }
+    if (persistent) {
+        for (int i = 0; i < steps; ++i)
+            if (int rc = mega_step(m, B, st)) return rc;
+    } else if (!m->use_graph) {
         for (int i = 0; i < steps; ++i)
             if (int rc = decode_step(m, B, st)) return rc;
     } else if (m->graph == nullptr || m->graph_B != B || m->graph_stream != st) {
@@ -464,9 +549,20 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
         m->graph_B = B;
         m->graph_stream = st;
     }
-    if (m->use_graph)
+    if (!persistent && m->use_graph)
         for (int i = 0; i < steps; ++i) XFT_CHECK_HIP(hipGraphLaunch(m->graph, st));
     XFT_CHECK_HIP(hipStreamSynchronize(st));
+    if (persistent) {
+        int aborted = 0;
+        XFT_CHECK_HIP(hipMemcpy(&aborted, m->mega_sync + 1, 4, hipMemcpyDeviceToHost));
+        if (aborted) {
+            // the kernel gave up at a barrier: the caches and the residual stream are unusable
+            XFT_CHECK_HIP(hipMemset(m->mega_sync, 0, (size_t)(64 + kWsSlots) * sizeof(unsigned int)));
+            m->cur_B = 0;
+            set_error("xfthip_model_decode: the persistent decode kernel timed out at a device-wide barrier");
+            return 3;
+        }
+    }
     if (ids_out_host) {
         // the log holds the input id of every step; the outputs are rows 1..steps-1 plus the final ids
         std::vector<int> log((size_t)steps * B);
@@ -476,6 +572,35 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
     }
     m->cur_pos += steps;
     return 0;
+}
+
+int xfthip_model_use_persistent(xfthip_model_t m, int enable) {
+    XFT_REQUIRE(m != nullptr, "xfthip_model_use_persistent: null model");
+    m->use_persistent = enable != 0;
+    return 0;
+}
+
+int xfthip_model_persistent_trace(xfthip_model_t m, unsigned long long *ticks_host, int capacity) {
+    XFT_REQUIRE(m && capacity >= 0, "xfthip_model_persistent_trace: bad argument");
+    const int need = 5 * m->cfg.layers + 3;
+    if (ticks_host == nullptr) {
+        // arm: later persistent steps record their barrier times
+        if (!m->mega_trace) {
+            XFT_CHECK_HIP(hipMalloc((void **)&m->mega_trace, (size_t)need * 8));
+            XFT_CHECK_HIP(hipMemset(m->mega_trace, 0, (size_t)need * 8));
+            m->mega_trace_cap = need;
+        }
+        return 0;
+    }
+    XFT_REQUIRE(m->mega_trace != nullptr, "xfthip_model_persistent_trace: tracing was not armed");
+    XFT_REQUIRE(capacity >= need, "xfthip_model_persistent_trace: capacity %d < %d entries", capacity, need);
+    XFT_CHECK_HIP(hipMemcpy(ticks_host, m->mega_trace, (size_t)need * 8, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+int xfthip_model_decode_mode(xfthip_model_t m) {
+    if (!m) return -1;
+    return m->mega_state == 1 && m->use_persistent ? 2 : (m->use_graph ? 1 : 0);
 }
 
 int xfthip_model_use_graph(xfthip_model_t m, int enable) {

@@ -204,6 +204,7 @@ def test_persistent_decode_multi_step_call(xh, orc):
     kernel, no host work between them) returns the ids of single-step calls."""
     B, S, steps, vocab = 2, 20, 16, 1000
     model, _ = build_small_model(xh, orc, 0, 12)
+    model.use_persistent(True)
     ids = np.random.default_rng(37).integers(0, vocab, (B, S)).astype(np.int32)
     model.prefill(ids)
     one = np.stack([model.decode(1, B)[0] for _ in range(steps)])

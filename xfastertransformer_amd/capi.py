@@ -359,7 +359,7 @@ class Model:
             return None
         n = 5 * self.cfg.layers + 3
         out = np.zeros(n, np.uint64)
-        check(lib.xfthip_model_persistent_trace(self.h, _hp(out), n))
+        check(lib.xfthip_model_persistent_trace(self.h, _hp(out), len(out)))
         return out.astype(np.float64) * 1e-8
 
     def decode_mode(self):

@@ -99,48 +99,17 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
     const int blk_begin = wg_begin + wave * wbase + (wave < wrem ? wave : wrem);
     const int blk_end = blk_begin + wbase + (wave < wrem ? 1 : 0);
 
-    // Q fragments (B operand): lane (col, g) holds 8 dims per MFMA step
-    HFrag qf[4];
-    {
-        const uint16_t *qrow = p.q + ((size_t)b * p.S + cs) * p.qStride + (size_t)(kvh * p.G + cj) * D;
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            const int d0 = INT8 ? 64 * (s >> 1) + 16 * g + 8 * (s & 1) : 32 * s + 8 * g;
-            if (cvalid) {
-                uint32_t raw[4];
-                if constexpr (COH) {
-                    ld_dev16(qrow + d0, raw);
-                } else {
-                    const u32x4 r4 = *(const u32x4 *)(qrow + d0);
-                    raw[0] = r4[0], raw[1] = r4[1], raw[2] = r4[2], raw[3] = r4[3];
-                }
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float lo = u2f(raw[i] << 16), hi = u2f(raw[i] & 0xFFFF0000u);
-                    qf[s].u[i] = pack_f16(lo, hi);
-                }
-            } else {
-                qf[s].q = u32x4 {0u, 0u, 0u, 0u};
-            }
-        }
-    }
-
     const size_t bh = (size_t)b * p.kv.H + kvh;
     const ATTN_GLOBAL char *kbase = (const ATTN_GLOBAL char *)p.kv.k + bh * p.kv.S * D * (INT8 ? 1 : 2);
     const ATTN_GLOBAL char *vbase = (const ATTN_GLOBAL char *)p.kv.v + bh * p.kv.S * D * (INT8 ? 1 : 2);
     const ATTN_GLOBAL float *ksc = INT8 ? (const ATTN_GLOBAL float *)p.kv.kscale + bh * p.kv.S : nullptr;
     const ATTN_GLOBAL float *vsc = INT8 ? (const ATTN_GLOBAL float *)p.kv.vscale + bh * p.kv.S : nullptr;
 
-    float m_run = kNegBig, l_run = 0.0f;
-    f32x4 o[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] = f32x4 {0.f, 0.f, 0.f, 0.f};
-
-    for (int blk = blk_begin; blk < blk_end; ++blk) {
+    // K (2 token tiles x 4 steps), V (8 dim tiles) and the scales of one block of 32 tokens
+    HFrag kf[2][4], vf[8];
+    f32x4 ks[2], vs[2];
+    auto load_block = [&](const int blk) {
         const int t0 = blk << 5;
-        // ---- loads: K (2 token tiles x 4 steps), V (8 dim tiles), scales ----
-        HFrag kf[2][4], vf[8];
-        f32x4 ks[2], vs[2];
         if constexpr (INT8) {
 #pragma unroll
             for (int a = 0; a < 2; ++a) {
@@ -176,6 +145,46 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
                 vf[dt].q = *(const ATTN_GLOBAL u32x4 *)src;
             }
         }
+    };
+
+    // Q fragments (B operand): lane (col, g) holds 8 dims per MFMA step.  The raw loads go out
+    // first, then the first block's K / V loads, and only then is q converted, so that the two
+    // round trips overlap.
+    HFrag qf[4];
+    uint32_t qraw[4][4];
+    {
+        const uint16_t *qrow = p.q + ((size_t)b * p.S + cs) * p.qStride + (size_t)(kvh * p.G + cj) * D;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const int d0 = INT8 ? 64 * (s >> 1) + 16 * g + 8 * (s & 1) : 32 * s + 8 * g;
+            qraw[s][0] = qraw[s][1] = qraw[s][2] = qraw[s][3] = 0u;
+            if (cvalid) {
+                if constexpr (COH) {
+                    ld_dev16(qrow + d0, qraw[s]);
+                } else {
+                    const u32x4 r4 = *(const u32x4 *)(qrow + d0);
+                    qraw[s][0] = r4[0], qraw[s][1] = r4[1], qraw[s][2] = r4[2], qraw[s][3] = r4[3];
+                }
+            }
+        }
+    }
+    if (blk_begin < blk_end) load_block(blk_begin);
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float lo = u2f(qraw[s][i] << 16), hi = u2f(qraw[s][i] & 0xFFFF0000u);
+            qf[s].u[i] = pack_f16(lo, hi);
+        }
+
+    float m_run = kNegBig, l_run = 0.0f;
+    f32x4 o[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = f32x4 {0.f, 0.f, 0.f, 0.f};
+
+    for (int blk = blk_begin; blk < blk_end; ++blk) {
+        const int t0 = blk << 5;
+        if (blk != blk_begin) load_block(blk);
 
         // ---- scores S^T[token = t0 + 16a + 4g + r][col] ----
         f32x4 sc[2];
@@ -322,15 +331,26 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
     const float *base = p.ws + group * p.nsplit * kSlotFloats;
     float *s_f = &s_o[0][0][0]; // [nsplit][16] factors, reusing the output staging area
     float *s_linv = s_f + 64 * 16;
+    float *s_pm = s_linv + 16, *s_pl = s_pm + 64 * 16; // [nsplit][16] partial maxima and sums
+    // one load per thread (independent round trips), then the per-column arithmetic from LDS
+    for (int v = threadIdx.x; v < p.nsplit * 32; v += 64 * NW) {
+        const int s = v >> 5, e = v & 31;
+        const float x = ws_ld(&base[(size_t)s * kSlotFloats + e]);
+        if (e < 16)
+            s_pm[s * 16 + e] = x;
+        else
+            s_pl[s * 16 + e - 16] = x;
+    }
+    wg_sync();
     if (threadIdx.x < 16) {
         const int col = threadIdx.x;
         float m = kNegBig;
-        for (int s = 0; s < p.nsplit; ++s) m = fmaxf(m, ws_ld(&base[(size_t)s * kSlotFloats + col]));
+        for (int s = 0; s < p.nsplit; ++s) m = fmaxf(m, s_pm[s * 16 + col]);
         float l = 0.0f;
         for (int s = 0; s < p.nsplit; ++s) {
-            const float f = fast_exp(ws_ld(&base[(size_t)s * kSlotFloats + col]) - m);
+            const float f = fast_exp(s_pm[s * 16 + col] - m);
             s_f[s * 16 + col] = f;
-            l += ws_ld(&base[(size_t)s * kSlotFloats + 16 + col]) * f;
+            l += s_pl[s * 16 + col] * f;
         }
         s_linv[col] = 1.0f / l;
     }
@@ -340,7 +360,14 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
         const int cc = cg * 16 + col;
         if (cc >= ncols) continue;
         float acc = 0.0f;
-        for (int s = 0; s < p.nsplit; ++s) acc = fmaf(ws_ld(&base[(size_t)s * kSlotFloats + 32 + col * D + d]), s_f[s * 16 + col], acc);
+        for (int s0 = 0; s0 < p.nsplit; s0 += 4) {
+            float t[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) t[u] = s0 + u < p.nsplit ? ws_ld(&base[(size_t)(s0 + u) * kSlotFloats + 32 + col * D + d]) : 0.0f;
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (s0 + u < p.nsplit) acc = fmaf(t[u], s_f[(s0 + u) * 16 + col], acc);
+        }
         const int s_tok = cc / p.G, j = cc % p.G;
         const size_t idx = ((size_t)b * p.S + s_tok) * p.oStride + (size_t)(kvh * p.G + j) * D + d;
         if constexpr (COH)

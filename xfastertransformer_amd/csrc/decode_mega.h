@@ -31,7 +31,9 @@ struct MegaParams {
     float *logits;
     int *idlog; // [steps][M]
     int *step;
-    unsigned int *counter;
+    int act_pitch; // LDS activation row pitch (elements): max K of any phase + 8
+    int red_off; // byte offset of the K-slice partial sums behind the activation rows
+    unsigned int *counter; // [0] global arrivals, [64 * (1 + g)] arrivals of the workgroups with blockIdx % 8 == g
     int *abort_flag;
     unsigned int spin_limit;
     unsigned long long *trace; // optional: [0] kernel start, [i] time workgroup 0 left barrier i (100 MHz ticks)
@@ -39,7 +41,8 @@ struct MegaParams {
 };
 
 // occupancy of the kernel (workgroups per compute unit) and its launch (preceded by the counter reset)
-int mega_decode_max_blocks(int *blocks_per_cu);
-int mega_decode_launch(const MegaParams &p, int grid, hipStream_t stream);
+size_t mega_lds_bytes(int M, int act_pitch);
+int mega_decode_max_blocks(int *blocks_per_cu, size_t lds_bytes);
+int mega_decode_launch(const MegaParams &p, int grid, size_t lds_bytes, hipStream_t stream);
 
 } // namespace xfthip

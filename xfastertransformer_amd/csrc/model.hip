@@ -123,7 +123,10 @@ struct xfthip_model {
     int mega_state = 0, mega_grid = 0;
     MegaLayer *mega_layers = nullptr;
     float *mega_ws = nullptr;
-    unsigned int *mega_sync = nullptr; // [0] barrier counter, [1] abort flag, [64..] attention tickets
+    unsigned int *mega_sync = nullptr; // [0, 640) barrier counters, [16] abort flag, [1024, ...) attention tickets
+    int mega_lds_B = 0; // batch the kernel's LDS size was last set up for
+    size_t mega_lds = 0;
+    int mega_pitch = 0;
     unsigned long long *mega_trace = nullptr;
     int mega_trace_cap = 0;
 };
@@ -137,7 +140,7 @@ static int mega_prepare(xfthip_model *m) {
     const xfthip_model_config &c = m->cfg;
     m->mega_state = -1;
     if (c.kv_dtype != XFTHIP_FP16 || c.head_size != 128) return 0;
-    if (c.hidden > 4096 || c.hidden % 64 != 0 || c.intermediate % 16 != 0 || c.vocab <= 0) return 0;
+    if (c.hidden > 8192 || c.hidden % 64 != 0 || c.intermediate % 16 != 0 || c.vocab <= 0) return 0;
     if (!m->lm_head || m->lm_head->pw.kind != XFTHIP_W_BF16 || !m->embedding) return 0;
     std::vector<MegaLayer> tab(c.layers);
     for (int l = 0; l < c.layers; ++l) {
@@ -154,22 +157,40 @@ static int mega_prepare(xfthip_model *m) {
         t.kv = m->caches[l]->kv;
     }
     if (m->lm_head->pw.KT % 4 != 0) return 0;
-    int per_cu = 0;
-    if (int rc = mega_decode_max_blocks(&per_cu)) return rc;
-    if (per_cu < 1) return 0;
     m->mega_grid = device_cu_count();
+    if (m->mega_grid < 8) return 0;
+    int kmax = c.hidden > c.intermediate ? c.hidden : c.intermediate;
+    if (c.q_heads * c.head_size > kmax) kmax = c.q_heads * c.head_size;
+    m->mega_pitch = kmax + 8;
+    m->mega_lds_B = 0;
     if (!m->mega_layers) XFT_CHECK_HIP(hipMalloc((void **)&m->mega_layers, tab.size() * sizeof(MegaLayer)));
     XFT_CHECK_HIP(hipMemcpy(m->mega_layers, tab.data(), tab.size() * sizeof(MegaLayer), hipMemcpyHostToDevice));
     if (!m->mega_ws) XFT_CHECK_HIP(hipMalloc((void **)&m->mega_ws, (size_t)kWsSlots * kSlotFloats * sizeof(float)));
     if (!m->mega_sync) {
-        XFT_CHECK_HIP(hipMalloc((void **)&m->mega_sync, (size_t)(64 + kWsSlots) * sizeof(unsigned int)));
-        XFT_CHECK_HIP(hipMemset(m->mega_sync, 0, (size_t)(64 + kWsSlots) * sizeof(unsigned int)));
+        XFT_CHECK_HIP(hipMalloc((void **)&m->mega_sync, (size_t)(1024 + kWsSlots) * sizeof(unsigned int)));
+        XFT_CHECK_HIP(hipMemset(m->mega_sync, 0, (size_t)(1024 + kWsSlots) * sizeof(unsigned int)));
     }
     m->mega_state = 1;
     return 0;
 }
 
-static int mega_step(xfthip_model *m, int B, hipStream_t st) {
+// LDS of the kernel depends on the batch; returns 0 with *ok = false when it does not fit
+static int mega_fit(xfthip_model *m, int B, bool *ok) {
+    *ok = false;
+    if (m->mega_lds_B != B) {
+        const size_t lds = mega_lds_bytes(B, m->mega_pitch);
+        if (lds > (size_t)160 * 1024) return 0;
+        int per_cu = 0;
+        if (int rc = mega_decode_max_blocks(&per_cu, lds)) return rc;
+        if (per_cu < 1) return 0;
+        m->mega_lds = lds;
+        m->mega_lds_B = B;
+    }
+    *ok = true;
+    return 0;
+}
+
+static int mega_step(xfthip_model *m, int B, int position, hipStream_t st) {
     const xfthip_model_config &c = m->cfg;
     MegaParams p = {};
     p.layers = m->mega_layers;
@@ -177,18 +198,25 @@ static int mega_step(xfthip_model *m, int B, hipStream_t st) {
     p.x = m->x, p.q = m->qkv, p.att = m->att, p.h = m->h, p.pos = m->pos;
     p.cosT = m->cosT, p.sinT = m->sinT;
     p.rms_eps = c.rms_eps, p.scale = 1.0f / sqrtf((float)c.head_size);
-    p.ws = m->mega_ws, p.tickets = m->mega_sync + 64;
-    int nsplit = m->mega_grid / (B * c.kv_heads);
-    nsplit = nsplit < 1 ? 1 : (nsplit > 16 ? 16 : nsplit);
+    p.ws = m->mega_ws, p.tickets = m->mega_sync + 1024;
+    // a unit is 8 waves: one token block of 32 per wave keeps its load chain at a single round
+    // trip, so the context is split as far as there are workgroups
+    const int nblk = (position + 1 + 31) / 32;
+    int nsplit = (nblk + 7) / 8;
+    const int room = m->mega_grid / (B * c.kv_heads);
+    nsplit = nsplit > room ? room : nsplit;
+    nsplit = nsplit < 1 ? 1 : (nsplit > 64 ? 64 : nsplit);
     while (nsplit > 1 && (size_t)B * c.kv_heads * nsplit > (size_t)kWsSlots) --nsplit;
     p.nsplit = nsplit;
+    p.act_pitch = m->mega_pitch;
+    p.red_off = (int)((((size_t)B * m->mega_pitch * 2) + 15) & ~(size_t)15);
     p.embedding = m->embedding, p.ids = m->ids, p.final_norm = m->final_norm;
     p.lm_head = m->lm_head->pw.packed, p.kt_lm = m->lm_head->pw.KT, p.vocab = c.vocab;
     p.logits = m->logits, p.idlog = m->idlog, p.step = m->step;
-    p.counter = m->mega_sync, p.abort_flag = (int *)(m->mega_sync + 1);
+    p.counter = m->mega_sync, p.abort_flag = (int *)(m->mega_sync + 16);
     p.spin_limit = 400000u;
     p.trace = m->mega_trace, p.trace_cap = m->mega_trace_cap;
-    return mega_decode_launch(p, m->mega_grid, st);
+    return mega_decode_launch(p, m->mega_grid, m->mega_lds, st);
 }
 
 static int upload_f32(float **dst, const float *src, size_t n) {
@@ -510,11 +538,12 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
     if (m->use_persistent && B <= 4 && (size_t)B * c.kv_heads <= (size_t)kWsSlots) {
         if (m->mega_state == 0)
             if (int rc = mega_prepare(m)) return rc;
-        persistent = m->mega_state == 1;
+        if (m->mega_state == 1)
+            if (int rc = mega_fit(m, B, &persistent)) return rc;
     }
     if (persistent) {
         for (int i = 0; i < steps; ++i)
-            if (int rc = mega_step(m, B, st)) return rc;
+            if (int rc = mega_step(m, B, m->cur_pos + i, st)) return rc;
     } else if (!m->use_graph) {
         for (int i = 0; i < steps; ++i)
             if (int rc = decode_step(m, B, st)) return rc;
@@ -554,10 +583,10 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
     XFT_CHECK_HIP(hipStreamSynchronize(st));
     if (persistent) {
         int aborted = 0;
-        XFT_CHECK_HIP(hipMemcpy(&aborted, m->mega_sync + 1, 4, hipMemcpyDeviceToHost));
+        XFT_CHECK_HIP(hipMemcpy(&aborted, m->mega_sync + 16, 4, hipMemcpyDeviceToHost));
         if (aborted) {
             // the kernel gave up at a barrier: the caches and the residual stream are unusable
-            XFT_CHECK_HIP(hipMemset(m->mega_sync, 0, (size_t)(64 + kWsSlots) * sizeof(unsigned int)));
+            XFT_CHECK_HIP(hipMemset(m->mega_sync, 0, (size_t)(1024 + kWsSlots) * sizeof(unsigned int)));
             m->cur_B = 0;
             set_error("xfthip_model_decode: the persistent decode kernel timed out at a device-wide barrier");
             return 3;

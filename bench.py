@@ -140,6 +140,8 @@ def main():
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--weights", choices=["int8", "uint4"], default="int8")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-fusion", action="store_true", help="run RMSNorm / RoPE + cache append as their own kernels instead of inside the decode GEMVs")
+    ap.add_argument("--persistent", action="store_true", help="run each decode step as the single persistent kernel (experimental)")
     ap.add_argument("--eager", action="store_true", help="launch decode kernels one by one instead of replaying the captured graph (for per-kernel profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -155,6 +157,10 @@ def main():
 
     if args.eager:
         model.use_graph(False)
+    if args.no_fusion:
+        model.use_fusion(False)
+    if args.persistent:
+        model.use_persistent(True)
     rng = np.random.default_rng(3)
     ids = rng.integers(0, CFG["vocab"], (B, args.prompt)).astype(np.int32)
     t0 = time.time()

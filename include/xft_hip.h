@@ -314,6 +314,13 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
 /* enable (default) or disable replaying the decode step as a captured HIP graph; with 0 every
  * step launches its kernels one by one (for per-kernel profiling) */
 int xfthip_model_use_graph(xfthip_model_t m, int enable);
+/* enable (default) or disable the decode-step fusions: RMSNorm as the prologue of the QKV and
+ * gate/up GEMVs (up to 4 rows) and RoPE + cache append as the epilogue of the QKV GEMV (one new
+ * token per sequence, FP16 cache).  Disabled, the step runs xfthip_rmsnorm / xfthip_gemm /
+ * xfthip_rope_kvstore one after the other; results agree to the last bit of the bf16 hand-over
+ * points except for the fp32 summation order inside the norm.  The reference keeps these as
+ * separate calls (src/layers/attention.h:322-460, src/layers/mlp_llama.h:200-260). */
+int xfthip_model_use_fusion(xfthip_model_t m, int enable);
 /* Decode of up to 4 sequences with INT8 symmetric layer weights, FP16 cache and a BF16 lm_head runs
  * as ONE persistent kernel per step (device-wide barriers instead of launches).  enable = 0 falls
  * back to the per-kernel step (captured in a HIP graph when xfthip_model_use_graph allows).

@@ -199,6 +199,35 @@ def test_persistent_decode_matches_per_kernel_decode(xh, orc, B, S):
             break
 
 
+@pytest.mark.parametrize("kind,B", [(0, 1), (0, 3), (1, 2), (2, 4)])
+def test_fused_decode_step_matches_unfused(xh, orc, kind, B):
+    """The decode-step fusions (RMSNorm as the GEMV prologue, RoPE + cache append as the QKV
+    GEMV's epilogue) keep every bf16 hand-over point of the unfused step; only the fp32 summation
+    order inside the norm differs.  Logits of every step within 1e-2, ids equal unless the
+    top-2 logits are that close."""
+    S, steps, vocab = 21, 10, 1000
+    model, _ = build_small_model(xh, orc, kind, 13, layers=3, B=4)
+    ids = np.random.default_rng(38).integers(0, vocab, (B, S)).astype(np.int32)
+    runs = []
+    for fused in (False, True):
+        model.use_fusion(fused)
+        model.prefill(ids)
+        out, lg = [], []
+        for t in range(steps):
+            out.append(model.decode(1, B)[0])
+            lg.append(model.logits(B))
+        runs.append((np.stack(out), np.stack(lg)))
+    (ids_u, lg_u), (ids_f, lg_f) = runs
+    for t in range(steps):
+        err = float(np.abs(lg_u[t] - lg_f[t]).max())
+        assert err < 1e-2, (t, err)
+        if not np.array_equal(ids_u[t], ids_f[t]):
+            for b in np.nonzero(ids_u[t] != ids_f[t])[0]:
+                gap = float(abs(lg_u[t][b, ids_u[t][b]] - lg_u[t][b, ids_f[t][b]]))
+                assert gap < 2e-2, (t, b, gap)
+            break
+
+
 def test_persistent_decode_multi_step_call(xh, orc):
     """One xfthip_model_decode call for many steps (back-to-back launches of the persistent
     kernel, no host work between them) returns the ids of single-step calls."""

@@ -39,16 +39,21 @@ def build_hip(force=True):
     objdir = os.path.join(CSRC, "build")
     os.makedirs(objdir, exist_ok=True)
     objs = []
-    procs = []
+    todo = []
     for s in srcs:
         o = os.path.join(objdir, os.path.basename(s) + ".o")
         objs.append(o)
         if force or _stale(o, [s] + [d for d in deps if d.endswith(".h")]):
-            cmd = [HIPCC] + HIP_FLAGS + ["-c", s, "-o", o]
-            print("+", " ".join(cmd), flush=True)
-            procs.append((s, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+            todo.append((s, [HIPCC] + HIP_FLAGS + ["-c", s, "-o", o]))
+    # at most `jobs` compilers at a time (the template-heavy units take a minute or two each)
+    jobs = max(1, min(8, os.cpu_count() or 1))
     failed = False
-    for s, pr in procs:
+    running = []
+    built = bool(todo)
+
+    def reap(pr_s):
+        nonlocal failed
+        s, pr = pr_s
         out, _ = pr.communicate()
         out = "\n".join(l for l in out.splitlines() if "not a recognized feature" not in l)
         if out.strip():
@@ -56,9 +61,16 @@ def build_hip(force=True):
         if pr.returncode != 0:
             failed = True
             print("FAILED:", s)
+
+    while todo or running:
+        while todo and len(running) < jobs:
+            s, cmd = todo.pop(0)
+            print("+", " ".join(cmd), flush=True)
+            running.append((s, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        reap(running.pop(0))
     if failed:
         raise RuntimeError("hipcc failed")
-    if force or procs or not os.path.exists(LIB_HIP):
+    if force or built or not os.path.exists(LIB_HIP):
         _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_HIP] + objs)
     return LIB_HIP
 

@@ -349,6 +349,9 @@ class Model:
     def use_graph(self, enable):
         check(lib.xfthip_model_use_graph(self.h, int(bool(enable))))
 
+    def use_fusion(self, enable):
+        check(lib.xfthip_model_use_fusion(self.h, int(bool(enable))))
+
     def use_persistent(self, enable):
         check(lib.xfthip_model_use_persistent(self.h, int(bool(enable))))
 

@@ -20,6 +20,7 @@
 #include "attention_dev.h"
 #include "decode_mega.h"
 #include "kvcache.h"
+#include "qgemm.h"
 
 namespace xfthip {
 
@@ -118,6 +119,7 @@ struct xfthip_model {
     int graph_B = 0;
     hipStream_t graph_stream = nullptr;
     bool use_graph = true;
+    bool fuse_decode = true; // RMSNorm prologue / RoPE + cache-append epilogue inside the decode GEMVs
     // persistent whole-step decode kernel: 0 = not examined yet, 1 = usable, -1 = configuration not covered
     bool use_persistent = false;
     int mega_state = 0, mega_grid = 0;
@@ -248,16 +250,48 @@ static int attention_block(xfthip_model *m, int idx, const float *x_in, int in_s
     const int qcols = c.q_heads * c.head_size, kvcols = c.kv_heads * c.head_size;
     const int qkv_cols = qcols + 2 * kvcols;
     int rc;
-    if (do_norm) {
-        if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, x_in, XFTHIP_F32, L.ln1, T, c.hidden, in_stride, c.hidden, c.rms_eps, st))) return rc;
-    } else {
-        hipLaunchKernelGGL(narrow_rows_kernel, dim3(T), dim3(256), 0, st, x_in, in_stride, m->xn, c.hidden);
+    // Decode step (one new token per sequence, a handful of rows): the norm runs as the QKV
+    // GEMV's prologue and the rotation + cache append as its epilogue, which takes two launches
+    // (and their gaps) out of every layer.
+    const PackedWeight &wq = L.qkv->pw;
+    const bool small = m->fuse_decode && wq.kind != XFTHIP_W_W8A8;
+    const bool fuse_norm = small && do_norm && skinny_can_fuse_norm(wq, T);
+    const bool fuse_rope = small && S == 1 && T <= 16 && c.kv_dtype == XFTHIP_FP16 && !L.qkv_bias && c.head_size == 128
+            && wq.KT * ktile_of(wq.kind) == wq.K;
+    if (!fuse_norm) {
+        if (do_norm) {
+            if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, x_in, XFTHIP_F32, L.ln1, T, c.hidden, in_stride, c.hidden, c.rms_eps, st))) return rc;
+        } else {
+            hipLaunchKernelGGL(narrow_rows_kernel, dim3(T), dim3(256), 0, st, x_in, in_stride, m->xn, c.hidden);
+        }
     }
-    if ((rc = xfthip_gemm(L.qkv, T, m->xn, c.hidden, m->qkv, qkv_cols, XFTHIP_BF16, L.qkv_bias ? XFTHIP_EPI_BIAS : XFTHIP_EPI_NONE,
-                 L.qkv_bias, nullptr, 0, XFTHIP_F32, 1.0f, st)))
-        return rc;
-    if ((rc = xfthip_rope_kvstore(m->caches[idx], m->qkv, XFTHIP_BF16, qkv_cols, B, S, c.q_heads, m->cosT, m->sinT, past, past_dev, st)))
-        return rc;
+    if (fuse_norm || fuse_rope) {
+        SkinnyParams sp = {};
+        sp.M = T;
+        sp.A = m->xn;
+        sp.lda = c.hidden;
+        sp.C = m->qkv;
+        sp.ldc = qkv_cols;
+        sp.c_dtype = XFTHIP_BF16;
+        sp.epi = L.qkv_bias ? XFTHIP_EPI_BIAS : XFTHIP_EPI_NONE;
+        sp.bias = L.qkv_bias;
+        sp.gamma = 1.0f;
+        if (fuse_norm) {
+            sp.norm_x = x_in, sp.ldx = in_stride, sp.norm_w = L.ln1, sp.norm_eps = c.rms_eps;
+        }
+        if (fuse_rope) {
+            sp.rope = 1, sp.cosT = m->cosT, sp.sinT = m->sinT, sp.pos_dev = past_dev, sp.pos_host = past;
+            sp.qH = c.q_heads, sp.kvH = c.kv_heads, sp.kv = m->caches[idx]->kv;
+        }
+        if ((rc = qgemm_skinny(wq, sp, st))) return rc;
+    } else {
+        if ((rc = xfthip_gemm(L.qkv, T, m->xn, c.hidden, m->qkv, qkv_cols, XFTHIP_BF16, L.qkv_bias ? XFTHIP_EPI_BIAS : XFTHIP_EPI_NONE,
+                     L.qkv_bias, nullptr, 0, XFTHIP_F32, 1.0f, st)))
+            return rc;
+    }
+    if (!fuse_rope)
+        if ((rc = xfthip_rope_kvstore(m->caches[idx], m->qkv, XFTHIP_BF16, qkv_cols, B, S, c.q_heads, m->cosT, m->sinT, past, past_dev, st)))
+            return rc;
     xfthip_kvcache_t attend = m->caches[idx];
     if (c.kv_dtype == XFTHIP_INT8 && S > 1 && past == 0 && past_dev == nullptr) {
         if ((rc = rope_kvstore_impl(m->prefill_cache, m->qkv, XFTHIP_BF16, qkv_cols, B, S, c.q_heads, m->cosT, m->sinT, 0, nullptr,
@@ -280,13 +314,27 @@ static int mlp_block(xfthip_model *m, int idx, const float *x_in, int in_stride,
     XFT_REQUIRE(L.gateup && L.down, "layer %d has no MLP weights attached", idx);
     XFT_REQUIRE(!do_norm || L.ln2, "layer %d has no MLP norm weight", idx);
     int rc;
-    if (do_norm) {
-        // epsilon 1e-6 is hard-coded on the MLP side of the reference (src/layers/mlp_llama.h:212)
-        if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, x_in, XFTHIP_F32, L.ln2, T, c.hidden, in_stride, c.hidden, 1e-6f, st))) return rc;
+    const PackedWeight &wg = L.gateup->pw;
+    // epsilon 1e-6 is hard-coded on the MLP side of the reference (src/layers/mlp_llama.h:212)
+    if (m->fuse_decode && do_norm && wg.kind != XFTHIP_W_W8A8 && skinny_can_fuse_norm(wg, T)) {
+        SkinnyParams sp = {};
+        sp.M = T;
+        sp.A = m->xn;
+        sp.lda = c.hidden;
+        sp.C = m->h;
+        sp.ldc = c.intermediate;
+        sp.c_dtype = XFTHIP_BF16;
+        sp.gateup = 1;
+        sp.norm_x = x_in, sp.ldx = in_stride, sp.norm_w = L.ln2, sp.norm_eps = 1e-6f;
+        if ((rc = qgemm_skinny(wg, sp, st))) return rc;
     } else {
-        hipLaunchKernelGGL(narrow_rows_kernel, dim3(T), dim3(256), 0, st, x_in, in_stride, m->xn, c.hidden);
+        if (do_norm) {
+            if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, x_in, XFTHIP_F32, L.ln2, T, c.hidden, in_stride, c.hidden, 1e-6f, st))) return rc;
+        } else {
+            hipLaunchKernelGGL(narrow_rows_kernel, dim3(T), dim3(256), 0, st, x_in, in_stride, m->xn, c.hidden);
+        }
+        if ((rc = xfthip_gemm_gateup_silu(L.gateup, T, m->xn, c.hidden, m->h, c.intermediate, XFTHIP_BF16, st))) return rc;
     }
-    if ((rc = xfthip_gemm_gateup_silu(L.gateup, T, m->xn, c.hidden, m->h, c.intermediate, XFTHIP_BF16, st))) return rc;
     return xfthip_gemm(L.down, T, m->h, c.intermediate, x_out, out_stride, XFTHIP_F32, XFTHIP_EPI_RESIDENTIAL, nullptr, x_in, in_stride,
             XFTHIP_F32, 1.0f, st);
 }
@@ -630,6 +678,16 @@ int xfthip_model_persistent_trace(xfthip_model_t m, unsigned long long *ticks_ho
 int xfthip_model_decode_mode(xfthip_model_t m) {
     if (!m) return -1;
     return m->mega_state == 1 && m->use_persistent ? 2 : (m->use_graph ? 1 : 0);
+}
+
+int xfthip_model_use_fusion(xfthip_model_t m, int enable) {
+    XFT_REQUIRE(m != nullptr, "xfthip_model_use_fusion: null model");
+    m->fuse_decode = enable != 0;
+    if (m->graph) {
+        (void)hipGraphExecDestroy(m->graph);
+        m->graph = nullptr;
+    }
+    return 0;
 }
 
 int xfthip_model_use_graph(xfthip_model_t m, int enable) {

@@ -1,6 +1,7 @@
 // Parameter block shared by the weight-only GEMM kernels and their C-ABI entry points.
 #pragma once
 #include "common.h"
+#include "kvcache.h"
 
 namespace xfthip {
 
@@ -19,9 +20,29 @@ struct SkinnyParams {
     int ldres, res_dtype;
     float gamma;
     int gateup; // 1: combine tile pairs as silu(gate)*up, N counts cat columns
+
+    // ---- fusions of the decode step (M <= 4, skinny kernel only) ----
+    // RMSNorm prologue: when norm_x is set, A is ignored and every workgroup normalises the M rows
+    // of norm_x (fp32, row pitch ldx) with norm_w / norm_eps into LDS itself (same arithmetic as
+    // the rmsnorm kernel, bf16 result) while its first weight tiles are in flight.
+    const float *norm_x;
+    int ldx;
+    const float *norm_w;
+    float norm_eps;
+    // RoPE + cache append epilogue of the QKV projection (one new token per sequence, FP16 cache):
+    // column tiles are paired (d, d + 64) within a head, the rotated query goes to C as bf16
+    // (row pitch ldc, q_heads * 128 columns), rotated keys and the values go to the cache at
+    // position pos_dev[m] (or pos_host when pos_dev is null).  The tables hold 64 entries a row.
+    int rope;
+    const float *cosT, *sinT;
+    const int *pos_dev;
+    int pos_host;
+    int qH, kvH;
+    KvView kv;
 };
 
 int qgemm_skinny(const PackedWeight &pw, const SkinnyParams &p, hipStream_t stream); // M <= 32
+bool skinny_can_fuse_norm(const PackedWeight &pw, int M); // may SkinnyParams::norm_x be used
 int qgemm_mfma(const PackedWeight &pw, const SkinnyParams &p, hipStream_t stream); // any M, built for M > 32
 
 int gemm_w8a8_from_bf16(xfthip_weight_t w, int M, const void *A, int lda, void *C, int ldc, int c_dtype, int epilogue,

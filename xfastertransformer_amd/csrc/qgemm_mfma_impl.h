@@ -1,0 +1,399 @@
+// Kernel template of the dequant-fused weight-only GEMM for many activation rows (M > 32), the
+// prefill shape.  Included by one translation unit per weight kind (qgemm_mfma_*.hip) so that
+// the instantiations compile in parallel.
+// Replaces MMHelper::compute* (reference src/utils/matmul_helper.h:565-1705) at large M, where
+// the reference switches to AMX (oneDNN) kernels.  MFMA-bound.
+//
+// A workgroup of 4 wavefronts computes a (4*WN*16 columns) x (WM*16 rows) output tile.  Each
+// wave owns WN column tiles and streams their packed codes from global memory straight into
+// registers (the same 1-KiB tile layout the M <= 32 kernel uses: one 128-bit load per lane is an
+// MFMA "A" operand after widening), so weights never pass through LDS.  The activation rows are
+// shared by the 4 waves: staged through a double-buffered, padded LDS tile and read back as
+// 128-bit "B" operands.  Widening cost (12 VALU ops per 16 codes) is amortised over WM MFMAs.
+// Scale / zero-point / bias / activation / residual are applied in the epilogue.
+#pragma once
+#include <type_traits>
+
+#include "qgemm.h"
+
+namespace xfthip {
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+union MFrag {
+    bf16x8 v;
+    uint32_t u[4];
+    u32x4 q;
+};
+
+__device__ inline uint32_t pack_hi16_m(float lo, float hi) {
+    return __builtin_amdgcn_perm(f2u(hi), f2u(lo), 0x07060302u);
+}
+
+__constant__ float c_nf4_big[16] = {-1.0f, -0.6961928009986877f, -0.5250730514526367f, -0.39491748809814453f,
+        -0.28444138169288635f, -0.18477343022823334f, -0.09105003625154495f, 0.0f, 0.07958029955625534f,
+        0.16093020141124725f, 0.24611230194568634f, 0.33791524171829224f, 0.44070982933044434f,
+        0.5626170039176941f, 0.7229568362236023f, 1.0f};
+
+__device__ inline float silu_big(float x) {
+    return x / (1.0f + fast_exp(-x));
+}
+
+// MFMA shape: v_mfma_f32_32x32x16_bf16 with the activations as the "A" operand (rows = tokens)
+// and the widened weights as "B" (columns = output columns), so a lane's accumulators are
+// D[m = 8 (j/4) + 4 h + j%4][n = lane & 31] (h = lane >> 5): consecutive lanes hold consecutive
+// output columns and the epilogue stores 64-byte row segments.
+//
+// KIND: weight kind; WN: 32-column tiles per wave (4 waves per block split the columns);
+// WM: 32-row activation tiles per block (shared by the waves through LDS); NEED_SUM: accumulate
+// row sums of A for the zero-point term; KTAIL: K is not a whole number of tiles.
+template <int KIND>
+struct StepTraits;
+template <>
+struct StepTraits<XFTHIP_W_INT8> {
+    static constexpr int KTILE = 64, GROUPS = 4, SUB = 1, WREGS = 2; // 8 bytes per lane per k group
+};
+template <>
+struct StepTraits<XFTHIP_W_UINT4> {
+    static constexpr int KTILE = 128, GROUPS = 4, SUB = 2, WREGS = 4; // 16 bytes per lane per k group, 2 MFMAs
+};
+template <>
+struct StepTraits<XFTHIP_W_NF4> {
+    static constexpr int KTILE = 128, GROUPS = 4, SUB = 2, WREGS = 4;
+};
+template <>
+struct StepTraits<XFTHIP_W_BF16> {
+    static constexpr int KTILE = 32, GROUPS = 2, SUB = 1, WREGS = 4;
+};
+
+template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL>
+__global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nblocks_n, int nblocks_m) {
+    using T = StepTraits<KIND>;
+    constexpr int KTILE = T::KTILE, GROUPS = T::GROUPS, SUB = T::SUB, WREGS = T::WREGS;
+    constexpr int ROWS = 32 * WM;
+    constexpr int ROWB = KTILE * 2 + 16; // padded LDS row pitch in bytes
+    constexpr int CHUNKS_PER_ROW = KTILE / 8; // 16-byte chunks
+    constexpr int TOTAL_CHUNKS = ROWS * CHUNKS_PER_ROW;
+    constexpr int ALOADS = TOTAL_CHUNKS / 256;
+    static_assert(TOTAL_CHUNKS % 256 == 0, "activation tile must split evenly over the block");
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int h = lane >> 5, nl = lane & 31;
+
+    // block -> (column block, row block): blocks that share a column block sit on the same XCD
+    // (block ids round-robin over the 8 XCDs), so their weight reads hit that XCD's L2
+    int nb, mb;
+    {
+        const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
+        const int nb8 = (nblocks_n + 7) >> 3;
+        nb = (slot / nblocks_m) + xcd * nb8;
+        mb = slot % nblocks_m;
+        if (slot / nblocks_m >= nb8 || nb >= nblocks_n) return;
+    }
+    const int n32_0 = (nb * 4 + wave) * WN; // first 32-column tile of this wave
+    const int m0 = mb * ROWS;
+
+    uint2 *lut = nullptr;
+    unsigned char *abuf_base = lds;
+    if constexpr (KIND == XFTHIP_W_NF4) {
+        lut = (uint2 *)lds;
+        abuf_base = lds + 2048;
+        {
+            const int i = threadIdx.x;
+            const float c0 = c_nf4_big[i & 15], c1 = c_nf4_big[i >> 4];
+            const uint32_t h0 = f32_to_bf16_ref(c0), h1 = f32_to_bf16_ref(c1);
+            const uint32_t l0 = f32_to_bf16_ref(c0 - bf16_to_f32((uint16_t)h0));
+            const uint32_t l1 = f32_to_bf16_ref(c1 - bf16_to_f32((uint16_t)h1));
+            lut[i] = make_uint2(h0 | (h1 << 16), l0 | (l1 << 16));
+        }
+    }
+
+    f32x16 acc[WN][WM];
+    f32x16 accS[WM];
+#pragma unroll
+    for (int t = 0; t < WN; ++t)
+#pragma unroll
+        for (int m = 0; m < WM; ++m)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) acc[t][m][j] = 0.0f;
+#pragma unroll
+    for (int m = 0; m < WM; ++m)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) accS[m][j] = 0.0f;
+    MFrag ones;
+    ones.u[0] = ones.u[1] = ones.u[2] = ones.u[3] = 0x3F803F80u;
+
+    // weight source of this lane: 16-column packed tile (2 per 32-column MFMA tile), chunk of
+    // its column inside the tile, and which 8-byte half (INT8) / dword pair (4-bit) it uses
+    const uint8_t *wbase[WN];
+#pragma unroll
+    for (int t = 0; t < WN; ++t) {
+        int nt = (n32_0 + t) * 2 + (nl >> 4);
+        nt = nt < p.NTILES ? nt : p.NTILES - 1;
+        wbase[t] = p.packed + (size_t)nt * p.KT * 1024 + (nl & 15) * 16 + (KIND == XFTHIP_W_INT8 ? 8 * h : 0);
+    }
+    constexpr int ROW_STEP = 256 / CHUNKS_PER_ROW;
+    const int a_kc = threadIdx.x % CHUNKS_PER_ROW;
+    const int a_row0 = threadIdx.x / CHUNKS_PER_ROW;
+    uint32_t a_off[ALOADS];
+#pragma unroll
+    for (int i = 0; i < ALOADS; ++i) {
+        int row = m0 + a_row0 + i * ROW_STEP;
+        row = row < p.M ? row : p.M - 1;
+        a_off[i] = (uint32_t)row * (uint32_t)p.lda + a_kc * 8;
+    }
+
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+    uint32_t wreg[2][GROUPS][WN][WREGS];
+    u32x4 areg[ALOADS];
+
+    auto load_w = [&](int buf, int kt) {
+#pragma unroll
+        for (int gq = 0; gq < GROUPS; ++gq)
+#pragma unroll
+            for (int t = 0; t < WN; ++t) {
+                if constexpr (KIND == XFTHIP_W_INT8) {
+                    const uint2 v = *(const uint2 *)(wbase[t] + (size_t)kt * 1024 + gq * 256);
+                    wreg[buf][gq][t][0] = v.x;
+                    wreg[buf][gq][t][1] = v.y;
+                } else if constexpr (KIND == XFTHIP_W_BF16) {
+                    // chunk g = 2 s + h holds k = 8 g .. 8 g + 7
+                    const u32x4 v = *(const u32x4 *)(wbase[t] + (size_t)kt * 1024 + (2 * gq + h) * 256);
+                    wreg[buf][gq][t][0] = v[0]; wreg[buf][gq][t][1] = v[1]; wreg[buf][gq][t][2] = v[2]; wreg[buf][gq][t][3] = v[3];
+                } else {
+                    const u32x4 v = *(const u32x4 *)(wbase[t] + (size_t)kt * 1024 + gq * 256);
+                    wreg[buf][gq][t][0] = v[0]; wreg[buf][gq][t][1] = v[1]; wreg[buf][gq][t][2] = v[2]; wreg[buf][gq][t][3] = v[3];
+                }
+            }
+    };
+    auto load_a = [&](int kt) {
+#pragma unroll
+        for (int i = 0; i < ALOADS; ++i) {
+            if constexpr (KTAIL) {
+                const int k = kt * KTILE + a_kc * 8;
+                const bool v = k < p.K;
+                const u32x4 a = *(const u32x4 *)(p.A + a_off[i] + (v ? (size_t)kt * KTILE : (size_t)0) - (v ? 0 : a_kc * 8));
+                areg[i] = v ? a : zero4;
+            } else {
+                areg[i] = *(const u32x4 *)(p.A + a_off[i] + (size_t)kt * KTILE);
+            }
+        }
+    };
+    auto store_a = [&](int buf) {
+        unsigned char *dst = abuf_base + buf * (ROWS * ROWB);
+#pragma unroll
+        for (int i = 0; i < ALOADS; ++i) *(u32x4 *)(dst + (a_row0 + i * ROW_STEP) * ROWB + a_kc * 16) = areg[i];
+    };
+    // one MFMA k step = 16 k: lane (row/col, h) holds k = kbase + 8 h .. + 8
+    auto compute = [&](int wb, int ab) {
+        const unsigned char *src = abuf_base + ab * (ROWS * ROWB) + nl * ROWB;
+#pragma unroll
+        for (int gq = 0; gq < GROUPS; ++gq) {
+#pragma unroll
+            for (int sb = 0; sb < SUB; ++sb) {
+                // k offset of this step inside the tile
+                const int koff = (KIND == XFTHIP_W_INT8) ? 16 * gq + 8 * h
+                        : (KIND == XFTHIP_W_BF16)        ? 16 * gq + 8 * h
+                                                         : 32 * gq + 16 * sb + 8 * h;
+                MFrag a[WM];
+#pragma unroll
+                for (int m = 0; m < WM; ++m) a[m].q = *(const u32x4 *)(src + m * 32 * ROWB + koff * 2);
+#pragma unroll
+                for (int t = 0; t < WN; ++t) {
+                    MFrag whi, wlo;
+                    if constexpr (KIND == XFTHIP_W_INT8) {
+                        const uint32_t x = wreg[wb][gq][t][0], y = wreg[wb][gq][t][1];
+                        whi.u[0] = pack_hi16_m((float)(int)(int8_t)(x), (float)(int)(int8_t)(x >> 8));
+                        whi.u[1] = pack_hi16_m((float)(int)(int8_t)(x >> 16), (float)((int)x >> 24));
+                        whi.u[2] = pack_hi16_m((float)(int)(int8_t)(y), (float)(int)(int8_t)(y >> 8));
+                        whi.u[3] = pack_hi16_m((float)(int)(int8_t)(y >> 16), (float)((int)y >> 24));
+                    } else if constexpr (KIND == XFTHIP_W_BF16) {
+                        whi.u[0] = wreg[wb][gq][t][0]; whi.u[1] = wreg[wb][gq][t][1];
+                        whi.u[2] = wreg[wb][gq][t][2]; whi.u[3] = wreg[wb][gq][t][3];
+                    } else {
+                        // codes 16 sb + 8 h .. + 8 of the lane's 32-code chunk = dword 2 sb + h
+                        const uint32_t x0 = wreg[wb][gq][t][2 * sb], x1 = wreg[wb][gq][t][2 * sb + 1];
+                        const uint32_t x = h ? x1 : x0;
+                        if constexpr (KIND == XFTHIP_W_UINT4) {
+                            whi.u[0] = (x & 0x000F000Fu) | 0x43004300u;
+                            whi.u[1] = ((x >> 4) & 0x000F000Fu) | 0x43004300u;
+                            whi.u[2] = ((x >> 8) & 0x000F000Fu) | 0x43004300u;
+                            whi.u[3] = ((x >> 12) & 0x000F000Fu) | 0x43004300u;
+                        } else {
+                            const uint2 e0 = lut[x & 0xFF], e1 = lut[(x >> 8) & 0xFF], e2 = lut[(x >> 16) & 0xFF], e3 = lut[x >> 24];
+                            whi.u[0] = e0.x; whi.u[1] = e1.x; whi.u[2] = e2.x; whi.u[3] = e3.x;
+                            wlo.u[0] = e0.y; wlo.u[1] = e1.y; wlo.u[2] = e2.y; wlo.u[3] = e3.y;
+                        }
+                    }
+#pragma unroll
+                    for (int m = 0; m < WM; ++m) {
+                        if constexpr (KIND == XFTHIP_W_NF4)
+                            acc[t][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[m].v, wlo.v, acc[t][m], 0, 0, 0);
+                        acc[t][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[m].v, whi.v, acc[t][m], 0, 0, 0);
+                    }
+                }
+                if constexpr (NEED_SUM) {
+#pragma unroll
+                    for (int m = 0; m < WM; ++m) accS[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[m].v, ones.v, accS[m], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+#define XFT_FENCE() __builtin_amdgcn_sched_barrier(0)
+    const int kt_n = (p.K + KTILE - 1) / KTILE;
+    load_w(0, 0);
+    load_a(0);
+    store_a(0);
+    __syncthreads();
+    int kt = 0;
+    for (; kt + 2 <= kt_n - 1; kt += 2) {
+        load_w(1, kt + 1);
+        load_a(kt + 1);
+        XFT_FENCE();
+        compute(0, 0);
+        XFT_FENCE();
+        store_a(1);
+        __syncthreads();
+        load_w(0, kt + 2);
+        load_a(kt + 2);
+        XFT_FENCE();
+        compute(1, 1);
+        XFT_FENCE();
+        store_a(0);
+        __syncthreads();
+    }
+    if (kt + 1 < kt_n) {
+        load_w(1, kt + 1);
+        load_a(kt + 1);
+        XFT_FENCE();
+        compute(0, 0);
+        XFT_FENCE();
+        store_a(1);
+        __syncthreads();
+        compute(1, 1);
+    } else {
+        compute(0, 0);
+    }
+#undef XFT_FENCE
+
+    // ---- epilogue: lane holds C[m0 + 32 mt + 8 (j/4) + 4 h + j%4][32 (n32_0 + t) + nl] ----
+    auto run_epilogue = [&](auto epi_tag) {
+        constexpr int EPI = decltype(epi_tag)::value;
+#pragma unroll
+        for (int t = 0; t < WN; ++t) {
+            const int np = (n32_0 + t) * 32 + nl;
+            const bool nvalid = np < p.N;
+            float s = 1.0f, z = 0.0f, bv = 0.0f;
+            if constexpr (KIND != XFTHIP_W_BF16) s = p.scale[np < p.NTILES * 16 ? np : 0];
+            if constexpr (KIND == XFTHIP_W_UINT4 || (KIND == XFTHIP_W_INT8 && NEED_SUM)) z = p.zero ? p.zero[np < p.NTILES * 16 ? np : 0] : 0.0f;
+            if constexpr (EPI == XFTHIP_EPI_BIAS || EPI == XFTHIP_EPI_RESIDENTIAL || EPI == XFTHIP_EPI_RESEXT) bv = (p.bias && nvalid) ? p.bias[np] : 0.0f;
+#pragma unroll
+            for (int m = 0; m < WM; ++m) {
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const int row = m0 + 32 * m + 8 * (j >> 2) + 4 * h + (j & 3);
+                    if (row >= p.M || !nvalid) continue;
+                    float x = acc[t][m][j];
+                    if constexpr (KIND == XFTHIP_W_UINT4) {
+                        x = fmaf(s, x - 128.0f * accS[m][j], z * accS[m][j]);
+                    } else if constexpr (KIND == XFTHIP_W_INT8) {
+                        x = s * x;
+                        if constexpr (NEED_SUM) x = fmaf(z, accS[m][j], x);
+                    } else if constexpr (KIND == XFTHIP_W_NF4) {
+                        x = s * x;
+                    }
+                    if constexpr (EPI == XFTHIP_EPI_BIAS) x += bv;
+                    if constexpr (EPI == XFTHIP_EPI_SILU) x = silu_big(x);
+                    if constexpr (EPI == XFTHIP_EPI_GELU) {
+                        const float e = fast_exp(1.702f * x);
+                        x = e / (e + 1.0f) * x;
+                    }
+                    if constexpr (EPI == XFTHIP_EPI_RESMUL) x *= load_as_f32(p.res, p.res_dtype, (size_t)row * p.ldres + np);
+                    if constexpr (EPI == XFTHIP_EPI_RESIDENTIAL) x = (x + bv) + load_as_f32(p.res, p.res_dtype, (size_t)row * p.ldres + np);
+                    if constexpr (EPI == XFTHIP_EPI_RESEXT) x = fmaf(p.gamma, load_as_f32(p.res, p.res_dtype, (size_t)row * p.ldres + np), x + bv);
+                    store_from_f32(p.C, p.c_dtype, (size_t)row * p.ldc + np, x);
+                }
+            }
+        }
+    };
+    if (p.gateup) {
+        // packed columns alternate 16 gate / 16 up: lanes nl < 16 hold gate, nl >= 16 the matching up
+#pragma unroll
+        for (int t = 0; t < WN; ++t) {
+            const int np = (n32_0 + t) * 32 + nl;
+            const int out_col = (n32_0 + t) * 16 + (nl & 15);
+            float s = 1.0f, z = 0.0f;
+            if constexpr (KIND != XFTHIP_W_BF16) s = p.scale[np < p.NTILES * 16 ? np : 0];
+            if constexpr (KIND == XFTHIP_W_UINT4 || (KIND == XFTHIP_W_INT8 && NEED_SUM)) z = p.zero ? p.zero[np < p.NTILES * 16 ? np : 0] : 0.0f;
+#pragma unroll
+            for (int m = 0; m < WM; ++m) {
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const int row = m0 + 32 * m + 8 * (j >> 2) + 4 * h + (j & 3);
+                    float x = acc[t][m][j];
+                    if constexpr (KIND == XFTHIP_W_UINT4) {
+                        x = fmaf(s, x - 128.0f * accS[m][j], z * accS[m][j]);
+                    } else if constexpr (KIND == XFTHIP_W_INT8) {
+                        x = s * x;
+                        if constexpr (NEED_SUM) x = fmaf(z, accS[m][j], x);
+                    } else if constexpr (KIND == XFTHIP_W_NF4) {
+                        x = s * x;
+                    }
+                    const float other = __shfl_xor(x, 16, 64); // gate <-> up partner
+                    if (nl < 16 && row < p.M && out_col < p.N / 2)
+                        store_from_f32(p.C, p.c_dtype, (size_t)row * p.ldc + out_col, other * silu_big(x));
+                }
+            }
+        }
+        return;
+    }
+    switch (p.epi) {
+        case XFTHIP_EPI_BIAS: run_epilogue(std::integral_constant<int, XFTHIP_EPI_BIAS> {}); break;
+        case XFTHIP_EPI_SILU: run_epilogue(std::integral_constant<int, XFTHIP_EPI_SILU> {}); break;
+        case XFTHIP_EPI_GELU: run_epilogue(std::integral_constant<int, XFTHIP_EPI_GELU> {}); break;
+        case XFTHIP_EPI_RESMUL: run_epilogue(std::integral_constant<int, XFTHIP_EPI_RESMUL> {}); break;
+        case XFTHIP_EPI_RESIDENTIAL: run_epilogue(std::integral_constant<int, XFTHIP_EPI_RESIDENTIAL> {}); break;
+        case XFTHIP_EPI_RESEXT: run_epilogue(std::integral_constant<int, XFTHIP_EPI_RESEXT> {}); break;
+        default: run_epilogue(std::integral_constant<int, XFTHIP_EPI_NONE> {}); break;
+    }
+}
+
+template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL>
+static int launch_big2(const SkinnyParams &p, hipStream_t stream) {
+    using T = StepTraits<KIND>;
+    constexpr int ROWS = 32 * WM, ROWB = T::KTILE * 2 + 16;
+    const int n32 = (p.NTILES + 1) / 2;
+    const int nblocks_n = (n32 + 4 * WN - 1) / (4 * WN);
+    const int nblocks_m = (p.M + ROWS - 1) / ROWS;
+    const int nb8 = (nblocks_n + 7) / 8;
+    const int blocks = nb8 * 8 * nblocks_m;
+    const size_t smem = 2 * ROWS * ROWB + (KIND == XFTHIP_W_NF4 ? 2048 : 0);
+    hipLaunchKernelGGL((qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL>), dim3(blocks), dim3(256), smem, stream, p, nblocks_n,
+            nblocks_m);
+    XFT_CHECK_HIP(hipGetLastError());
+    return 0;
+}
+
+template <int KIND, int WN, int WM, bool NEED_SUM>
+static int launch_big(const SkinnyParams &p, hipStream_t stream) {
+    if (p.K % StepTraits<KIND>::KTILE != 0) return launch_big2<KIND, WN, WM, NEED_SUM, true>(p, stream);
+    return launch_big2<KIND, WN, WM, NEED_SUM, false>(p, stream);
+}
+
+template <int KIND, bool NEED_SUM>
+static int dispatch_big_tile(const SkinnyParams &p, hipStream_t stream) {
+    const int cus = device_cu_count();
+    // block tile = (4*WN*32 columns) x (WM*32 rows); take the largest that gives every CU a block
+    const int n32 = (p.NTILES + 1) / 2;
+    const long t_large = (long)((n32 + 7) / 8) * ((p.M + 127) / 128);
+    const long t_mid = (long)((n32 + 3) / 4) * ((p.M + 127) / 128);
+    if (t_large >= cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
+    if (t_mid >= cus) return launch_big<KIND, 1, 4, NEED_SUM>(p, stream);
+    return launch_big<KIND, 1, 2, NEED_SUM>(p, stream);
+}
+
+} // namespace
+} // namespace xfthip

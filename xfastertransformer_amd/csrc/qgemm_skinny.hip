@@ -1,412 +1,36 @@
 // Dequant-fused weight-only GEMM for few activation rows (M <= 32): the decode-time shape.
 // Replaces MMHelper::compute* (reference src/utils/matmul_helper.h:565-1705) for
-// INT8 / UINT4 / NF4 / BF16 weights against bf16 activations.
-//
-// HBM-bound: every weight byte is read exactly once with 128-bit loads.  One wavefront
-// owns NT column tiles (16 output columns each) and a slice of K; the weight tile is the
-// MFMA "A" operand (rows = output columns), the activation rows are the "B" operand
-// (columns = tokens, padded to 16), so D[n][m] accumulates in 4 VGPRs per tile.  The
-// integer codes are widened to bf16 in registers (exact: |code| < 256 fits 8 significant
-// bits), per-column scale / zero-point are applied once in the epilogue.  The K slices of
-// one column block are summed through LDS in a fixed order (deterministic).
+// INT8 / UINT4 / NF4 / BF16 weights against bf16 activations.  The kernel lives in
+// qgemm_skinny_impl.h; this file checks the fused options and picks the weight kind.
 #include "qgemm.h"
 
 namespace xfthip {
 
+int qgemm_skinny_int8(const SkinnyParams &p, hipStream_t stream);
+int qgemm_skinny_uint4(const SkinnyParams &p, hipStream_t stream);
+int qgemm_skinny_nf4(const SkinnyParams &p, hipStream_t stream);
+int qgemm_skinny_bf16(const SkinnyParams &p, hipStream_t stream);
 
-template <int KIND>
-struct KindTraits;
-template <>
-struct KindTraits<XFTHIP_W_INT8> {
-    static constexpr int MPT = 2, KL = 16, KTILE = 64;
-};
-template <>
-struct KindTraits<XFTHIP_W_UINT4> {
-    static constexpr int MPT = 4, KL = 32, KTILE = 128;
-};
-template <>
-struct KindTraits<XFTHIP_W_NF4> {
-    static constexpr int MPT = 4, KL = 32, KTILE = 128;
-};
-template <>
-struct KindTraits<XFTHIP_W_BF16> {
-    static constexpr int MPT = 1, KL = 8, KTILE = 32;
-};
-
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
-union Frag {
-    bf16x8 v;
-    uint32_t u[4];
-    u32x4 q;
-};
-
-// two fp32 -> packed bf16 pair by truncation (exact for small integers)
-__device__ inline uint32_t pack_hi16(float lo, float hi) {
-    return __builtin_amdgcn_perm(f2u(hi), f2u(lo), 0x07060302u);
+// LDS of the RMSNorm prologue: M rows of K + 8 bf16 values
+static inline size_t skinny_norm_lds_bytes(int M, int K) {
+    return (size_t)M * (K + 8) * 2;
 }
 
-// Widen the codes of MFMA step `i` of a lane's 16-byte chunk to 8 bf16 values.
-template <int KIND>
-__device__ inline bf16x8 widen(const u32x4 &w, int i, const uint32_t *lut) {
-    Frag f;
-    Frag src;
-    src.q = w;
-    const uint32_t *wd = src.u;
-    if constexpr (KIND == XFTHIP_W_INT8) {
-        uint32_t a = wd[2 * i], b = wd[2 * i + 1];
-        f.u[0] = pack_hi16((float)(int)(int8_t)(a), (float)(int)(int8_t)(a >> 8));
-        f.u[1] = pack_hi16((float)(int)(int8_t)(a >> 16), (float)((int)a >> 24));
-        f.u[2] = pack_hi16((float)(int)(int8_t)(b), (float)(int)(int8_t)(b >> 8));
-        f.u[3] = pack_hi16((float)(int)(int8_t)(b >> 16), (float)((int)b >> 24));
-    } else if constexpr (KIND == XFTHIP_W_UINT4) {
-        // 0x4300 | u is the bf16 value 128 + u; the 128 is removed in the epilogue
-        uint32_t a = wd[i];
-        f.u[0] = (a & 0x000F000Fu) | 0x43004300u;
-        f.u[1] = ((a >> 4) & 0x000F000Fu) | 0x43004300u;
-        f.u[2] = ((a >> 8) & 0x000F000Fu) | 0x43004300u;
-        f.u[3] = ((a >> 12) & 0x000F000Fu) | 0x43004300u;
-    } else if constexpr (KIND == XFTHIP_W_NF4) {
-        (void)lut; // NF4 goes through widen_nf4
-    } else {
-        f.q = w;
-    }
-    return f.v;
-}
-
-// NF4: a code value is not a bf16 number, so it is split into hi + lo bf16 parts (16
-// significant bits, relative error 2^-17) and multiplied with two MFMAs.  The table maps a
-// byte (two codes) to {hi pair, lo pair}.
-__device__ inline void widen_nf4(const u32x4 &w, int i, const uint2 *lut, bf16x8 &hi, bf16x8 &lo) {
-    Frag src, h, l;
-    src.q = w;
-    const uint32_t a = src.u[i];
-    const uint2 e0 = lut[a & 0xFF], e1 = lut[(a >> 8) & 0xFF], e2 = lut[(a >> 16) & 0xFF], e3 = lut[a >> 24];
-    h.u[0] = e0.x; h.u[1] = e1.x; h.u[2] = e2.x; h.u[3] = e3.x;
-    l.u[0] = e0.y; l.u[1] = e1.y; l.u[2] = e2.y; l.u[3] = e3.y;
-    hi = h.v;
-    lo = l.v;
-}
-
-__device__ inline float silu_f(float x) {
-    return x / (1.0f + fast_exp(-x));
-}
-
-// NF4 code values (QLoRA appendix E), split into bf16 hi + lo parts for the MFMA
-__constant__ float c_nf4_gemm[16] = {-1.0f, -0.6961928009986877f, -0.5250730514526367f, -0.39491748809814453f,
-        -0.28444138169288635f, -0.18477343022823334f, -0.09105003625154495f, 0.0f, 0.07958029955625534f,
-        0.16093020141124725f, 0.24611230194568634f, 0.33791524171829224f, 0.44070982933044434f,
-        0.5626170039176941f, 0.7229568362236023f, 1.0f};
-
-// KIND: weight kind; NT: column tiles per wave; MT: 16-row activation tiles (1 or 2);
-// U: k tiles per load batch (the packed K extent is padded to whole batches);
-// NEED_SUM: also accumulate the row sums of A (zero-point term); KTAIL: K is not a whole
-// number of tiles, activation loads past K are masked.  blockDim.x = 64 * (K slices).
-template <int KIND, int NT, int MT, int U, bool NEED_SUM, bool KTAIL>
-__global__ __launch_bounds__(512) void qgemm_skinny_kernel(SkinnyParams p) {
-    using T = KindTraits<KIND>;
-    constexpr int MPT = T::MPT, KL = T::KL, KTILE = T::KTILE;
-    extern __shared__ float smem[];
-
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int nwaves = blockDim.x >> 6;
-    const int g = lane >> 4, ml = lane & 15;
-    constexpr bool need_sum = NEED_SUM;
-
-    uint2 *lut = nullptr;
-    if constexpr (KIND == XFTHIP_W_NF4) {
-        // 256-entry table: byte -> {bf16 hi parts of (low, high) nibble, bf16 lo parts}
-        lut = (uint2 *)smem;
-        for (int i = threadIdx.x; i < 256; i += blockDim.x) {
-            const float c0 = c_nf4_gemm[i & 15], c1 = c_nf4_gemm[i >> 4];
-            const uint32_t h0 = f32_to_bf16_ref(c0), h1 = f32_to_bf16_ref(c1);
-            const uint32_t l0 = f32_to_bf16_ref(c0 - bf16_to_f32((uint16_t)h0));
-            const uint32_t l1 = f32_to_bf16_ref(c1 - bf16_to_f32((uint16_t)h1));
-            lut[i] = make_uint2(h0 | (h1 << 16), l0 | (l1 << 16));
-        }
-        __syncthreads();
-    }
-    float *red = smem + (KIND == XFTHIP_W_NF4 ? 512 : 0);
-
-    // K slice of this wave: balanced split of the KT / U load batches
-    const int nbatch = p.KT / U;
-    const int base = nbatch / nwaves, rem = nbatch % nwaves;
-    const int b_begin = wave * base + (wave < rem ? wave : rem);
-    const int nb = base + (wave < rem ? 1 : 0);
-    const int nt0 = blockIdx.x * NT;
-
-    f32x4 acc[NT][MT];
-    f32x4 accS[MT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int m = 0; m < MT; ++m) acc[t][m] = f32x4 {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int m = 0; m < MT; ++m) accS[m] = f32x4 {0.f, 0.f, 0.f, 0.f};
-
-    Frag ones;
-    ones.u[0] = ones.u[1] = ones.u[2] = ones.u[3] = 0x3F803F80u;
-
-    // Every load below is unconditional: out-of-range column tiles and activation rows are
-    // clamped to the last valid one (their results are never stored), so the loop body is
-    // straight-line code and the loads of the next batch stay in flight during the MFMAs.
-    const uint8_t *wbase[NT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-        int nt = nt0 + t;
-        nt = nt < p.NTILES ? nt : p.NTILES - 1;
-        wbase[t] = p.packed + (size_t)nt * p.KT * 1024 + lane * 16;
-    }
-    const uint16_t *abase[MT];
-#pragma unroll
-    for (int m = 0; m < MT; ++m) {
-        int row = m * 16 + ml;
-        row = row < p.M ? row : p.M - 1;
-        abase[m] = p.A + (size_t)row * p.lda + g * KL;
-    }
-
-    const u32x4 zero4 = {0u, 0u, 0u, 0u};
-    u32x4 wbuf[2][U][NT];
-    u32x4 abuf[2][U][MT][MPT];
-
-    auto issue = [&](int buf, int batch) {
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int kt = batch * U + u;
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-                wbuf[buf][u][t] = __builtin_nontemporal_load((const u32x4 *)(wbase[t] + (size_t)kt * 1024));
-#pragma unroll
-            for (int m = 0; m < MT; ++m) {
-#pragma unroll
-                for (int i = 0; i < MPT; ++i) {
-                    int koff = kt * KTILE + 8 * i;
-                    if constexpr (KTAIL) {
-                        // chunk is inside the row iff koff + 8 <= K - g*KL; otherwise read the row
-                        // start (always valid) and discard it
-                        const bool v = koff + 8 <= p.K - g * KL;
-                        const u32x4 a = *(const u32x4 *)(abase[m] + (v ? koff : -g * KL));
-                        abuf[buf][u][m][i] = v ? a : zero4;
-                    } else {
-                        abuf[buf][u][m][i] = *(const u32x4 *)(abase[m] + koff);
-                    }
-                }
-            }
-        }
-    };
-    auto compute = [&](int buf) {
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-#pragma unroll
-            for (int i = 0; i < MPT; ++i) {
-                Frag a[MT];
-#pragma unroll
-                for (int m = 0; m < MT; ++m) a[m].q = abuf[buf][u][m][i];
-#pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    if constexpr (KIND == XFTHIP_W_NF4) {
-                        bf16x8 whi, wlo;
-                        widen_nf4(wbuf[buf][u][t], i, lut, whi, wlo);
-#pragma unroll
-                        for (int m = 0; m < MT; ++m) {
-                            acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wlo, a[m].v, acc[t][m], 0, 0, 0);
-                            acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(whi, a[m].v, acc[t][m], 0, 0, 0);
-                        }
-                    } else {
-                        bf16x8 wv = widen<KIND>(wbuf[buf][u][t], i, nullptr);
-#pragma unroll
-                        for (int m = 0; m < MT; ++m)
-                            acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, a[m].v, acc[t][m], 0, 0, 0);
-                    }
-                }
-                if constexpr (need_sum) {
-#pragma unroll
-                    for (int m = 0; m < MT; ++m)
-                        accS[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, a[m].v, accS[m], 0, 0, 0);
-                }
-            }
-        }
-    };
-
-    // sched_barrier keeps the compiler from sinking the next batch's loads below the MFMAs of
-    // the current one: all loads of a batch are issued back to back, then the math runs.
-#define XFT_FENCE() __builtin_amdgcn_sched_barrier(0)
-    if (nb > 0) {
-        issue(0, b_begin);
-        XFT_FENCE();
-        int b = 1; // next batch to issue; buffer 0 holds batch b - 1
-        for (; b + 1 < nb; b += 2) {
-            issue(1, b_begin + b);
-            XFT_FENCE();
-            compute(0);
-            XFT_FENCE();
-            issue(0, b_begin + b + 1);
-            XFT_FENCE();
-            compute(1);
-            XFT_FENCE();
-        }
-        if (b < nb) {
-            issue(1, b_begin + b);
-            XFT_FENCE();
-            compute(0);
-            XFT_FENCE();
-            compute(1);
-        } else {
-            compute(0);
-        }
-    }
-#undef XFT_FENCE
-
-    // ---- cross-wave reduction through LDS: red[wave][m][n] -------------------------------
-    constexpr int ROWS = 16 * MT, COLS = 16 * NT, LD = COLS + 1;
-    float *mine = red + (size_t)wave * (ROWS * LD + ROWS);
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int m = 0; m < MT; ++m)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) mine[(m * 16 + ml) * LD + t * 16 + 4 * g + r] = acc[t][m][r];
-    if (g == 0) {
-#pragma unroll
-        for (int m = 0; m < MT; ++m) mine[ROWS * LD + m * 16 + ml] = accS[m][0];
-    }
-    __syncthreads();
-
-    const int stride = ROWS * LD + ROWS;
-    auto total = [&](int m, int c) {
-        float s = 0.0f;
-        for (int w = 0; w < nwaves; ++w) s += red[(size_t)w * stride + m * LD + c];
-        return s;
-    };
-    auto total_sum = [&](int m) {
-        float s = 0.0f;
-        for (int w = 0; w < nwaves; ++w) s += red[(size_t)w * stride + ROWS * LD + m];
-        return s;
-    };
-    auto column_value = [&](int m, int c, float sumA) {
-        const int np = nt0 * 16 + c;
-        float v = total(m, c);
-        if constexpr (KIND == XFTHIP_W_BF16) return v;
-        const float s = p.scale[np];
-        if constexpr (KIND == XFTHIP_W_UINT4) {
-            const float z = p.zero ? p.zero[np] : 0.0f;
-            return fmaf(s, v - 128.0f * sumA, z * sumA);
-        } else if constexpr (KIND == XFTHIP_W_INT8) {
-            v = s * v;
-            if constexpr (need_sum) v = fmaf(p.zero[np], sumA, v);
-            return v;
-        } else {
-            return s * v;
-        }
-    };
-
-    if (!p.gateup) {
-        for (int v = threadIdx.x; v < ROWS * COLS; v += blockDim.x) {
-            const int m = v / COLS, c = v % COLS;
-            const int np = nt0 * 16 + c;
-            if (m >= p.M || np >= p.N) continue;
-            const float sumA = need_sum ? total_sum(m) : 0.0f;
-            float x = column_value(m, c, sumA);
-            switch (p.epi) {
-                case XFTHIP_EPI_BIAS: x += p.bias[np]; break;
-                case XFTHIP_EPI_SILU: x = silu_f(x); break;
-                case XFTHIP_EPI_GELU: {
-                    float e = fast_exp(1.702f * x);
-                    x = e / (e + 1.0f) * x;
-                    break;
-                }
-                case XFTHIP_EPI_RESMUL: x *= load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + np); break;
-                case XFTHIP_EPI_RESIDENTIAL:
-                    if (p.bias) x += p.bias[np];
-                    x += load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + np);
-                    break;
-                case XFTHIP_EPI_RESEXT:
-                    if (p.bias) x += p.bias[np];
-                    x = fmaf(p.gamma, load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + np), x);
-                    break;
-                default: break;
-            }
-            store_from_f32(p.C, p.c_dtype, (size_t)m * p.ldc + np, x);
-        }
-    } else if constexpr (NT >= 2) {
-        // tile pairs (2j, 2j+1) hold gate / up columns [16 j', 16 j' + 16)
-        constexpr int PAIRS = NT / 2;
-        for (int v = threadIdx.x; v < ROWS * PAIRS * 16; v += blockDim.x) {
-            const int m = v / (PAIRS * 16), rr = v % (PAIRS * 16);
-            const int pr = rr >> 4, c = rr & 15;
-            const int out_col = (blockIdx.x * PAIRS + pr) * 16 + c;
-            if (m >= p.M || out_col >= p.N / 2) continue;
-            const float sumA = need_sum ? total_sum(m) : 0.0f;
-            const float gate = column_value(m, pr * 32 + c, sumA);
-            const float up = column_value(m, pr * 32 + 16 + c, sumA);
-            store_from_f32(p.C, p.c_dtype, (size_t)m * p.ldc + out_col, up * silu_f(gate));
-        }
-    }
-}
-
-// k tiles per load batch, sized so that two batches of weight + activation fragments stay in
-// registers (256 VGPRs per lane at 8 waves per block)
-template <int KIND, int MT>
-constexpr int batch_tiles() {
-    if (KIND == XFTHIP_W_INT8) return MT == 1 ? 4 : 2;
-    if (KIND == XFTHIP_W_BF16) return MT == 1 ? 4 : 2;
-    return MT == 1 ? 2 : 1;
-}
-
-template <int KIND, int NT, int MT, int U, bool NEED_SUM, bool KTAIL>
-static int launch(const SkinnyParams &p, int kslices, hipStream_t stream) {
-    constexpr int ROWS = 16 * MT, COLS = 16 * NT;
-    size_t smem = (size_t)kslices * (ROWS * (COLS + 1) + ROWS) * sizeof(float) + (KIND == XFTHIP_W_NF4 ? 2048 : 0);
-    int blocks = (p.NTILES + NT - 1) / NT;
-    hipLaunchKernelGGL((qgemm_skinny_kernel<KIND, NT, MT, U, NEED_SUM, KTAIL>), dim3(blocks), dim3(64 * kslices), smem,
-            stream, p);
-    XFT_CHECK_HIP(hipGetLastError());
-    return 0;
-}
-
-template <int KIND, int NT, int MT, bool NEED_SUM>
-static int dispatch_tail(const SkinnyParams &p, int kslices, hipStream_t stream) {
-    constexpr int U = batch_tiles<KIND, MT>();
-    if (p.KT * KindTraits<KIND>::KTILE != p.K)
-        return launch<KIND, NT, MT, U, NEED_SUM, true>(p, kslices, stream);
-    return launch<KIND, NT, MT, U, NEED_SUM, false>(p, kslices, stream);
-}
-
-template <int KIND, int NT, int MT>
-static int dispatch_sum(const SkinnyParams &p, int kslices, hipStream_t stream) {
-    if constexpr (KIND == XFTHIP_W_UINT4) {
-        return dispatch_tail<KIND, NT, MT, true>(p, kslices, stream);
-    } else if constexpr (KIND == XFTHIP_W_INT8) {
-        if (p.zero) return dispatch_tail<KIND, NT, MT, true>(p, kslices, stream);
-        return dispatch_tail<KIND, NT, MT, false>(p, kslices, stream);
-    } else {
-        return dispatch_tail<KIND, NT, MT, false>(p, kslices, stream);
-    }
-}
-
-template <int KIND>
-static int dispatch_shape(const SkinnyParams &p, hipStream_t stream) {
-    const int cus = device_cu_count();
-    const int mt = (p.M + 15) / 16;
-    // column tiles per wave: 2 when that still leaves at least 2 blocks per CU (gate/up needs pairs)
-    const bool wide = p.gateup || (p.NTILES / 2 >= 2 * cus);
-    // K slices per block: aim at two load batches per wave, at most 8 waves
-    const int u = (mt == 1) ? batch_tiles<KIND, 1>() : batch_tiles<KIND, 2>();
-    const int nbatch = p.KT / u;
-    int kslices = (nbatch + 1) / 2;
-    if (kslices < 1) kslices = 1;
-    if (kslices > 8) kslices = 8;
-    if (mt == 1) {
-        if (wide) return dispatch_sum<KIND, 2, 1>(p, kslices, stream);
-        return dispatch_sum<KIND, 1, 1>(p, kslices, stream);
-    }
-    if (wide) return dispatch_sum<KIND, 2, 2>(p, kslices, stream);
-    return dispatch_sum<KIND, 1, 2>(p, kslices, stream);
+bool skinny_can_fuse_norm(const PackedWeight &pw, int M) {
+    return M <= 4 && pw.kind != XFTHIP_W_W8A8 && pw.KT * ktile_of(pw.kind) == pw.K && pw.K % 4 == 0
+            && skinny_norm_lds_bytes(M, pw.K) <= (size_t)36 * 1024;
 }
 
 int qgemm_skinny(const PackedWeight &pw, const SkinnyParams &p0, hipStream_t stream) {
     SkinnyParams p = p0;
+    if (p.norm_x && !skinny_can_fuse_norm(pw, p.M)) {
+        set_error("qgemm_skinny: RMSNorm prologue not available for M=%d K=%d kind=%d", p.M, pw.K, pw.kind);
+        return 2;
+    }
+    if (p.rope && (p.M > 16 || p.gateup || (p.qH + 2 * p.kvH) * 128 != pw.N || p.kv.int8 != 0 || p.kv.D != 128)) {
+        set_error("qgemm_skinny: RoPE / cache-append epilogue needs M <= 16, head size 128, an FP16 cache and a [K, (q+2kv)*128] weight");
+        return 2;
+    }
     p.packed = pw.packed;
     p.scale = pw.scale;
     p.zero = pw.zero;
@@ -415,10 +39,10 @@ int qgemm_skinny(const PackedWeight &pw, const SkinnyParams &p0, hipStream_t str
     p.K = pw.K;
     p.N = pw.N;
     switch (pw.kind) {
-        case XFTHIP_W_INT8: return dispatch_shape<XFTHIP_W_INT8>(p, stream);
-        case XFTHIP_W_UINT4: return dispatch_shape<XFTHIP_W_UINT4>(p, stream);
-        case XFTHIP_W_NF4: return dispatch_shape<XFTHIP_W_NF4>(p, stream);
-        case XFTHIP_W_BF16: return dispatch_shape<XFTHIP_W_BF16>(p, stream);
+        case XFTHIP_W_INT8: return qgemm_skinny_int8(p, stream);
+        case XFTHIP_W_UINT4: return qgemm_skinny_uint4(p, stream);
+        case XFTHIP_W_NF4: return qgemm_skinny_nf4(p, stream);
+        case XFTHIP_W_BF16: return qgemm_skinny_bf16(p, stream);
         default: set_error("qgemm_skinny: weight kind %d not supported", pw.kind); return 2;
     }
 }

@@ -67,23 +67,45 @@ def build_model(xh, kind, batch, max_seq, prompt):
     return model, layer_weights, lmw, host, shapes
 
 
-def time_gemm_kernel(xh, layer_weights, which, M, iters):
-    """Average duration of one launch of the weight-only GEMM over the distinct per-layer weights
-    `which` (indices into a layer's [qkv, o, gateup, down]), HIP events on the launch stream."""
-    c = CFG
-    K_max = max(c["hidden"], c["inter"])
-    A = xh.DeviceBuffer.from_numpy(xh.f32_to_bf16_bits(np.random.default_rng(1).standard_normal((M, K_max)).astype(np.float32)))
-    out = xh.DeviceBuffer(M * 2 * c["inter"] * 4)
+class GemvHarness:
+    """Launches the decode GEMVs exactly as the decode step does, one kernel at a time:
+    index 0 QKV (RMSNorm prologue, RoPE + cache-append epilogue), 1 out-projection, 2 gate/up
+    (RMSNorm prologue, SwiGLU), 3 down projection."""
 
-    def launch(w, i):
-        if i == 2:
-            xh.gemm_gateup_silu(w, A.ptr, M, w.K, out.ptr, w.N // 2, xh.BF16)
+    def __init__(self, xh, M):
+        c = CFG
+        self.xh, self.M = xh, M
+        rng = np.random.default_rng(1)
+        k_max = max(c["hidden"], c["inter"])
+        self.A = xh.DeviceBuffer.from_numpy(xh.f32_to_bf16_bits(rng.standard_normal((M, k_max)).astype(np.float32)))
+        self.x = xh.DeviceBuffer.from_numpy(rng.standard_normal((M, c["hidden"])).astype(np.float32))
+        self.g = xh.DeviceBuffer.from_numpy(np.ones(c["hidden"], np.float32))
+        self.out = xh.DeviceBuffer(M * 2 * c["inter"] * 4)
+        self.cache = xh.KVCache(xh.FP16, M, c["kv_heads"], 64, c["head"])
+        self.tables = xh.RopeTables(c["head"], 64)
+        self.fused = M <= 4
+
+    def launch(self, w, i):
+        xh, c, M = self.xh, CFG, self.M
+        if i == 0 and self.fused:
+            xh.gemm_qkv_rmsnorm_rope(w, self.cache, self.x.ptr, M, c["hidden"], self.g.ptr, 1e-6, self.out.ptr,
+                                     c["q_heads"] * c["head"], c["q_heads"], self.tables, 7)
+        elif i == 2 and self.fused:
+            xh.gemm_gateup_silu_rmsnorm(w, self.x.ptr, M, c["hidden"], self.g.ptr, 1e-6, self.out.ptr, w.N // 2, xh.BF16)
+        elif i == 2:
+            xh.gemm_gateup_silu(w, self.A.ptr, M, w.K, self.out.ptr, w.N // 2, xh.BF16)
         else:
-            xh.gemm(w, A.ptr, M, w.K, out.ptr, w.N, xh.BF16)
+            xh.gemm(w, self.A.ptr, M, w.K, self.out.ptr, w.N, xh.BF16)
 
+
+def time_gemm_kernel(xh, layer_weights, which, M, iters):
+    """Average duration of one launch of the weight-only GEMV over the distinct per-layer weights
+    `which` (indices into a layer's [qkv, o, gateup, down]), HIP events on the launch stream, and
+    its algorithmic bytes (the packed weight, the activation rows in, the result rows out)."""
+    h = GemvHarness(xh, M)
     for ws in layer_weights:
         for i in which:
-            launch(ws[i], i)
+            h.launch(ws[i], i)
     xh.synchronize()
     t = xh.Timer()
     n = 0
@@ -91,12 +113,90 @@ def time_gemm_kernel(xh, layer_weights, which, M, iters):
     for _ in range(iters):
         for ws in layer_weights:
             for i in which:
-                launch(ws[i], i)
+                h.launch(ws[i], i)
                 n += 1
     ms = t.stop()
-    byts = sum(layer_weights[0][i].bytes() + 2 * M * layer_weights[0][i].K
+    in_bytes = lambda i, w: (4 if (h.fused and i in (0, 2)) else 2) * M * w.K
+    byts = sum(layer_weights[0][i].bytes() + in_bytes(i, layer_weights[0][i])
                + 2 * M * (layer_weights[0][i].N // (2 if i == 2 else 1)) for i in which) / len(which)
     return ms * 1e3 / n, byts
+
+
+PMC_COPY_BYTES = 256 << 20
+
+
+def pmc_workload(xh, layer_weights, M):
+    """What `rocprofv3 --pmc FETCH_SIZE` (and, in a second run, WRITE_SIZE) is pointed at: 8 launches
+    of the library's plain copy kernel over PMC_COPY_BYTES (known traffic: that many bytes read and
+    as many written), then one launch of the decode GEMV over every layer's weights (distinct
+    memory each time, so nothing is served from a cache)."""
+    src = xh.DeviceBuffer(PMC_COPY_BYTES)
+    dst = xh.DeviceBuffer(PMC_COPY_BYTES)
+    src.zero()
+    xh.synchronize()
+    for _ in range(8):
+        xh.copy_kernel(dst.ptr, src.ptr, PMC_COPY_BYTES)
+    xh.synchronize()
+    for which in ((0,), (1, 3), (2,)):
+        time_gemm_kernel(xh, layer_weights, which, M, 1)
+    xh.synchronize()
+
+
+TRAFFIC_FILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "qgemm_skinny_int8_bs1_hbm_traffic.txt")
+
+
+def pmc_summary(fetch_csv, write_csv):
+    """Turns the two counter CSVs of `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --output-format csv --
+    python3 bench.py --pmc-workload` into the summary kept under profiles/ (runs on the CPU)."""
+    import csv
+
+    def per_kernel(path, counter):
+        acc = {}
+        with open(path, newline="") as f:
+            for r in csv.DictReader(f):
+                if r["Counter_Name"] != counter:
+                    continue
+                name = r["Kernel_Name"]
+                if "stream_copy_kernel" in name:
+                    key = "copy"
+                elif "qgemm_skinny_kernel<" in name:
+                    # <KIND, NT, MT, U, NEED_SUM, KTAIL, NORM, ROPE>
+                    targs = name.split("qgemm_skinny_kernel<")[1].split(">")[0].replace(" ", "").split(",")
+                    key = "qkv" if targs[7] in ("true", "1") else ("wide" if targs[1] == "2" else "narrow")
+                else:
+                    continue
+                acc.setdefault(key, []).append(float(r["Counter_Value"]))
+        return {k: (sum(v) / len(v), len(v)) for k, v in acc.items()}
+
+    fetch, write = per_kernel(fetch_csv, "FETCH_SIZE"), per_kernel(write_csv, "WRITE_SIZE")
+    copy_kib = PMC_COPY_BYTES / 1024.0
+    sf, sw = copy_kib / fetch["copy"][0], copy_kib / write["copy"][0]
+    print("HBM traffic per launch of the M=1 INT8 weight-only GEMV (qgemm_skinny_kernel), from hardware counters")
+    print("commands (each its own run, as the counter blocks cannot be split over passes):")
+    print("  rocprofv3 --pmc FETCH_SIZE --output-format csv -d gpurun_out/pmc_fetch -- python3 bench.py --pmc-workload")
+    print("  rocprofv3 --pmc WRITE_SIZE --output-format csv -d gpurun_out/pmc_write -- python3 bench.py --pmc-workload")
+    print("  python bench.py --pmc-summary <fetch counter_collection.csv> <write counter_collection.csv>")
+    print("calibration: the library's plain copy kernel over %d KiB read %.1f (FETCH_SIZE) and wrote %.1f (WRITE_SIZE) counter units"
+          % (copy_kib, fetch["copy"][0], write["copy"][0]))
+    print("scale factors (KiB per counter unit): FETCH_SIZE %.4f  WRITE_SIZE %.4f" % (sf, sw))
+    for key, label in (("qkv", "norm + qkv + RoPE / cache append (2 column tiles per wave)"),
+                       ("narrow", "out-proj / down (1 column tile per wave), mean over the two shapes"),
+                       ("wide", "norm + gate/up + SwiGLU (2 column tiles per wave)")):
+        fb, wb = fetch[key][0] * sf * 1024.0, write[key][0] * sw * 1024.0
+        print("%s: %d launches, fetch %.0f B + write %.0f B" % (label, fetch[key][1], fb, wb))
+        print("traffic_bytes %s=%d" % (key, round(fb + wb)))
+
+
+def measured_traffic(key):
+    """HBM bytes per launch recorded by the last counter run (see pmc_summary), or None."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            for line in f:
+                if line.startswith("traffic_bytes %s=" % key):
+                    return int(line.split("=")[1])
+    except OSError:
+        pass
+    return None
 
 
 def cpu_baseline(kind, host, shapes, batch):
@@ -142,8 +242,13 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fusion", action="store_true", help="run RMSNorm / RoPE + cache append as their own kernels instead of inside the decode GEMVs")
     ap.add_argument("--persistent", action="store_true", help="run each decode step as the single persistent kernel (experimental)")
+    ap.add_argument("--pmc-workload", action="store_true", help="counter workload for rocprofv3 --pmc: a plain copy kernel of known size, then every distinct decode GEMV of the model once; prints no result line")
+    ap.add_argument("--pmc-summary", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"), help="summarise the two counter CSVs of the --pmc-workload runs (CPU only)")
     ap.add_argument("--eager", action="store_true", help="launch decode kernels one by one instead of replaying the captured graph (for per-kernel profiling)")
     args = ap.parse_args()
+    if args.pmc_summary:
+        pmc_summary(*args.pmc_summary)
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (no collectives are part of it)", file=sys.stderr)
         sys.exit(2)
@@ -155,6 +260,9 @@ def main():
     max_seq = args.prompt + args.warmup + args.steps + 1
     model, layer_weights, lmw, host, shapes = build_model(xh, kind, B, max_seq, args.prompt)
 
+    if args.pmc_workload:
+        pmc_workload(xh, layer_weights, B)
+        return
     if args.eager:
         model.use_graph(False)
     if args.no_fusion:
@@ -184,14 +292,18 @@ def main():
     kv_bytes = CFG["layers"] * 2 * B * ctx * CFG["kv_heads"] * CFG["head"] * 2
     step_bytes = wbytes + kv_bytes
 
-    # dominant kernel: the M<=32 weight-only GEMM; the two instantiations the layer uses
-    narrow_us, narrow_bytes = time_gemm_kernel(xh, layer_weights, (0, 1, 3), B, 4)
-    wide_us, wide_bytes = time_gemm_kernel(xh, layer_weights, (2,), B, 4)
-    dom = dict(name="qgemm_skinny_kernel (qkv, out-proj, down)", us=narrow_us, bytes=narrow_bytes, launches=3)
-    alt = dict(name="qgemm_skinny_kernel (gate/up + SwiGLU)", us=wide_us, bytes=wide_bytes, launches=1)
-    if alt["us"] * alt["launches"] > dom["us"] * dom["launches"]:
-        dom, alt = alt, dom
+    # dominant kernel: the M<=32 weight-only GEMV, in the three forms the decode step launches it
+    groups = []
+    for key, name, which in (("qkv", "qgemm_skinny_kernel (norm + qkv + RoPE/cache append)", (0,)),
+                             ("narrow", "qgemm_skinny_kernel (out-proj, down)", (1, 3)),
+                             ("wide", "qgemm_skinny_kernel (norm + gate/up + SwiGLU)", (2,))):
+        us, byts = time_gemm_kernel(xh, layer_weights, which, B, 4)
+        groups.append(dict(name=name, us=us, bytes=byts, launches=len(which), key=key))
+    groups.sort(key=lambda g: -g["us"] * g["launches"])
+    dom, others = groups[0], groups[1:]
     achieved = dom["bytes"] / dom["us"] / 1e3
+    # counter-measured HBM bytes per launch exist for the configuration the counters were run on
+    traffic = measured_traffic(dom["key"]) if (args.weights == "int8" and B == 1) else None
 
     result = {
         "metric": "decode tok/s (7B-shape, INT8/INT4 wts, bs1/32); qGEMM % HBM roofline",
@@ -213,11 +325,11 @@ def main():
         "step_hbm_bytes": int(step_bytes),
         "step_hbm_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "roofline": {"bound": "hbm", "kernel": dom["name"], "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "avg_launch_us": round(dom["us"], 3), "bytes_per_launch": int(dom["bytes"])},
-        "other_kernels": [{"kernel": alt["name"], "avg_launch_us": round(alt["us"], 3),
-                           "bytes_per_launch": int(alt["bytes"]),
-                           "frac": round(alt["bytes"] / alt["us"] / 1e3 / HBM_PEAK_GBS, 4)}],
+        "other_kernels": [{"kernel": g["name"], "launches_per_layer": g["launches"], "avg_launch_us": round(g["us"], 3),
+                           "bytes_per_launch": int(g["bytes"]),
+                           "frac": round(g["bytes"] / g["us"] / 1e3 / HBM_PEAK_GBS, 4)} for g in others],
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(kind, host, shapes, B)

@@ -65,6 +65,10 @@ int xfthip_free(void *ptr);
 int xfthip_memcpy_h2d(void *dst, const void *src_host, size_t bytes, xfthip_stream_t stream);
 int xfthip_memcpy_d2h(void *dst_host, const void *src, size_t bytes, xfthip_stream_t stream);
 int xfthip_memcpy_d2d(void *dst, const void *src, size_t bytes, xfthip_stream_t stream);
+/* Device-to-device copy by a plain kernel of this library (16 bytes per lane; pointers and size
+ * 16-byte aligned): reads `bytes` and writes `bytes`, which makes it the reference point when
+ * hardware counters of HBM traffic are scaled.  No counterpart in the reference. */
+int xfthip_copy_kernel(void *dst, const void *src, size_t bytes, xfthip_stream_t stream);
 int xfthip_memset(void *dst, int value, size_t bytes, xfthip_stream_t stream);
 int xfthip_stream_create(xfthip_stream_t *stream);
 int xfthip_stream_destroy(xfthip_stream_t stream);
@@ -127,6 +131,28 @@ int xfthip_gemm(xfthip_weight_t w, int M, const void *A, int lda, void *C, int l
  */
 int xfthip_gemm_gateup_silu(xfthip_weight_t w, int M, const void *A, int lda, void *out, int ldo, int out_dtype,
         xfthip_stream_t stream);
+
+/*
+ * The two decode-step fusions of the M <= 32 kernel, for up to 4 activation rows (the model
+ * driver uses them when it decodes; they are entry points of their own so that they can be
+ * tested and timed alone).  The reference runs the norm, the projection, the rotation and the
+ * cache write as separate calls (src/layers/rms_norm.cpp:54-110, src/layers/attention.h:322-460,
+ * src/layers/mlp_llama.h:200-260); the bf16 hand-over points between them are kept.
+ *
+ * xfthip_gemm_gateup_silu_rmsnorm: out = silu(n W_gate) * (n W_up) with
+ *   n = bf16(x * rsqrt(mean(x^2) + eps) * norm_weight), x fp32 [M, K] with row pitch ldx.
+ *
+ * xfthip_gemm_qkv_rmsnorm_rope: one new token per sequence (row m belongs to sequence m of the
+ * cache).  qkv = bf16(n W); the query heads are rotated (tables of xfthip_rope_tables_create,
+ * 64 entries a row) and written as bf16 to q_out [M, q_heads * 128] (row pitch ldq); the rotated
+ * key heads and the value heads are appended to `cache` (FP16 cache, head size 128) at
+ * position_dev[m], or at `position` for every row when position_dev is NULL.
+ */
+int xfthip_gemm_gateup_silu_rmsnorm(xfthip_weight_t w, int M, const float *x, int ldx, const float *norm_weight, float eps,
+        void *out, int ldo, int out_dtype, xfthip_stream_t stream);
+int xfthip_gemm_qkv_rmsnorm_rope(xfthip_weight_t w, xfthip_kvcache_t cache, int M, const float *x, int ldx,
+        const float *norm_weight, float eps, void *q_out, int ldq, int q_heads, const float *cos_table,
+        const float *sin_table, int position, const int *position_dev, xfthip_stream_t stream);
 
 
 /*

@@ -50,6 +50,10 @@ def device_info():
     return name.value.decode(), cus.value, mem.value
 
 
+def copy_kernel(dst_ptr, src_ptr, nbytes, stream=None):
+    check(lib.xfthip_copy_kernel(dst_ptr, src_ptr, C.c_size_t(nbytes), stream))
+
+
 def synchronize():
     check(lib.xfthip_device_synchronize())
 
@@ -281,6 +285,16 @@ class KVCache:
             self.free()
         except Exception:
             pass
+
+
+def gemm_gateup_silu_rmsnorm(w, x_dev, M, ldx, norm_w_dev, eps, out_dev, ldo, out_dtype, stream=None):
+    check(lib.xfthip_gemm_gateup_silu_rmsnorm(w.h, M, x_dev, ldx, norm_w_dev, C.c_float(eps), out_dev, ldo, out_dtype, stream))
+
+
+def gemm_qkv_rmsnorm_rope(w, cache, x_dev, M, ldx, norm_w_dev, eps, q_dev, ldq, q_heads, tables, position, pos_dev=None,
+                          stream=None):
+    check(lib.xfthip_gemm_qkv_rmsnorm_rope(w.h, cache.h, M, x_dev, ldx, norm_w_dev, C.c_float(eps), q_dev, ldq, q_heads,
+                                           tables.cos, tables.sin, position, pos_dev, stream))
 
 
 def rope_kvstore(cache, qkv_dev, dtype, stride, B, S, q_heads, tables, past, past_dev=None, stream=None):

@@ -68,4 +68,52 @@ int xfthip_gemm_gateup_silu(xfthip_weight_t w, int M, const void *A, int lda, vo
     return qgemm_mfma(pw, p, (hipStream_t)stream);
 }
 
+int xfthip_gemm_gateup_silu_rmsnorm(xfthip_weight_t w, int M, const float *x, int ldx, const float *norm_weight, float eps,
+        void *out, int ldo, int out_dtype, xfthip_stream_t stream) {
+    XFT_REQUIRE(w && x && norm_weight && out, "xfthip_gemm_gateup_silu_rmsnorm: null argument");
+    const PackedWeight &pw = w->pw;
+    XFT_REQUIRE(pw.flags & XFTHIP_WF_GATEUP, "xfthip_gemm_gateup_silu_rmsnorm: weight was not created with XFTHIP_WF_GATEUP");
+    XFT_REQUIRE(M > 0 && skinny_can_fuse_norm(pw, M),
+            "xfthip_gemm_gateup_silu_rmsnorm: needs 1 <= M <= 4, K a whole number of weight tiles and M rows of K in 36 KB of LDS (M=%d K=%d)",
+            M, pw.K);
+    XFT_REQUIRE(ldx >= pw.K && ldx % 4 == 0 && ((uintptr_t)x & 15) == 0, "xfthip_gemm_gateup_silu_rmsnorm: x rows must be 16-byte aligned, ldx >= K");
+    XFT_REQUIRE(ldo >= pw.N / 2, "xfthip_gemm_gateup_silu_rmsnorm: ldo=%d < I=%d", ldo, pw.N / 2);
+    XFT_REQUIRE(out_dtype == XFTHIP_F32 || out_dtype == XFTHIP_BF16, "xfthip_gemm_gateup_silu_rmsnorm: out_dtype must be f32 or bf16");
+    SkinnyParams p = {};
+    p.M = M;
+    p.C = out;
+    p.ldc = ldo;
+    p.c_dtype = out_dtype;
+    p.gateup = 1;
+    p.norm_x = x, p.ldx = ldx, p.norm_w = norm_weight, p.norm_eps = eps;
+    return qgemm_skinny(pw, p, (hipStream_t)stream);
+}
+
+int xfthip_gemm_qkv_rmsnorm_rope(xfthip_weight_t w, xfthip_kvcache_t cache, int M, const float *x, int ldx, const float *norm_weight,
+        float eps, void *q_out, int ldq, int q_heads, const float *cos_table, const float *sin_table, int position,
+        const int *position_dev, xfthip_stream_t stream) {
+    XFT_REQUIRE(w && cache && x && norm_weight && q_out && cos_table && sin_table, "xfthip_gemm_qkv_rmsnorm_rope: null argument");
+    const PackedWeight &pw = w->pw;
+    const KvView &kv = cache->kv;
+    XFT_REQUIRE(!(pw.flags & XFTHIP_WF_GATEUP) && pw.kind != XFTHIP_W_W8A8, "xfthip_gemm_qkv_rmsnorm_rope: unsupported weight");
+    XFT_REQUIRE(M > 0 && M <= kv.B && skinny_can_fuse_norm(pw, M),
+            "xfthip_gemm_qkv_rmsnorm_rope: needs 1 <= M <= min(4, cache batch) and K a whole number of weight tiles (M=%d K=%d)", M, pw.K);
+    XFT_REQUIRE(!kv.int8 && kv.D == 128, "xfthip_gemm_qkv_rmsnorm_rope: needs an FP16 cache with head size 128");
+    XFT_REQUIRE(q_heads > 0 && (q_heads + 2 * kv.H) * 128 == pw.N, "xfthip_gemm_qkv_rmsnorm_rope: weight has %d columns, expected (%d + 2 * %d) * 128",
+            pw.N, q_heads, kv.H);
+    XFT_REQUIRE(ldx >= pw.K && ldx % 4 == 0 && ((uintptr_t)x & 15) == 0, "xfthip_gemm_qkv_rmsnorm_rope: x rows must be 16-byte aligned, ldx >= K");
+    XFT_REQUIRE(ldq >= q_heads * 128, "xfthip_gemm_qkv_rmsnorm_rope: ldq=%d < %d", ldq, q_heads * 128);
+    XFT_REQUIRE(position_dev != nullptr || (position >= 0 && position < cache->maxSeq),
+            "xfthip_gemm_qkv_rmsnorm_rope: position %d outside the cache (max_seq %d)", position, cache->maxSeq);
+    SkinnyParams p = {};
+    p.M = M;
+    p.C = q_out;
+    p.ldc = ldq;
+    p.c_dtype = XFTHIP_BF16;
+    p.norm_x = x, p.ldx = ldx, p.norm_w = norm_weight, p.norm_eps = eps;
+    p.rope = 1, p.cosT = cos_table, p.sinT = sin_table, p.pos_dev = position_dev, p.pos_host = position;
+    p.qH = q_heads, p.kvH = kv.H, p.kv = kv;
+    return qgemm_skinny(pw, p, (hipStream_t)stream);
+}
+
 } // extern "C"

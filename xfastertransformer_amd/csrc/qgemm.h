@@ -20,6 +20,7 @@ struct SkinnyParams {
     int ldres, res_dtype;
     float gamma;
     int gateup; // 1: combine tile pairs as silu(gate)*up, N counts cat columns
+    int nblocks; // column blocks of the launch (set by the launcher)
 
     // ---- fusions of the decode step (M <= 4, skinny kernel only) ----
     // RMSNorm prologue: when norm_x is set, A is ignored and every workgroup normalises the M rows

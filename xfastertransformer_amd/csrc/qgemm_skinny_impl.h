@@ -148,308 +148,349 @@ __global__ __launch_bounds__(512) void qgemm_skinny_kernel(SkinnyParams p) {
     const int base = nbatch / nwaves, rem = nbatch % nwaves;
     const int b_begin = wave * base + (wave < rem ? wave : rem);
     const int nb = base + (wave < rem ? 1 : 0);
-    const int nt0 = blockIdx.x * NT;
-    // column tile t of this block; the RoPE epilogue pairs dims (d, d + 64) of a head, then V tiles
-    const int rope_pairs = ROPE ? (p.qH + p.kvH) * 4 : 0;
-    auto tile_of = [&](int t) {
-        if constexpr (ROPE) {
-            const int it = blockIdx.x;
-            return it < rope_pairs ? (it >> 2) * 8 + (it & 3) + 4 * t : (p.qH + p.kvH) * 8 + 2 * (it - rope_pairs) + t;
-        }
-        return nt0 + t;
-    };
-
-    f32x4 acc[NT][MT];
-    f32x4 accS[MT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int m = 0; m < MT; ++m) acc[t][m] = f32x4 {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int m = 0; m < MT; ++m) accS[m] = f32x4 {0.f, 0.f, 0.f, 0.f};
-
-    Frag ones;
-    ones.u[0] = ones.u[1] = ones.u[2] = ones.u[3] = 0x3F803F80u;
-
-    // Every load below is unconditional: out-of-range column tiles and activation rows are
-    // clamped to the last valid one (their results are never stored), so the loop body is
-    // straight-line code and the loads of the next batch stay in flight during the MFMAs.
-    const uint8_t *wbase[NT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-        int nt = tile_of(t);
-        nt = nt < p.NTILES ? nt : p.NTILES - 1;
-        wbase[t] = p.packed + (size_t)nt * p.KT * 1024 + lane * 16;
-    }
-    const uint16_t *abase[MT];
-#pragma unroll
-    for (int m = 0; m < MT; ++m) {
-        int row = m * 16 + ml;
-        row = row < p.M ? row : p.M - 1;
-        abase[m] = p.A + (size_t)row * p.lda + g * KL;
-    }
-
-    const u32x4 zero4 = {0u, 0u, 0u, 0u};
-    u32x4 wbuf[2][U][NT];
-    u32x4 abuf[2][U][MT][MPT];
-
-    auto issue = [&](int buf, int batch) {
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int kt = batch * U + u;
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-                wbuf[buf][u][t] = __builtin_nontemporal_load((const u32x4 *)(wbase[t] + (size_t)kt * 1024));
-            if constexpr (NORM) continue; // activations are read from LDS in compute()
-#pragma unroll
-            for (int m = 0; m < MT; ++m) {
-#pragma unroll
-                for (int i = 0; i < MPT; ++i) {
-                    int koff = kt * KTILE + 8 * i;
-                    if constexpr (KTAIL) {
-                        // chunk is inside the row iff koff + 8 <= K - g*KL; otherwise read the row
-                        // start (always valid) and discard it
-                        const bool v = koff + 8 <= p.K - g * KL;
-                        const u32x4 a = *(const u32x4 *)(abase[m] + (v ? koff : -g * KL));
-                        abuf[buf][u][m][i] = v ? a : zero4;
-                    } else {
-                        abuf[buf][u][m][i] = *(const u32x4 *)(abase[m] + koff);
-                    }
-                }
-            }
-        }
-    };
+    // With the norm prologue the grid is one workgroup per compute unit and each walks over
+    // several column blocks, so that the prologue is paid once per workgroup rather than once per
+    // column block; the plain kernel is launched with one workgroup per column block.
+    bool first = true;
     uint16_t *xn = nullptr; // NORM: [M][K + 8] bf16 behind the reduction area
     int xn_row = 0;
-    auto compute = [&](int buf, int batch) {
-        (void)batch;
+    // column tile t of column block `it`; the RoPE epilogue pairs dims (d, d + 64) of a head, then V tiles
+    const int rope_pairs = ROPE ? (p.qH + p.kvH) * 4 : 0;
+    auto tile_index = [&](int it, int t) {
+        if constexpr (ROPE) return it < rope_pairs ? (it >> 2) * 8 + (it & 3) + 4 * t : (p.qH + p.kvH) * 8 + 2 * (it - rope_pairs) + t;
+        return it * NT + t;
+    };
+    // Every weight load is unconditional: out-of-range column tiles are clamped to the last valid
+    // one (their results are never stored).
+    const uint8_t *wbase[NT];
+    auto set_wbase = [&](int it) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
+        for (int t = 0; t < NT; ++t) {
+            int nt = tile_index(it, t);
+            nt = nt < p.NTILES ? nt : p.NTILES - 1;
+            wbase[t] = p.packed + (size_t)nt * p.KT * 1024 + lane * 16;
+        }
+    };
+    u32x4 wbuf[2][U][NT];
+    bool pre_issued = false; // NORM: the first batch of this block went out before the previous block's epilogue
+    auto run_block = [&](const int blk) {
+        const int nt0 = blk * NT;
+        auto tile_of = [&](int t) { return tile_index(blk, t); };
+
+        f32x4 acc[NT][MT];
+        f32x4 accS[MT];
 #pragma unroll
-            for (int i = 0; i < MPT; ++i) {
-                Frag a[MT];
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int m = 0; m < MT; ++m) acc[t][m] = f32x4 {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int m = 0; m < MT; ++m) accS[m] = f32x4 {0.f, 0.f, 0.f, 0.f};
+
+        Frag ones;
+        ones.u[0] = ones.u[1] = ones.u[2] = ones.u[3] = 0x3F803F80u;
+
+        // Activation loads are unconditional too (rows clamped to the last valid one), so the loop
+        // body is straight-line code and the loads of the next batch stay in flight during the MFMAs.
+        if (!pre_issued) set_wbase(blk);
+        const uint16_t *abase[MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            int row = m * 16 + ml;
+            row = row < p.M ? row : p.M - 1;
+            abase[m] = p.A + (size_t)row * p.lda + g * KL;
+        }
+
+        const u32x4 zero4 = {0u, 0u, 0u, 0u};
+        u32x4 abuf[2][U][MT][MPT];
+
+        auto issue = [&](int buf, int batch) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int kt = batch * U + u;
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+                    wbuf[buf][u][t] = __builtin_nontemporal_load((const u32x4 *)(wbase[t] + (size_t)kt * 1024));
+                if constexpr (NORM) continue; // activations are read from LDS in compute()
 #pragma unroll
                 for (int m = 0; m < MT; ++m) {
-                    if constexpr (NORM)
-                        a[m].q = *(const u32x4 *)(xn + xn_row + (batch * U + u) * KTILE + g * KL + 8 * i);
-                    else
-                        a[m].q = abuf[buf][u][m][i];
-                }
 #pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    if constexpr (KIND == XFTHIP_W_NF4) {
-                        bf16x8 whi, wlo;
-                        widen_nf4(wbuf[buf][u][t], i, lut, whi, wlo);
-#pragma unroll
-                        for (int m = 0; m < MT; ++m) {
-                            acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wlo, a[m].v, acc[t][m], 0, 0, 0);
-                            acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(whi, a[m].v, acc[t][m], 0, 0, 0);
+                    for (int i = 0; i < MPT; ++i) {
+                        int koff = kt * KTILE + 8 * i;
+                        if constexpr (KTAIL) {
+                            // chunk is inside the row iff koff + 8 <= K - g*KL; otherwise read the row
+                            // start (always valid) and discard it
+                            const bool v = koff + 8 <= p.K - g * KL;
+                            const u32x4 a = *(const u32x4 *)(abase[m] + (v ? koff : -g * KL));
+                            abuf[buf][u][m][i] = v ? a : zero4;
+                        } else {
+                            abuf[buf][u][m][i] = *(const u32x4 *)(abase[m] + koff);
                         }
-                    } else {
-                        bf16x8 wv = widen<KIND>(wbuf[buf][u][t], i, nullptr);
-#pragma unroll
-                        for (int m = 0; m < MT; ++m)
-                            acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, a[m].v, acc[t][m], 0, 0, 0);
                     }
                 }
-                if constexpr (need_sum) {
+            }
+        };
+        auto compute = [&](int buf, int batch) {
+            (void)batch;
 #pragma unroll
-                    for (int m = 0; m < MT; ++m)
-                        accS[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, a[m].v, accS[m], 0, 0, 0);
+            for (int u = 0; u < U; ++u) {
+#pragma unroll
+                for (int i = 0; i < MPT; ++i) {
+                    Frag a[MT];
+#pragma unroll
+                    for (int m = 0; m < MT; ++m) {
+                        if constexpr (NORM)
+                            a[m].q = *(const u32x4 *)(xn + xn_row + (batch * U + u) * KTILE + g * KL + 8 * i);
+                        else
+                            a[m].q = abuf[buf][u][m][i];
+                    }
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                        if constexpr (KIND == XFTHIP_W_NF4) {
+                            bf16x8 whi, wlo;
+                            widen_nf4(wbuf[buf][u][t], i, lut, whi, wlo);
+#pragma unroll
+                            for (int m = 0; m < MT; ++m) {
+                                acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wlo, a[m].v, acc[t][m], 0, 0, 0);
+                                acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(whi, a[m].v, acc[t][m], 0, 0, 0);
+                            }
+                        } else {
+                            bf16x8 wv = widen<KIND>(wbuf[buf][u][t], i, nullptr);
+#pragma unroll
+                            for (int m = 0; m < MT; ++m)
+                                acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, a[m].v, acc[t][m], 0, 0, 0);
+                        }
+                    }
+                    if constexpr (need_sum) {
+#pragma unroll
+                        for (int m = 0; m < MT; ++m)
+                            accS[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, a[m].v, accS[m], 0, 0, 0);
+                    }
                 }
             }
-        }
-    };
+        };
 
-    // sched_barrier keeps the compiler from sinking the next batch's loads below the MFMAs of
-    // the current one: all loads of a batch are issued back to back, then the math runs.
+        // sched_barrier keeps the compiler from sinking the next batch's loads below the MFMAs of
+        // the current one: all loads of a batch are issued back to back, then the math runs.
 #define XFT_FENCE() __builtin_amdgcn_sched_barrier(0)
-    if (nb > 0) {
-        issue(0, b_begin);
-        XFT_FENCE();
-    }
-    if constexpr (NORM) {
-        // RMSNorm of the M rows into LDS while the first weight tiles are on their way; same
-        // arithmetic as rmsnorm_vec_kernel: y = bf16((x * rstd) * w)
-        float *part = red + (size_t)nwaves * (16 * MT * (16 * NT + 1) + 16 * MT);
-        xn = (uint16_t *)(part + 16);
-        const int pitch = p.K + 8;
-        xn_row = (ml < p.M ? ml : p.M - 1) * pitch;
-        for (int m = 0; m < p.M; ++m) {
-            const float *row = p.norm_x + (size_t)m * p.ldx;
-            float sq = 0.0f;
-            for (int c = threadIdx.x * 4; c < p.K; c += blockDim.x * 4) {
-                const float4 v = *(const float4 *)(row + c);
-                sq = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, sq))));
-            }
+        if (nb > 0 && !pre_issued) {
+            issue(0, b_begin);
+            XFT_FENCE();
+        }
+        // Per-column scale / zero point of the epilogue, fetched now (behind the first weight
+        // batch) instead of after the reduction, where their latency would be exposed.
+        float e_scale[NT], e_zero[NT];
 #pragma unroll
-            for (int off = 32; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
-            if (lane == 0) part[(m & 1) * 8 + wave] = sq;
-            __syncthreads();
-            float tot = 0.0f;
-            for (int w = 0; w < nwaves; ++w) tot += part[(m & 1) * 8 + w];
-            const float var = 1.0f / sqrtf(tot / (float)p.K + p.norm_eps);
-            for (int c = threadIdx.x * 4; c < p.K; c += blockDim.x * 4) {
-                const float4 v = *(const float4 *)(row + c);
-                const float4 w = *(const float4 *)(p.norm_w + c);
-                const uint32_t lo = f32_to_bf16_ref((v.x * var) * w.x) | ((uint32_t)f32_to_bf16_ref((v.y * var) * w.y) << 16);
-                const uint32_t hi = f32_to_bf16_ref((v.z * var) * w.z) | ((uint32_t)f32_to_bf16_ref((v.w * var) * w.w) << 16);
-                *(uint2 *)(xn + (size_t)m * pitch + c) = make_uint2(lo, hi);
+        for (int t = 0; t < NT; ++t) {
+            e_scale[t] = 0.0f, e_zero[t] = 0.0f;
+            if constexpr (KIND != XFTHIP_W_BF16) {
+                int nt = tile_of(t);
+                nt = nt < p.NTILES ? nt : p.NTILES - 1;
+                e_scale[t] = p.scale[nt * 16 + (lane & 15)];
+                if ((KIND == XFTHIP_W_UINT4 || need_sum) && p.zero) e_zero[t] = p.zero[nt * 16 + (lane & 15)];
             }
         }
-        __syncthreads();
-    }
-    if (nb > 0) {
-        int b = 1; // next batch to issue; buffer 0 holds batch b - 1
-        for (; b + 1 < nb; b += 2) {
-            issue(1, b_begin + b);
-            XFT_FENCE();
-            compute(0, b_begin + b - 1);
-            XFT_FENCE();
-            issue(0, b_begin + b + 1);
-            XFT_FENCE();
-            compute(1, b_begin + b);
-            XFT_FENCE();
+        if (NORM && first) {
+            // RMSNorm of the M rows into LDS while the first weight tiles are on their way; same
+            // arithmetic as rmsnorm_vec_kernel: y = bf16((x * rstd) * w)
+            float *part = red + (size_t)nwaves * (16 * MT * (16 * NT + 1) + 16 * MT);
+            xn = (uint16_t *)(part + 16);
+            const int pitch = p.K + 8;
+            xn_row = (ml < p.M ? ml : p.M - 1) * pitch;
+            for (int m = 0; m < p.M; ++m) {
+                const float *row = p.norm_x + (size_t)m * p.ldx;
+                float sq = 0.0f;
+                for (int c = threadIdx.x * 4; c < p.K; c += blockDim.x * 4) {
+                    const float4 v = *(const float4 *)(row + c);
+                    sq = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, sq))));
+                }
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
+                if (lane == 0) part[(m & 1) * 8 + wave] = sq;
+                __syncthreads();
+                float tot = 0.0f;
+                for (int w = 0; w < nwaves; ++w) tot += part[(m & 1) * 8 + w];
+                const float var = 1.0f / sqrtf(tot / (float)p.K + p.norm_eps);
+                for (int c = threadIdx.x * 4; c < p.K; c += blockDim.x * 4) {
+                    const float4 v = *(const float4 *)(row + c);
+                    const float4 w = *(const float4 *)(p.norm_w + c);
+                    const uint32_t lo = f32_to_bf16_ref((v.x * var) * w.x) | ((uint32_t)f32_to_bf16_ref((v.y * var) * w.y) << 16);
+                    const uint32_t hi = f32_to_bf16_ref((v.z * var) * w.z) | ((uint32_t)f32_to_bf16_ref((v.w * var) * w.w) << 16);
+                    *(uint2 *)(xn + (size_t)m * pitch + c) = make_uint2(lo, hi);
+                }
+            }
+            __syncthreads();
         }
-        if (b < nb) {
-            issue(1, b_begin + b);
-            XFT_FENCE();
-            compute(0, b_begin + b - 1);
-            XFT_FENCE();
-            compute(1, b_begin + b);
-        } else {
-            compute(0, b_begin + b - 1);
+        if (nb > 0) {
+            int b = 1; // next batch to issue; buffer 0 holds batch b - 1
+            for (; b + 1 < nb; b += 2) {
+                issue(1, b_begin + b);
+                XFT_FENCE();
+                compute(0, b_begin + b - 1);
+                XFT_FENCE();
+                issue(0, b_begin + b + 1);
+                XFT_FENCE();
+                compute(1, b_begin + b);
+                XFT_FENCE();
+            }
+            if (b < nb) {
+                issue(1, b_begin + b);
+                XFT_FENCE();
+                compute(0, b_begin + b - 1);
+                XFT_FENCE();
+                compute(1, b_begin + b);
+            } else {
+                compute(0, b_begin + b - 1);
+            }
         }
-    }
+        if constexpr (NORM) {
+            // the next column block's first batch goes out before this block's reduction and epilogue
+            const int nxt = blk + gridDim.x;
+            pre_issued = nxt < p.nblocks;
+            if (pre_issued) {
+                set_wbase(nxt);
+                if (nb > 0) issue(0, b_begin);
+                XFT_FENCE();
+            }
+        }
 #undef XFT_FENCE
 
-    // ---- cross-wave reduction through LDS: red[wave][m][n] -------------------------------
-    constexpr int ROWS = 16 * MT, COLS = 16 * NT, LD = COLS + 1;
-    float *mine = red + (size_t)wave * (ROWS * LD + ROWS);
+        // ---- cross-wave reduction through LDS: red[wave][m][n] -------------------------------
+        constexpr int ROWS = 16 * MT, COLS = 16 * NT, LD = COLS + 1;
+        float *mine = red + (size_t)wave * (ROWS * LD + ROWS);
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
+        for (int t = 0; t < NT; ++t)
 #pragma unroll
-        for (int m = 0; m < MT; ++m)
+            for (int m = 0; m < MT; ++m)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) mine[(m * 16 + ml) * LD + t * 16 + 4 * g + r] = acc[t][m][r];
-    if (g == 0) {
+                for (int r = 0; r < 4; ++r) mine[(m * 16 + ml) * LD + t * 16 + 4 * g + r] = acc[t][m][r];
+        if (g == 0) {
 #pragma unroll
-        for (int m = 0; m < MT; ++m) mine[ROWS * LD + m * 16 + ml] = accS[m][0];
-    }
-    __syncthreads();
+            for (int m = 0; m < MT; ++m) mine[ROWS * LD + m * 16 + ml] = accS[m][0];
+        }
+        __syncthreads();
 
-    const int stride = ROWS * LD + ROWS;
-    auto total = [&](int m, int c) {
-        float s = 0.0f;
-        for (int w = 0; w < nwaves; ++w) s += red[(size_t)w * stride + m * LD + c];
-        return s;
-    };
-    auto total_sum = [&](int m) {
-        float s = 0.0f;
-        for (int w = 0; w < nwaves; ++w) s += red[(size_t)w * stride + ROWS * LD + m];
-        return s;
-    };
-    auto column_value = [&](int m, int c, float sumA) {
-        const int np = tile_of(c >> 4) * 16 + (c & 15);
-        float v = total(m, c);
-        if constexpr (KIND == XFTHIP_W_BF16) return v;
-        const float s = p.scale[np];
-        if constexpr (KIND == XFTHIP_W_UINT4) {
-            const float z = p.zero ? p.zero[np] : 0.0f;
-            return fmaf(s, v - 128.0f * sumA, z * sumA);
-        } else if constexpr (KIND == XFTHIP_W_INT8) {
-            v = s * v;
-            if constexpr (need_sum) v = fmaf(p.zero[np], sumA, v);
-            return v;
-        } else {
-            return s * v;
-        }
-    };
+        const int stride = ROWS * LD + ROWS;
+        auto total = [&](int m, int c) {
+            float s = 0.0f;
+            for (int w = 0; w < nwaves; ++w) s += red[(size_t)w * stride + m * LD + c];
+            return s;
+        };
+        auto total_sum = [&](int m) {
+            float s = 0.0f;
+            for (int w = 0; w < nwaves; ++w) s += red[(size_t)w * stride + ROWS * LD + m];
+            return s;
+        };
+        // (c & 15 equals threadIdx.x & 15 for every caller, so the scales fetched at the start of
+        // the block are the ones this thread needs)
+        auto column_value = [&](int m, int c, float sumA) {
+            float v = total(m, c);
+            if constexpr (KIND == XFTHIP_W_BF16) return v;
+            const float s = e_scale[c >> 4];
+            if constexpr (KIND == XFTHIP_W_UINT4) {
+                return fmaf(s, v - 128.0f * sumA, e_zero[c >> 4] * sumA);
+            } else if constexpr (KIND == XFTHIP_W_INT8) {
+                v = s * v;
+                if constexpr (need_sum) v = fmaf(e_zero[c >> 4], sumA, v);
+                return v;
+            } else {
+                return s * v;
+            }
+        };
 
-    if constexpr (ROPE) {
-        // one new token per sequence: row m is sequence m at position pos
-        const int it = blockIdx.x;
-        const int qcols = p.qH * 128;
-        if (it < rope_pairs) {
-            const int hh = it >> 2, jj = it & 3;
-            for (int v = threadIdx.x; v < p.M * 16; v += blockDim.x) {
-                const int m = v >> 4, c = v & 15;
+        if constexpr (ROPE) {
+            // one new token per sequence: row m is sequence m at position pos
+            const int it = blk;
+            const int qcols = p.qH * 128;
+            if (it < rope_pairs) {
+                const int hh = it >> 2, jj = it & 3;
+                for (int v = threadIdx.x; v < p.M * 16; v += blockDim.x) {
+                    const int m = v >> 4, c = v & 15;
+                    const float sumA = need_sum ? total_sum(m) : 0.0f;
+                    // the projection's output is bf16 in the reference (the rotation reads it back)
+                    const float lo = bf16_to_f32(f32_to_bf16_ref(column_value(m, c, sumA)));
+                    const float hi = bf16_to_f32(f32_to_bf16_ref(column_value(m, 16 + c, sumA)));
+                    const int i = jj * 16 + c, pos = p.pos_dev ? p.pos_dev[m] : p.pos_host;
+                    const float cs = p.cosT[(size_t)pos * 64 + i], sn = p.sinT[(size_t)pos * 64 + i];
+                    // reference: fmsub(q, cos, qHalf*sin) ; fmadd(qHalf, cos, q*sin)
+                    const float nlo = fmaf(lo, cs, -(hi * sn)), nhi = fmaf(hi, cs, lo * sn);
+                    if (hh < p.qH) {
+                        uint16_t *dst = (uint16_t *)p.C + (size_t)m * p.ldc + hh * 128;
+                        dst[i] = f32_to_bf16_ref(nlo);
+                        dst[i + 64] = f32_to_bf16_ref(nhi);
+                    } else if (pos < p.kv.S) {
+                        const size_t bh = (size_t)m * p.kv.H + (hh - p.qH);
+                        uint16_t *dst = (uint16_t *)p.kv.k + (bh * p.kv.S + pos) * 128;
+                        dst[i] = f32_to_fp16_bits(nlo);
+                        dst[i + 64] = f32_to_fp16_bits(nhi);
+                    }
+                }
+            } else {
+                for (int v = threadIdx.x; v < p.M * 32; v += blockDim.x) {
+                    const int m = v >> 5, cc = v & 31;
+                    const int vt = 2 * (it - rope_pairs) + (cc >> 4);
+                    const float sumA = need_sum ? total_sum(m) : 0.0f;
+                    const float val = bf16_to_f32(f32_to_bf16_ref(column_value(m, cc, sumA)));
+                    const int pos = p.pos_dev ? p.pos_dev[m] : p.pos_host;
+                    if (pos < p.kv.S) {
+                        const size_t bh = (size_t)m * p.kv.H + (vt >> 3);
+                        const int d = (vt & 7) * 16 + (cc & 15);
+                        uint16_t *dst = (uint16_t *)p.kv.v + (bh * (p.kv.S / 32) + (pos >> 5)) * (size_t)128 * 32 + (size_t)d * 32 + v_slot(pos & 31);
+                        *dst = f32_to_fp16_bits(val);
+                    }
+                }
+            }
+            (void)qcols;
+        } else if (!p.gateup) {
+            for (int v = threadIdx.x; v < ROWS * COLS; v += blockDim.x) {
+                const int m = v / COLS, c = v % COLS;
+                const int np = nt0 * 16 + c;
+                if (m >= p.M || np >= p.N) continue;
                 const float sumA = need_sum ? total_sum(m) : 0.0f;
-                // the projection's output is bf16 in the reference (the rotation reads it back)
-                const float lo = bf16_to_f32(f32_to_bf16_ref(column_value(m, c, sumA)));
-                const float hi = bf16_to_f32(f32_to_bf16_ref(column_value(m, 16 + c, sumA)));
-                const int i = jj * 16 + c, pos = p.pos_dev ? p.pos_dev[m] : p.pos_host;
-                const float cs = p.cosT[(size_t)pos * 64 + i], sn = p.sinT[(size_t)pos * 64 + i];
-                // reference: fmsub(q, cos, qHalf*sin) ; fmadd(qHalf, cos, q*sin)
-                const float nlo = fmaf(lo, cs, -(hi * sn)), nhi = fmaf(hi, cs, lo * sn);
-                if (hh < p.qH) {
-                    uint16_t *dst = (uint16_t *)p.C + (size_t)m * p.ldc + hh * 128;
-                    dst[i] = f32_to_bf16_ref(nlo);
-                    dst[i + 64] = f32_to_bf16_ref(nhi);
-                } else if (pos < p.kv.S) {
-                    const size_t bh = (size_t)m * p.kv.H + (hh - p.qH);
-                    uint16_t *dst = (uint16_t *)p.kv.k + (bh * p.kv.S + pos) * 128;
-                    dst[i] = f32_to_fp16_bits(nlo);
-                    dst[i + 64] = f32_to_fp16_bits(nhi);
+                float x = column_value(m, c, sumA);
+                switch (p.epi) {
+                    case XFTHIP_EPI_BIAS: x += p.bias[np]; break;
+                    case XFTHIP_EPI_SILU: x = silu_f(x); break;
+                    case XFTHIP_EPI_GELU: {
+                        float e = fast_exp(1.702f * x);
+                        x = e / (e + 1.0f) * x;
+                        break;
+                    }
+                    case XFTHIP_EPI_RESMUL: x *= load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + np); break;
+                    case XFTHIP_EPI_RESIDENTIAL:
+                        if (p.bias) x += p.bias[np];
+                        x += load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + np);
+                        break;
+                    case XFTHIP_EPI_RESEXT:
+                        if (p.bias) x += p.bias[np];
+                        x = fmaf(p.gamma, load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + np), x);
+                        break;
+                    default: break;
                 }
+                store_from_f32(p.C, p.c_dtype, (size_t)m * p.ldc + np, x);
             }
-        } else {
-            for (int v = threadIdx.x; v < p.M * 32; v += blockDim.x) {
-                const int m = v >> 5, cc = v & 31;
-                const int vt = 2 * (it - rope_pairs) + (cc >> 4);
+        } else if constexpr (NT >= 2) {
+            // tile pairs (2j, 2j+1) hold gate / up columns [16 j', 16 j' + 16)
+            constexpr int PAIRS = NT / 2;
+            for (int v = threadIdx.x; v < ROWS * PAIRS * 16; v += blockDim.x) {
+                const int m = v / (PAIRS * 16), rr = v % (PAIRS * 16);
+                const int pr = rr >> 4, c = rr & 15;
+                const int out_col = (blk * PAIRS + pr) * 16 + c;
+                if (m >= p.M || out_col >= p.N / 2) continue;
                 const float sumA = need_sum ? total_sum(m) : 0.0f;
-                const float val = bf16_to_f32(f32_to_bf16_ref(column_value(m, cc, sumA)));
-                const int pos = p.pos_dev ? p.pos_dev[m] : p.pos_host;
-                if (pos < p.kv.S) {
-                    const size_t bh = (size_t)m * p.kv.H + (vt >> 3);
-                    const int d = (vt & 7) * 16 + (cc & 15);
-                    uint16_t *dst = (uint16_t *)p.kv.v + (bh * (p.kv.S / 32) + (pos >> 5)) * (size_t)128 * 32 + (size_t)d * 32 + v_slot(pos & 31);
-                    *dst = f32_to_fp16_bits(val);
-                }
+                const float gate = column_value(m, pr * 32 + c, sumA);
+                const float up = column_value(m, pr * 32 + 16 + c, sumA);
+                store_from_f32(p.C, p.c_dtype, (size_t)m * p.ldc + out_col, up * silu_f(gate));
             }
         }
-        (void)qcols;
-    } else if (!p.gateup) {
-        for (int v = threadIdx.x; v < ROWS * COLS; v += blockDim.x) {
-            const int m = v / COLS, c = v % COLS;
-            const int np = nt0 * 16 + c;
-            if (m >= p.M || np >= p.N) continue;
-            const float sumA = need_sum ? total_sum(m) : 0.0f;
-            float x = column_value(m, c, sumA);
-            switch (p.epi) {
-                case XFTHIP_EPI_BIAS: x += p.bias[np]; break;
-                case XFTHIP_EPI_SILU: x = silu_f(x); break;
-                case XFTHIP_EPI_GELU: {
-                    float e = fast_exp(1.702f * x);
-                    x = e / (e + 1.0f) * x;
-                    break;
-                }
-                case XFTHIP_EPI_RESMUL: x *= load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + np); break;
-                case XFTHIP_EPI_RESIDENTIAL:
-                    if (p.bias) x += p.bias[np];
-                    x += load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + np);
-                    break;
-                case XFTHIP_EPI_RESEXT:
-                    if (p.bias) x += p.bias[np];
-                    x = fmaf(p.gamma, load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + np), x);
-                    break;
-                default: break;
-            }
-            store_from_f32(p.C, p.c_dtype, (size_t)m * p.ldc + np, x);
+        if constexpr (NORM) {
+            first = false;
+            __syncthreads(); // the next column block reuses the reduction area
         }
-    } else if constexpr (NT >= 2) {
-        // tile pairs (2j, 2j+1) hold gate / up columns [16 j', 16 j' + 16)
-        constexpr int PAIRS = NT / 2;
-        for (int v = threadIdx.x; v < ROWS * PAIRS * 16; v += blockDim.x) {
-            const int m = v / (PAIRS * 16), rr = v % (PAIRS * 16);
-            const int pr = rr >> 4, c = rr & 15;
-            const int out_col = (blockIdx.x * PAIRS + pr) * 16 + c;
-            if (m >= p.M || out_col >= p.N / 2) continue;
-            const float sumA = need_sum ? total_sum(m) : 0.0f;
-            const float gate = column_value(m, pr * 32 + c, sumA);
-            const float up = column_value(m, pr * 32 + 16 + c, sumA);
-            store_from_f32(p.C, p.c_dtype, (size_t)m * p.ldc + out_col, up * silu_f(gate));
-        }
+    };
+    if constexpr (NORM) {
+        for (int blk = blockIdx.x; blk < p.nblocks; blk += gridDim.x) run_block(blk);
+    } else {
+        run_block(blockIdx.x);
     }
 }
 
@@ -469,8 +510,14 @@ static int launch(const SkinnyParams &p, int kslices, hipStream_t stream) {
     if (NORM) smem += 64 + skinny_norm_lds_bytes(p.M, p.K);
     int blocks = (p.NTILES + NT - 1) / NT;
     if (ROPE) blocks = (p.qH + 2 * p.kvH) * 4; // rotation pairs of the query and key heads, then value tile pairs
+    SkinnyParams q = p;
+    q.nblocks = blocks;
+    if (NORM) {
+        const int cus = device_cu_count();
+        blocks = blocks < cus ? blocks : cus;
+    }
     hipLaunchKernelGGL((qgemm_skinny_kernel<KIND, NT, MT, U, NEED_SUM, KTAIL, NORM, ROPE>), dim3(blocks), dim3(64 * kslices), smem,
-            stream, p);
+            stream, q);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }

@@ -28,6 +28,15 @@ int device_cu_count() {
 
 using namespace xfthip;
 
+namespace xfthip {
+typedef uint32_t cp16 __attribute__((ext_vector_type(4)));
+// plain grid-stride copy, 16 bytes per lane: the known-traffic kernel that HBM byte counters are
+// calibrated against
+__global__ void stream_copy_kernel(const cp16 *__restrict__ src, cp16 *__restrict__ dst, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+} // namespace xfthip
+
 extern "C" {
 
 const char *xfthip_last_error(void) {
@@ -96,6 +105,18 @@ int xfthip_memcpy_d2h(void *dst_host, const void *src, size_t bytes, xfthip_stre
 int xfthip_memcpy_d2d(void *dst, const void *src, size_t bytes, xfthip_stream_t stream) {
     if (bytes == 0) return 0;
     XFT_CHECK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream));
+    return 0;
+}
+
+int xfthip_copy_kernel(void *dst, const void *src, size_t bytes, xfthip_stream_t stream) {
+    XFT_REQUIRE(dst && src && bytes % 16 == 0 && (((uintptr_t)dst | (uintptr_t)src) & 15) == 0,
+            "xfthip_copy_kernel: pointers and size must be 16-byte aligned");
+    if (bytes == 0) return 0;
+    const size_t n = bytes / 16;
+    const int blocks = (int)((n + 1023) / 1024 < 8192 ? (n + 1023) / 1024 : 8192);
+    hipLaunchKernelGGL(xfthip::stream_copy_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const xfthip::cp16 *)src,
+            (xfthip::cp16 *)dst, n);
+    XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }
 

@@ -62,10 +62,12 @@ struct AttnLds {
 };
 
 // wg_sync: a barrier over the block.
-// COH: the unit runs inside a kernel whose other workgroups produced q and will consume the
-// output in the same launch: q, the split partials and the output then go through
-// device-coherent accesses (ld_dev / st_dev) and the ticket needs no cache maintenance.  The
-// cache rows appended in the same launch must have been written with st_dev as well.
+// COH: q, the split partials and a bf16 output go through device-coherent accesses (ld_dev /
+// st_dev), and the ticket hand-over between the workgroups of a split needs no cache maintenance:
+// the alternative, a device-scope fence by every thread, writes back and invalidates the whole L2
+// of the XCD and costs several microseconds per launch.  It also lets the unit run inside a
+// kernel whose other workgroups produced q and will consume the output in the same launch (the
+// cache rows appended in that launch must then have been written with st_dev as well).
 template <bool INT8, int NW, bool COH = false, typename Sync>
 __device__ inline void attn_unit(const AttnParams &p, const int split, const int kvh, const int cg, const int b, AttnLds<NW> &L,
         const Sync &wg_sync) {
@@ -287,7 +289,7 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
         if (p.nsplit == 1) {
             const int s_tok = cc / p.G, j = cc % p.G;
             const size_t idx = ((size_t)b * p.S + s_tok) * p.oStride + (size_t)(kvh * p.G + j) * D + d;
-            if constexpr (COH)
+            if (COH && p.out_dtype == XFTHIP_BF16)
                 st_dev((uint16_t *)p.out + idx, f32_to_bf16_ref(acc / l));
             else
                 store_from_f32(p.out, p.out_dtype, idx, acc / l);
@@ -370,7 +372,7 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
         }
         const int s_tok = cc / p.G, j = cc % p.G;
         const size_t idx = ((size_t)b * p.S + s_tok) * p.oStride + (size_t)(kvh * p.G + j) * D + d;
-        if constexpr (COH)
+        if (COH && p.out_dtype == XFTHIP_BF16)
             st_dev((uint16_t *)p.out + idx, f32_to_bf16_ref(acc * s_linv[col]));
         else
             store_from_f32(p.out, p.out_dtype, idx, acc * s_linv[col]);

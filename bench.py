@@ -294,9 +294,10 @@ def main():
 
     # dominant kernel: the M<=32 weight-only GEMV, in the three forms the decode step launches it
     groups = []
-    for key, name, which in (("qkv", "qgemm_skinny_kernel (norm + qkv + RoPE/cache append)", (0,)),
+    fused = B <= 4  # beyond 4 rows the norm and the rotation run as kernels of their own
+    for key, name, which in (("qkv", "qgemm_skinny_kernel (norm + qkv + RoPE/cache append)" if fused else "qgemm_skinny_kernel (qkv)", (0,)),
                              ("narrow", "qgemm_skinny_kernel (out-proj, down)", (1, 3)),
-                             ("wide", "qgemm_skinny_kernel (norm + gate/up + SwiGLU)", (2,))):
+                             ("wide", "qgemm_skinny_kernel (norm + gate/up + SwiGLU)" if fused else "qgemm_skinny_kernel (gate/up + SwiGLU)", (2,))):
         us, byts = time_gemm_kernel(xh, layer_weights, which, B, 4)
         groups.append(dict(name=name, us=us, bytes=byts, launches=len(which), key=key))
     groups.sort(key=lambda g: -g["us"] * g["launches"])

@@ -164,3 +164,16 @@ def test_kvstore_rejects_overflow(xh):
         xh.rope_kvstore(cache, dev.ptr, xh.BF16, (8 + 4) * 128, 1, 4, 8, None, 14)
     with pytest.raises(xh.XftHipError):
         xh.rope_kvstore(cache, dev.ptr, xh.BF16, (8 + 4) * 128, 2, 1, 8, None, 0)
+
+
+def test_copy_kernel_copies_and_checks_alignment(xh):
+    rng = np.random.default_rng(17)
+    a = rng.integers(0, 2 ** 31, 3 * 4096 + 4, dtype=np.int64).astype(np.uint32)
+    src = xh.DeviceBuffer.from_numpy(a)
+    dst = xh.DeviceBuffer(a.nbytes)
+    dst.zero()
+    xh.copy_kernel(dst.ptr, src.ptr, a.nbytes)
+    xh.synchronize()
+    assert np.array_equal(dst.to_numpy(np.uint32, a.shape), a)
+    with pytest.raises(xh.XftHipError):
+        xh.copy_kernel(dst.ptr, src.ptr, 24)  # not a multiple of 16 bytes

@@ -24,7 +24,7 @@ namespace xfthip {
 template <bool INT8>
 __global__ __launch_bounds__(256) void attn_kernel(AttnParams p) {
     __shared__ AttnLds<4> lds;
-    attn_unit<INT8, 4, true>(p, blockIdx.x, blockIdx.y % p.kv.H, blockIdx.y / p.kv.H, blockIdx.z, lds, [] { __syncthreads(); });
+    attn_unit<INT8, 4>(p, blockIdx.x, blockIdx.y % p.kv.H, blockIdx.y / p.kv.H, blockIdx.z, lds, [] { __syncthreads(); });
 }
 
 static float *g_ws = nullptr;

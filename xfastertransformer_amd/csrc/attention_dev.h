@@ -62,13 +62,13 @@ struct AttnLds {
 };
 
 // wg_sync: a barrier over the block.
-// COH: q, the split partials and a bf16 output go through device-coherent accesses (ld_dev /
-// st_dev), and the ticket hand-over between the workgroups of a split needs no cache maintenance:
-// the alternative, a device-scope fence by every thread, writes back and invalidates the whole L2
-// of the XCD and costs several microseconds per launch.  It also lets the unit run inside a
-// kernel whose other workgroups produced q and will consume the output in the same launch (the
-// cache rows appended in that launch must then have been written with st_dev as well).
-template <bool INT8, int NW, bool COH = false, typename Sync>
+// q, the split partials and a bf16 output go through device-coherent accesses (ld_dev / st_dev),
+// and the ticket hand-over between the workgroups of a split needs no cache maintenance: the
+// alternative, a device-scope fence by every thread, writes back and invalidates the whole L2 of
+// the XCD and costs several microseconds per launch.  It also lets the unit run inside a kernel
+// whose other workgroups produced q and will consume the output in the same launch (the cache
+// rows appended in that launch must then have been written with st_dev as well).
+template <bool INT8, int NW, typename Sync>
 __device__ inline void attn_unit(const AttnParams &p, const int split, const int kvh, const int cg, const int b, AttnLds<NW> &L,
         const Sync &wg_sync) {
     constexpr int D = 128;
@@ -161,12 +161,7 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
             const int d0 = INT8 ? 64 * (s >> 1) + 16 * g + 8 * (s & 1) : 32 * s + 8 * g;
             qraw[s][0] = qraw[s][1] = qraw[s][2] = qraw[s][3] = 0u;
             if (cvalid) {
-                if constexpr (COH) {
-                    ld_dev16(qrow + d0, qraw[s]);
-                } else {
-                    const u32x4 r4 = *(const u32x4 *)(qrow + d0);
-                    qraw[s][0] = r4[0], qraw[s][1] = r4[1], qraw[s][2] = r4[2], qraw[s][3] = r4[3];
-                }
+                ld_dev16(qrow + d0, qraw[s]);
             }
         }
     }
@@ -289,21 +284,15 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
         if (p.nsplit == 1) {
             const int s_tok = cc / p.G, j = cc % p.G;
             const size_t idx = ((size_t)b * p.S + s_tok) * p.oStride + (size_t)(kvh * p.G + j) * D + d;
-            if (COH && p.out_dtype == XFTHIP_BF16)
+            if (p.out_dtype == XFTHIP_BF16)
                 st_dev((uint16_t *)p.out + idx, f32_to_bf16_ref(acc / l));
             else
                 store_from_f32(p.out, p.out_dtype, idx, acc / l);
-        } else if constexpr (COH) {
+        } else {
             st_dev(&slot[32 + col * D + d], acc);
             if (d == 0) {
                 st_dev(&slot[col], m);
                 st_dev(&slot[16 + col], l);
-            }
-        } else {
-            slot[32 + col * D + d] = acc;
-            if (d == 0) {
-                slot[col] = m;
-                slot[16 + col] = l;
             }
         }
     }
@@ -313,21 +302,13 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
     // (no waiting: every workgroup publishes its partial, takes a ticket and leaves; the one
     // holding the last ticket sees all partials and resets the counter for the next launch)
     unsigned int &s_ticket = L.s_ticket;
-    if constexpr (COH)
-        dev_drain();
-    else
-        __threadfence();
+    dev_drain();
     wg_sync();
     if (threadIdx.x == 0) s_ticket = atomicAdd(&p.tickets[group], 1u);
     wg_sync();
     if (s_ticket != (unsigned int)(p.nsplit - 1)) return;
-    if constexpr (COH) {
-        if (threadIdx.x == 0) st_dev(&p.tickets[group], 0u);
-    } else {
-        __threadfence();
-        if (threadIdx.x == 0) p.tickets[group] = 0u;
-    }
-    auto ws_ld = [](const float *q) { return COH ? ld_dev(q) : *q; };
+    if (threadIdx.x == 0) st_dev(&p.tickets[group], 0u);
+    auto ws_ld = [](const float *q) { return ld_dev(q); };
     // factors first (one thread per column, then per (split, column)), so that the wide pass over
     // the partial outputs is a plain weighted sum with independent loads
     const float *base = p.ws + group * p.nsplit * kSlotFloats;
@@ -372,7 +353,7 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
         }
         const int s_tok = cc / p.G, j = cc % p.G;
         const size_t idx = ((size_t)b * p.S + s_tok) * p.oStride + (size_t)(kvh * p.G + j) * D + d;
-        if (COH && p.out_dtype == XFTHIP_BF16)
+        if (p.out_dtype == XFTHIP_BF16)
             st_dev((uint16_t *)p.out + idx, f32_to_bf16_ref(acc * s_linv[col]));
         else
             store_from_f32(p.out, p.out_dtype, idx, acc * s_linv[col]);

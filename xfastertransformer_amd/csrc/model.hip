@@ -47,18 +47,29 @@ __global__ void gather_last_kernel(const float *__restrict__ x, float *__restric
 
 // first maximum per row: strict '>' inside a thread's ascending scan, lower index wins ties
 // across threads
-__global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ logits, int cols, int *__restrict__ ids) {
+// advance_pos / advance_step (may be null): the decode step's position and step counters, bumped
+// here so that the step needs no launches of its own for them
+__global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ logits, int cols, int *__restrict__ ids,
+        int *advance_pos, int *advance_step) {
     __shared__ float sv[1024];
     __shared__ int si[1024];
     const float *p = logits + (size_t)blockIdx.x * cols;
     float bv = -INFINITY;
     int bi = 0x7FFFFFFF;
-    for (int j = threadIdx.x; j < cols; j += blockDim.x) {
-        const float v = p[j];
+    auto take = [&](float v, int j) {
         if (v > bv || bi == 0x7FFFFFFF) {
             bv = v;
             bi = j;
         }
+    };
+    const bool vec = ((cols & 3) == 0) && ((((uintptr_t)p) & 15) == 0);
+    if (vec) {
+        for (int j = threadIdx.x * 4; j < cols; j += blockDim.x * 4) {
+            const float4 v = *(const float4 *)(p + j);
+            take(v.x, j), take(v.y, j + 1), take(v.z, j + 2), take(v.w, j + 3);
+        }
+    } else {
+        for (int j = threadIdx.x; j < cols; j += blockDim.x) take(p[j], j);
     }
     sv[threadIdx.x] = bv;
     si[threadIdx.x] = bi;
@@ -74,12 +85,22 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ 
         }
         __syncthreads();
     }
-    if (threadIdx.x == 0) ids[blockIdx.x] = si[0];
+    if (threadIdx.x == 0) {
+        ids[blockIdx.x] = si[0];
+        if (advance_pos) advance_pos[blockIdx.x] += 1;
+        if (advance_step && blockIdx.x == 0) advance_step[0] += 1;
+    }
 }
 
-__global__ void advance_kernel(int *pos, int n, int by) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) pos[i] += by;
+// start of a decode step: log the input id of sequence blockIdx.x and embed it
+__global__ void decode_begin_kernel(const uint16_t *__restrict__ table, const int *__restrict__ ids, float *__restrict__ x, int hidden,
+        int vocab, int *__restrict__ log, const int *__restrict__ step) {
+    const int b = blockIdx.x;
+    int id = ids[b];
+    if (threadIdx.x == 0) log[(size_t)step[0] * gridDim.x + b] = id;
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    const uint16_t *row = table + (size_t)id * hidden;
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) x[(size_t)b * hidden + c] = fp16_bits_to_f32(row[c]);
 }
 
 __global__ void fill_int_kernel(int *p, int n, int v) {
@@ -87,10 +108,6 @@ __global__ void fill_int_kernel(int *p, int n, int v) {
     if (i < n) p[i] = v;
 }
 
-__global__ void record_ids_kernel(const int *ids, int *log, const int *step, int B) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < B) log[(size_t)step[0] * B + i] = ids[i];
-}
 
 } // namespace xfthip
 
@@ -346,35 +363,47 @@ static int layer_forward(xfthip_model *m, int idx, const float *x_in, int in_str
     return mlp_block(m, idx, x_out, out_stride, x_out, out_stride, B * S, true, st);
 }
 
-static int head_forward(xfthip_model *m, const float *xrows, int B, hipStream_t st) {
+// final norm + lm_head + greedy pick; advance: also bump the decode step's position / step counters
+static int head_forward(xfthip_model *m, const float *xrows, int B, bool advance, hipStream_t st) {
     const xfthip_model_config &c = m->cfg;
     int rc;
-    if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, xrows, XFTHIP_F32, m->final_norm, B, c.hidden, c.hidden, c.hidden, c.rms_eps, st))) return rc;
-    if ((rc = xfthip_gemm(m->lm_head, B, m->xn, c.hidden, m->logits, c.vocab, XFTHIP_F32, XFTHIP_EPI_NONE, nullptr, nullptr, 0, XFTHIP_F32,
-                 1.0f, st)))
-        return rc;
-    return xfthip_argmax(m->logits, B, c.vocab, m->ids, st);
+    const PackedWeight &wl = m->lm_head->pw;
+    if (m->fuse_decode && wl.kind != XFTHIP_W_W8A8 && skinny_can_fuse_norm(wl, B)) {
+        SkinnyParams sp = {};
+        sp.M = B;
+        sp.C = m->logits;
+        sp.ldc = c.vocab;
+        sp.c_dtype = XFTHIP_F32;
+        sp.epi = XFTHIP_EPI_NONE;
+        sp.gamma = 1.0f;
+        sp.norm_x = xrows, sp.ldx = c.hidden, sp.norm_w = m->final_norm, sp.norm_eps = c.rms_eps;
+        if ((rc = qgemm_skinny(wl, sp, st))) return rc;
+    } else {
+        if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, xrows, XFTHIP_F32, m->final_norm, B, c.hidden, c.hidden, c.hidden, c.rms_eps, st))) return rc;
+        if ((rc = xfthip_gemm(m->lm_head, B, m->xn, c.hidden, m->logits, c.vocab, XFTHIP_F32, XFTHIP_EPI_NONE, nullptr, nullptr, 0,
+                     XFTHIP_F32, 1.0f, st)))
+            return rc;
+    }
+    hipLaunchKernelGGL(argmax_kernel, dim3(B), dim3(1024), 0, st, m->logits, c.vocab, m->ids, advance ? m->pos : nullptr,
+            advance ? m->step : nullptr);
+    XFT_CHECK_HIP(hipGetLastError());
+    return 0;
 }
 
 // the decode step that gets captured: everything reads its position from device memory
 static int decode_step(xfthip_model *m, int B, hipStream_t st) {
     const xfthip_model_config &c = m->cfg;
-    hipLaunchKernelGGL(record_ids_kernel, dim3((B + 63) / 64), dim3(64), 0, st, m->ids, m->idlog, m->step, B);
-    hipLaunchKernelGGL(embed_kernel, dim3(B), dim3(256), 0, st, m->embedding, m->ids, m->x, c.hidden, c.vocab);
+    hipLaunchKernelGGL(decode_begin_kernel, dim3(B), dim3(256), 0, st, m->embedding, m->ids, m->x, c.hidden, c.vocab, m->idlog, m->step);
     for (int l = 0; l < c.layers; ++l)
         if (int rc = layer_forward(m, l, m->x, c.hidden, m->x, c.hidden, B, 1, 0, m->pos, st)) return rc;
-    if (int rc = head_forward(m, m->x, B, st)) return rc;
-    hipLaunchKernelGGL(advance_kernel, dim3((B + 63) / 64), dim3(64), 0, st, m->pos, B, 1);
-    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(64), 0, st, m->step, 1, 1);
-    XFT_CHECK_HIP(hipGetLastError());
-    return 0;
+    return head_forward(m, m->x, B, true, st);
 }
 
 extern "C" {
 
 int xfthip_argmax(const float *logits, int rows, int cols, int *ids_dev, xfthip_stream_t stream) {
     XFT_REQUIRE(logits && ids_dev && rows > 0 && cols > 0, "xfthip_argmax: bad argument");
-    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, logits, cols, ids_dev);
+    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, logits, cols, ids_dev, (int *)nullptr, (int *)nullptr);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }
@@ -561,7 +590,7 @@ int xfthip_model_prefill(xfthip_model_t m, const int *ids_host, int B, int S, fl
     for (int l = 0; l < c.layers; ++l)
         if (int rc = layer_forward(m, l, m->x, c.hidden, m->x, c.hidden, B, S, 0, nullptr, st)) return rc;
     hipLaunchKernelGGL(gather_last_kernel, dim3(B), dim3(256), 0, st, m->x, m->xlast, S, c.hidden);
-    if (int rc = head_forward(m, m->xlast, B, st)) return rc;
+    if (int rc = head_forward(m, m->xlast, B, false, st)) return rc;
     hipLaunchKernelGGL(fill_int_kernel, dim3((B + 63) / 64), dim3(64), 0, st, m->pos, B, S);
     hipLaunchKernelGGL(fill_int_kernel, dim3(1), dim3(64), 0, st, m->step, 1, 0);
     XFT_CHECK_HIP(hipGetLastError());

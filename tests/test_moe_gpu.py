@@ -30,7 +30,8 @@ def test_top2_selection_and_weights(xh, orc):
     logits = rng.standard_normal((300, 8)).astype(np.float32)
     logits[5] = [1, 5, 5, 0, 5, -1, 2, 2]  # ties: the lower index wins
     logits[6] = [3, 3, 3, 3, 3, 3, 3, 3]
-    sel, w = xh.moe_top2(xh.DeviceBuffer.from_numpy(logits).ptr, 300, 8)
+    dev = xh.DeviceBuffer.from_numpy(logits)  # kept alive across the call: a temporary would be freed before the kernel runs
+    sel, w = xh.moe_top2(dev.ptr, 300, 8)
     esel, ew = orc.moe_top2(logits)
     assert np.array_equal(sel, esel)
     assert list(sel[5]) == [1, 2] and list(sel[6]) == [0, 1]

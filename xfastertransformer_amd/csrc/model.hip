@@ -367,23 +367,12 @@ static int layer_forward(xfthip_model *m, int idx, const float *x_in, int in_str
 static int head_forward(xfthip_model *m, const float *xrows, int B, bool advance, hipStream_t st) {
     const xfthip_model_config &c = m->cfg;
     int rc;
-    const PackedWeight &wl = m->lm_head->pw;
-    if (m->fuse_decode && wl.kind != XFTHIP_W_W8A8 && skinny_can_fuse_norm(wl, B)) {
-        SkinnyParams sp = {};
-        sp.M = B;
-        sp.C = m->logits;
-        sp.ldc = c.vocab;
-        sp.c_dtype = XFTHIP_F32;
-        sp.epi = XFTHIP_EPI_NONE;
-        sp.gamma = 1.0f;
-        sp.norm_x = xrows, sp.ldx = c.hidden, sp.norm_w = m->final_norm, sp.norm_eps = c.rms_eps;
-        if ((rc = qgemm_skinny(wl, sp, st))) return rc;
-    } else {
-        if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, xrows, XFTHIP_F32, m->final_norm, B, c.hidden, c.hidden, c.hidden, c.rms_eps, st))) return rc;
-        if ((rc = xfthip_gemm(m->lm_head, B, m->xn, c.hidden, m->logits, c.vocab, XFTHIP_F32, XFTHIP_EPI_NONE, nullptr, nullptr, 0,
-                     XFTHIP_F32, 1.0f, st)))
-            return rc;
-    }
+    // (the norm stays a kernel of its own here: as a prologue of the 2000-tile lm_head GEMV it cost
+    // 3 us more than it saved)
+    if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, xrows, XFTHIP_F32, m->final_norm, B, c.hidden, c.hidden, c.hidden, c.rms_eps, st))) return rc;
+    if ((rc = xfthip_gemm(m->lm_head, B, m->xn, c.hidden, m->logits, c.vocab, XFTHIP_F32, XFTHIP_EPI_NONE, nullptr, nullptr, 0, XFTHIP_F32,
+                 1.0f, st)))
+        return rc;
     hipLaunchKernelGGL(argmax_kernel, dim3(B), dim3(1024), 0, st, m->logits, c.vocab, m->ids, advance ? m->pos : nullptr,
             advance ? m->step : nullptr);
     XFT_CHECK_HIP(hipGetLastError());

@@ -168,6 +168,25 @@ def test_decode_graph_replays_match_eager_layers(xh, orc, persistent):
         full = np.concatenate([full, nxt.reshape(B, 1)], 1)
 
 
+def test_decode_graph_recaptured_when_the_split_count_changes(xh, orc):
+    """The attention split count is fixed when the decode step is captured and follows the
+    sequence length in steps of 128 tokens: decoding across such a boundary (and with a cache much
+    longer than the sequence) must still equal the eager recomputation of every token."""
+    B, S, steps, vocab = 2, 122, 10, 1000
+    model, _ = build_small_model(xh, orc, 0, 9, max_seq=1024)
+    ids = np.random.default_rng(39).integers(0, vocab, (B, S)).astype(np.int32)
+    first, _ = model.prefill(ids)
+    seq = [first]
+    for t in range(steps):
+        seq.append(model.decode(1, B)[0])
+    graph_ids = np.stack(seq, 1)
+    full = ids
+    for t in range(steps + 1):
+        nxt, _ = model.prefill(full)
+        assert np.array_equal(nxt, graph_ids[:, t]), t
+        full = np.concatenate([full, nxt.reshape(B, 1)], 1)
+
+
 @pytest.mark.parametrize("B,S", [(1, 40), (4, 9), (3, 33)])
 def test_persistent_decode_matches_per_kernel_decode(xh, orc, B, S):
     """The persistent whole-step kernel and the per-kernel decode step compute the same step

@@ -44,8 +44,10 @@ int attention_workspace_init() {
 
 using namespace xfthip;
 
-extern "C" int xfthip_attention(xfthip_kvcache_t c, const void *q, int qStride, void *out, int oStride, int out_dtype,
-        int B, int S, int qHeads, float scale, int past, const int *past_dev, xfthip_stream_t stream) {
+// len_hint: upper bound of the visible sequence length when the positions live in device memory
+// (0 = unknown, the cache length is assumed); it only steers the split count
+int xfthip::attention_launch(xfthip_kvcache_t c, const void *q, int qStride, void *out, int oStride, int out_dtype, int B, int S,
+        int qHeads, float scale, int past, const int *past_dev, int len_hint, hipStream_t stream) {
     XFT_REQUIRE(c && q && out, "xfthip_attention: null argument");
     XFT_REQUIRE(B > 0 && B <= c->kv.B, "xfthip_attention: batch %d exceeds cache batch %d", B, c->kv.B);
     XFT_REQUIRE(S > 0 && qHeads > 0 && qHeads % c->kv.H == 0, "xfthip_attention: bad S=%d or qHeads=%d (kvHeads=%d)", S, qHeads,
@@ -74,15 +76,9 @@ extern "C" int xfthip_attention(xfthip_kvcache_t c, const void *q, int qStride, 
     // split the KV sequence so that the launch has ~4 workgroups per CU, each wave keeping at
     // least one 32-token block; the longest visible sequence is bounded by the cache length
     // when the real one lives in device memory
-    const int len = past_dev ? c->maxSeq : past + S;
-    const int nblk = (len + 31) / 32;
+    const int len = past_dev ? ((len_hint > 0 && len_hint < c->maxSeq) ? len_hint : c->maxSeq) : past + S;
     const int wgs = B * c->kv.H * p.CG;
-    int nsplit = (4 * device_cu_count() + wgs - 1) / wgs;
-    const int cap = (nblk + 3) / 4;
-    if (nsplit > cap) nsplit = cap;
-    if (nsplit > 64) nsplit = 64;
-    if (nsplit < 1) nsplit = 1;
-    while (nsplit > 1 && (size_t)wgs * nsplit > (size_t)kWsSlots) --nsplit;
+    const int nsplit = attention_split_count(len, wgs);
     p.nsplit = nsplit;
     if (nsplit > 1)
         if (int rc = attention_workspace_init()) return rc;
@@ -90,9 +86,25 @@ extern "C" int xfthip_attention(xfthip_kvcache_t c, const void *q, int qStride, 
     p.tickets = g_tickets;
     dim3 grid(nsplit, c->kv.H * p.CG, B);
     if (c->kv.int8)
-        hipLaunchKernelGGL(attn_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, p);
+        hipLaunchKernelGGL(attn_kernel<true>, grid, dim3(256), 0, stream, p);
     else
-        hipLaunchKernelGGL(attn_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, p);
+        hipLaunchKernelGGL(attn_kernel<false>, grid, dim3(256), 0, stream, p);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
+}
+
+int xfthip::attention_split_count(int len, int units) {
+    const int nblk = (len + 31) / 32;
+    int nsplit = (4 * device_cu_count() + units - 1) / units;
+    const int cap = (nblk + 3) / 4;
+    if (nsplit > cap) nsplit = cap;
+    if (nsplit > 64) nsplit = 64;
+    if (nsplit < 1) nsplit = 1;
+    while (nsplit > 1 && (size_t)units * nsplit > (size_t)kWsSlots) --nsplit;
+    return nsplit;
+}
+
+extern "C" int xfthip_attention(xfthip_kvcache_t c, const void *q, int qStride, void *out, int oStride, int out_dtype,
+        int B, int S, int qHeads, float scale, int past, const int *past_dev, xfthip_stream_t stream) {
+    return attention_launch(c, q, qStride, out, oStride, out_dtype, B, S, qHeads, scale, past, past_dev, 0, (hipStream_t)stream);
 }

@@ -148,6 +148,11 @@ int device_cu_count();
 // allocates the split-KV merge workspace of the attention kernel (idempotent; must not run
 // during stream capture)
 int attention_workspace_init();
+// the attention launch behind xfthip_attention, with a length hint for callers whose positions live
+// in device memory, and the split count it picks for `units` (batch x kv head x column group) workgroups
+int attention_launch(xfthip_kvcache_t c, const void *q, int qStride, void *out, int oStride, int out_dtype, int B, int S,
+        int qHeads, float scale, int past, const int *past_dev, int len_hint, hipStream_t stream);
+int attention_split_count(int len, int units);
 
 } // namespace xfthip
 

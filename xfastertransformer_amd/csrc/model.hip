@@ -134,6 +134,8 @@ struct xfthip_model {
     int cur_B = 0, cur_pos = 0;
     hipGraphExec_t graph = nullptr;
     int graph_B = 0;
+    int graph_nsplit = 0; // attention split count the captured step was built with
+    int len_hint = 0; // upper bound of the sequence length during the current decode call (0 = unknown)
     hipStream_t graph_stream = nullptr;
     bool use_graph = true;
     bool fuse_decode = true; // RMSNorm prologue / RoPE + cache-append epilogue inside the decode GEMVs
@@ -316,8 +318,8 @@ static int attention_block(xfthip_model *m, int idx, const float *x_in, int in_s
             return rc;
         attend = m->prefill_cache;
     }
-    if ((rc = xfthip_attention(attend, m->qkv, qkv_cols, m->att, qcols, XFTHIP_BF16, B, S, c.q_heads,
-                 1.0f / sqrtf((float)c.head_size), past, past_dev, st)))
+    if ((rc = attention_launch(attend, m->qkv, qkv_cols, m->att, qcols, XFTHIP_BF16, B, S, c.q_heads, 1.0f / sqrtf((float)c.head_size), past,
+                 past_dev, past_dev ? m->len_hint : 0, st)))
         return rc;
     return xfthip_gemm(L.o, T, m->att, qcols, x_out, out_stride, XFTHIP_F32, XFTHIP_EPI_RESIDENTIAL, L.o_bias, x_in, in_stride,
             XFTHIP_F32, 1.0f, st);
@@ -600,6 +602,11 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
     hipStream_t st = (hipStream_t)stream;
     const int B = m->cur_B;
     hipLaunchKernelGGL(fill_int_kernel, dim3(1), dim3(64), 0, st, m->step, 1, 0);
+    // the positions are read from device memory, but the attention split count is fixed at launch
+    // (capture) time: it follows an upper bound of the length, rounded up so that the graph is
+    // re-captured only every 128 tokens
+    m->len_hint = ((m->cur_pos + steps + 127) / 128) * 128;
+    const int nsplit = attention_split_count(m->len_hint < c.max_seq ? m->len_hint : c.max_seq, B * c.kv_heads);
     bool persistent = false;
     if (m->use_persistent && B <= 4 && (size_t)B * c.kv_heads <= (size_t)kWsSlots) {
         if (m->mega_state == 0)
@@ -613,7 +620,7 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
     } else if (!m->use_graph) {
         for (int i = 0; i < steps; ++i)
             if (int rc = decode_step(m, B, st)) return rc;
-    } else if (m->graph == nullptr || m->graph_B != B || m->graph_stream != st) {
+    } else if (m->graph == nullptr || m->graph_B != B || m->graph_stream != st || m->graph_nsplit != nsplit) {
         if (m->graph) {
             (void)hipGraphExecDestroy(m->graph);
             m->graph = nullptr;
@@ -642,6 +649,7 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
         if (own) (void)hipStreamDestroy(cap);
         XFT_CHECK_HIP(e);
         m->graph_B = B;
+        m->graph_nsplit = nsplit;
         m->graph_stream = st;
     }
     if (!persistent && m->use_graph)

@@ -94,6 +94,10 @@ class GemvHarness:
             xh.gemm_gateup_silu_rmsnorm(w, self.x.ptr, M, c["hidden"], self.g.ptr, 1e-6, self.out.ptr, w.N // 2, xh.BF16)
         elif i == 2:
             xh.gemm_gateup_silu(w, self.A.ptr, M, w.K, self.out.ptr, w.N // 2, xh.BF16)
+        elif i in (1, 3):
+            # out-projection / down projection: fp32 result + fp32 residual, as in the layer
+            xh.gemm(w, self.A.ptr, M, w.K, self.out.ptr, w.N, xh.F32, epi=xh.EPI_RESIDENTIAL, res=self.x.ptr, ldres=c["hidden"],
+                    res_dtype=xh.F32)
         else:
             xh.gemm(w, self.A.ptr, M, w.K, self.out.ptr, w.N, xh.BF16)
 
@@ -117,8 +121,10 @@ def time_gemm_kernel(xh, layer_weights, which, M, iters):
                 n += 1
     ms = t.stop()
     in_bytes = lambda i, w: (4 if (h.fused and i in (0, 2)) else 2) * M * w.K
-    byts = sum(layer_weights[0][i].bytes() + in_bytes(i, layer_weights[0][i])
-               + 2 * M * (layer_weights[0][i].N // (2 if i == 2 else 1)) for i in which) / len(which)
+    # result rows: bf16, except the fp32 result + fp32 residual of out-proj / down
+    out_bytes = lambda i, w: (8 * M * w.N) if i in (1, 3) else 2 * M * (w.N // (2 if i == 2 else 1))
+    byts = sum(layer_weights[0][i].bytes() + in_bytes(i, layer_weights[0][i]) + out_bytes(i, layer_weights[0][i])
+               for i in which) / len(which)
     return ms * 1e3 / n, byts
 
 

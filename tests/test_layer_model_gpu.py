@@ -262,6 +262,20 @@ def test_persistent_decode_multi_step_call(xh, orc):
     assert np.array_equal(one, many)
 
 
+def test_persistent_trace_reports_increasing_barrier_times(xh, orc):
+    layers = 2
+    model, _ = build_small_model(xh, orc, 0, 14, layers=layers)
+    model.use_persistent(True)
+    model.persistent_trace(arm=True)
+    model.prefill(np.random.default_rng(40).integers(0, 1000, (2, 12)).astype(np.int32))
+    model.decode(3, 2)
+    assert model.decode_mode() == 2
+    t = model.persistent_trace()
+    # kernel start, then one entry per barrier: embedding, 5 per layer, lm_head
+    assert t.shape == (5 * layers + 3,)
+    assert np.all(np.diff(t) > 0) and (t[-1] - t[0]) < 0.1
+
+
 def test_model_rejects_bad_use(xh, orc):
     model, _ = build_small_model(xh, orc, 0, 7, layers=1)
     with pytest.raises(xh.XftHipError):

@@ -44,7 +44,7 @@ def synth_codes(rng, kind, K, N):
     return q, scale, zero
 
 
-def build_model(xh, kind, batch, max_seq, prompt):
+def build_model(xh, kind, batch, max_seq, prompt, kv_int8=False):
     c = CFG
     rng = np.random.default_rng(3)
     qkv_cols = (c["q_heads"] + 2 * c["kv_heads"]) * c["head"]
@@ -52,7 +52,7 @@ def build_model(xh, kind, batch, max_seq, prompt):
               (c["inter"], c["hidden"])]
     host = [synth_codes(rng, kind, K, N) for K, N in shapes]
     model = xh.Model(c["layers"], c["hidden"], c["inter"], c["q_heads"], c["kv_heads"], c["head"], vocab=c["vocab"],
-                     max_batch=batch, max_seq=max_seq, max_tokens=batch * prompt, kv_dtype=xh.FP16)
+                     max_batch=batch, max_seq=max_seq, max_tokens=batch * prompt, kv_dtype=xh.INT8 if kv_int8 else xh.FP16)
     ones = np.ones(c["hidden"], np.float32)
     layer_weights = []
     for l in range(c["layers"]):
@@ -245,6 +245,7 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--weights", choices=["int8", "uint4"], default="int8")
+    ap.add_argument("--kv", choices=["fp16", "int8"], default="fp16", help="KV cache format")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fusion", action="store_true", help="run RMSNorm / RoPE + cache append as their own kernels instead of inside the decode GEMVs")
     ap.add_argument("--persistent", action="store_true", help="run each decode step as the single persistent kernel (experimental)")
@@ -264,7 +265,7 @@ def main():
     kind = 0 if args.weights == "int8" else 1
     B = args.batch
     max_seq = args.prompt + args.warmup + args.steps + 1
-    model, layer_weights, lmw, host, shapes = build_model(xh, kind, B, max_seq, args.prompt)
+    model, layer_weights, lmw, host, shapes = build_model(xh, kind, B, max_seq, args.prompt, args.kv == "int8")
 
     if args.pmc_workload:
         pmc_workload(xh, layer_weights, B)
@@ -295,7 +296,8 @@ def main():
     # algorithmic HBM bytes of one decode step at the mean context of the timed region
     wbytes = sum(w.bytes() for w in layer_weights[0]) * CFG["layers"] + lmw.bytes()
     ctx = args.prompt + args.warmup + args.steps / 2.0
-    kv_bytes = CFG["layers"] * 2 * B * ctx * CFG["kv_heads"] * CFG["head"] * 2
+    kv_elem = (1 + 4.0 / CFG["head"]) if args.kv == "int8" else 2  # INT8 code + one fp32 scale per (token, head)
+    kv_bytes = CFG["layers"] * 2 * B * ctx * CFG["kv_heads"] * CFG["head"] * kv_elem
     step_bytes = wbytes + kv_bytes
 
     # dominant kernel: the M<=32 weight-only GEMV, in the three forms the decode step launches it
@@ -325,9 +327,9 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16 activations x %s weights, fp32 accumulate" % args.weights,
         "data": "synthetic",
-        "config": {"workload": "configs[3]: 32-layer Llama-2-7B-shape, %s weight-only, FP16 KV, batch %d, "
-                               "%d-token prompt, greedy decode" % (args.weights.upper(), B, args.prompt),
-                   "batch": B, "prompt": args.prompt, "weights": args.weights},
+        "config": {"workload": "configs[3]: 32-layer Llama-2-7B-shape, %s weight-only, %s KV, batch %d, "
+                               "%d-token prompt, greedy decode" % (args.weights.upper(), args.kv.upper(), B, args.prompt),
+                   "batch": B, "prompt": args.prompt, "weights": args.weights, "kv": args.kv},
         "ttft_ms": round(ttft_ms, 2),
         "step_hbm_bytes": int(step_bytes),
         "step_hbm_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),

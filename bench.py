@@ -1,7 +1,9 @@
 #!/usr/bin/env python3
 """Decode-throughput benchmark of the MI355X decoder-layer hot path.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--weights int8|uint4]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--weights int8|uint4] [--kv fp16|int8]
+                    [--eager | --no-fusion | --persistent]        (variants of the decode step)
+                    [--pmc-workload | --pmc-summary FETCH_CSV WRITE_CSV]   (hardware-counter traffic)
 
 Workload (BASELINE.json configs[3]): a 32-layer Llama-2-7B-shape model with random weights
 (vocab 32000, hidden 4096, intermediate 11008, 32 heads), weight-only INT8 (or UINT4)
@@ -10,8 +12,9 @@ decode.  One "step" is one decode step of the whole batch (one graph replay); th
 decoded tokens per second with every weight and the KV cache resident in HBM.
 
 One JSON line goes to stdout.  Besides the driver's fields it carries
-  roofline     the dominant kernel (the M<=32 weight-only GEMM) timed live with HIP events
-               on the launch stream, in algorithmic bytes per launch
+  roofline     the dominant kernel of the step (one of the three forms of the M<=32 weight-only
+               GEMV) timed live with HIP events on the launch stream, in algorithmic bytes per
+               launch; traffic = counter-measured HBM bytes per launch (profiles/)
   cpu_baseline this repository's CPU restatement of the reference's arithmetic (the oracle),
                timed on the host cores on a bounded sample of the same workload
 """

@@ -513,7 +513,8 @@ static int launch(const SkinnyParams &p, int kslices, hipStream_t stream) {
     SkinnyParams q = p;
     q.nblocks = blocks;
     if (NORM) {
-        const int cus = device_cu_count();
+        // one workgroup of 8 waves per CU, or two of 4
+        const int cus = device_cu_count() * (kslices <= 4 ? 2 : 1);
         blocks = blocks < cus ? blocks : cus;
     }
     hipLaunchKernelGGL((qgemm_skinny_kernel<KIND, NT, MT, U, NEED_SUM, KTAIL, NORM, ROPE>), dim3(blocks), dim3(64 * kslices), smem,
@@ -531,6 +532,18 @@ static int dispatch_tail(const SkinnyParams &p, int kslices, hipStream_t stream)
             return 2;
         }
         return launch<KIND, NT, MT, U, NEED_SUM, true, false>(p, kslices, stream);
+    }
+    if constexpr (MT == 1 && (KIND == XFTHIP_W_UINT4 || KIND == XFTHIP_W_NF4)) {
+        // 4-bit codes with the norm prologue: no activation registers are needed, so a batch can
+        // hold 4 tiles (512 k) like the INT8 kernel's, which doubles the bytes a wave has in flight
+        if (p.norm_x && p.KT % 4 == 0) {
+            int ks = (p.KT / 4 + 1) / 2;
+            ks = ks < 1 ? 1 : (ks > 8 ? 8 : ks);
+            if constexpr (NT == 2) {
+                if (p.rope) return launch<KIND, NT, MT, 4, NEED_SUM, false, true, true>(p, ks, stream);
+            }
+            if (!p.rope) return launch<KIND, NT, MT, 4, NEED_SUM, false, true, false>(p, ks, stream);
+        }
     }
     if constexpr (MT == 1 && NT == 2) {
         if (p.rope) {

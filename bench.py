@@ -5,7 +5,7 @@
                     [--eager | --no-fusion | --persistent]        (variants of the decode step)
                     [--pmc-workload | --pmc-summary FETCH_CSV WRITE_CSV]   (hardware-counter traffic)
 
-Workload (BASELINE.json configs[3]): a 32-layer Llama-2-7B-shape model with random weights
+Workload (configs[3] of the benchmark definition): a 32-layer Llama-2-7B-shape model with random weights
 (vocab 32000, hidden 4096, intermediate 11008, 32 heads), weight-only INT8 (or UINT4)
 per-channel codes against bf16 activations, FP16 KV cache, a 512-token prompt, then greedy
 decode.  One "step" is one decode step of the whole batch (one graph replay); the value is
@@ -182,8 +182,8 @@ def pmc_summary(fetch_csv, write_csv):
     sf, sw = copy_kib / fetch["copy"][0], copy_kib / write["copy"][0]
     print("HBM traffic per launch of the M=1 INT8 weight-only GEMV (qgemm_skinny_kernel), from hardware counters")
     print("commands (each its own run, as the counter blocks cannot be split over passes):")
-    print("  rocprofv3 --pmc FETCH_SIZE --output-format csv -d gpurun_out/pmc_fetch -- python3 bench.py --pmc-workload")
-    print("  rocprofv3 --pmc WRITE_SIZE --output-format csv -d gpurun_out/pmc_write -- python3 bench.py --pmc-workload")
+    print("  rocprofv3 --pmc FETCH_SIZE --output-format csv -d <outdir>/pmc_fetch -- python3 bench.py --pmc-workload")
+    print("  rocprofv3 --pmc WRITE_SIZE --output-format csv -d <outdir>/pmc_write -- python3 bench.py --pmc-workload")
     print("  python bench.py --pmc-summary <fetch counter_collection.csv> <write counter_collection.csv>")
     print("calibration: the library's plain copy kernel over %d KiB read %.1f (FETCH_SIZE) and wrote %.1f (WRITE_SIZE) counter units"
           % (copy_kib, fetch["copy"][0], write["copy"][0]))

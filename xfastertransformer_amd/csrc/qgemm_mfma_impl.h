@@ -392,6 +392,12 @@ static int dispatch_big_tile(const SkinnyParams &p, hipStream_t stream) {
     const long t_mid = (long)((n32 + 3) / 4) * ((p.M + 127) / 128);
     if (t_large >= cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
     if (t_mid >= cus) return launch_big<KIND, 1, 4, NEED_SUM>(p, stream);
+    // Few rows against a deep K (512 tokens x 4096 columns): 64-row tiles give one workgroup per CU
+    // whose k loop is a chain of load latencies; 32-row tiles put two on a CU, which overlap.
+    if constexpr (KIND != XFTHIP_W_BF16) {
+        const long t_small = (long)((n32 + 3) / 4) * ((p.M + 63) / 64);
+        if (t_small < 2 * cus) return launch_big<KIND, 1, 1, NEED_SUM>(p, stream);
+    }
     return launch_big<KIND, 1, 2, NEED_SUM>(p, stream);
 }
 

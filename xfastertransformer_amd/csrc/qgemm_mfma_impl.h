@@ -21,6 +21,17 @@ namespace {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
+// f32_to_bf16_ref() without its early returns: the same bits for every input (RNE on normals,
+// subnormals to signed zero, infinities kept, NaN quieted), as selects, so that the eight
+// conversions of an output chunk do not become eight divergent branch ladders.
+__device__ inline uint32_t f32_to_bf16_sel(float f) {
+    const uint32_t u = __float_as_uint(f), a = u & 0x7FFFFFFFu, top = u >> 16;
+    uint32_t r = (u + 0x7FFFu + (top & 1u)) >> 16;
+    r = a < 0x00800000u ? (top & 0x8000u) : r;
+    r = a >= 0x7F800000u ? (top | (a > 0x7F800000u ? 0x40u : 0u)) : r;
+    return r;
+}
+
 union MFrag {
     bf16x8 v;
     uint32_t u[4];
@@ -280,73 +291,163 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
 #undef XFT_FENCE
 
     // ---- epilogue: lane holds C[m0 + 32 mt + 8 (j/4) + 4 h + j%4][32 (n32_0 + t) + nl] ----
+    // A lane owns 16 rows of ONE column.  Finishing and storing every element from the accumulator
+    // registers costs a 64-bit index, bounds tests and a type conversion in 128 unrolled copies a
+    // lane, which made the epilogue of a 2048 x 4096 result take 23 us (the k loop of K = 4096: 75).
+    // Instead each wave drops one 32-row block of scaled results at a time, as fp32, into an LDS
+    // patch of its own (one ds_write with a constant offset per element), then walks the patch in
+    // 8-column chunks, consecutive lanes along a row: residual, conversion and 16-byte stores run
+    // in that short loop.
+    constexpr int OPITCH = 32 * WN * 4 + 32; // patch row pitch in bytes
+    __syncthreads(); // every wave is past its last read of the activation tiles
+    unsigned char *obuf = abuf_base + wave * (32 * OPITCH);
+    const bool c_wide = (((size_t)p.C | ((size_t)p.ldc * (p.c_dtype == XFTHIP_F32 ? 4 : 2))) & 15) == 0;
+    const bool res_wide = (((size_t)p.res | ((size_t)p.ldres * (p.res_dtype == XFTHIP_F32 ? 4 : 2))) & 15) == 0;
+    auto wave_sync = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    auto put_at = [&](float *base, int t_cols, int j, float x) { base[(8 * (j >> 2) + (j & 3)) * (OPITCH / 4) + t_cols] = x; };
+    // rows [32 m, 32 m + 32) of the patch, strip_cols wide, go to output columns col0 .. col_end - 1
+    auto flush = [&](auto epi_tag, int m, int col0, int strip_cols, int col_end) {
+        constexpr int EPI = decltype(epi_tag)::value;
+        constexpr bool HAS_RES = EPI == XFTHIP_EPI_RESMUL || EPI == XFTHIP_EPI_RESIDENTIAL || EPI == XFTHIP_EPI_RESEXT;
+        wave_sync();
+        const int cpr = strip_cols >> 3; // 8-column chunks a row: 2, 4 or 8
+        const int cpr_log2 = __builtin_ctz(cpr);
+        for (int idx = lane; idx < 32 * cpr; idx += 64) {
+            const int r = idx >> cpr_log2, ch = idx & (cpr - 1);
+            const int row = m0 + 32 * m + r;
+            const int c = col0 + 8 * ch;
+            if (row >= p.M || c >= col_end) continue;
+            const float *src = (const float *)(obuf + r * OPITCH) + 8 * ch;
+            const f32x4 lo = *(const f32x4 *)src, hi = *(const f32x4 *)(src + 4);
+            float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            const bool full = c + 8 <= col_end;
+            if constexpr (HAS_RES) {
+                const size_t ri = (size_t)row * p.ldres + c;
+                float rv[8];
+                if (full && res_wide) {
+                    if (p.res_dtype == XFTHIP_F32) {
+                        const f32x4 r0 = *(const f32x4 *)((const float *)p.res + ri), r1 = *(const f32x4 *)((const float *)p.res + ri + 4);
+                        rv[0] = r0[0], rv[1] = r0[1], rv[2] = r0[2], rv[3] = r0[3], rv[4] = r1[0], rv[5] = r1[1], rv[6] = r1[2], rv[7] = r1[3];
+                    } else {
+                        const u32x4 rr = *(const u32x4 *)((const uint16_t *)p.res + ri);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint16_t b0 = (uint16_t)rr[e], b1 = (uint16_t)(rr[e] >> 16);
+                            rv[2 * e] = p.res_dtype == XFTHIP_BF16 ? bf16_to_f32(b0) : fp16_bits_to_f32(b0);
+                            rv[2 * e + 1] = p.res_dtype == XFTHIP_BF16 ? bf16_to_f32(b1) : fp16_bits_to_f32(b1);
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) rv[e] = c + e < col_end ? load_as_f32(p.res, p.res_dtype, ri + e) : 0.0f;
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    if constexpr (EPI == XFTHIP_EPI_RESMUL) v[e] *= rv[e];
+                    if constexpr (EPI == XFTHIP_EPI_RESIDENTIAL) v[e] = v[e] + rv[e];
+                    if constexpr (EPI == XFTHIP_EPI_RESEXT) v[e] = fmaf(p.gamma, rv[e], v[e]);
+                }
+            }
+            const size_t ci = (size_t)row * p.ldc + c;
+            if (full && c_wide) {
+                if (p.c_dtype == XFTHIP_F32) {
+                    const f32x4 o0 = {v[0], v[1], v[2], v[3]}, o1 = {v[4], v[5], v[6], v[7]};
+                    *(f32x4 *)((float *)p.C + ci) = o0;
+                    *(f32x4 *)((float *)p.C + ci + 4) = o1;
+                } else {
+                    u32x4 o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t b0 = p.c_dtype == XFTHIP_BF16 ? f32_to_bf16_sel(v[2 * e]) : f32_to_fp16_bits(v[2 * e]);
+                        const uint32_t b1 = p.c_dtype == XFTHIP_BF16 ? f32_to_bf16_sel(v[2 * e + 1]) : f32_to_fp16_bits(v[2 * e + 1]);
+                        o[e] = b0 | (b1 << 16);
+                    }
+                    *(u32x4 *)((uint16_t *)p.C + ci) = o;
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (c + e < col_end) store_from_f32(p.C, p.c_dtype, ci + e, v[e]);
+            }
+        }
+        wave_sync();
+    };
     auto run_epilogue = [&](auto epi_tag) {
         constexpr int EPI = decltype(epi_tag)::value;
+        float s[WN], z[WN], bv[WN];
 #pragma unroll
         for (int t = 0; t < WN; ++t) {
             const int np = (n32_0 + t) * 32 + nl;
-            const bool nvalid = np < p.N;
-            float s = 1.0f, z = 0.0f, bv = 0.0f;
-            if constexpr (KIND != XFTHIP_W_BF16) s = p.scale[np < p.NTILES * 16 ? np : 0];
-            if constexpr (KIND == XFTHIP_W_UINT4 || (KIND == XFTHIP_W_INT8 && NEED_SUM)) z = p.zero ? p.zero[np < p.NTILES * 16 ? np : 0] : 0.0f;
-            if constexpr (EPI == XFTHIP_EPI_BIAS || EPI == XFTHIP_EPI_RESIDENTIAL || EPI == XFTHIP_EPI_RESEXT) bv = (p.bias && nvalid) ? p.bias[np] : 0.0f;
+            s[t] = 1.0f, z[t] = 0.0f, bv[t] = 0.0f;
+            if constexpr (KIND != XFTHIP_W_BF16) s[t] = p.scale[np < p.NTILES * 16 ? np : 0];
+            if constexpr (KIND == XFTHIP_W_UINT4 || (KIND == XFTHIP_W_INT8 && NEED_SUM)) z[t] = p.zero ? p.zero[np < p.NTILES * 16 ? np : 0] : 0.0f;
+            if constexpr (EPI == XFTHIP_EPI_BIAS || EPI == XFTHIP_EPI_RESIDENTIAL || EPI == XFTHIP_EPI_RESEXT) bv[t] = (p.bias && np < p.N) ? p.bias[np] : 0.0f;
+        }
+        float *put_base = (float *)(obuf + 4 * h * OPITCH) + nl;
 #pragma unroll
-            for (int m = 0; m < WM; ++m) {
+        for (int m = 0; m < WM; ++m) {
+#pragma unroll
+            for (int t = 0; t < WN; ++t) {
 #pragma unroll
                 for (int j = 0; j < 16; ++j) {
-                    const int row = m0 + 32 * m + 8 * (j >> 2) + 4 * h + (j & 3);
-                    if (row >= p.M || !nvalid) continue;
                     float x = acc[t][m][j];
                     if constexpr (KIND == XFTHIP_W_UINT4) {
-                        x = fmaf(s, x - 128.0f * accS[m][j], z * accS[m][j]);
+                        x = fmaf(s[t], x - 128.0f * accS[m][j], z[t] * accS[m][j]);
                     } else if constexpr (KIND == XFTHIP_W_INT8) {
-                        x = s * x;
-                        if constexpr (NEED_SUM) x = fmaf(z, accS[m][j], x);
+                        x = s[t] * x;
+                        if constexpr (NEED_SUM) x = fmaf(z[t], accS[m][j], x);
                     } else if constexpr (KIND == XFTHIP_W_NF4) {
-                        x = s * x;
+                        x = s[t] * x;
                     }
-                    if constexpr (EPI == XFTHIP_EPI_BIAS) x += bv;
+                    if constexpr (EPI == XFTHIP_EPI_BIAS || EPI == XFTHIP_EPI_RESIDENTIAL || EPI == XFTHIP_EPI_RESEXT) x += bv[t];
                     if constexpr (EPI == XFTHIP_EPI_SILU) x = silu_big(x);
                     if constexpr (EPI == XFTHIP_EPI_GELU) {
                         const float e = fast_exp(1.702f * x);
                         x = e / (e + 1.0f) * x;
                     }
-                    if constexpr (EPI == XFTHIP_EPI_RESMUL) x *= load_as_f32(p.res, p.res_dtype, (size_t)row * p.ldres + np);
-                    if constexpr (EPI == XFTHIP_EPI_RESIDENTIAL) x = (x + bv) + load_as_f32(p.res, p.res_dtype, (size_t)row * p.ldres + np);
-                    if constexpr (EPI == XFTHIP_EPI_RESEXT) x = fmaf(p.gamma, load_as_f32(p.res, p.res_dtype, (size_t)row * p.ldres + np), x + bv);
-                    store_from_f32(p.C, p.c_dtype, (size_t)row * p.ldc + np, x);
+                    put_at(put_base, 32 * t, j, x); // the residual operand joins in flush()
                 }
             }
+            flush(epi_tag, m, n32_0 * 32, 32 * WN, p.N);
         }
     };
     if (p.gateup) {
         // packed columns alternate 16 gate / 16 up: lanes nl < 16 hold gate, nl >= 16 the matching up
+        float s[WN], z[WN];
 #pragma unroll
         for (int t = 0; t < WN; ++t) {
             const int np = (n32_0 + t) * 32 + nl;
-            const int out_col = (n32_0 + t) * 16 + (nl & 15);
-            float s = 1.0f, z = 0.0f;
-            if constexpr (KIND != XFTHIP_W_BF16) s = p.scale[np < p.NTILES * 16 ? np : 0];
-            if constexpr (KIND == XFTHIP_W_UINT4 || (KIND == XFTHIP_W_INT8 && NEED_SUM)) z = p.zero ? p.zero[np < p.NTILES * 16 ? np : 0] : 0.0f;
+            s[t] = 1.0f, z[t] = 0.0f;
+            if constexpr (KIND != XFTHIP_W_BF16) s[t] = p.scale[np < p.NTILES * 16 ? np : 0];
+            if constexpr (KIND == XFTHIP_W_UINT4 || (KIND == XFTHIP_W_INT8 && NEED_SUM)) z[t] = p.zero ? p.zero[np < p.NTILES * 16 ? np : 0] : 0.0f;
+        }
+        // gate lanes write output column 16 t + nl of the strip; the up lanes' copies of the
+        // product land in the unused columns behind the strip, which flush() never reads
+        float *put_base = (float *)(obuf + 4 * h * OPITCH) + (nl < 16 ? nl : 16 * WN + (nl - 16));
 #pragma unroll
-            for (int m = 0; m < WM; ++m) {
+        for (int m = 0; m < WM; ++m) {
+#pragma unroll
+            for (int t = 0; t < WN; ++t) {
 #pragma unroll
                 for (int j = 0; j < 16; ++j) {
-                    const int row = m0 + 32 * m + 8 * (j >> 2) + 4 * h + (j & 3);
                     float x = acc[t][m][j];
                     if constexpr (KIND == XFTHIP_W_UINT4) {
-                        x = fmaf(s, x - 128.0f * accS[m][j], z * accS[m][j]);
+                        x = fmaf(s[t], x - 128.0f * accS[m][j], z[t] * accS[m][j]);
                     } else if constexpr (KIND == XFTHIP_W_INT8) {
-                        x = s * x;
-                        if constexpr (NEED_SUM) x = fmaf(z, accS[m][j], x);
+                        x = s[t] * x;
+                        if constexpr (NEED_SUM) x = fmaf(z[t], accS[m][j], x);
                     } else if constexpr (KIND == XFTHIP_W_NF4) {
-                        x = s * x;
+                        x = s[t] * x;
                     }
                     const float other = __shfl_xor(x, 16, 64); // gate <-> up partner
-                    if (nl < 16 && row < p.M && out_col < p.N / 2)
-                        store_from_f32(p.C, p.c_dtype, (size_t)row * p.ldc + out_col, other * silu_big(x));
+                    put_at(put_base, 16 * t, j, other * silu_big(x));
                 }
             }
+            flush(std::integral_constant<int, XFTHIP_EPI_NONE> {}, m, n32_0 * 16, 16 * WN, p.N / 2);
         }
         return;
     }
@@ -370,7 +471,9 @@ static int launch_big2(const SkinnyParams &p, hipStream_t stream) {
     const int nblocks_m = (p.M + ROWS - 1) / ROWS;
     const int nb8 = (nblocks_n + 7) / 8;
     const int blocks = nb8 * 8 * nblocks_m;
-    const size_t smem = 2 * ROWS * ROWB + (KIND == XFTHIP_W_NF4 ? 2048 : 0);
+    // the activation double buffer, reused after the k loop by the four waves' output patches
+    const size_t pipe = 2 * ROWS * ROWB, patches = 4 * 32 * (32 * WN * 4 + 32);
+    const size_t smem = (pipe > patches ? pipe : patches) + (KIND == XFTHIP_W_NF4 ? 2048 : 0);
     hipLaunchKernelGGL((qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL>), dim3(blocks), dim3(256), smem, stream, p, nblocks_n,
             nblocks_m);
     XFT_CHECK_HIP(hipGetLastError());

@@ -489,19 +489,35 @@ static int launch_big(const SkinnyParams &p, hipStream_t stream) {
 template <int KIND, bool NEED_SUM>
 static int dispatch_big_tile(const SkinnyParams &p, hipStream_t stream) {
     const int cus = device_cu_count();
-    // block tile = (4*WN*32 columns) x (WM*32 rows); take the largest that gives every CU a block
+    // Block tile = (4*WN*32 columns) x (WM*32 rows).  The choices below are the measured winners on
+    // 4096x{4096,12288,22016} and 11008x4096 weights at 512, 1024 and 2048 rows: 128-row tiles only
+    // pay once there are many row blocks to share a weight tile's trip through L2; below that,
+    // more and smaller workgroups per CU (whose k loops overlap) win by up to 1.5x.
     const int n32 = (p.NTILES + 1) / 2;
     const long t_large = (long)((n32 + 7) / 8) * ((p.M + 127) / 128);
     const long t_mid = (long)((n32 + 3) / 4) * ((p.M + 127) / 128);
-    if (t_large >= cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
-    if (t_mid >= cus) return launch_big<KIND, 1, 4, NEED_SUM>(p, stream);
-    // Few rows against a deep K (512 tokens x 4096 columns): 64-row tiles give one workgroup per CU
-    // whose k loop is a chain of load latencies; 32-row tiles put two on a CU, which overlap.
-    if constexpr (KIND != XFTHIP_W_BF16) {
-        const long t_small = (long)((n32 + 3) / 4) * ((p.M + 63) / 64);
-        if (t_small < 2 * cus) return launch_big<KIND, 1, 1, NEED_SUM>(p, stream);
+    const long t_small = (long)((n32 + 3) / 4) * ((p.M + 63) / 64);
+    if constexpr (KIND == XFTHIP_W_BF16) {
+        if (t_large >= cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
+        if (t_mid >= cus) return launch_big<KIND, 1, 4, NEED_SUM>(p, stream);
+        return launch_big<KIND, 1, 2, NEED_SUM>(p, stream);
+    } else if constexpr (KIND == XFTHIP_W_INT8) {
+        if (p.M > 1024) {
+            if (t_large >= 2 * cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
+            if (t_mid >= cus) return launch_big<KIND, 1, 4, NEED_SUM>(p, stream);
+        }
+    } else {
+        // 4-bit kinds: the 128 x 128 tile holds half the accumulators of the 128 x 256 one at the
+        // same occupancy (LDS for the 128-deep k tile) and never won
+        if (p.M > 512 && t_large >= cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
     }
-    return launch_big<KIND, 1, 2, NEED_SUM>(p, stream);
+    if constexpr (KIND != XFTHIP_W_BF16) {
+        // Few rows against a deep K (512 tokens x 4096 columns): 64-row tiles would leave one
+        // workgroup per CU, whose k loop is then a chain of load latencies; 32-row tiles put two
+        // on a CU.
+        if (t_small < 2 * cus) return launch_big<KIND, 1, 1, NEED_SUM>(p, stream);
+        return launch_big<KIND, 1, 2, NEED_SUM>(p, stream);
+    }
 }
 
 } // namespace

@@ -201,6 +201,35 @@ def gemm_f32(A, W, epi=EPI_NONE, bias=None, res=None, gamma=1.0):
     return Cm
 
 
+_DEQ_CACHE = {}
+
+
+def blas_gemm(w, A, epi=EPI_NONE, bias=None, res=None, gamma=1.0):
+    """A . deq(w) with numpy's sgemm on the weight dequantised once per QWeight object (kept until
+    clear_blas_cache()); epilogues NONE / BIAS / RESIDENTIAL / RESEXT as apply_epilogue has them."""
+    if isinstance(w, QWeight):
+        key = id(w)
+        if key not in _DEQ_CACHE:
+            _DEQ_CACHE[key] = (w, dequant(w))
+        Wd = _DEQ_CACHE[key][1]
+    else:
+        Wd = f32(w)
+    out = f32(A) @ Wd
+    if epi == EPI_BIAS:
+        out += f32(bias)
+    elif epi in (EPI_RESIDENTIAL, EPI_RESEXT):
+        if bias is not None:
+            out += f32(bias)
+        out += f32(res) if epi == EPI_RESIDENTIAL else np.float32(gamma) * f32(res)
+    elif epi != EPI_NONE:
+        raise ValueError("blas_gemm: epilogue %d not offered" % epi)
+    return out
+
+
+def clear_blas_cache():
+    _DEQ_CACHE.clear()
+
+
 def w8a8_quantize_rows(A):
     A = f32(A)
     M, K = A.shape
@@ -357,7 +386,7 @@ class LlamaLayerOracle:
     kernel error from the declared precision of the activation format."""
 
     def __init__(self, hidden, inter, q_heads, kv_heads, head, wqkv, wo, wgateup, wdown, ln1, ln2, kv_int8=0,
-                 batch=1, max_seq=256, eps=1e-6, rope_base=10000, max_pos=2048, rounding="fp32"):
+                 batch=1, max_seq=256, eps=1e-6, rope_base=10000, max_pos=2048, rounding="fp32", gemm="oracle"):
         self.hidden, self.inter, self.qh, self.kvh, self.D = hidden, inter, q_heads, kv_heads, head
         self.wqkv, self.wo, self.wgateup, self.wdown = wqkv, wo, wgateup, wdown
         self.ln1, self.ln2, self.eps = f32(ln1), f32(ln2), eps
@@ -365,11 +394,17 @@ class LlamaLayerOracle:
         self.vc = KVCache(kv_int8, batch, kv_heads, max_seq, head)
         self.cos, self.sin = rope_tables(head, max_pos, rope_base)
         self.rounding = rounding
+        # gemm="blas": C = A . deq(W) through the BLAS sgemm behind numpy on the weight dequantised
+        # once (orc_dequant), for shapes where the scalar orc_qgemm would take minutes; same closed
+        # form, fp32 accumulation in another order (tests/test_oracle_pins.py compares the two)
+        self.gemm = gemm
 
     def _r(self, x):
         return round_bf16(x) if self.rounding == "bf16" else x
 
     def _mm(self, w, a, **kw):
+        if self.gemm == "blas":
+            return blas_gemm(w, a, **kw)
         if isinstance(w, QWeight):
             return qgemm(w, a, **kw)
         return gemm_f32(a, w, **kw)
@@ -411,6 +446,7 @@ class LlamaModelOracle:
     def __init__(self, layers, embedding_fp16, final_norm, lm_head_f32, eps=1e-6):
         self.layers, self.emb, self.fn, self.lm, self.eps = layers, embedding_fp16, f32(final_norm), lm_head_f32, eps
         self.rounding = layers[0].rounding
+        self.gemm = layers[0].gemm
 
     def step(self, ids, B, S, past):
         x = from_fp16(self.emb[np.asarray(ids).reshape(-1)])
@@ -420,7 +456,7 @@ class LlamaModelOracle:
         xn = rmsnorm(last, self.fn, self.eps)
         if self.rounding == "bf16":
             xn = round_bf16(xn)
-        logits = gemm_f32(xn, self.lm)
+        logits = f32(xn) @ f32(self.lm) if self.gemm == "blas" else gemm_f32(xn, self.lm)
         return logits, argmax(logits)
 
 

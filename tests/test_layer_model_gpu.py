@@ -26,18 +26,30 @@ def _cos(a, b):
 
 
 def _check_layer_output(got, ref):
-    """Layer-output bar.  Cosine >= 0.9999 as stated.  The stated max-abs 2e-2 is below what a
-    bf16 activation format can represent at this shape: outputs reach |y| ~ 11 (bf16 quantum
-    0.0625 there) and the CPU oracle run with fp32 activations differs from the same oracle
-    with activations narrowed to bf16 at the GEMM inputs by max-abs 0.073 / rms 0.0135 (one
-    narrowing alone, the normalised input of the QKV GEMM, gives 0.053).  The bar applied is
-    therefore rms error <= 2e-2 and max-abs <= 2e-2 per unit of output rms, with a hard cap
-    of 0.1; the measured values are printed."""
+    """Bar against the oracle that keeps fp32 activations end to end (the reference's data flow).
+    Cosine >= 0.9999 as stated.  The stated max-abs 2e-2 is below what a bf16 activation format can
+    represent at this shape: outputs reach |y| ~ 11 (bf16 quantum 0.0625 there) and the CPU oracle
+    run with fp32 activations differs from the same oracle with activations narrowed to bf16 at the
+    GEMM inputs by max-abs 0.073 / rms 0.0135 (one narrowing alone, the normalised input of the QKV
+    GEMM, gives 0.053).  Against this oracle the bar is therefore rms error <= 2e-2 and max-abs <=
+    4e-2 per unit of output rms with a hard cap of 0.1; _check_layer_output_bf16_points() applies
+    the stated 2e-2 where it is meaningful."""
     err = np.abs(got - ref)
     rms_ref = float(np.sqrt((ref.astype(np.float64) ** 2).mean()))
     assert _cos(got, ref) >= 0.9999
     assert float(np.sqrt((err.astype(np.float64) ** 2).mean())) <= 2e-2
     assert err.max() <= min(0.1, 2e-2 * max(1.0, rms_ref) * 2.0), (err.max(), rms_ref)
+
+
+def _check_layer_output_bf16_points(got, ref16):
+    """The stated layer tolerance (max-abs 2e-2, cosine >= 0.9999) against the oracle that narrows
+    activations to bf16 at the same five hand-over points as the GPU pipeline: what is left is
+    kernel error (summation order, exp, fp16 probabilities) plus the occasional bf16 rounding of an
+    intermediate that lands on the other side."""
+    err = float(np.abs(got - ref16).max())
+    assert _cos(got, ref16) >= 0.9999
+    assert err <= 2e-2, err
+    return err
 
 
 def make_layer_weights(orc, rng, kind, hidden, inter, qh, kvh, D):
@@ -81,15 +93,16 @@ def test_llama7b_layer_prefill_then_decode(xh, orc, kind, kv_int8):
     print("prefill max-abs vs fp32-activation oracle", np.abs(got - e32).max(), "vs bf16-point oracle",
           np.abs(got - e16).max(), flush=True)
     _check_layer_output(got, e32)
-    _check_layer_output(got, e16)
-    worst = 0.0
+    _check_layer_output_bf16_points(got, e16)
+    worst = worst16 = 0.0
     for t in range(steps):
         x = orc.round_bf16(rng.standard_normal((1, hidden)))
         got = run(x, 1, S0 + t)
-        e32 = ref32.forward(x, 1, 1, S0 + t)
+        e32, e16 = ref32.forward(x, 1, 1, S0 + t), ref16.forward(x, 1, 1, S0 + t)
         worst = max(worst, float(np.abs(got - e32).max()))
         _check_layer_output(got, e32)
-    print("decode worst max-abs", worst, flush=True)
+        worst16 = max(worst16, _check_layer_output_bf16_points(got, e16))
+    print("decode worst max-abs vs fp32-activation oracle", worst, "vs bf16-point oracle", worst16, flush=True)
 
 
 def build_small_model(xh, orc, kind, seed, layers=2, hidden=512, inter=1408, qh=4, kvh=2, vocab=1000, B=2,
@@ -123,23 +136,27 @@ def test_small_model_greedy_decode_matches_oracle(xh, orc, kind):
     first, logits = model.prefill(ids, want_logits=True)
     elogits, efirst = ref.step(ids, B, S, 0)
     assert np.abs(logits - elogits).max() < 2e-2 and _cos(logits, elogits) >= 0.9999
-    # a token may only differ where the oracle's top-2 logits are closer than the tolerance
-    def same_or_tied(g, e, lg):
+    # The oracle is teacher-forced with the GPU's tokens, so every one of the steps is checked: the
+    # GPU's choice must be the oracle's best logit or within the logit tolerance of it.
+    def check_ids(g, lg):
+        same = 0
         for b in range(B):
-            if g[b] != e[b]:
-                assert abs(lg[b, g[b]] - lg[b, e[b]]) < 4e-2, (b, g[b], e[b])
-                return False
-        return True
-    assert same_or_tied(first, efirst, elogits)
+            best = int(lg[b].argmax())
+            assert lg[b, g[b]] >= lg[b, best] - 4e-2, (b, int(g[b]), best, float(lg[b, best] - lg[b, g[b]]))
+            same += int(g[b] == best)
+        return same
+    exact = check_ids(first, elogits)
     got = model.decode(steps, B)
-    cur = efirst
+    cur = first
+    verified = 0
     for t in range(steps):
-        elogits, nxt = ref.step(cur.reshape(B, 1), B, 1, S + t)
-        if not same_or_tied(got[t], nxt, elogits):
-            break  # sequences legitimately diverge after a near-tie
-        cur = nxt
-    else:
-        assert np.array_equal(got[-1], cur)
+        elogits, _ = ref.step(cur.reshape(B, 1), B, 1, S + t)
+        exact += check_ids(got[t], elogits)
+        cur = got[t]
+        verified += 1
+    assert verified == steps
+    print(f"greedy ids equal to the oracle's best in {exact} of {(steps + 1) * B} choices", flush=True)
+    assert exact >= (steps + 1) * B - 3
 
 
 @pytest.mark.parametrize("persistent", [False, True])

@@ -407,6 +407,14 @@ class Model:
             pass
 
 
+def argmax(logits_dev, rows, cols, stream=None):
+    """First-maximum argmax of fp32 logits [rows, cols] in device memory; returns host int32 [rows]."""
+    ids = DeviceBuffer(rows * 4)
+    check(lib.xfthip_argmax(logits_dev, rows, cols, ids.ptr, stream))
+    synchronize()
+    return ids.to_numpy(np.int32, (rows,))
+
+
 # ---------------------------------------------------------------------------- W8A8
 def w8a8_quantize_rows(A_dev, a_dtype, M, K, lda, stream=None):
     """Returns device buffers (qa [M, ldq], scale, zero, sum) and ldq."""

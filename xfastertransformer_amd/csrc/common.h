@@ -9,6 +9,7 @@
 #include <string>
 
 #include "../../include/xft_hip.h"
+#include "bf16_convert.h"
 
 namespace xfthip {
 
@@ -84,16 +85,8 @@ __host__ __device__ inline int logical_col(int np, int inter) {
 __device__ inline uint32_t f2u(float f) { return __float_as_uint(f); }
 __device__ inline float u2f(uint32_t u) { return __uint_as_float(u); }
 
-// fp32 -> bf16 exactly as the reference's bfloat16_t assignment (include/bfloat16.h:40-65):
-// RNE on normals, subnormals flushed to signed zero, NaN quieted.
-__device__ inline uint16_t f32_to_bf16_ref(float f) {
-    uint32_t u = f2u(f);
-    uint32_t a = u & 0x7FFFFFFFu;
-    if (a > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
-    if (a == 0x7F800000u) return (uint16_t)(u >> 16);
-    if (a < 0x00800000u) return (uint16_t)((u >> 16) & 0x8000u);
-    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
-}
+// fp32 -> bf16 exactly as the reference's bfloat16_t assignment (bf16_convert.h)
+__device__ inline uint16_t f32_to_bf16_ref(float f) { return f32_bits_to_bf16_ref(f2u(f)); }
 __device__ inline float bf16_to_f32(uint16_t b) { return u2f((uint32_t)b << 16); }
 
 __device__ inline uint16_t f32_to_fp16_bits(float f) {

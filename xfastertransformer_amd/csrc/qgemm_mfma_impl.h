@@ -21,16 +21,8 @@ namespace {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-// f32_to_bf16_ref() without its early returns: the same bits for every input (RNE on normals,
-// subnormals to signed zero, infinities kept, NaN quieted), as selects, so that the eight
-// conversions of an output chunk do not become eight divergent branch ladders.
-__device__ inline uint32_t f32_to_bf16_sel(float f) {
-    const uint32_t u = __float_as_uint(f), a = u & 0x7FFFFFFFu, top = u >> 16;
-    uint32_t r = (u + 0x7FFFu + (top & 1u)) >> 16;
-    r = a < 0x00800000u ? (top & 0x8000u) : r;
-    r = a >= 0x7F800000u ? (top | (a > 0x7F800000u ? 0x40u : 0u)) : r;
-    return r;
-}
+// f32_to_bf16_ref() as selects (bf16_convert.h): the same bits for every input
+__device__ inline uint32_t f32_to_bf16_sel(float f) { return f32_bits_to_bf16_sel(__float_as_uint(f)); }
 
 union MFrag {
     bf16x8 v;

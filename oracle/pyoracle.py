@@ -207,14 +207,25 @@ _DEQ_CACHE = {}
 def blas_gemm(w, A, epi=EPI_NONE, bias=None, res=None, gamma=1.0):
     """A . deq(w) with numpy's sgemm on the weight dequantised once per QWeight object (kept until
     clear_blas_cache()); epilogues NONE / BIAS / RESIDENTIAL / RESEXT as apply_epilogue has them."""
-    if isinstance(w, QWeight):
+    A = f32(A)
+    Wd = None
+    if not isinstance(w, QWeight):
+        Wd = f32(w)
+    elif A.shape[0] > 8 or w.kind not in (W_INT8, W_UINT4):
         key = id(w)
         if key not in _DEQ_CACHE:
             _DEQ_CACHE[key] = (w, dequant(w))
         Wd = _DEQ_CACHE[key][1]
+    if A.shape[0] <= 8 and isinstance(w, QWeight) and w.kind in (W_INT8, W_UINT4):
+        # few rows: stream the integer codes once (a quarter or an eighth of the fp32 bytes)
+        out = np.empty((A.shape[0], w.N), np.float32)
+        rc = lib.orc_qgemm_skinny(w.kind, A.shape[0], w.N, w.K, p(A), w.K, p(w.q), p(w.scale), p(w.zero), p(out), w.N)
+        assert rc == 0
+    elif A.shape[0] <= 8:
+        # one threaded sgemv per row (the skinny sgemm of the BLAS behind numpy runs on one core)
+        out = np.stack([a @ Wd for a in A])
     else:
-        Wd = f32(w)
-    out = f32(A) @ Wd
+        out = A @ Wd
     if epi == EPI_BIAS:
         out += f32(bias)
     elif epi in (EPI_RESIDENTIAL, EPI_RESEXT):

@@ -379,6 +379,54 @@ ORC_API void orc_qgemm_f64(int kind, int M, int N, int K, const float *A, int ld
         }
 }
 
+/* The same closed form for a few activation rows (M <= 8) at full-model sizes, where orc_qgemm's
+ * per-element dequantisation would take a second per call: C = A * (scale*q + zero) evaluated as
+ * scale * (A * q) + zero * sum(A), the integer codes streamed once with a vectorisable inner loop.
+ * fp32 accumulation in k order; differs from orc_qgemm only in where the scale multiplies
+ * (tests/test_oracle_pins.py compares the two).  INT8 and UINT4 only. */
+ORC_API int orc_qgemm_skinny(int kind, int M, int N, int K, const float *A, int lda, const void *q, const float *scale,
+        const float *zero, float *C, int ldc) {
+    enum { NB = 128, MMAX = 8 };
+    if (M > MMAX || (kind != ORC_W_INT8 && kind != ORC_W_UINT4) || (N & 1)) return 1;
+    float sumA[MMAX];
+    for (int m = 0; m < M; ++m) {
+        float s = 0.0f;
+        for (int64_t k = 0; k < K; ++k) s += A[(int64_t)m * lda + k];
+        sumA[m] = s;
+    }
+#pragma omp parallel for schedule(static)
+    for (int n0 = 0; n0 < N; n0 += NB) {
+        float acc[MMAX][NB];
+        float w[NB];
+        const int nb = (N - n0 < NB) ? N - n0 : NB;
+        for (int m = 0; m < M; ++m)
+            for (int j = 0; j < nb; ++j) acc[m][j] = 0.0f;
+        for (int64_t k = 0; k < K; ++k) {
+            if (kind == ORC_W_INT8) {
+                const int8_t *row = (const int8_t *)q + k * N + n0;
+#pragma omp simd
+                for (int j = 0; j < nb; ++j) w[j] = (float)row[j];
+            } else {
+                const uint8_t *row = (const uint8_t *)q + (k * N + n0) / 2;
+#pragma omp simd
+                for (int j = 0; j < nb / 2; ++j) {
+                    w[2 * j] = (float)(row[j] & 0xF);
+                    w[2 * j + 1] = (float)(row[j] >> 4);
+                }
+            }
+            for (int m = 0; m < M; ++m) {
+                const float a = A[(int64_t)m * lda + k];
+#pragma omp simd
+                for (int j = 0; j < nb; ++j) acc[m][j] += a * w[j];
+            }
+        }
+        for (int m = 0; m < M; ++m)
+            for (int j = 0; j < nb; ++j)
+                C[(int64_t)m * ldc + n0 + j] = scale[n0 + j] * acc[m][j] + (zero ? zero[n0 + j] * sumA[m] : 0.0f);
+    }
+    return 0;
+}
+
 /* Plain fp32 GEMM against an fp32 [K,N] weight, same accumulation order. */
 ORC_API void orc_gemm_f32(int M, int N, int K, const float *A, int lda, const float *W, int ldw, float *C, int ldc,
         int epi, const float *bias, const float *res, int ldres, float gamma) {

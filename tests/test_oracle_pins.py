@@ -538,13 +538,19 @@ def test_layer_and_model_oracle_vs_float64_numpy(kind, gemm):
     orc.clear_blas_cache()
 
 
-def test_blas_gemm_matches_scalar_oracle_gemm():
+@pytest.mark.parametrize("M", [1, 3, 9])
+def test_blas_gemm_matches_scalar_oracle_gemm(M):
+    """Both fast GEMM routes of the full-size model oracle (numpy sgemm on the dequantised weight for
+    many rows, orc_qgemm_skinny on the integer codes for up to 8) against the scalar orc_qgemm."""
     rng = np.random.default_rng(302)
-    M, K, N = 9, 640, 112
+    K, N = 640, 112
     A = orc.round_bf16(rng.standard_normal((M, K)))
     bias, res = rng.standard_normal(N).astype(np.float32), rng.standard_normal((M, N)).astype(np.float32)
     for kind in (orc.W_INT8, orc.W_UINT4, orc.W_NF4):
         w = orc.quantize(kind, (rng.standard_normal((K, N)) * 0.02).astype(np.float32))
+        if kind == orc.W_INT8:
+            w.zero = (rng.standard_normal(N) * 0.01).astype(np.float32)
+        assert np.abs(orc.qgemm(w, A)).max() > 0.5
         for epi, kw in ((orc.EPI_NONE, {}), (orc.EPI_BIAS, dict(bias=bias)), (orc.EPI_RESIDENTIAL, dict(res=res)),
                         (orc.EPI_RESIDENTIAL, dict(res=res, bias=bias)), (orc.EPI_RESEXT, dict(res=res, gamma=0.3))):
             assert np.abs(orc.blas_gemm(w, A, epi, **kw) - orc.qgemm(w, A, epi, **kw)).max() < 1e-4

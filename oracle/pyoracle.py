@@ -397,7 +397,8 @@ class LlamaLayerOracle:
     kernel error from the declared precision of the activation format."""
 
     def __init__(self, hidden, inter, q_heads, kv_heads, head, wqkv, wo, wgateup, wdown, ln1, ln2, kv_int8=0,
-                 batch=1, max_seq=256, eps=1e-6, rope_base=10000, max_pos=2048, rounding="fp32", gemm="oracle"):
+                 batch=1, max_seq=256, eps=1e-6, rope_base=10000, max_pos=2048, rounding="fp32", gemm="oracle",
+                 prefill_attention="flash"):
         self.hidden, self.inter, self.qh, self.kvh, self.D = hidden, inter, q_heads, kv_heads, head
         self.wqkv, self.wo, self.wgateup, self.wdown = wqkv, wo, wgateup, wdown
         self.ln1, self.ln2, self.eps = f32(ln1), f32(ln2), eps
@@ -409,6 +410,11 @@ class LlamaLayerOracle:
         # once (orc_dequant), for shapes where the scalar orc_qgemm would take minutes; same closed
         # form, fp32 accumulation in another order (tests/test_oracle_pins.py compares the two)
         self.gemm = gemm
+        # prefill_attention="cache": a prefill from position 0 also takes the route the reference
+        # takes when a past exists (crossAttnByHead: rows go to the FP16/INT8 cache first, fp32 scores
+        # and probabilities over the cache) instead of the flash-style path, which narrows K, V and
+        # the probabilities to bf16.  This is the precision the GPU attention kernel works at.
+        self.prefill_attention = prefill_attention
 
     def _r(self, x):
         return round_bf16(x) if self.rounding == "bf16" else x
@@ -436,7 +442,7 @@ class LlamaLayerOracle:
         v = np.ascontiguousarray(qkv[:, qcols + kvcols:])
         q = self._r(q)
         scale = 1.0 / np.sqrt(self.D)
-        if past == 0 and S > 1:
+        if past == 0 and S > 1 and self.prefill_attention == "flash":
             att = flash_prefill(q, to_bf16(k), to_bf16(v), self.qh, self.kvh, self.D, [S] * B, [0] * B, scale)
             for b in range(B):
                 self.kc.store(b, 0, k[b * S:(b + 1) * S])

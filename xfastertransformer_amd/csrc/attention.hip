@@ -27,16 +27,29 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnParams p) {
     attn_unit<INT8, 4>(p, blockIdx.x, blockIdx.y % p.kv.H, blockIdx.y / p.kv.H, blockIdx.z, lds, [] { __syncthreads(); });
 }
 
-static float *g_ws = nullptr;
-static unsigned int *g_tickets = nullptr;
+// Split-KV merge workspace: `slots` partial-result slots of kSlotFloats floats and one ticket per
+// column group.  The library keeps one for plain xfthip_attention calls (allocated on first use);
+// a model owns its own, so that two models on two streams never share partials or tickets.
+static AttnWorkspace g_shared_ws;
+
+int attention_workspace_create(AttnWorkspace *w, int slots) {
+    w->ws = nullptr, w->tickets = nullptr, w->slots = 0;
+    XFT_CHECK_HIP(hipMalloc((void **)&w->ws, (size_t)slots * kSlotFloats * sizeof(float)));
+    XFT_CHECK_HIP(hipMalloc((void **)&w->tickets, (size_t)slots * sizeof(unsigned int)));
+    XFT_CHECK_HIP(hipMemset(w->tickets, 0, (size_t)slots * sizeof(unsigned int)));
+    XFT_CHECK_HIP(hipDeviceSynchronize());
+    w->slots = slots;
+    return 0;
+}
+
+void attention_workspace_destroy(AttnWorkspace *w) {
+    if (w->ws) (void)hipFree(w->ws);
+    if (w->tickets) (void)hipFree(w->tickets);
+    w->ws = nullptr, w->tickets = nullptr, w->slots = 0;
+}
 
 int attention_workspace_init() {
-    if (g_ws == nullptr) XFT_CHECK_HIP(hipMalloc((void **)&g_ws, (size_t)kWsSlots * kSlotFloats * sizeof(float)));
-    if (g_tickets == nullptr) {
-        XFT_CHECK_HIP(hipMalloc((void **)&g_tickets, (size_t)kWsSlots * sizeof(unsigned int)));
-        XFT_CHECK_HIP(hipMemset(g_tickets, 0, (size_t)kWsSlots * sizeof(unsigned int)));
-        XFT_CHECK_HIP(hipDeviceSynchronize());
-    }
+    if (g_shared_ws.slots == 0) return attention_workspace_create(&g_shared_ws, kWsSlots);
     return 0;
 }
 
@@ -45,9 +58,12 @@ int attention_workspace_init() {
 using namespace xfthip;
 
 // len_hint: upper bound of the visible sequence length when the positions live in device memory
-// (0 = unknown, the cache length is assumed); it only steers the split count
+// (0 = unknown, the cache length is assumed); it only steers the split count.
+// wsp: the workspace to merge splits through (nullptr = the library's shared one, allocated on first
+// use).  strict: fail instead of lowering the split count when the workspace is too small.
 int xfthip::attention_launch(xfthip_kvcache_t c, const void *q, int qStride, void *out, int oStride, int out_dtype, int B, int S,
-        int qHeads, float scale, int past, const int *past_dev, int len_hint, hipStream_t stream) {
+        int qHeads, float scale, int past, const int *past_dev, int len_hint, hipStream_t stream, const AttnWorkspace *wsp,
+        bool strict) {
     XFT_REQUIRE(c && q && out, "xfthip_attention: null argument");
     XFT_REQUIRE(B > 0 && B <= c->kv.B, "xfthip_attention: batch %d exceeds cache batch %d", B, c->kv.B);
     XFT_REQUIRE(S > 0 && qHeads > 0 && qHeads % c->kv.H == 0, "xfthip_attention: bad S=%d or qHeads=%d (kvHeads=%d)", S, qHeads,
@@ -78,12 +94,21 @@ int xfthip::attention_launch(xfthip_kvcache_t c, const void *q, int qStride, voi
     // when the real one lives in device memory
     const int len = past_dev ? ((len_hint > 0 && len_hint < c->maxSeq) ? len_hint : c->maxSeq) : past + S;
     const int wgs = B * c->kv.H * p.CG;
-    const int nsplit = attention_split_count(len, wgs);
+    int nsplit = attention_split_count(len, wgs);
+    if (nsplit > 1) {
+        if (wsp == nullptr) {
+            if (int rc = attention_workspace_init()) return rc;
+            wsp = &g_shared_ws;
+        }
+        if ((size_t)wgs * nsplit > (size_t)wsp->slots) {
+            XFT_REQUIRE(!strict, "xfthip_attention: %d column groups x %d sequence splits need %zu partial-result slots, the workspace holds %d",
+                    wgs, nsplit, (size_t)wgs * nsplit, wsp->slots);
+            while (nsplit > 1 && (size_t)wgs * nsplit > (size_t)wsp->slots) --nsplit;
+        }
+    }
     p.nsplit = nsplit;
-    if (nsplit > 1)
-        if (int rc = attention_workspace_init()) return rc;
-    p.ws = g_ws;
-    p.tickets = g_tickets;
+    p.ws = wsp ? wsp->ws : nullptr;
+    p.tickets = wsp ? wsp->tickets : nullptr;
     dim3 grid(nsplit, c->kv.H * p.CG, B);
     if (c->kv.int8)
         hipLaunchKernelGGL(attn_kernel<true>, grid, dim3(256), 0, stream, p);
@@ -106,5 +131,6 @@ int xfthip::attention_split_count(int len, int units) {
 
 extern "C" int xfthip_attention(xfthip_kvcache_t c, const void *q, int qStride, void *out, int oStride, int out_dtype,
         int B, int S, int qHeads, float scale, int past, const int *past_dev, xfthip_stream_t stream) {
-    return attention_launch(c, q, qStride, out, oStride, out_dtype, B, S, qHeads, scale, past, past_dev, 0, (hipStream_t)stream);
+    return attention_launch(c, q, qStride, out, oStride, out_dtype, B, S, qHeads, scale, past, past_dev, 0, (hipStream_t)stream,
+            nullptr, false);
 }

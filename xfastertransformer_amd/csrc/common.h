@@ -138,13 +138,24 @@ __device__ inline void dev_drain() {
 __device__ inline float fast_exp(float x) { return __expf(x); }
 
 int device_cu_count();
-// allocates the split-KV merge workspace of the attention kernel (idempotent; must not run
-// during stream capture)
+// Split-KV merge workspace of the attention kernel: partial (max, sum, output) slots and one
+// ticket per column group (tickets are zero between launches).
+struct AttnWorkspace {
+    float *ws = nullptr;
+    unsigned int *tickets = nullptr;
+    int slots = 0;
+};
+int attention_workspace_create(AttnWorkspace *w, int slots); // allocates; not for use during stream capture
+void attention_workspace_destroy(AttnWorkspace *w);
+// allocates the library's shared workspace (idempotent; must not run during stream capture)
 int attention_workspace_init();
 // the attention launch behind xfthip_attention, with a length hint for callers whose positions live
-// in device memory, and the split count it picks for `units` (batch x kv head x column group) workgroups
+// in device memory, the workspace to use (nullptr = the shared one) and whether a workspace that is
+// too small is an error (otherwise the split count is lowered to fit)
 int attention_launch(xfthip_kvcache_t c, const void *q, int qStride, void *out, int oStride, int out_dtype, int B, int S,
-        int qHeads, float scale, int past, const int *past_dev, int len_hint, hipStream_t stream);
+        int qHeads, float scale, int past, const int *past_dev, int len_hint, hipStream_t stream, const AttnWorkspace *wsp = nullptr,
+        bool strict = false);
+// the split count the launch picks for `units` (batch x kv head x column group) workgroups
 int attention_split_count(int len, int units);
 
 } // namespace xfthip

@@ -120,6 +120,7 @@ struct xfthip_model {
     // INT8 KV: the first-token pass attends over unquantised keys/values, as the reference's
     // flash path does on its bf16 copies (src/layers/attention.h:1121-1188); they live here
     xfthip_kvcache_t prefill_cache = nullptr;
+    AttnWorkspace attn_ws; // split-KV partials and tickets of this model's attention launches
     float *cosT = nullptr, *sinT = nullptr;
     // scratch
     uint16_t *xn = nullptr, *qkv = nullptr, *att = nullptr, *h = nullptr;
@@ -319,7 +320,7 @@ static int attention_block(xfthip_model *m, int idx, const float *x_in, int in_s
         attend = m->prefill_cache;
     }
     if ((rc = attention_launch(attend, m->qkv, qkv_cols, m->att, qcols, XFTHIP_BF16, B, S, c.q_heads, 1.0f / sqrtf((float)c.head_size), past,
-                 past_dev, past_dev ? m->len_hint : 0, st)))
+                 past_dev, past_dev ? m->len_hint : 0, st, &m->attn_ws)))
         return rc;
     return xfthip_gemm(L.o, T, m->att, qcols, x_out, out_stride, XFTHIP_F32, XFTHIP_EPI_RESIDENTIAL, L.o_bias, x_in, in_stride,
             XFTHIP_F32, 1.0f, st);
@@ -419,7 +420,7 @@ int xfthip_model_create(const xfthip_model_config *cfg, xfthip_model_t *out) {
     };
     for (int l = 0; l < c.layers; ++l)
         if (int rc = xfthip_kvcache_create(c.kv_dtype, c.max_batch, c.kv_heads, c.max_seq, c.head_size, &m->caches[l])) return fail(rc);
-    if (int rc = attention_workspace_init()) return fail(rc);
+    if (int rc = attention_workspace_create(&m->attn_ws, kWsSlots)) return fail(rc);
     if (c.kv_dtype == XFTHIP_INT8)
         if (int rc = xfthip_kvcache_create(XFTHIP_FP16, c.max_batch, c.kv_heads, c.max_seq, c.head_size, &m->prefill_cache)) return fail(rc);
     if (int rc = xfthip_rope_tables_create(c.head_size, c.max_pos_embed, c.rope_base, 1.0f, &m->cosT, &m->sinT)) return fail(rc);
@@ -453,6 +454,7 @@ int xfthip_model_destroy(xfthip_model_t m) {
     if (m->graph) (void)hipGraphExecDestroy(m->graph);
     for (auto c : m->caches) xfthip_kvcache_destroy(c);
     xfthip_kvcache_destroy(m->prefill_cache);
+    attention_workspace_destroy(&m->attn_ws);
     for (auto &L : m->layers) {
         if (L.ln1) (void)hipFree(L.ln1);
         if (L.ln2) (void)hipFree(L.ln2);
@@ -527,6 +529,12 @@ int xfthip_model_set_head(xfthip_model_t m, const uint16_t *embedding_fp16_host,
     XFT_REQUIRE(c.vocab > 0, "xfthip_model_set_head: model was created without a vocabulary");
     XFT_REQUIRE(lm_head->pw.K == c.hidden && lm_head->pw.N == c.vocab, "xfthip_model_set_head: lm_head is [%d,%d], expected [%d,%d]",
             lm_head->pw.K, lm_head->pw.N, c.hidden, c.vocab);
+    // a captured decode step holds the addresses of the buffers replaced below
+    if (m->graph) {
+        XFT_CHECK_HIP(hipDeviceSynchronize());
+        (void)hipGraphExecDestroy(m->graph);
+        m->graph = nullptr;
+    }
     if (m->embedding) (void)hipFree(m->embedding);
     m->embedding = nullptr;
     const size_t eb = (size_t)c.vocab * c.hidden * 2;

@@ -250,6 +250,20 @@ int xfthip_rope_kvstore(xfthip_kvcache_t c, void *qkv, int dtype, int stride, in
 int xfthip_attention(xfthip_kvcache_t c, const void *q, int qStride, void *out, int oStride, int out_dtype, int B,
         int S, int qHeads, float scale, int past, const int *past_dev, xfthip_stream_t stream);
 
+/*
+ * xfthip_attention for callers that cannot allocate (code under HIP graph capture, serving loops
+ * and harnesses that forbid hipMalloc): same arguments, same kernel and same split of the KV
+ * sequence, but the partial results and tickets of the split merge live in a statically allocated
+ * device array of the library (1024 partial-result slots, about 8.5 MB per GPU, held until the
+ * process ends) instead of the workspace xfthip_attention allocates on first use.  The call
+ * allocates and frees nothing.  A shape whose split needs more than 1024 slots (column groups
+ * B * kvHeads * ceil(S * qHeads / kvHeads / 16) times sequence splits) is rejected with an error
+ * that says so.  All calls on one GPU share the array: calls that overlap on one GPU (two streams)
+ * race; calls on one stream do not.  No counterpart in the reference.
+ */
+int xfthip_attention_static(xfthip_kvcache_t c, const void *q, int qStride, void *out, int oStride, int out_dtype, int B,
+        int S, int qHeads, float scale, int past, const int *past_dev, xfthip_stream_t stream);
+
 
 /* ---- decoder layers and the model driver -------------------------------------------- */
 typedef struct xfthip_model *xfthip_model_t;

@@ -309,6 +309,13 @@ def attention(cache, q_dev, q_stride, out_dev, o_stride, out_dtype, B, S, q_head
                                C.c_float(scale), past, past_dev, stream))
 
 
+def attention_static(cache, q_dev, q_stride, out_dev, o_stride, out_dtype, B, S, q_heads, scale, past, past_dev=None,
+                     stream=None):
+    """xfthip_attention through the statically allocated split workspace (allocates nothing)."""
+    check(lib.xfthip_attention_static(cache.h, q_dev, q_stride, out_dev, o_stride, out_dtype, B, S, q_heads,
+                                      C.c_float(scale), past, past_dev, stream))
+
+
 # ---------------------------------------------------------------------------- model driver
 class ModelConfig(C.Structure):
     _fields_ = [("layers", C.c_int), ("hidden", C.c_int), ("intermediate", C.c_int), ("q_heads", C.c_int),

@@ -17,6 +17,8 @@
 // INT8 caches are widened to fp16 in registers (exact); the per-token key scale multiplies
 // the score column, the value scale multiplies the probability (gemm_kernel_ext.cpp:471-500,
 // gemm_kernel_ext2.cpp:75-91).
+#include <mutex>
+
 #include "attention_dev.h"
 
 namespace xfthip {
@@ -50,6 +52,36 @@ void attention_workspace_destroy(AttnWorkspace *w) {
 
 int attention_workspace_init() {
     if (g_shared_ws.slots == 0) return attention_workspace_create(&g_shared_ws, kWsSlots);
+    return 0;
+}
+
+// ---- statically allocated workspace of xfthip_attention_static ---------------------------------
+// Device memory that exists from the moment the code object is loaded: callers that must not
+// allocate (stream capture, serving loops that forbid hipMalloc) get the split-KV partials and the
+// tickets from here.  Each device holds its own copy at its own address; in host code the array's
+// name is only a handle for hipGetSymbolAddress, never a pointer to pass to a kernel.
+constexpr int kStaticSlots = 1024;
+constexpr size_t kStaticTicketOffset = (size_t)kStaticSlots * kSlotFloats * sizeof(float);
+static __device__ __align__(256) unsigned char scratch[kStaticTicketOffset + (size_t)kStaticSlots * sizeof(unsigned int)];
+
+constexpr int kMaxDevices = 64;
+static void *g_scratch_ptr[kMaxDevices] = {};
+static std::mutex g_scratch_mu;
+
+// Resolves (once per device, with that device current) the device address of `scratch` and clears
+// the tickets.  Allocates nothing.  Called by xfthip_init and by the entry point's first call on a device.
+int attention_static_scratch_init() {
+    int dev = -1;
+    XFT_CHECK_HIP(hipGetDevice(&dev));
+    XFT_REQUIRE(dev >= 0 && dev < kMaxDevices, "attention_static_scratch_init: device index %d out of range", dev);
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (g_scratch_ptr[dev] != nullptr) return 0;
+    void *ptr = nullptr;
+    XFT_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    XFT_REQUIRE(ptr != nullptr, "attention_static_scratch_init: no device address for the static scratch");
+    XFT_CHECK_HIP(hipMemset((unsigned char *)ptr + kStaticTicketOffset, 0, (size_t)kStaticSlots * sizeof(unsigned int)));
+    XFT_CHECK_HIP(hipDeviceSynchronize());
+    g_scratch_ptr[dev] = ptr;
     return 0;
 }
 
@@ -101,7 +133,9 @@ int xfthip::attention_launch(xfthip_kvcache_t c, const void *q, int qStride, voi
             wsp = &g_shared_ws;
         }
         if ((size_t)wgs * nsplit > (size_t)wsp->slots) {
-            XFT_REQUIRE(!strict, "xfthip_attention: %d column groups x %d sequence splits need %zu partial-result slots, the workspace holds %d",
+            XFT_REQUIRE(!strict,
+                    "xfthip_attention_static: %d column groups x %d sequence splits need %zu partial-result slots, the static "
+                    "scratch holds %d; use xfthip_attention for this shape",
                     wgs, nsplit, (size_t)wgs * nsplit, wsp->slots);
             while (nsplit > 1 && (size_t)wgs * nsplit > (size_t)wsp->slots) --nsplit;
         }
@@ -133,4 +167,19 @@ extern "C" int xfthip_attention(xfthip_kvcache_t c, const void *q, int qStride, 
         int B, int S, int qHeads, float scale, int past, const int *past_dev, xfthip_stream_t stream) {
     return attention_launch(c, q, qStride, out, oStride, out_dtype, B, S, qHeads, scale, past, past_dev, 0, (hipStream_t)stream,
             nullptr, false);
+}
+
+extern "C" int xfthip_attention_static(xfthip_kvcache_t c, const void *q, int qStride, void *out, int oStride, int out_dtype,
+        int B, int S, int qHeads, float scale, int past, const int *past_dev, xfthip_stream_t stream) {
+    int dev = -1;
+    XFT_CHECK_HIP(hipGetDevice(&dev));
+    XFT_REQUIRE(dev >= 0 && dev < kMaxDevices, "xfthip_attention_static: device index %d out of range", dev);
+    if (g_scratch_ptr[dev] == nullptr)
+        if (int rc = attention_static_scratch_init()) return rc;
+    AttnWorkspace w;
+    w.ws = (float *)g_scratch_ptr[dev];
+    w.tickets = (unsigned int *)((unsigned char *)g_scratch_ptr[dev] + kStaticTicketOffset);
+    w.slots = kStaticSlots;
+    return attention_launch(c, q, qStride, out, oStride, out_dtype, B, S, qHeads, scale, past, past_dev, 0, (hipStream_t)stream, &w,
+            true);
 }

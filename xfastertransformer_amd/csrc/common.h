@@ -149,6 +149,9 @@ int attention_workspace_create(AttnWorkspace *w, int slots); // allocates; not f
 void attention_workspace_destroy(AttnWorkspace *w);
 // allocates the library's shared workspace (idempotent; must not run during stream capture)
 int attention_workspace_init();
+// resolves the device address of the statically allocated workspace behind xfthip_attention_static
+// for the current device (idempotent, allocates nothing)
+int attention_static_scratch_init();
 // the attention launch behind xfthip_attention, with a length hint for callers whose positions live
 // in device memory, the workspace to use (nullptr = the shared one) and whether a workspace that is
 // too small is an error (otherwise the split count is lowered to fit)

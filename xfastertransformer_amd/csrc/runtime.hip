@@ -56,7 +56,9 @@ int xfthip_init(int device) {
             "xfthip_init: this library is built for gfx950 only, device %d is %s", device, prop.gcnArchName);
     g_device = device;
     g_cus = prop.multiProcessorCount;
-    return 0;
+    // the statically allocated attention workspace: resolve its address on this device now, so
+    // that xfthip_attention_static never has to during a stream capture
+    return attention_static_scratch_init();
 }
 
 int xfthip_finalize(void) {

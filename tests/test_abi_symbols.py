@@ -39,7 +39,7 @@ def test_c_abi_exports_every_declared_symbol():
 
 
 @pytest.mark.skipif(not os.path.exists(LIB_LAYERS), reason="host library not built")
-def test_host_layer_exports_reference_entry_points():
+def test_host_layer_exports_reference_entry_points(tmp_path):
     out = subprocess.check_output(["nm", "-DC", "--defined-only", LIB_LAYERS], text=True)
     for fn in ("xft::invokeLayerLLaMA(", "xft::invokeAttentionLLaMA(", "xft::invokeMLPLLaMA(", "xft::invokeGemm(",
                "xft::invokeRmsNorm(", "xft::invokeRotaryEmbedding("):
@@ -69,10 +69,8 @@ def test_host_layer_exports_reference_entry_points():
         return 0;
     }
     '''
-    work = os.path.join(ROOT, "_work")
-    os.makedirs(work, exist_ok=True)
-    cpp = os.path.join(work, "link_check.cpp")
-    exe = os.path.join(work, "link_check")
+    cpp = str(tmp_path / "link_check.cpp")
+    exe = str(tmp_path / "link_check")
     open(cpp, "w").write(src)
     subprocess.check_call(["g++", "-std=c++17", "-I" + os.path.join(ROOT, "include"), cpp, "-o", exe, "-L" + PKG,
                            "-lxft_layers", "-lxft_hip", "-Wl,-rpath," + PKG])

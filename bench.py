@@ -3,6 +3,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--weights int8|uint4] [--kv fp16|int8]
                     [--eager | --no-fusion | --persistent]        (variants of the decode step)
+                    [--no-extras] [--no-cpu-baseline]
+                    [--prefill-gemm | --attention | --moe]        (one of the extra measurements alone, one JSON line)
                     [--pmc-workload | --pmc-summary FETCH_CSV WRITE_CSV]   (hardware-counter traffic)
 
 Workload (configs[3] of the benchmark definition): a 32-layer Llama-2-7B-shape model with random weights
@@ -15,8 +17,12 @@ One JSON line goes to stdout.  Besides the driver's fields it carries
   roofline     the dominant kernel of the step (one of the three forms of the M<=32 weight-only
                GEMV) timed live with HIP events on the launch stream, in algorithmic bytes per
                launch; traffic = counter-measured HBM bytes per launch (profiles/)
-  cpu_baseline this repository's CPU restatement of the reference's arithmetic (the oracle),
+  cpu_baseline this repository's CPU restatement of the reference's data flow
+               (oracle/xft_cpu_baseline.c, compiled on this machine with -O3 -march=native -fopenmp),
                timed on the host cores on a bounded sample of the same workload
+  extra        the other points the metric names, measured in the same run: decode at batch 32 and
+               with UINT4 weights, the weight-only GEMM sweep at 2048 rows against the bf16 MFMA
+               peak, the GQA attention sweep, and the sparse-MLP layer
 """
 import argparse
 import json
@@ -30,6 +36,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
 
 CFG = dict(layers=32, hidden=4096, inter=11008, q_heads=32, kv_heads=32, head=128, vocab=32000)
 
@@ -208,36 +215,241 @@ def measured_traffic(key):
     return None
 
 
-def cpu_baseline(kind, host, shapes, batch):
-    """The oracle's decode step of one layer (GEMMs + norm + SwiGLU; attention over a short
-    context is negligible next to 202 MB of weights), extrapolated to 32 layers + lm_head."""
-    from oracle import pyoracle as orc
+def _cpu_model_name():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown CPU"
+
+
+def _build_cpu_baseline_lib():
+    """oracle/xft_cpu_baseline.c compiled for THIS machine's vector ISA (gcc -O3 -march=native -fopenmp)
+    into a temporary directory; the generic build kept next to the oracle is the fallback."""
+    import ctypes
+    import subprocess
+    import tempfile
+    src = os.path.join(ROOT, "oracle", "xft_cpu_baseline.c")
+    out = os.path.join(tempfile.mkdtemp(prefix="xft_cpu_baseline_"), "libxft_cpu_baseline.so")
+    flags = "-O3 -march=native -fopenmp"
+    try:
+        subprocess.check_call(["gcc"] + flags.split() + ["-fPIC", "-shared", "-fno-math-errno", "-std=gnu11", src, "-o", out, "-lm"],
+                              stderr=subprocess.DEVNULL)
+        return ctypes.CDLL(out), flags
+    except (OSError, subprocess.CalledProcessError):
+        return ctypes.CDLL(os.path.join(ROOT, "oracle", "libxft_cpu_baseline.so")), "-O3 -mavx2 -mfma -mf16c -fopenmp (prebuilt)"
+
+
+def cpu_model(lib, cfg, kind, layer_arrays, ln1, ln2, final_norm, emb_fp16, lm_bf16, kcache, vcache, batch, max_seq):
+    """The cpu_model struct of oracle/xft_cpu_baseline.c.  layer_arrays[i] (i = qkv, o, gate/up, down) is
+    a list over layers of (codes, scale, zero-or-None) numpy arrays; returns (struct, objects to keep alive)."""
+    import ctypes as C
+    L = cfg["layers"]
+
+    class CpuModel(C.Structure):
+        _fields_ = [("kind", C.c_int), ("layers", C.c_int), ("hidden", C.c_int), ("inter", C.c_int), ("heads", C.c_int),
+                    ("kv_heads", C.c_int), ("head", C.c_int), ("vocab", C.c_int), ("max_seq", C.c_int),
+                    ("wq", C.POINTER(C.c_void_p) * 4), ("ws", C.POINTER(C.c_void_p) * 4), ("wz", C.POINTER(C.c_void_p) * 4),
+                    ("ln1", C.c_void_p), ("ln2", C.c_void_p), ("final_norm", C.c_void_p), ("embedding", C.c_void_p),
+                    ("lm_head", C.c_void_p), ("kcache", C.c_void_p), ("vcache", C.c_void_p), ("batch", C.c_int)]
+
+    keep = [layer_arrays, ln1, ln2, final_norm, emb_fp16, lm_bf16, kcache, vcache]
+    ptr = lambda a: a.ctypes.data_as(C.c_void_p)
+
+    def table(arrs):
+        t = (C.c_void_p * L)(*[a.ctypes.data for a in arrs])
+        keep.append(t)
+        return C.cast(t, C.POINTER(C.c_void_p))
+
+    m = CpuModel()
+    m.kind, m.layers, m.hidden, m.inter = kind, L, cfg["hidden"], cfg["inter"]
+    m.heads, m.kv_heads, m.head, m.vocab = cfg["q_heads"], cfg["kv_heads"], cfg["head"], cfg["vocab"]
+    m.max_seq, m.batch = max_seq, batch
+    for i, per_layer in enumerate(layer_arrays):
+        m.wq[i] = table([w[0] for w in per_layer])
+        m.ws[i] = table([w[1] for w in per_layer])
+        m.wz[i] = table([w[2] for w in per_layer]) if per_layer[0][2] is not None else None
+    m.ln1, m.ln2, m.final_norm = ptr(ln1), ptr(ln2), ptr(final_norm)
+    m.embedding, m.lm_head, m.kcache, m.vcache = ptr(emb_fp16), ptr(lm_bf16), ptr(kcache), ptr(vcache)
+    lib.cpu_num_threads.restype = C.c_int
+    lib.cpu_scratch_floats.restype = C.c_int64
+    return m, keep
+
+
+def cpu_baseline(kind, host, shapes, batch, prompt, budget_s=15.0):
+    """Greedy decode steps of the whole 32-layer model on the host cores (every layer its own copy of
+    the weights, FP16 cache filled up to the prompt length), as many as fit the time budget."""
+    import ctypes as C
+    lib, flags = _build_cpu_baseline_lib()
     c = CFG
-    ws = [orc.QWeight(kind, K, N, q, s, z) for (K, N), (q, s, z) in zip(shapes, host)]
+    L = c["layers"]
+    steps_max = 24
+    max_seq = prompt + steps_max + 2
+    # distinct memory per layer: nothing stays in a cache from one layer to the next
+    layer_arrays = [[(q.copy(), sc, z) for _ in range(L)] for (q, sc, z) in host]
     rng = np.random.default_rng(5)
-    x = rng.standard_normal((batch, c["hidden"])).astype(np.float32)
     ones = np.ones(c["hidden"], np.float32)
+    emb = (rng.standard_normal((c["vocab"], c["hidden"]), dtype=np.float32) * 0.02).astype(np.float16).view(np.uint16)
+    lm = ((rng.standard_normal((c["hidden"], c["vocab"]), dtype=np.float32) * 0.02).view(np.uint32) >> 16).astype(np.uint16)
+    cache_shape = (L, batch, c["kv_heads"], max_seq, c["head"])
+    kc = rng.standard_normal(cache_shape, dtype=np.float32).astype(np.float16).view(np.uint16)
+    vc = rng.standard_normal(cache_shape, dtype=np.float32).astype(np.float16).view(np.uint16)
+    m, keep = cpu_model(lib, c, kind, layer_arrays, ones, ones, ones, emb, lm, kc, vc, batch, max_seq)
+    scratch = np.zeros(int(lib.cpu_scratch_floats(C.byref(m))), np.float32)
+    ids = rng.integers(0, c["vocab"], batch).astype(np.int32)
+    ptr = lambda a: a.ctypes.data_as(C.c_void_p)
+    times = []
+    t_start = time.time()
+    for t in range(steps_max + 2):
+        t0 = time.time()
+        lib.cpu_decode_step(C.byref(m), ptr(ids), prompt + t, ptr(scratch))
+        if t >= 2:  # two warm-up steps
+            times.append(time.time() - t0)
+        if time.time() - t_start > budget_s and len(times) >= 3:
+            break
+    med = float(np.median(times))
+    return dict(value=round(batch / med, 3), unit="tok/s", cores=int(lib.cpu_num_threads()), kind="port",
+                sample="xFT-semantics CPU restatement (not the xDNN binary): %d greedy decode steps (median, after 2 warm-up steps) "
+                       "of the full 32-layer model at context %d, batch %d, every layer its own weights; gcc %s on %s"
+                       % (len(times), prompt, batch, flags, _cpu_model_name()))
 
-    def layer_step():
-        xn = orc.rmsnorm(x, ones)
-        qkv = orc.qgemm(ws[0], xn)
-        att = qkv[:, :c["hidden"]].copy()
-        x1 = orc.qgemm(ws[1], att, orc.EPI_RESIDENTIAL, res=x)
-        h = orc.silu_sum(orc.qgemm(ws[2], orc.rmsnorm(x1, ones)))
-        return orc.qgemm(ws[3], h, orc.EPI_RESIDENTIAL, res=x1)
 
-    layer_step()
+# ---------------------------------------------------------------------------- extra measurements
+def decode_run(xh, kind, B, prompt, steps, warmup, kv_int8=False):
+    """tok/s of greedy decode for one (weights, batch) point, with its share of the HBM roofline."""
+    max_seq = prompt + warmup + steps + 1
+    model, layer_weights, lmw, _, _ = build_model(xh, kind, B, max_seq, prompt, kv_int8)
+    ids = np.random.default_rng(3).integers(0, CFG["vocab"], (B, prompt)).astype(np.int32)
+    model.prefill(ids)
+    model.decode_untracked(warmup)
+    xh.synchronize()
     t0 = time.time()
-    n = 0
-    while time.time() - t0 < 12.0 and n < 50:
-        layer_step()
-        n += 1
-    per_layer = (time.time() - t0) / n
-    # lm_head: fp32 GEMM of the same byte count per row as one more 131 M-element matrix
-    step = per_layer * (c["layers"] + c["hidden"] * c["vocab"] / 202375168.0)
-    return dict(value=round(batch / step, 3), unit="tok/s", cores=orc.num_threads(), kind="port",
-                sample=f"{n} decode steps of 1 of 32 layers (INT8/UINT4 weight-only GEMMs, RMSNorm, SwiGLU), "
-                       f"extrapolated x32 + lm_head; attention over the cache not timed")
+    model.decode_untracked(steps)
+    xh.synchronize()
+    dt = time.time() - t0
+    wbytes = sum(w.bytes() for w in layer_weights[0]) * CFG["layers"] + lmw.bytes()
+    ctx = prompt + warmup + steps / 2.0
+    kv_elem = (1 + 4.0 / CFG["head"]) if kv_int8 else 2
+    step_bytes = wbytes + CFG["layers"] * 2 * B * ctx * CFG["kv_heads"] * CFG["head"] * kv_elem
+    ms = dt * 1e3 / steps
+    out = dict(weights="int8" if kind == 0 else "uint4", batch=B, kv="int8" if kv_int8 else "fp16", tok_s=round(B * steps / dt, 1),
+               ms_per_step=round(ms, 4), step_hbm_bytes=int(step_bytes),
+               step_hbm_frac=round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4))
+    model.free()
+    for ws in layer_weights:
+        for w in ws:
+            w.free()
+    lmw.free()
+    return out
+
+
+def prefill_gemm_sweep(xh, M=2048, nweights=8, iters=3):
+    """The weight-only GEMM sweep at M rows (bf16 in, bf16 out): every (N, K) x kind of the sweep
+    launched back to back over `nweights` distinct weights (more than the 256 MB the Infinity Cache
+    holds for every case but 4096 x 4096 UINT4/NF4, which get twice as many), HIP events on the
+    launch stream; TFLOP/s = 2 M N K / time, against the published dense bf16 MFMA peak."""
+    rng = np.random.default_rng(1)
+    res = []
+    for (N, K) in ((4096, 4096), (11008, 4096), (4096, 11008)):
+        A = xh.DeviceBuffer.from_numpy(xh.f32_to_bf16_bits(rng.standard_normal((M, K), dtype=np.float32)))
+        Cd = xh.DeviceBuffer(M * N * 2)
+        for kind, name in ((xh.W_INT8, "int8"), (xh.W_UINT4, "uint4"), (xh.W_NF4, "nf4")):
+            q, sc, z = synth_codes(rng, 0 if kind == xh.W_INT8 else 1, K, N)
+            if kind == xh.W_NF4:
+                z = None
+            nw = nweights * (2 if (kind != xh.W_INT8 and N * K <= 4096 * 4096) else 1)
+            ws = [xh.Weight(kind, K, N, q, sc, z) for _ in range(nw)]
+            for w in ws:
+                xh.gemm(w, A.ptr, M, K, Cd.ptr, N, xh.BF16)
+            xh.synchronize()
+            t = xh.Timer()
+            t.start()
+            for _ in range(iters):
+                for w in ws:
+                    xh.gemm(w, A.ptr, M, K, Cd.ptr, N, xh.BF16)
+            us = t.stop() * 1e3 / (iters * nw)
+            tf = 2.0 * M * N * K / us / 1e6
+            res.append(dict(kind=name, M=M, N=N, K=K, avg_launch_us=round(us, 2), tflops=round(tf, 1),
+                            frac_of_bf16_mfma_peak=round(tf / MFMA_BF16_PEAK_TFLOPS, 4)))
+            for w in ws:
+                w.free()
+    return res
+
+
+def attention_sweep(xh, iters=10):
+    """GQA attention, 32 query / 8 KV heads, head size 128: decode at batch 1 / 16 / 64 and context
+    1024 / 4096 / 16384 over FP16 and INT8 caches (achieved GB/s against B ctx 8 128 2 e bytes, e = 2
+    or 1 + 4/128) and the causal prefill of 4 x 2048 tokens (TFLOP/s on the causal-halved flops)."""
+    qh, kvh, D = 32, 8, 128
+    scale = 1.0 / np.sqrt(D)
+    out = []
+    for int8 in (0, 1):
+        for B in (1, 16, 64):
+            cache = xh.KVCache(xh.INT8 if int8 else xh.FP16, B, kvh, 16384, D)
+            q = xh.DeviceBuffer(B * qh * D * 2)
+            q.zero()
+            o = xh.DeviceBuffer(B * qh * D * 2)
+            for ctx in (1024, 4096, 16384):
+                for _ in range(2):
+                    xh.attention(cache, q.ptr, qh * D, o.ptr, qh * D, xh.BF16, B, 1, qh, scale, ctx - 1)
+                xh.synchronize()
+                t = xh.Timer()
+                t.start()
+                for _ in range(iters):
+                    xh.attention(cache, q.ptr, qh * D, o.ptr, qh * D, xh.BF16, B, 1, qh, scale, ctx - 1)
+                us = t.stop() * 1e3 / iters
+                byts = B * ctx * kvh * D * 2 * ((1 + 4.0 / D) if int8 else 2) + B * qh * D * 2 * 2
+                out.append(dict(phase="decode", kv="int8" if int8 else "fp16", batch=B, ctx=ctx, avg_launch_us=round(us, 2),
+                                gbs=round(byts / us / 1e3, 1), frac_of_hbm_peak=round(byts / us / 1e3 / HBM_PEAK_GBS, 4)))
+            cache.free()
+    B, S = 4, 2048
+    cache = xh.KVCache(xh.FP16, B, kvh, S, D)
+    stride = (qh + 2 * kvh) * D
+    qkv = xh.DeviceBuffer(B * S * stride * 2)
+    qkv.zero()
+    o = xh.DeviceBuffer(B * S * qh * D * 2)
+    xh.rope_kvstore(cache, qkv.ptr, xh.BF16, stride, B, S, qh, None, 0)
+    xh.attention(cache, qkv.ptr, stride, o.ptr, qh * D, xh.BF16, B, S, qh, scale, 0)
+    xh.synchronize()
+    t = xh.Timer()
+    t.start()
+    for _ in range(3):
+        xh.attention(cache, qkv.ptr, stride, o.ptr, qh * D, xh.BF16, B, S, qh, scale, 0)
+    us = t.stop() * 1e3 / 3
+    flops = 4.0 * B * qh * S * S * D / 2
+    out.append(dict(phase="prefill", kv="fp16", batch=B, seq=S, avg_launch_us=round(us, 1), tflops=round(flops / us / 1e6, 1),
+                    frac_of_bf16_mfma_peak=round(flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)))
+    return out
+
+
+def moe_layer(xh, iters=5):
+    """Mixtral-8x7B-shape sparse MLP: hidden 4096, FFN 14336, 8 experts, top-2, INT8 per-channel expert
+    weights, 256 tokens with N(0,1) router logits.  1.409 GB of expert weights and 180.4 GFLOP per pass."""
+    H, I, E, T = 4096, 14336, 8, 256
+    rng = np.random.default_rng(4)
+    moe = xh.MoE(H, I, E, T, np.zeros((H, E), np.float32), np.ones(H, np.float32))
+    gq, gs, _ = synth_codes(rng, 0, H, 2 * I)
+    dq, ds, _ = synth_codes(rng, 0, I, H)
+    for e in range(E):
+        moe.set_expert(e, xh.Weight(xh.W_INT8, H, 2 * I, gq, gs, None, flags=xh.WF_GATEUP), xh.Weight(xh.W_INT8, I, H, dq, ds, None))
+    x = xh.DeviceBuffer.from_numpy(rng.standard_normal((T, H), dtype=np.float32))
+    y = xh.DeviceBuffer(T * H * 4)
+    lg = xh.DeviceBuffer.from_numpy(rng.standard_normal((T, E), dtype=np.float32))
+    moe.forward(x.ptr, y.ptr, T, True, lg.ptr)
+    xh.synchronize()
+    t0 = time.time()
+    for _ in range(iters):
+        moe.forward(x.ptr, y.ptr, T, True, lg.ptr)
+    xh.synchronize()
+    us = (time.time() - t0) * 1e6 / iters
+    wbytes, flops = 8 * (4096 * 28672 + 14336 * 4096), 512 * 3 * 2 * 4096 * 14336
+    moe.free()
+    return dict(tokens=T, experts=E, us_per_layer=round(us, 1), weight_gbs=round(wbytes / us / 1e3, 1),
+                frac_of_hbm_peak=round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4), tflops=round(flops / us / 1e6, 1),
+                note="wall time of xfthip_moe_forward (it synchronises once for the per-expert row counts)")
 
 
 def main():
@@ -255,6 +467,10 @@ def main():
     ap.add_argument("--pmc-workload", action="store_true", help="counter workload for rocprofv3 --pmc: a plain copy kernel of known size, then every distinct decode GEMV of the model once; prints no result line")
     ap.add_argument("--pmc-summary", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"), help="summarise the two counter CSVs of the --pmc-workload runs (CPU only)")
     ap.add_argument("--eager", action="store_true", help="launch decode kernels one by one instead of replaying the captured graph (for per-kernel profiling)")
+    ap.add_argument("--no-extras", action="store_true", help="skip the extra measurements (batch 32 / UINT4 decode, GEMM sweep, attention sweep, sparse MLP)")
+    ap.add_argument("--prefill-gemm", action="store_true", help="only the weight-only GEMM sweep at M = 1, 8, 32, 256, 2048 (one JSON line)")
+    ap.add_argument("--attention", action="store_true", help="only the GQA attention sweep (one JSON line)")
+    ap.add_argument("--moe", action="store_true", help="only the sparse-MLP layer (one JSON line)")
     args = ap.parse_args()
     if args.pmc_summary:
         pmc_summary(*args.pmc_summary)
@@ -265,6 +481,15 @@ def main():
 
     from xfastertransformer_amd import capi as xh
     xh.init(0)
+    if args.prefill_gemm:
+        print(json.dumps({"prefill_gemm": [r for M in (256, 2048) for r in prefill_gemm_sweep(xh, M)], "peak_tflops": MFMA_BF16_PEAK_TFLOPS}))
+        return
+    if args.attention:
+        print(json.dumps({"attention": attention_sweep(xh), "hbm_peak_gbs": HBM_PEAK_GBS, "peak_tflops": MFMA_BF16_PEAK_TFLOPS}))
+        return
+    if args.moe:
+        print(json.dumps({"moe": moe_layer(xh)}))
+        return
     kind = 0 if args.weights == "int8" else 1
     B = args.batch
     max_seq = args.prompt + args.warmup + args.steps + 1
@@ -334,7 +559,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16 activations x %s weights, fp32 accumulate" % args.weights,
-        "data": "synthetic",
+        "data": "synthetic: integer codes drawn as N(0, 0.02) weights quantise to, one layer's codes uploaded as 32 distinct device weights",
         "config": {"workload": "configs[3]: 32-layer Llama-2-7B-shape, %s weight-only, %s KV, batch %d, "
                                "%d-token prompt, greedy decode" % (args.weights.upper(), args.kv.upper(), B, args.prompt),
                    "batch": B, "prompt": args.prompt, "weights": args.weights, "kv": args.kv},
@@ -344,13 +569,29 @@ def main():
         "step_hbm_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "roofline": {"bound": "hbm", "kernel": dom["name"], "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "traffic_source": "recorded counter run, profiles/qgemm_skinny_int8_bs1_hbm_traffic.txt (not measured in this run)",
                      "avg_launch_us": round(dom["us"], 3), "bytes_per_launch": int(dom["bytes"])},
         "other_kernels": [{"kernel": g["name"], "launches_per_layer": g["launches"], "avg_launch_us": round(g["us"], 3),
                            "bytes_per_launch": int(g["bytes"]),
                            "frac": round(g["bytes"] / g["us"] / 1e3 / HBM_PEAK_GBS, 4)} for g in others],
     }
+    if not args.no_extras:
+        # free the main model before the other points of the metric are built
+        model.free()
+        for ws in layer_weights:
+            for w in ws:
+                w.free()
+        lmw.free()
+        extra = {"decode": []}
+        for k2, b2 in ((0, 32), (1, 1), (1, 32)):
+            if (k2, b2) != (kind, B):
+                extra["decode"].append(decode_run(xh, k2, b2, args.prompt, 64, 8))
+        extra["prefill_gemm"] = prefill_gemm_sweep(xh, 2048)
+        extra["attention"] = attention_sweep(xh)
+        extra["moe"] = moe_layer(xh)
+        result["extra"] = extra
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(kind, host, shapes, B)
+        result["cpu_baseline"] = cpu_baseline(kind, host, shapes, B, args.prompt)
     print(json.dumps(result), flush=True)
 
 

@@ -1,5 +1,6 @@
 // Enumerations of the xFasterTransformer layer API (source-compatible with the reference's
 // include/dtype.h:18-56: same names, same order, same values).
+// The declarations follow intel/xFasterTransformer (Apache-2.0, Copyright (c) Intel Corporation).
 #pragma once
 
 namespace xft {

@@ -4,6 +4,7 @@
 // fp32 [hiddenSize, (attHeadNum + 2*kvHeadNum) * attHeadDim] host matrix (row stride = that
 // width), attnOutWeight is [attHeadNum*attHeadDim, hiddenSize].  The KV cache (FP16) belongs to
 // the callee and carries over between calls: pastSeqLen / step are supplied by the caller.
+// The declarations follow intel/xFasterTransformer (Apache-2.0, Copyright (c) Intel Corporation).
 #pragma once
 
 #include "dtype.h"

@@ -2,6 +2,7 @@
 // One Llama decoder layer: RMSNorm -> fused QKV -> RoPE -> causal attention over the callee's
 // FP16 KV cache -> out-proj + residual -> RMSNorm -> SwiGLU MLP + residual.  fp32 host
 // activations, fp32 host weights [in, out] (see layers_attention.h for the Q/K/V layout).
+// The declarations follow intel/xFasterTransformer (Apache-2.0, Copyright (c) Intel Corporation).
 #pragma once
 
 #include "dtype.h"

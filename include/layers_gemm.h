@@ -2,6 +2,7 @@
 // MI355X build: A, B (row-major [K,N], or [N,K] when transB), C, bias and res are HOST buffers
 // of the element type named by dt (bf16 or fp16); C = alpha * op(A) * op(B) + beta * C (+ bias)
 // (+ res).  B is converted and packed on every call, as the reference does.
+// The declarations follow intel/xFasterTransformer (Apache-2.0, Copyright (c) Intel Corporation).
 #pragma once
 
 #include "dtype.h"

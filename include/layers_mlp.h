@@ -3,6 +3,7 @@
 // [numTokens, stride]; the weights are fp32 host matrices [in, out] converted once per distinct
 // set of weight addresses.  dt selects the on-device weight format: bf16 (the reference's), or
 // the weight-only formats int8 / int4 / nf4 this build adds to the same entry point.
+// The declarations follow intel/xFasterTransformer (Apache-2.0, Copyright (c) Intel Corporation).
 #pragma once
 
 #include "dtype.h"

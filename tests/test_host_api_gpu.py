@@ -189,3 +189,92 @@ def test_invoke_gemm_bf16(host, orc, M, transB):
     exp = A.astype(np.float64) @ Bm.astype(np.float64)
     assert np.abs(orc.from_bf16(Cb) - exp).max() < 0.5  # gemm_kernel_ext_test.cpp tolerance for bf16
     assert (np.abs(orc.from_bf16(Cb) - exp) <= 1e-3 + np.abs(exp) * 2.0 ** -8).all()
+
+
+FP16, W8A8 = 2, 4  # xft::DataType
+
+
+def test_invoke_gemm_fp16_and_large_m(host, orc):
+    """fp16 invokeGemm (src/kernels/gemm_kernel_ext.cpp:503-517; the reference's test tolerance is 0.05)
+    and the 1024-row case of its bf16 test.  fp16 operands are multiplied exactly (hi + lo bf16 split),
+    so the result is within one fp16 rounding of the float64 product."""
+    M, N, K = 1024, 512, 1024
+    rng = np.random.default_rng(3)
+    A = orc.from_fp16(orc.to_fp16(rng.uniform(-1, 1, (M, K))))
+    Bm = orc.from_fp16(orc.to_fp16(rng.uniform(-1, 1, (K, N))))
+    exp = A.astype(np.float64) @ Bm.astype(np.float64)
+    for transB in (False, True):
+        Ah, Bh = orc.to_fp16(A), orc.to_fp16(Bm.T.copy() if transB else Bm)
+        Ch = np.zeros((M, N), np.uint16)
+        host["gemm"](FP16, False, transB, M, N, K, 1.0, ptr(Ah), K, ptr(Bh), 0.0, ptr(Ch), N, None, None, -1)
+        got = orc.from_fp16(Ch)
+        assert np.abs(got - exp).max() < 0.05
+        assert (np.abs(got - exp) <= 2e-3 + np.abs(exp) * 2.0 ** -10).all()
+    Ab, Bb = orc.to_bf16(orc.round_bf16(A)), orc.to_bf16(orc.round_bf16(Bm))
+    Cb = np.zeros((M, N), np.uint16)
+    host["gemm"](BF16, False, False, M, N, K, 1.0, ptr(Ab), K, ptr(Bb), 0.0, ptr(Cb), N, None, None, -1)
+    expb = orc.round_bf16(A).astype(np.float64) @ orc.round_bf16(Bm).astype(np.float64)
+    assert np.abs(orc.from_bf16(Cb) - expb).max() < 0.5
+
+
+def test_invoke_layer_llama_w8a8_fp16_and_unsupported(host, orc, capfd):
+    hidden, inter, qh, kvh, D = 1024, 2816, 8, 8, 128
+    rng = np.random.default_rng(17)
+    qkv, wo, gate, up, down = _layer_weights(rng, hidden, inter, qh, kvh, D)
+    ln1 = rng.uniform(0.8, 1.2, hidden).astype(np.float32)
+    ln2 = rng.uniform(0.8, 1.2, hidden).astype(np.float32)
+    qcols, kvcols = qh * D, kvh * D
+
+    def call(dt, x, S, past, step, weights=(qkv, wo, gate, up, down)):
+        q_, o_, g_, u_, d_ = weights
+        out = np.full_like(x, 7.0)
+        host["layer"](dt, SILU, RMS, 1, S, D, qh, kvh, 32, 32, past, past + S, step, hidden, inter, ptr(out), hidden, ptr(x),
+                      hidden, ptr(ln1), None, ptr(q_), C.c_void_p(q_.ctypes.data + qcols * 4),
+                      C.c_void_p(q_.ctypes.data + (qcols + kvcols) * 4), ptr(o_), ptr(ln2), None, ptr(g_), ptr(u_), ptr(d_),
+                      None, None, None, None)
+        return out
+
+    # W8A8: per-row INT8 activations against per-column INT8 weights (matmul_helper.h:2762-2965)
+    ow = [orc.quantize(orc.W_W8A8, w) for w in (qkv, wo, np.concatenate([gate, up], 1), down)]
+    ref = orc.LlamaLayerOracle(hidden, inter, qh, kvh, D, *ow, ln1, ln2, max_seq=32)
+    past = 0
+    for step, S in enumerate((18, 1, 1)):
+        x = rng.standard_normal((S, hidden)).astype(np.float32)
+        out = call(W8A8, x, S, past, step)
+        exp = ref.forward(x, 1, S, past)
+        err = np.abs(out - exp)
+        # the GPU quantises the bf16 activation rows, the oracle the fp32 ones: codes differ by one now and then
+        assert _cos(out, exp) >= 0.9995 and err.max() < 0.15 and np.sqrt((err ** 2).mean()) < 3e-2, (step, err.max())
+        past += S
+    # fp16 is served (weights held as bf16): same result as dt = bf16 on copies of the same weights
+    x = rng.standard_normal((5, hidden)).astype(np.float32)
+    copies = tuple(w.copy() for w in (qkv, wo, gate, up, down))
+    a = call(FP16, x, 5, 0, 0)
+    b = call(BF16, x, 5, 0, 0, copies)
+    assert np.array_equal(a, b) and not (a == 7.0).all()
+    # a type no entry point serves: the reference's message, output untouched
+    capfd.readouterr()
+    c = call(FP32, x, 5, 0, 0)
+    assert (c == 7.0).all()
+    assert "unsupported data type" in capfd.readouterr().out
+
+
+def test_invoke_rotary_embedding_reads_the_second_half_of_the_tables(host, orc):
+    """The public tables are [maxPosition, dim]: the second half of a head must use columns
+    [dim/2, dim) (src/layers/rotary_embedding_api.cpp:35-47), also when they differ from the first half."""
+    rng = np.random.default_rng(19)
+    T, heads, D = 3, 2, 8
+    q = rng.standard_normal((T, heads * D)).astype(np.float32)
+    k = rng.standard_normal((T, heads * D)).astype(np.float32)
+    cos = rng.uniform(-1, 1, (6, D)).astype(np.float32)
+    sin = rng.uniform(-1, 1, (6, D)).astype(np.float32)
+    pos = np.array([5, 0, 2], np.int64)
+    eq, ek = q.copy().reshape(T, heads, D), k.copy().reshape(T, heads, D)
+    h = D // 2
+    for buf in (eq, ek):
+        for t in range(T):
+            a, b = buf[t, :, :h].copy(), buf[t, :, h:].copy()
+            buf[t, :, :h] = a * cos[pos[t], :h] - b * sin[pos[t], :h]
+            buf[t, :, h:] = b * cos[pos[t], h:] + a * sin[pos[t], h:]
+    host["rope"](FP32, ptr(pos), ptr(q), ptr(k), ptr(cos), ptr(sin), D, heads * D, heads * D, T, heads, D, heads)
+    assert np.abs(q - eq.reshape(T, -1)).max() < 1e-6 and np.abs(k - ek.reshape(T, -1)).max() < 1e-6

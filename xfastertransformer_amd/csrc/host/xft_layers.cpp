@@ -7,9 +7,11 @@
 // mutex serialises each invoke*LLaMA; weights are fp32 host matrices [in, out], converted once
 // on first sight and cached for the life of the process under a key made of their addresses
 // plus dims and dt; activations are fp32 host buffers; the KV cache (FP16) is owned here and
-// the caller supplies pastSeqLen / step.  Beyond the reference: dt may also be int8, int4 or
-// nf4, which selects the weight-only formats (the reference's entry points silently ignore
-// every dt but bf16 / fp16).
+// the caller supplies pastSeqLen / step.  Beyond the reference: dt may also be int8, w8a8, int4
+// or nf4, which selects the weight-only / W8A8 formats (the reference's entry points print
+// ">> unsupported data type" for every dt but bf16 / fp16, decoder_layer.cpp:172-206).
+// dt = fp16 is served with the weights narrowed to bf16 (8 significant bits instead of fp16's
+// 11): this build has no fp16 weight kind; a one-line notice says so once.
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -68,14 +70,20 @@ float from_bf16(uint16_t b) {
     return f;
 }
 
-// weight kind for a DataType, or -1
+// weight kind for a DataType; -1 (after the reference's own message) for a type no entry point serves
 int kind_of(xft::DataType dt) {
     switch (dt) {
         case xft::DataType::bf16: return XFTHIP_W_BF16;
+        case xft::DataType::fp16: {
+            static std::once_flag once;
+            std::call_once(once, [] { printf(">> fp16 weights are held as bf16 by this build\n"); });
+            return XFTHIP_W_BF16;
+        }
         case xft::DataType::int8: return XFTHIP_W_INT8;
+        case xft::DataType::w8a8: return XFTHIP_W_W8A8;
         case xft::DataType::int4: return XFTHIP_W_UINT4;
         case xft::DataType::nf4: return XFTHIP_W_NF4;
-        default: return -1;
+        default: printf(">> unsupported data type\n"); return -1;
     }
 }
 
@@ -202,7 +210,7 @@ void invokeLayerLLaMA(DataType dt, ActivationType at, NormType nt, int batchSize
     (void)ln1Beta; (void)ln2Beta; (void)currentSeqLen; (void)step;
 
     const int kind = kind_of(dt);
-    if (kind < 0) return; // the reference's dispatch has no else-branch either (decoder_layer.cpp:172-206)
+    if (kind < 0) return; // message printed, output untouched, as the reference (decoder_layer.cpp:172-206)
     if (nt != NormType::RMS) {
         printf(">> unsupported norm type (this build implements RMSNorm layers)\n");
         return;
@@ -224,7 +232,7 @@ void invokeLayerLLaMA(DataType dt, ActivationType at, NormType nt, int batchSize
         e.qkv = make_weight(kind, hiddenSize, qCols + 2 * kvCols, qkv.data(), XFTHIP_WF_NONE);
         e.o = make_weight(kind, qCols, hiddenSize, (const float *)attnOutWeight, XFTHIP_WF_NONE);
         auto gu = concat_gateup((const float *)gateWeight, (const float *)upWeight, hiddenSize, intermediateSize);
-        e.gateup = make_weight(kind, hiddenSize, 2 * intermediateSize, gu.data(), XFTHIP_WF_GATEUP);
+        e.gateup = make_weight(kind, hiddenSize, 2 * intermediateSize, gu.data(), kind == XFTHIP_W_W8A8 ? XFTHIP_WF_NONE : XFTHIP_WF_GATEUP);
         e.down = make_weight(kind, intermediateSize, hiddenSize, (const float *)downWeight, XFTHIP_WF_NONE);
         e.ln1.assign(ln1Gamma, ln1Gamma + hiddenSize);
         e.ln2.assign(ln2Gamma, ln2Gamma + hiddenSize);
@@ -297,7 +305,7 @@ void invokeMLPLLaMA(DataType dt, ActivationType at, int numTokens, int hiddenSiz
     Entry &e = hub[key.str()];
     if (!e.hasMlp) {
         auto gu = concat_gateup((const float *)gateWeight, (const float *)upWeight, hiddenSize, intermediateSize);
-        e.gateup = make_weight(kind, hiddenSize, 2 * intermediateSize, gu.data(), XFTHIP_WF_GATEUP);
+        e.gateup = make_weight(kind, hiddenSize, 2 * intermediateSize, gu.data(), kind == XFTHIP_W_W8A8 ? XFTHIP_WF_NONE : XFTHIP_WF_GATEUP);
         e.down = make_weight(kind, intermediateSize, hiddenSize, (const float *)downWeight, XFTHIP_WF_NONE);
         e.hasMlp = true;
         // head geometry is irrelevant to the MLP block; one 128-wide head keeps the scratch small
@@ -382,41 +390,110 @@ void invokeRotaryEmbedding(DataType dt, const int64_t *positionIds, void *query,
     for (void *p : {dq, dk, dc, ds, dp}) xfthip_free(p);
 }
 
+// fp16 bit pattern -> float (IEEE binary16)
+static float from_fp16(uint16_t h) {
+    const uint32_t sgn = (uint32_t)(h & 0x8000u) << 16, ex = (h >> 10) & 31u;
+    uint32_t man = h & 1023u, u;
+    if (ex == 0) {
+        if (man == 0) {
+            u = sgn;
+        } else {
+            int sh = 0;
+            while (!(man & 1024u)) man <<= 1, ++sh;
+            u = sgn | ((uint32_t)(113 - sh) << 23) | ((man & 1023u) << 13);
+        }
+    } else if (ex == 31) {
+        u = sgn | 0x7F800000u | (man << 13);
+    } else {
+        u = sgn | ((ex + 112u) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+// float -> fp16 bit pattern, round to nearest even
+static uint16_t to_fp16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    const uint32_t sgn = (u >> 16) & 0x8000u, a = u & 0x7FFFFFFFu;
+    if (a >= 0x47800000u) return (uint16_t)(sgn | (a > 0x7F800000u ? 0x7E00u : 0x7C00u));
+    if (a < 0x38800000u) {
+        if (a < 0x33000000u) return (uint16_t)sgn;
+        const uint32_t man = (a & 0x7FFFFFu) | 0x800000u;
+        const int sh = 126 - (int)(a >> 23);
+        uint32_t r = man >> sh;
+        const uint32_t rem = man & ((1u << sh) - 1), half = 1u << (sh - 1);
+        if (rem > half || (rem == half && (r & 1u))) ++r;
+        return (uint16_t)(sgn | r);
+    }
+    const uint32_t r = a - 0x38000000u;
+    uint32_t man = r >> 13;
+    const uint32_t rem = r & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (man & 1u))) ++man;
+    return (uint16_t)(sgn | man);
+}
+
 void invokeGemm(DataType dt, bool transA, bool transB, int M, int N, int K, float alpha, void *A, int lda, void *B, float beta, void *C,
         int ldc, void *bias, void *res, int ldres) {
     // the reference accepts bias / res but never reads them (src/utils/matmul_helper.h:63-101)
     (void)bias; (void)res; (void)ldres;
-    if (dt != DataType::bf16) {
-        printf(">> invokeGemm: only bf16 is offered by this build\n");
+    if (dt != DataType::bf16 && dt != DataType::fp16) {
+        printf(">> invokeGemm: only bf16 and fp16 are offered (as in the reference, src/kernels/gemm_kernel_ext.cpp:503-517)\n");
         return;
     }
     ensure_init();
+    const bool half = dt == DataType::fp16;
     const uint16_t *a = (const uint16_t *)A, *b = (const uint16_t *)B;
-    // op(B) as [K, N] bf16, op(A) as dense [M, Kp] with Kp a multiple of 8
-    std::vector<uint16_t> bm((size_t)K * N);
-    for (int k = 0; k < K; ++k)
-        for (int n = 0; n < N; ++n) bm[(size_t)k * N + n] = transB ? b[(size_t)n * K + k] : b[(size_t)k * N + n];
+    auto a_at = [&](int m, int k) { return transA ? a[(size_t)k * M + m] : a[(size_t)m * lda + k]; };
+    auto b_at = [&](int k, int n) { return transB ? b[(size_t)n * K + k] : b[(size_t)k * N + n]; };
+    // The device GEMM multiplies bf16 by bf16.  An fp16 value (11 significant bits) is the exact sum of
+    // two bf16 values hi + lo, so the fp16 product runs as one bf16 GEMM over a tripled k extent:
+    // [Ah | Ah | Al] x [Bh ; Bl ; Bh] = Ah Bh + Ah Bl + Al Bh (the dropped Al Bl term is below 2^-16 of
+    // the product).  bf16 runs as it is.
+    const int parts = half ? 3 : 1;
     const int Kp = (K + 7) / 8 * 8;
-    std::vector<uint16_t> am((size_t)M * Kp, 0);
+    auto split = [&](uint16_t h, uint16_t &hi, uint16_t &lo) {
+        const float f = from_fp16(h);
+        hi = to_bf16(f);
+        lo = to_bf16(f - from_bf16(hi));
+    };
+    std::vector<uint16_t> am((size_t)M * Kp * parts, 0), bp((size_t)Kp * parts * N, 0);
     for (int m = 0; m < M; ++m)
-        for (int k = 0; k < K; ++k) am[(size_t)m * Kp + k] = transA ? a[(size_t)k * M + m] : a[(size_t)m * lda + k];
-    std::vector<uint16_t> bp((size_t)Kp * N, 0);
-    memcpy(bp.data(), bm.data(), bm.size() * 2);
+        for (int k = 0; k < K; ++k) {
+            uint16_t *row = &am[(size_t)m * Kp * parts];
+            if (half) {
+                uint16_t hi, lo;
+                split(a_at(m, k), hi, lo);
+                row[k] = hi, row[Kp + k] = hi, row[2 * Kp + k] = lo;
+            } else {
+                row[k] = a_at(m, k);
+            }
+        }
+    for (int k = 0; k < K; ++k)
+        for (int n = 0; n < N; ++n) {
+            if (half) {
+                uint16_t hi, lo;
+                split(b_at(k, n), hi, lo);
+                bp[(size_t)k * N + n] = hi, bp[((size_t)Kp + k) * N + n] = lo, bp[((size_t)2 * Kp + k) * N + n] = hi;
+            } else {
+                bp[(size_t)k * N + n] = b_at(k, n);
+            }
+        }
     xfthip_weight_t w = nullptr;
-    CK(xfthip_weight_create(XFTHIP_W_BF16, Kp, N, bp.data(), nullptr, nullptr, XFTHIP_WF_NONE, &w));
+    CK(xfthip_weight_create(XFTHIP_W_BF16, Kp * parts, N, bp.data(), nullptr, nullptr, XFTHIP_WF_NONE, &w));
     void *da = nullptr, *dc = nullptr;
     CK(xfthip_malloc(&da, am.size() * 2));
     CK(xfthip_malloc(&dc, (size_t)M * N * 4));
     CK(xfthip_memcpy_h2d(da, am.data(), am.size() * 2, nullptr));
-    CK(xfthip_gemm(w, M, da, Kp, dc, N, XFTHIP_F32, XFTHIP_EPI_NONE, nullptr, nullptr, 0, XFTHIP_F32, 1.0f, nullptr));
+    CK(xfthip_gemm(w, M, da, Kp * parts, dc, N, XFTHIP_F32, XFTHIP_EPI_NONE, nullptr, nullptr, 0, XFTHIP_F32, 1.0f, nullptr));
     std::vector<float> acc((size_t)M * N);
     CK(xfthip_memcpy_d2h(acc.data(), dc, acc.size() * 4, nullptr));
     uint16_t *c = (uint16_t *)C;
     for (int m = 0; m < M; ++m)
         for (int n = 0; n < N; ++n) {
             float v = alpha * acc[(size_t)m * N + n];
-            if (beta != 0.0f) v += beta * from_bf16(c[(size_t)m * ldc + n]);
-            c[(size_t)m * ldc + n] = to_bf16(v);
+            if (beta != 0.0f) v += beta * (half ? from_fp16(c[(size_t)m * ldc + n]) : from_bf16(c[(size_t)m * ldc + n]));
+            c[(size_t)m * ldc + n] = half ? to_fp16(v) : to_bf16(v);
         }
     xfthip_free(da);
     xfthip_free(dc);

@@ -121,6 +121,12 @@ struct xfthip_model {
     // flash path does on its bf16 copies (src/layers/attention.h:1121-1188); they live here
     xfthip_kvcache_t prefill_cache = nullptr;
     AttnWorkspace attn_ws; // split-KV partials and tickets of this model's attention launches
+    // W8A8 layers: int8 activation rows + per-row (scale, zero, sum), and the [tokens, 2 * inter]
+    // bf16 result of the gate/up projection (which runs as a plain GEMM for this kind)
+    int8_t *w8a8_qa = nullptr;
+    size_t w8a8_qa_bytes = 0;
+    float *w8a8_stat = nullptr;
+    uint16_t *gu = nullptr;
     float *cosT = nullptr, *sinT = nullptr;
     // scratch
     uint16_t *xn = nullptr, *qkv = nullptr, *att = nullptr, *h = nullptr;
@@ -259,6 +265,47 @@ __global__ void narrow_rows_kernel(const float *__restrict__ in, int in_stride, 
     for (int c = threadIdx.x; c < cols; c += blockDim.x) orow[c] = xfthip::f32_to_bf16_ref(row[c]);
 }
 
+// h[t][i] = silu(gu[t][i]) * gu[t][inter + i] on bf16 rows: the SwiGLU of a gate/up projection that
+// ran as a plain GEMM (DecoderUtil::siluSum, src/utils/decoder_util.h:550-573)
+__global__ void silu_mul_kernel(const uint16_t *__restrict__ gu, uint16_t *__restrict__ h, int inter) {
+    const uint16_t *row = gu + (size_t)blockIdx.x * 2 * inter;
+    for (int i = threadIdx.x; i < inter; i += blockDim.x) {
+        const float g = bf16_to_f32(row[i]), u = bf16_to_f32(row[inter + i]);
+        h[(size_t)blockIdx.x * inter + i] = f32_to_bf16_ref(u * (g / (1.0f + fast_exp(-g))));
+    }
+}
+
+// xfthip_gemm for the model: W8A8 weights quantise their activation rows into the model's own
+// scratch (sized at attach time, so nothing is allocated or freed while a captured step exists)
+static int model_gemm(xfthip_model *m, xfthip_weight_t w, int M, const void *A, int lda, void *C, int ldc, int c_dtype, int epi,
+        const float *bias, const void *res, int ldres, int res_dtype, hipStream_t st) {
+    if (w->pw.kind == XFTHIP_W_W8A8) {
+        XFT_REQUIRE(m->w8a8_qa != nullptr, "model has a W8A8 weight but no activation scratch");
+        const int K = w->pw.K, ldq = (K + 15) / 16 * 16;
+        XFT_REQUIRE((size_t)M * ldq <= m->w8a8_qa_bytes, "W8A8 scratch too small for %d rows of %d", M, K);
+        float *sA = m->w8a8_stat, *zA = sA + m->cfg.max_tokens, *sumA = zA + m->cfg.max_tokens;
+        if (int rc = xfthip_w8a8_quantize_rows(A, XFTHIP_BF16, M, K, lda, m->w8a8_qa, ldq, sA, zA, sumA, st)) return rc;
+        return xfthip_gemm_w8a8(w, M, m->w8a8_qa, ldq, sA, zA, sumA, C, ldc, c_dtype, epi, bias, res, ldres, res_dtype, 1.0f, st);
+    }
+    return xfthip_gemm(w, M, A, lda, C, ldc, c_dtype, epi, bias, res, ldres, res_dtype, 1.0f, st);
+}
+
+// grows the model's W8A8 scratch for a weight with K input rows (called when weights are attached)
+static int w8a8_reserve(xfthip_model *m, const PackedWeight &pw, bool gateup) {
+    if (pw.kind != XFTHIP_W_W8A8) return 0;
+    const size_t need = (size_t)m->cfg.max_tokens * ((pw.K + 15) / 16 * 16);
+    if (need > m->w8a8_qa_bytes) {
+        XFT_CHECK_HIP(hipDeviceSynchronize());
+        if (m->w8a8_qa) (void)hipFree(m->w8a8_qa);
+        m->w8a8_qa = nullptr;
+        XFT_CHECK_HIP(hipMalloc((void **)&m->w8a8_qa, need));
+        m->w8a8_qa_bytes = need;
+    }
+    if (!m->w8a8_stat) XFT_CHECK_HIP(hipMalloc((void **)&m->w8a8_stat, (size_t)m->cfg.max_tokens * 3 * sizeof(float)));
+    if (gateup && !m->gu) XFT_CHECK_HIP(hipMalloc((void **)&m->gu, (size_t)m->cfg.max_tokens * pw.N * 2));
+    return 0;
+}
+
 // attention half of a layer: x_out = Attn(norm?(x_in)) * Wo + bias + x_in
 static int attention_block(xfthip_model *m, int idx, const float *x_in, int in_stride, float *x_out, int out_stride, int B,
         int S, int past, const int *past_dev, bool do_norm, hipStream_t st) {
@@ -305,8 +352,8 @@ static int attention_block(xfthip_model *m, int idx, const float *x_in, int in_s
         }
         if ((rc = qgemm_skinny(wq, sp, st))) return rc;
     } else {
-        if ((rc = xfthip_gemm(L.qkv, T, m->xn, c.hidden, m->qkv, qkv_cols, XFTHIP_BF16, L.qkv_bias ? XFTHIP_EPI_BIAS : XFTHIP_EPI_NONE,
-                     L.qkv_bias, nullptr, 0, XFTHIP_F32, 1.0f, st)))
+        if ((rc = model_gemm(m, L.qkv, T, m->xn, c.hidden, m->qkv, qkv_cols, XFTHIP_BF16, L.qkv_bias ? XFTHIP_EPI_BIAS : XFTHIP_EPI_NONE,
+                     L.qkv_bias, nullptr, 0, XFTHIP_F32, st)))
             return rc;
     }
     if (!fuse_rope)
@@ -322,8 +369,8 @@ static int attention_block(xfthip_model *m, int idx, const float *x_in, int in_s
     if ((rc = attention_launch(attend, m->qkv, qkv_cols, m->att, qcols, XFTHIP_BF16, B, S, c.q_heads, 1.0f / sqrtf((float)c.head_size), past,
                  past_dev, past_dev ? m->len_hint : 0, st, &m->attn_ws)))
         return rc;
-    return xfthip_gemm(L.o, T, m->att, qcols, x_out, out_stride, XFTHIP_F32, XFTHIP_EPI_RESIDENTIAL, L.o_bias, x_in, in_stride,
-            XFTHIP_F32, 1.0f, st);
+    return model_gemm(m, L.o, T, m->att, qcols, x_out, out_stride, XFTHIP_F32, XFTHIP_EPI_RESIDENTIAL, L.o_bias, x_in, in_stride,
+            XFTHIP_F32, st);
 }
 
 // MLP half of a layer: x_out = (silu(xn Wgate) * (xn Wup)) Wdown + x_in, xn = norm?(x_in)
@@ -353,10 +400,18 @@ static int mlp_block(xfthip_model *m, int idx, const float *x_in, int in_stride,
         } else {
             hipLaunchKernelGGL(narrow_rows_kernel, dim3(T), dim3(256), 0, st, x_in, in_stride, m->xn, c.hidden);
         }
-        if ((rc = xfthip_gemm_gateup_silu(L.gateup, T, m->xn, c.hidden, m->h, c.intermediate, XFTHIP_BF16, st))) return rc;
+        if (wg.kind == XFTHIP_W_W8A8) {
+            // cat(gate, up) as one plain int8 GEMM, then SwiGLU (the reference's own order of work)
+            if ((rc = model_gemm(m, L.gateup, T, m->xn, c.hidden, m->gu, 2 * c.intermediate, XFTHIP_BF16, XFTHIP_EPI_NONE, nullptr, nullptr, 0,
+                         XFTHIP_F32, st)))
+                return rc;
+            hipLaunchKernelGGL(silu_mul_kernel, dim3(T), dim3(256), 0, st, m->gu, m->h, c.intermediate);
+        } else if ((rc = xfthip_gemm_gateup_silu(L.gateup, T, m->xn, c.hidden, m->h, c.intermediate, XFTHIP_BF16, st))) {
+            return rc;
+        }
     }
-    return xfthip_gemm(L.down, T, m->h, c.intermediate, x_out, out_stride, XFTHIP_F32, XFTHIP_EPI_RESIDENTIAL, nullptr, x_in, in_stride,
-            XFTHIP_F32, 1.0f, st);
+    return model_gemm(m, L.down, T, m->h, c.intermediate, x_out, out_stride, XFTHIP_F32, XFTHIP_EPI_RESIDENTIAL, nullptr, x_in, in_stride,
+            XFTHIP_F32, st);
 }
 
 // one layer on device buffers (x_in may alias x_out)
@@ -461,7 +516,7 @@ int xfthip_model_destroy(xfthip_model_t m) {
         if (L.qkv_bias) (void)hipFree(L.qkv_bias);
         if (L.o_bias) (void)hipFree(L.o_bias);
     }
-    void *bufs[] = {m->mega_trace, m->mega_layers, m->mega_ws, m->mega_sync, m->cosT, m->sinT, m->xn, m->qkv, m->att, m->h, m->x, m->xlast, m->logits, m->ids, m->pos, m->step, m->idlog,
+    void *bufs[] = {m->w8a8_qa, m->w8a8_stat, m->gu, m->mega_trace, m->mega_layers, m->mega_ws, m->mega_sync, m->cosT, m->sinT, m->xn, m->qkv, m->att, m->h, m->x, m->xlast, m->logits, m->ids, m->pos, m->step, m->idlog,
             m->embedding, m->final_norm};
     for (void *b : bufs)
         if (b) (void)hipFree(b);
@@ -482,6 +537,8 @@ int xfthip_model_set_attention(xfthip_model_t m, int idx, xfthip_weight_t qkv, x
     LayerW &L = m->layers[idx];
     L.qkv = qkv;
     L.o = o;
+    if (int rc = w8a8_reserve(m, qkv->pw, false)) return rc;
+    if (int rc = w8a8_reserve(m, o->pw, false)) return rc;
     int rc;
     if ((rc = upload_f32(&L.ln1, ln1_host, c.hidden))) return rc;
     if ((rc = upload_f32(&L.qkv_bias, qkv_bias_host, qkv_cols))) return rc;
@@ -498,14 +555,20 @@ int xfthip_model_set_mlp(xfthip_model_t m, int idx, xfthip_weight_t gateup, xfth
     XFT_REQUIRE(m && gateup && down, "xfthip_model_set_mlp: null argument");
     XFT_REQUIRE(idx >= 0 && idx < m->cfg.layers, "xfthip_model_set_mlp: layer %d out of range", idx);
     const xfthip_model_config &c = m->cfg;
-    XFT_REQUIRE(gateup->pw.K == c.hidden && gateup->pw.N == 2 * c.intermediate && (gateup->pw.flags & XFTHIP_WF_GATEUP),
-            "xfthip_model_set_mlp: gate/up weight must be [%d,%d] created with XFTHIP_WF_GATEUP", c.hidden, 2 * c.intermediate);
+    // W8A8 gate/up weights stay in plain cat(gate, up) column order: the int8 GEMM has no fused SwiGLU
+    const bool gu_w8a8 = gateup->pw.kind == XFTHIP_W_W8A8;
+    XFT_REQUIRE(gateup->pw.K == c.hidden && gateup->pw.N == 2 * c.intermediate
+                    && (gu_w8a8 ? !(gateup->pw.flags & XFTHIP_WF_GATEUP) : (gateup->pw.flags & XFTHIP_WF_GATEUP) != 0),
+            "xfthip_model_set_mlp: gate/up weight must be [%d,%d] created with XFTHIP_WF_GATEUP (W8A8: without it)", c.hidden,
+            2 * c.intermediate);
     XFT_REQUIRE(down->pw.K == c.intermediate && down->pw.N == c.hidden, "xfthip_model_set_mlp: down weight is [%d,%d], expected [%d,%d]",
             down->pw.K, down->pw.N, c.intermediate, c.hidden);
     LayerW &L = m->layers[idx];
     L.gateup = gateup;
     L.down = down;
     if (int rc = upload_f32(&L.ln2, ln2_host, c.hidden)) return rc;
+    if (int rc = w8a8_reserve(m, gateup->pw, true)) return rc;
+    if (int rc = w8a8_reserve(m, down->pw, false)) return rc;
     if (m->graph) {
         (void)hipGraphExecDestroy(m->graph);
         m->graph = nullptr;

@@ -37,6 +37,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
+MFMA_INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA, published
 
 CFG = dict(layers=32, hidden=4096, inter=11008, q_heads=32, kv_heads=32, head=128, vocab=32000)
 
@@ -356,11 +357,11 @@ def prefill_gemm_sweep(xh, M=2048, nweights=8, iters=3):
     for (N, K) in ((4096, 4096), (11008, 4096), (4096, 11008)):
         A = xh.DeviceBuffer.from_numpy(xh.f32_to_bf16_bits(rng.standard_normal((M, K), dtype=np.float32)))
         Cd = xh.DeviceBuffer(M * N * 2)
-        for kind, name in ((xh.W_INT8, "int8"), (xh.W_UINT4, "uint4"), (xh.W_NF4, "nf4")):
-            q, sc, z = synth_codes(rng, 0 if kind == xh.W_INT8 else 1, K, N)
+        for kind, name in ((xh.W_INT8, "int8"), (xh.W_UINT4, "uint4"), (xh.W_NF4, "nf4"), (xh.W_W8A8, "w8a8")):
+            q, sc, z = synth_codes(rng, 0 if kind in (xh.W_INT8, xh.W_W8A8) else 1, K, N)
             if kind == xh.W_NF4:
                 z = None
-            nw = nweights * (2 if (kind != xh.W_INT8 and N * K <= 4096 * 4096) else 1)
+            nw = nweights * (2 if (kind in (xh.W_UINT4, xh.W_NF4) and N * K <= 4096 * 4096) else 1)
             ws = [xh.Weight(kind, K, N, q, sc, z) for _ in range(nw)]
             for w in ws:
                 xh.gemm(w, A.ptr, M, K, Cd.ptr, N, xh.BF16)
@@ -372,8 +373,12 @@ def prefill_gemm_sweep(xh, M=2048, nweights=8, iters=3):
                     xh.gemm(w, A.ptr, M, K, Cd.ptr, N, xh.BF16)
             us = t.stop() * 1e3 / (iters * nw)
             tf = 2.0 * M * N * K / us / 1e6
-            res.append(dict(kind=name, M=M, N=N, K=K, avg_launch_us=round(us, 2), tflops=round(tf, 1),
-                            frac_of_bf16_mfma_peak=round(tf / MFMA_BF16_PEAK_TFLOPS, 4)))
+            if kind == xh.W_W8A8:  # per-row activation quantisation + int8 MFMA GEMM, against the int8 peak
+                res.append(dict(kind=name, M=M, N=N, K=K, avg_launch_us=round(us, 2), tops=round(tf, 1),
+                                frac_of_int8_mfma_peak=round(tf / MFMA_INT8_PEAK_TOPS, 4)))
+            else:
+                res.append(dict(kind=name, M=M, N=N, K=K, avg_launch_us=round(us, 2), tflops=round(tf, 1),
+                                frac_of_bf16_mfma_peak=round(tf / MFMA_BF16_PEAK_TFLOPS, 4)))
             for w in ws:
                 w.free()
     return res

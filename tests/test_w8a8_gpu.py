@@ -69,3 +69,51 @@ def test_w8a8_gemm_vs_oracle(xh, orc, M, K, N):
     exp2 = orc.qgemm(w, A, orc.EPI_RESIDENTIAL, bias=bias, res=res)
     assert np.abs(cd.to_numpy(np.float32, (M, N)) - exp2).max() < 1e-5
     dw.free()
+
+
+@pytest.mark.parametrize("M,K,N", [(256, 4096, 1024), (2048, 1024, 1024), (100, 1008, 176), (2011, 512, 4096)])
+def test_w8a8_large_m_bit_exact(xh, orc, M, K, N):
+    """More than 32 rows take the block-tiled int8 MFMA kernel: the same integers and the same
+    dequantisation order as the M <= 32 kernel, so still bit-identical to the oracle."""
+    print(f"case M={M} K={K} N={N}", flush=True)
+    rng = np.random.default_rng(M + K + N)
+    w = orc.quantize(orc.W_W8A8, (rng.standard_normal((K, N)) * 0.02).astype(np.float32))
+    w.zero = (rng.standard_normal(N) * 0.002).astype(np.float32)
+    A = orc.round_bf16(rng.standard_normal((M, K)) + 0.2)
+    dw = xh.Weight(xh.W_W8A8, K, N, w.q, w.scale, w.zero)
+    ad = xh.DeviceBuffer.from_numpy(orc.to_bf16(A))
+    cd = xh.DeviceBuffer(M * N * 4)
+    xh.gemm(dw, ad.ptr, M, K, cd.ptr, N, xh.F32)
+    xh.synchronize()
+    got = cd.to_numpy(np.float32, (M, N))
+    exp = orc.qgemm(w, A)
+    assert np.array_equal(got.view(np.uint32), exp.view(np.uint32)), np.abs(got - exp).max()
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    qa, s, z, sm, ldq = xh.w8a8_quantize_rows(ad.ptr, xh.BF16, M, K, K)
+    rd, bd = xh.DeviceBuffer.from_numpy(res), xh.DeviceBuffer.from_numpy(bias)
+    for epi in (xh.EPI_RESIDENTIAL, xh.EPI_BIAS, xh.EPI_SILU):
+        xh.gemm_w8a8(dw, M, qa, ldq, s, z, sm, cd.ptr, N, xh.F32, epi, bd.ptr, rd.ptr, N)
+        xh.synchronize()
+        e2 = orc.qgemm(w, A, epi, bias=bias, res=res)
+        assert np.abs(cd.to_numpy(np.float32, (M, N)) - e2).max() < 2e-4
+    dw.free()
+
+
+def test_w8a8_model_shape_rows_2048(xh, orc):
+    """[2048, 4096] x [4096, 4096] at the model's size: sampled rows against the oracle (rows are
+    independent in this path), every output finite."""
+    M, K, N = 2048, 4096, 4096
+    rng = np.random.default_rng(5)
+    w = orc.quantize(orc.W_W8A8, (rng.standard_normal((K, N)) * 0.02).astype(np.float32))
+    A = orc.round_bf16(rng.standard_normal((M, K)))
+    dw = xh.Weight(xh.W_W8A8, K, N, w.q, w.scale, w.zero)
+    ad = xh.DeviceBuffer.from_numpy(orc.to_bf16(A))
+    cd = xh.DeviceBuffer(M * N * 4)
+    xh.gemm(dw, ad.ptr, M, K, cd.ptr, N, xh.F32)
+    xh.synchronize()
+    got = cd.to_numpy(np.float32, (M, N))
+    assert np.isfinite(got).all()
+    rows = np.array([0, 1, 31, 32, 127, 128, 1000, 2046, 2047])
+    exp = orc.qgemm(w, A[rows])
+    assert np.array_equal(got[rows].view(np.uint32), exp.view(np.uint32))

@@ -214,6 +214,188 @@ static int launch_w8a8(const W8A8Params &p, hipStream_t stream) {
     return 0;
 }
 
+// ---- many activation rows (M > 32): block-tiled int8 MFMA GEMM ------------------------------------
+// A workgroup of 4 waves computes a (4 * WN * 32 columns) x (WM * 32 rows) tile with
+// v_mfma_i32_32x32x32_i8.  The quantised activation rows are the "A" operand, shared by the four
+// waves through a double-buffered LDS tile (64 k bytes per row and step); the packed INT8 weight is
+// the "B" operand: lane (column nl, k half h) of k step s finds its 16 K-consecutive codes at
+// lane slot (2 s + h) * 16 + (nl & 15) of the 1-KiB tile of column tile nl >> 4, so weights go from
+// HBM to the matrix core with one 128-bit load per lane and no ALU work, and every weight tile is
+// read once per block of WM * 32 rows.  Integer accumulation is exact; the dequantisation is the
+// same expression, evaluated in the same order, as in the M <= 32 kernel: bit-identical results.
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+
+template <int WN, int WM>
+__global__ __launch_bounds__(256) void w8a8_mfma_kernel(W8A8Params p, int nblocks_n, int nblocks_m) {
+    constexpr int ROWS = 32 * WM, ROWB = 64 + 16; // padded LDS row pitch in bytes
+    constexpr int CHUNKS = ROWS * 4; // 16-byte chunks of an activation tile
+    constexpr int ALOADS = (CHUNKS + 255) / 256;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_a[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int h = lane >> 5, nl = lane & 31;
+    // block -> (column block, row block): blocks that share a column block sit on the same XCD
+    int nb, mb;
+    {
+        const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
+        const int nb8 = (nblocks_n + 7) >> 3;
+        nb = (slot / nblocks_m) + xcd * nb8;
+        mb = slot % nblocks_m;
+        if (slot / nblocks_m >= nb8 || nb >= nblocks_n) return;
+    }
+    const int n32_0 = (nb * 4 + wave) * WN;
+    const int m0 = mb * ROWS;
+
+    i32x16 acc[WN][WM];
+#pragma unroll
+    for (int t = 0; t < WN; ++t)
+#pragma unroll
+        for (int m = 0; m < WM; ++m)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) acc[t][m][j] = 0;
+
+    const uint8_t *wbase[WN];
+#pragma unroll
+    for (int t = 0; t < WN; ++t) {
+        int nt = (n32_0 + t) * 2 + (nl >> 4);
+        nt = nt < p.NTILES ? nt : p.NTILES - 1;
+        wbase[t] = p.packed + (size_t)nt * p.KT * 1024 + h * 256 + (nl & 15) * 16;
+    }
+    const int a_kc = threadIdx.x & 3, a_row0 = threadIdx.x >> 2;
+    const int8_t *a_src[ALOADS];
+#pragma unroll
+    for (int i = 0; i < ALOADS; ++i) {
+        int row = m0 + a_row0 + 64 * i;
+        row = row < p.M ? row : p.M - 1;
+        a_src[i] = p.qa + (size_t)row * p.ldq + a_kc * 16;
+    }
+    const i32x4 zero4 = {0, 0, 0, 0};
+    i32x4 wreg[2][2][WN], areg[ALOADS];
+    auto load_w = [&](int buf, int kt) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int t = 0; t < WN; ++t) wreg[buf][s][t] = *(const i32x4 *)(wbase[t] + (size_t)kt * 1024 + s * 512);
+    };
+    auto load_a = [&](int kt) {
+        // chunk inside the row iff kt * 64 + 16 a_kc + 16 <= K (K % 16 == 0); otherwise the row start is read and dropped
+        const bool v = kt * 64 + a_kc * 16 + 16 <= p.K;
+#pragma unroll
+        for (int i = 0; i < ALOADS; ++i) {
+            const i32x4 a = *(const i32x4 *)(a_src[i] + (v ? kt * 64 : -a_kc * 16));
+            areg[i] = v ? a : zero4;
+        }
+    };
+    auto store_a = [&](int buf) {
+        unsigned char *dst = lds_a + buf * (ROWS * ROWB);
+#pragma unroll
+        for (int i = 0; i < ALOADS; ++i)
+            if (a_row0 + 64 * i < ROWS) *(i32x4 *)(dst + (a_row0 + 64 * i) * ROWB + a_kc * 16) = areg[i];
+    };
+    auto compute = [&](int wb, int ab) {
+        const unsigned char *src = lds_a + ab * (ROWS * ROWB) + nl * ROWB + 16 * h;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            i32x4 a[WM];
+#pragma unroll
+            for (int m = 0; m < WM; ++m) a[m] = *(const i32x4 *)(src + m * 32 * ROWB + 32 * s);
+#pragma unroll
+            for (int t = 0; t < WN; ++t)
+#pragma unroll
+                for (int m = 0; m < WM; ++m) acc[t][m] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[m], wreg[wb][s][t], acc[t][m], 0, 0, 0);
+        }
+    };
+#define XFT_FENCE() __builtin_amdgcn_sched_barrier(0)
+    const int kt_n = (p.K + 63) / 64;
+    load_w(0, 0);
+    load_a(0);
+    store_a(0);
+    __syncthreads();
+    int kt = 0;
+    for (; kt + 2 <= kt_n - 1; kt += 2) {
+        load_w(1, kt + 1);
+        load_a(kt + 1);
+        XFT_FENCE();
+        compute(0, 0);
+        XFT_FENCE();
+        store_a(1);
+        __syncthreads();
+        load_w(0, kt + 2);
+        load_a(kt + 2);
+        XFT_FENCE();
+        compute(1, 1);
+        XFT_FENCE();
+        store_a(0);
+        __syncthreads();
+    }
+    if (kt + 1 < kt_n) {
+        load_w(1, kt + 1);
+        load_a(kt + 1);
+        XFT_FENCE();
+        compute(0, 0);
+        XFT_FENCE();
+        store_a(1);
+        __syncthreads();
+        compute(1, 1);
+    } else {
+        compute(0, 0);
+    }
+#undef XFT_FENCE
+
+    // ---- epilogue: lane holds C[m0 + 32 m + 8 (j / 4) + 4 h + j % 4][32 (n32_0 + t) + nl] ----------
+#pragma unroll
+    for (int t = 0; t < WN; ++t) {
+        const int np = (n32_0 + t) * 32 + nl;
+        if (np >= p.N) continue;
+        const float sB = p.scaleB[np], zB = p.zeroB ? p.zeroB[np] : 0.0f, sumB = p.sumB[np];
+        const float bias = p.bias ? p.bias[np] : 0.0f;
+#pragma unroll
+        for (int m = 0; m < WM; ++m) {
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int row = m0 + 32 * m + 8 * (j >> 2) + 4 * h + (j & 3);
+                if (row >= p.M) continue;
+                // C = s32*sA*sB + sumB*sB*zA + sumA*zB, evaluated left to right without contraction
+                const float t0 = ((float)acc[t][m][j] * p.sA[row]) * sB;
+                const float t1 = (sumB * sB) * p.zA[row];
+                const float t2 = p.sumA[row] * zB;
+                float x = (t0 + t1) + t2;
+                switch (p.epi) {
+                    case XFTHIP_EPI_BIAS: x += bias; break;
+                    case XFTHIP_EPI_SILU: x = x / (1.0f + fast_exp(-x)); break;
+                    case XFTHIP_EPI_GELU: {
+                        float e = fast_exp(1.702f * x);
+                        x = e / (e + 1.0f) * x;
+                        break;
+                    }
+                    case XFTHIP_EPI_RESMUL: x *= load_as_f32(p.res, p.res_dtype, (size_t)row * p.ldres + np); break;
+                    case XFTHIP_EPI_RESIDENTIAL:
+                        if (p.bias) x += bias;
+                        x += load_as_f32(p.res, p.res_dtype, (size_t)row * p.ldres + np);
+                        break;
+                    case XFTHIP_EPI_RESEXT:
+                        if (p.bias) x += bias;
+                        x = fmaf(p.gamma, load_as_f32(p.res, p.res_dtype, (size_t)row * p.ldres + np), x);
+                        break;
+                    default: break;
+                }
+                store_from_f32(p.C, p.c_dtype, (size_t)row * p.ldc + np, x);
+            }
+        }
+    }
+}
+
+template <int WN, int WM>
+static int launch_w8a8_mfma(const W8A8Params &p, hipStream_t stream) {
+    const int n32 = (p.NTILES + 1) / 2;
+    const int nblocks_n = (n32 + 4 * WN - 1) / (4 * WN);
+    const int nblocks_m = (p.M + 32 * WM - 1) / (32 * WM);
+    const int blocks = ((nblocks_n + 7) / 8) * 8 * nblocks_m;
+    const size_t smem = 2 * (size_t)(32 * WM) * (64 + 16);
+    hipLaunchKernelGGL((w8a8_mfma_kernel<WN, WM>), dim3(blocks), dim3(256), smem, stream, p, nblocks_n, nblocks_m);
+    XFT_CHECK_HIP(hipGetLastError());
+    return 0;
+}
+
 // scratch for the quantised activations of xfthip_gemm on a W8A8 weight (grown on demand)
 static int8_t *g_qa = nullptr;
 static float *g_qstat = nullptr;
@@ -251,6 +433,19 @@ int xfthip_gemm_w8a8(xfthip_weight_t w, int M, const int8_t *qa, int ldq, const 
     XFT_REQUIRE(!needs_res || (res && ldres >= pw.N), "xfthip_gemm_w8a8: epilogue %d needs res with ldres >= N", epilogue);
     const size_t csz = c_dtype == XFTHIP_F32 ? 4 : 2, rsz = res_dtype == XFTHIP_F32 ? 4 : 2;
     const int cus = device_cu_count();
+    if (M > 32) {
+        // block-tiled kernel: every weight tile is read once per 128 (or 64) rows
+        W8A8Params p = {};
+        p.packed = pw.packed, p.scaleB = pw.scale, p.zeroB = pw.zero, p.sumB = pw.colsum;
+        p.KT = pw.KT, p.NTILES = pw.NTILES, p.K = pw.K, p.N = pw.N, p.M = M;
+        p.qa = qa, p.ldq = ldq, p.sA = scaleA, p.zA = zeroA, p.sumA = sumA;
+        p.C = C, p.ldc = ldc, p.c_dtype = c_dtype, p.epi = epilogue, p.bias = bias;
+        p.res = res, p.ldres = ldres, p.res_dtype = res_dtype, p.gamma = gamma;
+        const int n32 = (pw.NTILES + 1) / 2;
+        const long t_large = (long)((n32 + 7) / 8) * ((M + 127) / 128);
+        if (t_large >= cus) return launch_w8a8_mfma<2, 4>(p, (hipStream_t)stream);
+        return launch_w8a8_mfma<1, 2>(p, (hipStream_t)stream);
+    }
     for (int m0 = 0; m0 < M; m0 += 32) {
         W8A8Params p = {};
         p.packed = pw.packed;

@@ -1,0 +1,100 @@
+// xft::Model / xft::AutoModel: a model directory on disk driven to generated token ids.
+// Source-compatible with the generation loop of the reference's include/models.h:25-133
+//     AutoModel model(path, xft::DataType::int8);
+//     model.config(maxLen); model.input(ids, batch);
+//     while (!model.isDone()) model.generate();
+//     auto out = model.finalize();
+// for Llama-family model directories (config.ini + .bin files as the reference's convert tools
+// write them, src/models/common_decoder.h:167-262, src/layers/decoder_block.h:205-343) on one
+// MI355X.  Greedy search and sampling (top-k / top-p / temperature, repetition penalty, stop
+// words) are served; beam search, prefix sharing and the sequence-id (continuous batching)
+// overloads print a message and exit(-1), the reference's style for an unsupported request.
+// The declarations follow intel/xFasterTransformer (Apache-2.0, Copyright (c) Intel Corporation).
+#pragma once
+
+#include <cstdint>
+#include <string>
+#include <tuple>
+#include <vector>
+
+#include "abstract_searcher.h"
+#include "dtype.h"
+
+namespace xft {
+
+struct ModelImpl; // device model, weights and searcher state (private to the library)
+
+class Model {
+public:
+    Model();
+    ~Model();
+    Model(const Model &) = delete;
+    Model &operator=(const Model &) = delete;
+
+    // inputIds_: batchSize_ prompts of equal length, row-major (models.cpp:99-115)
+    void input(std::vector<int32_t> &inputIds_, int batchSize_);
+
+    void config(int maxLen_ = -1, int numBeams_ = 1, int numBeamHypsToKeep_ = 1, float lenPenalty_ = 1.0,
+            bool doEarlyStopping_ = false, int eosTokenId_ = -1, int padTokenId_ = -1, bool doSample_ = false,
+            float temperature_ = 1.0, int topK_ = 50, float topP_ = 1.0, float repetitionPenalty_ = 1.0,
+            const std::vector<std::vector<int>> &stopWordsList_ = {});
+
+    void config(SearcherConfig &config_, const std::vector<std::vector<int>> &stopWordsList_ = {});
+
+    bool isDone();
+
+    // Logits of the next token: (host pointer to fp32 [batch, vocab], 0, vocab).  Only
+    // logitsAll = false is served (the last position of each sequence).
+    std::tuple<float *, int, int> forward(bool logitsAll = true);
+
+    // One step: the first call after input() runs the prompt, every later call one new token per
+    // sequence.  Returns the batch's next token ids (models.cpp:834-846).
+    std::vector<int32_t> generate();
+
+    bool isMaster() { return true; }
+
+    int getRank() { return 0; }
+
+    int getBatchSize() { return batchSize; }
+
+    int getSeqLen() { return seqLen; }
+
+    void setVocabSize(int vocabSize) { this->vocabSize = vocabSize; }
+
+    int getVocabSize() { return this->vocabSize; }
+
+    int getMaxSeqLen() { return maxSeqLen; }
+
+    SearcherConfig getConfig() { return configuration; }
+
+    // prompt + generated ids of every sequence, row-major [batch, current length]
+    std::vector<int32_t> finalize();
+
+    void exitSlaves() {}
+
+    bool setStopWords(std::vector<std::vector<int>> stopWordsList);
+
+    // not served by this build (print + exit(-1))
+    void setPrefix(std::vector<int32_t> &prefixIDs);
+    void unsetPrefix();
+    bool freeSeqs(std::vector<int> &seqIDs);
+    std::vector<int> set_input(std::vector<int32_t> &inputIds_, int batchSize_, SearcherConfig &config_,
+            const std::vector<std::vector<int>> &stopWordsList_ = {});
+
+protected:
+    ModelImpl *impl;
+    std::vector<int32_t> inputIds;
+    int batchSize;
+    int seqLen;
+    int vocabSize;
+    int maxSeqLen;
+    SearcherConfig configuration;
+    bool isNewInput;
+};
+
+class AutoModel : public Model {
+public:
+    AutoModel(std::string modelPath, xft::DataType dataType, xft::DataType KVCacheDataType = xft::DataType::fp16);
+};
+
+} // namespace xft

@@ -377,6 +377,11 @@ int xfthip_model_persistent_trace(xfthip_model_t m, unsigned long long *ticks_ho
 int xfthip_model_decode_mode(xfthip_model_t m);
 /* ids chosen by the last prefill / decode call (host int32 [B]) and the current position */
 int xfthip_model_last_ids(xfthip_model_t m, int *ids_host, int *position);
+/* Replace the ids the next decode step embeds (host int32 [B], each inside the vocabulary): for
+ * searchers that do not take the arg-max of the raw logits (sampling, repetition penalty, padding of
+ * finished sequences: the nextTokens vector GreedySearch / SampleSearch feed back,
+ * src/searchers/greedy_search.cpp:112-119, sample_search.cpp:74-90). */
+int xfthip_model_set_next_ids(xfthip_model_t m, const int *ids_host, xfthip_stream_t stream);
 /* fp32 logits of the last step, device pointer [B, vocab] (valid until the next call) */
 int xfthip_model_logits(xfthip_model_t m, const float **logits_dev);
 

@@ -76,6 +76,42 @@ def test_host_layer_exports_reference_entry_points(tmp_path):
                            "-lxft_layers", "-lxft_hip", "-Wl,-rpath," + PKG])
 
 
+@pytest.mark.skipif(not os.path.exists(LIB_LAYERS), reason="host library not built")
+def test_host_layer_exports_the_model_classes(tmp_path):
+    """xft::AutoModel / xft::Model as include/models.h declares them (the generation loop of the
+    reference's examples: config, input, generate until isDone, finalize) link against the library."""
+    out = subprocess.check_output(["nm", "-DC", "--defined-only", LIB_LAYERS], text=True)
+    for fn in ("xft::AutoModel::AutoModel(", "xft::Model::generate()", "xft::Model::isDone()", "xft::Model::finalize()",
+               "xft::Model::input(", "xft::Model::config(", "xft::Model::setStopWords(", "xft_automodel_create",
+               "xft_sample_candidates"):
+        assert fn in out, fn
+    src = r'''
+    #include "models.h"
+    int main(int argc, char **argv) {
+        if (argc > 100) {  // never executed: link check only
+            xft::AutoModel model(argv[1], xft::DataType::int8, xft::DataType::fp16);
+            std::vector<int32_t> ids = {1, 2, 3, 4};
+            model.config(/*maxLen*/ 16, /*numBeams*/ 1, 1, 1.0f, false, /*eos*/ 2, /*pad*/ 0, /*doSample*/ true, 0.8f, 40, 0.9f, 1.1f,
+                    {{5, 6}});
+            SearcherConfig cfg(32);
+            model.config(cfg);
+            model.input(ids, 2);
+            while (!model.isDone()) { std::vector<int32_t> next = model.generate(); (void)next; }
+            std::vector<int32_t> all = model.finalize();
+            return (int)all.size() + model.getVocabSize() + model.getMaxSeqLen() + model.getBatchSize() + model.getSeqLen()
+                    + model.getRank() + (int)model.isMaster() + model.getConfig().maxLen;
+        }
+        return 0;
+    }
+    '''
+    cpp = str(tmp_path / "model_link_check.cpp")
+    exe = str(tmp_path / "model_link_check")
+    open(cpp, "w").write(src)
+    subprocess.check_call(["g++", "-std=c++17", "-I" + os.path.join(ROOT, "include"), cpp, "-o", exe, "-L" + PKG,
+                           "-lxft_layers", "-lxft_hip", "-Wl,-rpath," + PKG])
+    assert subprocess.run([exe]).returncode == 0
+
+
 def test_package_refuses_to_import_without_the_library(tmp_path):
     """The Python binding has no CPU fallback: without libxft_hip.so the import raises."""
     import shutil

@@ -76,11 +76,11 @@ def build_hip(force=True):
 
 
 def build_host(force=True):
-    """The C++ host layer (xft::invoke* entry points) over the C-ABI; plain g++, no HIP headers."""
-    src = os.path.join(CSRC, "host", "xft_layers.cpp")
-    deps = [src] + glob.glob(os.path.join(ROOT, "include", "*.h")) + [LIB_HIP]
+    """The C++ host layer (xft::invoke* entry points, xft::AutoModel) over the C-ABI; plain g++, no HIP headers."""
+    srcs = sorted(glob.glob(os.path.join(CSRC, "host", "*.cpp")))
+    deps = srcs + glob.glob(os.path.join(CSRC, "host", "*.h")) + glob.glob(os.path.join(ROOT, "include", "*.h")) + [LIB_HIP]
     if force or _stale(LIB_LAYERS, deps):
-        _run([os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", src, "-o", LIB_LAYERS,
+        _run([os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"] + srcs + ["-o", LIB_LAYERS,
               "-L" + HERE, "-lxft_hip", "-Wl,-rpath,$ORIGIN"])
     return LIB_LAYERS
 

@@ -389,6 +389,10 @@ class Model:
     def decode_mode(self):
         return int(lib.xfthip_model_decode_mode(self.h))
 
+    def set_next_ids(self, ids, stream=None):
+        ids = np.ascontiguousarray(ids, np.int32)
+        check(lib.xfthip_model_set_next_ids(self.h, _hp(ids), stream))
+
     def last_ids(self, B):
         ids = np.empty(B, np.int32)
         pos = C.c_int()

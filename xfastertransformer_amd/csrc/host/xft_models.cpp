@@ -1,0 +1,881 @@
+// xft::Model / xft::AutoModel over the C-ABI of the gfx950 library: the on-disk model format of the
+// reference (config.ini + one .bin per tensor) loaded into a device-resident decoder stack, and
+// the searchers that turn its logits into token ids.
+//
+// Replaces, for Llama-family directories on one GPU:
+//   AutoModel::AutoModel / Model::input / config / generate / isDone / finalize (src/models/models.cpp:99-135,
+//   706-758, 834-846, 1014-1035), CommonDecoder's constructor (src/models/common_decoder.h:167-262: the
+//   config.ini keys), DecoderBlock's weight loading (src/layers/decoder_block.h:205-343: the file names and
+//   shapes), CommonDecoder::setEmbeddingWeights / setFinalLnWeight / setPredictorWeight
+//   (common_decoder.h:857-874, llama.cpp:46-51), GreedySearch and SampleSearch
+//   (src/searchers/greedy_search.cpp, sample_search.cpp) and the repetition penalty / stop-word helpers
+//   (src/searchers/search_utils.cpp:22-99).
+// Plain C++ (g++), no HIP headers.  Failures print a message and exit(-1), as the reference does.
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <functional>
+#include <map>
+#include <random>
+#include <set>
+#include <string>
+#include <vector>
+
+#include "../../../include/models.h"
+#include "../../../include/xft_hip.h"
+#include "host_util.h"
+
+using namespace xfthost;
+
+namespace {
+
+// ---- config.ini ---------------------------------------------------------------------------------
+// Section / key lookup is case-insensitive and the "first" section is the smallest name of an ordered
+// set, the behaviour of the INIReader the reference uses (models.cpp:1023: *reader.Sections().begin()).
+struct Ini {
+    std::set<std::string> sections;
+    std::map<std::string, std::string> values;
+    bool ok = false;
+
+    static std::string lower(std::string s) {
+        for (auto &c : s) c = (char)tolower((unsigned char)c);
+        return s;
+    }
+    static std::string trim(const std::string &s) {
+        size_t a = 0, b = s.size();
+        while (a < b && isspace((unsigned char)s[a])) ++a;
+        while (b > a && isspace((unsigned char)s[b - 1])) --b;
+        return s.substr(a, b - a);
+    }
+    explicit Ini(const std::string &path) {
+        FILE *f = fopen(path.c_str(), "r");
+        if (!f) return;
+        ok = true;
+        char line[4096];
+        std::string section;
+        while (fgets(line, sizeof(line), f)) {
+            std::string s = trim(line);
+            if (s.empty() || s[0] == ';' || s[0] == '#') continue;
+            if (s[0] == '[') {
+                const size_t e = s.find(']');
+                if (e == std::string::npos) continue;
+                section = trim(s.substr(1, e - 1));
+                sections.insert(section);
+                continue;
+            }
+            size_t eq = s.find_first_of("=:");
+            if (eq == std::string::npos) continue;
+            std::string key = trim(s.substr(0, eq)), val = trim(s.substr(eq + 1));
+            // an inline comment starts at " ;" or " #"
+            for (size_t i = 1; i < val.size(); ++i)
+                if ((val[i] == ';' || val[i] == '#') && isspace((unsigned char)val[i - 1])) {
+                    val = trim(val.substr(0, i));
+                    break;
+                }
+            values[lower(section) + "=" + lower(key)] = val;
+        }
+        fclose(f);
+    }
+    bool has(const std::string &sec, const std::string &key) const { return values.count(lower(sec) + "=" + lower(key)) != 0; }
+    std::string get(const std::string &sec, const std::string &key, const std::string &dflt = "") const {
+        auto it = values.find(lower(sec) + "=" + lower(key));
+        return it == values.end() ? dflt : it->second;
+    }
+    long get_int(const std::string &sec, const std::string &key, long dflt) const {
+        const std::string v = get(sec, key);
+        if (v.empty()) return dflt;
+        char *end = nullptr;
+        const long r = strtol(v.c_str(), &end, 0);
+        return end > v.c_str() ? r : dflt;
+    }
+    double get_float(const std::string &sec, const std::string &key, double dflt) const {
+        const std::string v = get(sec, key);
+        if (v.empty()) return dflt;
+        char *end = nullptr;
+        const double r = strtod(v.c_str(), &end);
+        return end > v.c_str() ? r : dflt;
+    }
+};
+
+bool file_exists(const std::string &p) {
+    FILE *f = fopen(p.c_str(), "rb");
+    if (!f) return false;
+    fclose(f);
+    return true;
+}
+
+// Reads `count` elements of `wtype` (fp32 / fp16 / bf16 as config.ini's weight_data_type names it,
+// src/utils/weight_util.h:37-67, 139-167) and widens them to fp32.  A missing optional file gives an
+// empty vector; a short or missing required file ends the process.
+std::vector<float> read_floats(const std::string &path, size_t count, xft::DataType wtype, bool required = true) {
+    std::vector<float> out;
+    FILE *f = fopen(path.c_str(), "rb");
+    if (!f) {
+        if (required) {
+            printf("Cannot open the weight file %s\n", path.c_str());
+            exit(-1);
+        }
+        return out;
+    }
+    out.resize(count);
+    size_t got = 0;
+    if (wtype == xft::DataType::fp32) {
+        got = fread(out.data(), 4, count, f);
+    } else {
+        std::vector<uint16_t> raw(count);
+        got = fread(raw.data(), 2, count, f);
+        if (wtype == xft::DataType::fp16)
+            for (size_t i = 0; i < got; ++i) out[i] = from_fp16(raw[i]);
+        else
+            for (size_t i = 0; i < got; ++i) out[i] = from_bf16(raw[i]);
+    }
+    fclose(f);
+    if (got != count) {
+        printf("Weight file %s holds %zu elements, %zu expected\n", path.c_str(), got, count);
+        exit(-1);
+    }
+    return out;
+}
+
+std::vector<uint8_t> read_bytes(const std::string &path, size_t count) {
+    std::vector<uint8_t> out(count);
+    FILE *f = fopen(path.c_str(), "rb");
+    if (!f) {
+        printf("Cannot open the weight file %s\n", path.c_str());
+        exit(-1);
+    }
+    const size_t got = fread(out.data(), 1, count, f);
+    fclose(f);
+    if (got != count) {
+        printf("Weight file %s holds %zu bytes, %zu expected\n", path.c_str(), got, count);
+        exit(-1);
+    }
+    return out;
+}
+
+const char *type_name(xft::DataType dt) {
+    switch (dt) {
+        case xft::DataType::fp32: return "fp32";
+        case xft::DataType::bf16: return "bf16";
+        case xft::DataType::fp16: return "fp16";
+        case xft::DataType::int8: return "int8";
+        case xft::DataType::w8a8: return "w8a8";
+        case xft::DataType::int4: return "int4";
+        case xft::DataType::nf4: return "nf4";
+        case xft::DataType::bf16_fp16: return "bf16_fp16";
+        case xft::DataType::bf16_int8: return "bf16_int8";
+        case xft::DataType::bf16_w8a8: return "bf16_w8a8";
+        case xft::DataType::bf16_int4: return "bf16_int4";
+        case xft::DataType::bf16_nf4: return "bf16_nf4";
+        case xft::DataType::w8a8_int8: return "w8a8_int8";
+        case xft::DataType::w8a8_int4: return "w8a8_int4";
+        case xft::DataType::w8a8_nf4: return "w8a8_nf4";
+        case xft::DataType::fp8_e4m3: return "fp8_e4m3";
+        default: return "unknown";
+    }
+}
+
+// One [K, N] matrix of the directory, in whichever form the files hold it.
+struct HostMatrix {
+    int K = 0, N = 0;
+    std::vector<float> w; // fp32 [K, N] (plain files)
+    int qkind = -1; // XFTHIP_W_INT8 / XFTHIP_W_UINT4 when the directory is pre-quantised
+    std::vector<uint8_t> q;
+    std::vector<float> scale, zero;
+};
+
+// horizontal concatenation of matrices with the same K: [K, sum N]
+HostMatrix hcat(const std::vector<const HostMatrix *> &parts) {
+    HostMatrix out;
+    out.K = parts[0]->K;
+    out.qkind = parts[0]->qkind;
+    for (auto *p : parts) out.N += p->N;
+    if (out.qkind < 0) {
+        out.w.resize((size_t)out.K * out.N);
+        int off = 0;
+        for (auto *p : parts) {
+            for (int k = 0; k < out.K; ++k) memcpy(&out.w[(size_t)k * out.N + off], &p->w[(size_t)k * p->N], sizeof(float) * p->N);
+            off += p->N;
+        }
+        return out;
+    }
+    const int per = out.qkind == XFTHIP_W_UINT4 ? 2 : 1; // columns per byte
+    out.q.resize((size_t)out.K * out.N / per);
+    int off = 0;
+    for (auto *p : parts) {
+        for (int k = 0; k < out.K; ++k)
+            memcpy(&out.q[((size_t)k * out.N + off) / per], &p->q[(size_t)k * p->N / per], (size_t)p->N / per);
+        out.scale.insert(out.scale.end(), p->scale.begin(), p->scale.end());
+        out.zero.insert(out.zero.end(), p->zero.begin(), p->zero.end());
+        off += p->N;
+    }
+    return out;
+}
+
+} // namespace
+
+namespace xft {
+
+struct ModelImpl {
+    std::string path, modelType;
+    xft::DataType fileType = xft::DataType::fp32;
+    int fileQuant = -1; // weight kind of pre-quantised files or -1
+    int wkind = XFTHIP_W_BF16;
+    int kvDtype = XFTHIP_FP16;
+    int layers = 0, hidden = 0, inter = 0, heads = 0, kvHeads = 0, headSize = 0, vocab = 0;
+    int maxPosEmbed = 0, maxPositions = 0, maxSeqLength = -1, startId = 0, endId = 0;
+    float eps = 1e-6f, ropeTheta = 10000.0f;
+
+    struct Layer {
+        xfthip_weight_t qkv = nullptr, o = nullptr, gateup = nullptr, down = nullptr;
+        std::vector<float> ln1, ln2, qkvBias, oBias;
+    };
+    std::vector<Layer> L;
+    std::vector<uint16_t> embedding;
+    std::vector<float> finalNorm;
+    xfthip_weight_t lmHead = nullptr;
+    size_t weightBytes = 0;
+
+    xfthip_model_t model = nullptr;
+    xfthip_model_config cfg {};
+
+    // searcher state (GreedySearch / SampleSearch members of the reference)
+    bool haveSearcher = false, sampling = false;
+    int maxLen = 0, eosTokenId = -1, padTokenId = -1, topK = 50;
+    float topP = 1.0f, temperatureInv = 1.0f, repetitionPenalty = 1.0f;
+    std::vector<std::vector<int>> stopWordsList, stopWordsIndex, cachedRepetVec;
+    std::vector<int> doneBatch, nextTokens, deviceIds;
+    std::vector<int32_t> output;
+    std::vector<float> logitsHost;
+    int step = 0, curLen = 0, batch = 0;
+    std::mt19937_64 rng {std::random_device {}()};
+
+    ModelImpl() {
+        // the reference seeds its sampler from std::random_device on every step (sample_search.cpp:229-231);
+        // XFT_SEED makes a run repeatable
+        if (const char *e = getenv("XFT_SEED")) rng.seed(strtoull(e, nullptr, 0));
+    }
+
+    ~ModelImpl() {
+        if (model) xfthip_model_destroy(model);
+        for (auto &l : L)
+            for (xfthip_weight_t w : {l.qkv, l.o, l.gateup, l.down})
+                if (w) xfthip_weight_destroy(w);
+        if (lmHead) xfthip_weight_destroy(lmHead);
+    }
+
+    std::string layer_file(int l, const std::string &name) const { return path + "/model.layers." + std::to_string(l) + "." + name; }
+
+    HostMatrix load_matrix(int l, const std::string &stem, int K, int N) const {
+        HostMatrix m;
+        m.K = K, m.N = N;
+        if (fileQuant >= 0) {
+            m.qkind = fileQuant;
+            m.q = read_bytes(layer_file(l, stem + ".qweight.0.bin"), (size_t)K * N / (fileQuant == XFTHIP_W_UINT4 ? 2 : 1));
+            m.zero = read_floats(layer_file(l, stem + ".zeros.0.bin"), N, xft::DataType::fp32);
+            m.scale = read_floats(layer_file(l, stem + ".scales.0.bin"), N, xft::DataType::fp32);
+        } else {
+            m.w = read_floats(layer_file(l, stem + ".weight.0.bin"), (size_t)K * N, fileType);
+        }
+        return m;
+    }
+
+    // Pre-quantised codes go to the device as they are when the requested type is the files' own
+    // (MMHelper::convertWeight's INT8->INT8 / UINT4->UINT4 copies, matmul_helper.h:284-315);
+    // anything else is dequantised (w = scale * q + zero) and converted like a plain matrix.
+    xfthip_weight_t to_device(HostMatrix &m, int flags) {
+        xfthip_weight_t h = nullptr;
+        if (m.qkind >= 0 && m.qkind == wkind) {
+            CK(xfthip_weight_create(wkind, m.K, m.N, m.q.data(), m.scale.data(), m.zero.data(), flags, &h));
+        } else {
+            if (m.qkind >= 0) {
+                m.w.resize((size_t)m.K * m.N);
+                for (int k = 0; k < m.K; ++k)
+                    for (int n = 0; n < m.N; ++n) {
+                        int code;
+                        if (m.qkind == XFTHIP_W_UINT4) {
+                            const uint8_t b = m.q[((size_t)k * m.N + n) / 2];
+                            code = (n & 1) ? (b >> 4) : (b & 15);
+                        } else {
+                            code = (int8_t)m.q[(size_t)k * m.N + n];
+                        }
+                        m.w[(size_t)k * m.N + n] = fmaf(m.scale[n], (float)code, m.zero[n]);
+                    }
+            }
+            h = make_weight(wkind, m.K, m.N, m.w.data(), flags);
+        }
+        weightBytes += xfthip_weight_bytes(h);
+        return h;
+    }
+
+    void load() {
+        const int qCols = heads * headSize, kvCols = kvHeads * headSize, qkvCols = qCols + 2 * kvCols;
+        L.resize(layers);
+        for (int l = 0; l < layers; ++l) {
+            Layer &y = L[l];
+            HostMatrix qkv = load_matrix(l, "attention.query_key_value", hidden, qkvCols);
+            y.qkv = to_device(qkv, XFTHIP_WF_NONE);
+            HostMatrix o = load_matrix(l, "attention.dense", qCols, hidden);
+            y.o = to_device(o, XFTHIP_WF_NONE);
+            if (file_exists(layer_file(l, fileQuant >= 0 ? "mlp.dense_h_to_4h.qweight.0.bin" : "mlp.dense_h_to_4h.weight.0.bin"))) {
+                printf("The model directory holds a two-matrix MLP (dense_h_to_4h); only gate/up/down MLPs are served.\n");
+                exit(-1);
+            }
+            {
+                HostMatrix gate = load_matrix(l, "mlp.gate_proj", hidden, inter);
+                HostMatrix up = load_matrix(l, "mlp.up_proj", hidden, inter);
+                HostMatrix gu = hcat({&gate, &up});
+                // the W8A8 path runs gate/up as one plain GEMM followed by silu(gate) * up
+                y.gateup = to_device(gu, wkind == XFTHIP_W_W8A8 ? XFTHIP_WF_NONE : XFTHIP_WF_GATEUP);
+            }
+            HostMatrix down = load_matrix(l, "mlp.down_proj", inter, hidden);
+            y.down = to_device(down, XFTHIP_WF_NONE);
+            y.ln1 = read_floats(layer_file(l, "input_layernorm.weight.bin"), hidden, fileType);
+            y.ln2 = read_floats(layer_file(l, "post_attention_layernorm.weight.bin"), hidden, fileType);
+            y.qkvBias = read_floats(layer_file(l, "attention.query_key_value.bias.0.bin"), qkvCols, fileType, false);
+            y.oBias = read_floats(layer_file(l, "attention.dense.bias.bin"), hidden, fileType, false);
+            if (file_exists(layer_file(l, "mlp.down_proj.bias.0.bin"))) {
+                printf("The model directory holds an MLP bias (layer %d); not served.\n", l);
+                exit(-1);
+            }
+        }
+        // embedding [vocab, hidden] kept in FP16 (src/layers/token_embedding.h:49-52)
+        {
+            std::vector<float> e = read_floats(path + "/model.wte.bin", (size_t)vocab * hidden, fileType);
+            embedding.resize(e.size());
+            for (size_t i = 0; i < e.size(); ++i) embedding[i] = to_fp16(e[i]);
+        }
+        finalNorm = read_floats(path + "/model.final_layernorm.weight.bin", hidden, fileType);
+        // lm_head is stored [vocab, hidden] (trans = true in DistLinear::setWeight, src/layers/dist_linear.h:55-80)
+        // and never quantised (common_decoder.h:1000-1001): transposed to [hidden, vocab] bf16 here
+        {
+            std::vector<float> w = read_floats(path + "/model.lm_head.weight.bin", (size_t)vocab * hidden, fileType);
+            std::vector<uint16_t> t((size_t)hidden * vocab);
+            for (int v = 0; v < vocab; ++v)
+                for (int h = 0; h < hidden; ++h) t[(size_t)h * vocab + v] = to_bf16(w[(size_t)v * hidden + h]);
+            CK(xfthip_weight_create(XFTHIP_W_BF16, hidden, vocab, t.data(), nullptr, nullptr, XFTHIP_WF_NONE, &lmHead));
+            weightBytes += xfthip_weight_bytes(lmHead);
+        }
+    }
+
+    // (re)build the device model when a call needs more batch / tokens / positions than it holds
+    void fit(int B, int S, int needLen) {
+        const bool grow = model == nullptr || B > cfg.max_batch || B * S > cfg.max_tokens || needLen > cfg.max_seq;
+        if (!grow) return;
+        if (model) CK(xfthip_model_destroy(model));
+        model = nullptr;
+        cfg.layers = layers, cfg.hidden = hidden, cfg.intermediate = inter;
+        cfg.q_heads = heads, cfg.kv_heads = kvHeads, cfg.head_size = headSize;
+        cfg.vocab = vocab;
+        cfg.max_batch = std::max(cfg.max_batch, B);
+        cfg.max_tokens = std::max(cfg.max_tokens, B * S);
+        cfg.max_seq = std::max(cfg.max_seq, needLen);
+        cfg.max_pos_embed = std::max(maxPosEmbed, cfg.max_seq);
+        cfg.rope_base = (int)ropeTheta;
+        cfg.kv_dtype = kvDtype;
+        cfg.rms_eps = eps;
+        CK(xfthip_model_create(&cfg, &model));
+        for (int l = 0; l < layers; ++l) {
+            Layer &y = L[l];
+            CK(xfthip_model_set_layer(model, l, y.qkv, y.o, y.gateup, y.down, y.ln1.data(), y.ln2.data(),
+                    y.qkvBias.empty() ? nullptr : y.qkvBias.data(), y.oBias.empty() ? nullptr : y.oBias.data()));
+        }
+        CK(xfthip_model_set_head(model, embedding.data(), finalNorm.data(), lmHead));
+    }
+
+    // ---- searchers ------------------------------------------------------------------------------
+    void fetch_logits() {
+        const float *dev = nullptr;
+        CK(xfthip_model_logits(model, &dev));
+        logitsHost.resize((size_t)batch * vocab);
+        CK(xfthip_memcpy_d2h(logitsHost.data(), dev, logitsHost.size() * 4, nullptr));
+    }
+
+    // search_utils.cpp:22-75 for one rank: the penalised set of a sequence is its prompt plus
+    // every token fed back so far
+    void repetition_penalty(float *logits) {
+        if (step == 1) {
+            const int S = (int)output.size() / batch;
+            cachedRepetVec.assign(batch, {});
+            for (int b = 0; b < batch; ++b) {
+                auto &v = cachedRepetVec[b];
+                v.assign(output.begin() + (size_t)b * S, output.begin() + (size_t)(b + 1) * S);
+                std::sort(v.begin(), v.end());
+                v.erase(std::unique(v.begin(), v.end()), v.end());
+            }
+        } else {
+            for (int b = 0; b < batch; ++b) {
+                auto &v = cachedRepetVec[b];
+                auto it = std::lower_bound(v.begin(), v.end(), nextTokens[b]);
+                if (it == v.end() || *it != nextTokens[b]) v.insert(it, nextTokens[b]);
+            }
+        }
+        for (int b = 0; b < batch; ++b)
+            for (int idx : cachedRepetVec[b]) {
+                if (idx < 0 || idx >= vocab) continue;
+                float &x = logits[(size_t)b * vocab + idx];
+                x = x < 0 ? x * repetitionPenalty : x / repetitionPenalty;
+            }
+    }
+
+    // greedy_search.cpp:270-287 / sample_search.cpp:245-265
+    void finish_tokens(std::vector<int> &ids) {
+        if (eosTokenId != -1)
+            for (int b = 0; b < batch; ++b) {
+                if (doneBatch[b] == 0) {
+                    if (ids[b] == eosTokenId) doneBatch[b] = 1;
+                } else if (doneBatch[b] > 0) {
+                    ids[b] = padTokenId;
+                } else {
+                    ids[b] = eosTokenId;
+                    doneBatch[b] = 1;
+                }
+            }
+        if (!stopWordsList.empty() && !stopWordsIndex.empty()) {
+            // search_utils.cpp:77-99
+            for (int b = 0; b < batch; ++b) {
+                if (doneBatch[b] != 0) continue;
+                for (size_t i = 0; i < stopWordsList.size(); ++i) {
+                    auto &words = stopWordsList[i];
+                    int &idx = stopWordsIndex[i][b];
+                    if (idx < (int)words.size()) {
+                        if (words[idx] == ids[b]) {
+                            if (++idx == (int)words.size()) doneBatch[b] = -1;
+                        } else {
+                            idx = 0;
+                        }
+                    } else {
+                        doneBatch[b] = -1;
+                    }
+                }
+            }
+        }
+    }
+};
+
+} // namespace xft
+
+// ---- the deterministic half of SampleSearch::sample (sample_search.cpp:154-226), exported so that it can
+// be checked on its own: the top-K candidates of one row (ordered by (value, id) descending, which
+// is what partial_sort with greater<pair<float,int>> produces), temperature, the top-P cut with
+// the reference's rule (at least 2 candidates; the candidate that crosses topP is left out once more
+// than 2 precede it) and the softmax over what is left.  Returns the number of candidates kept.
+extern "C" int xft_sample_candidates(const float *logits, int vocab, int topK, float topP, float temperature, int *ids_out,
+        float *probs_out) {
+    if (topK < 2) topK = 2;
+    if (topK > vocab) topK = vocab;
+    std::vector<std::pair<float, int>> el(vocab);
+    for (int j = 0; j < vocab; ++j) el[j] = std::make_pair(logits[j], j);
+    std::partial_sort(el.begin(), el.begin() + topK, el.end(), std::greater<std::pair<float, int>>());
+    const float tinv = 1 / temperature;
+    std::vector<float> vals(topK);
+    for (int j = 0; j < topK; ++j) {
+        vals[j] = el[j].first;
+        if (tinv != 1.0f) vals[j] *= tinv;
+        ids_out[j] = el[j].second;
+    }
+    int n = topK;
+    if (topP < 1.0f) {
+        std::vector<float> probs(topK);
+        float sum = 0, cur = 0;
+        for (int i = 0; i < topK; ++i) {
+            probs[i] = expf(vals[i]);
+            sum += probs[i];
+        }
+        const float inv = 1 / sum;
+        for (int i = 0; i < topK; ++i) {
+            cur += probs[i] * inv;
+            if (cur > topP) {
+                n = i > 2 ? i : 2;
+                break;
+            }
+        }
+    }
+    // softmax over the first n values (DecoderUtil::computeSoftmax, src/utils/decoder_util.h:298-340)
+    float mx = vals[0];
+    for (int i = 1; i < n; ++i) mx = std::max(mx, vals[i]);
+    float sum = 0;
+    for (int i = 0; i < n; ++i) {
+        probs_out[i] = expf(vals[i] - mx);
+        sum += probs_out[i];
+    }
+    const float inv = 1.0f / sum;
+    for (int i = 0; i < n; ++i) probs_out[i] *= inv;
+    return n;
+}
+
+// inverse-CDF draw of sample_search.cpp:232-243: the first candidate whose running sum reaches u
+extern "C" int xft_sample_pick(const int *ids, const float *probs, int n, float u) {
+    float cur = 0;
+    for (int i = 0; i < n; ++i) {
+        cur += probs[i];
+        if (cur >= u) return ids[i];
+    }
+    return ids[n - 1]; // rounding left the sum a hair under u
+}
+
+namespace xft {
+
+static void unsupported(const char *what) {
+    printf("%s is not supported by this build.\n", what);
+    exit(-1);
+}
+
+Model::Model() : impl(nullptr), batchSize(0), seqLen(0), vocabSize(0), maxSeqLen(0), isNewInput(false) {}
+
+Model::~Model() {
+    delete impl;
+}
+
+void Model::input(std::vector<int32_t> &inputIds_, int batchSize_) {
+    if (batchSize_ <= 0 || inputIds_.empty() || inputIds_.size() % (size_t)batchSize_ != 0) {
+        printf("Model::input: %zu ids do not form %d sequences of equal length.\n", inputIds_.size(), batchSize_);
+        exit(-1);
+    }
+    isNewInput = true;
+    batchSize = batchSize_;
+    seqLen = (int)(inputIds_.size() / (size_t)batchSize_);
+    inputIds = inputIds_;
+}
+
+void Model::config(int maxLen_, int numBeams_, int numBeamHypsToKeep_, float lenPenalty_, bool doEarlyStopping_, int eosTokenId_,
+        int padTokenId_, bool doSample_, float temperature_, int topK_, float topP_, float repetitionPenalty_,
+        const std::vector<std::vector<int>> &stopWordsList_) {
+    configuration.maxLen = maxLen_;
+    configuration.numBeams = numBeams_;
+    configuration.numBeamHypsToKeep = numBeamHypsToKeep_;
+    configuration.lenPenalty = lenPenalty_;
+    configuration.doEarlyStopping = doEarlyStopping_;
+    configuration.eosTokenId = eosTokenId_;
+    configuration.padTokenId = padTokenId_;
+    configuration.doSample = doSample_;
+    configuration.temperature = temperature_;
+    configuration.topK = topK_;
+    configuration.topP = topP_;
+    configuration.repetitionPenalty = repetitionPenalty_;
+    this->config(configuration, stopWordsList_);
+}
+
+void Model::config(SearcherConfig &config_, const std::vector<std::vector<int>> &stopWordsList_) {
+    isNewInput = true;
+    configuration = config_;
+    ModelImpl &s = *impl;
+    // getGenerationMode: one beam = greedy or sampling, more = beam search (searcher.h)
+    if (config_.numBeams != 1) unsupported("Beam search (numBeams != 1)");
+    s.sampling = config_.doSample;
+    s.maxLen = config_.maxLen;
+    s.eosTokenId = config_.eosTokenId == -1 ? s.endId : config_.eosTokenId;
+    s.padTokenId = config_.padTokenId == -1 ? s.eosTokenId : config_.padTokenId;
+    s.repetitionPenalty = config_.repetitionPenalty;
+    if (s.repetitionPenalty <= 0) {
+        printf("`repetitionPenalty` has to be a strictly positive float, but is %f.\n", s.repetitionPenalty);
+        exit(-1);
+    }
+    if (s.sampling) {
+        if (config_.temperature <= 0) {
+            printf("Temperature should greater than 0.\n");
+            exit(-1);
+        }
+        s.temperatureInv = 1 / config_.temperature;
+        s.topK = config_.topK < 2 ? 2 : config_.topK;
+        s.topP = config_.topP;
+    }
+    s.stopWordsList.clear();
+    s.stopWordsIndex.clear();
+    s.haveSearcher = true;
+    setStopWords(stopWordsList_);
+}
+
+bool Model::setStopWords(std::vector<std::vector<int>> stopWordsList) {
+    ModelImpl &s = *impl;
+    // a stop word that is only the EOS token is dropped (greedy_search.cpp:140-146)
+    s.stopWordsList.clear();
+    for (auto &w : stopWordsList)
+        if (!(w.size() == 1 && w[0] == s.eosTokenId)) s.stopWordsList.push_back(w);
+    return !s.stopWordsList.empty();
+}
+
+bool Model::isDone() {
+    ModelImpl &s = *impl;
+    if (!s.haveSearcher || inputIds.empty()) {
+        printf("Please set input and config first.\n");
+        exit(-1);
+    }
+    if (isNewInput) return false;
+    if (s.step == 0) return false;
+    if (s.curLen >= s.maxLen) return true;
+    for (int f : s.doneBatch)
+        if (f <= 0) return false;
+    return true;
+}
+
+std::tuple<float *, int, int> Model::forward(bool logitsAll) {
+    ModelImpl &s = *impl;
+    if (logitsAll) unsupported("Model::forward(logitsAll = true)");
+    if (inputIds.empty() || !isNewInput) unsupported("Model::forward without a new input");
+    s.batch = batchSize;
+    s.fit(batchSize, seqLen, std::max(seqLen + 1, s.maxLen));
+    s.logitsHost.resize((size_t)batchSize * s.vocab);
+    CK(xfthip_model_prefill(s.model, inputIds.data(), batchSize, seqLen, s.logitsHost.data(), nullptr));
+    return std::make_tuple(s.logitsHost.data(), 0, s.vocab);
+}
+
+std::vector<int32_t> Model::generate() {
+    ModelImpl &s = *impl;
+    if (!s.haveSearcher) {
+        printf("Please set the generation config by model.config().\n");
+        exit(-1);
+    }
+    if (inputIds.empty()) {
+        printf("Please set input tokens by model.input().\n");
+        exit(-1);
+    }
+    // the search runs on the host whenever the token is not simply the arg-max of the raw logits
+    const bool hostSearch = s.sampling || s.repetitionPenalty != 1.0f;
+    if (isNewInput) {
+        isNewInput = false;
+        s.step = 0;
+        s.batch = batchSize;
+        s.curLen = seqLen;
+        s.doneBatch.assign(batchSize, 0);
+        if (!s.stopWordsList.empty()) s.stopWordsIndex.assign(s.stopWordsList.size(), std::vector<int>(batchSize, 0));
+        s.output.assign(inputIds.begin(), inputIds.end());
+        if (s.maxLen > 0 && seqLen >= s.maxLen) {
+            // nothing to generate: the reference still runs the prompt and emits one token
+        }
+        s.fit(batchSize, seqLen, std::max(seqLen + 1, s.maxLen));
+        CK(xfthip_model_prefill(s.model, inputIds.data(), batchSize, seqLen, nullptr, nullptr));
+    } else {
+        // feed back what the searcher chose where it differs from the device's own arg-max
+        if (s.nextTokens != s.deviceIds) CK(xfthip_model_set_next_ids(s.model, s.nextTokens.data(), nullptr));
+        CK(xfthip_model_decode(s.model, 1, nullptr, nullptr));
+    }
+    s.step++;
+    s.deviceIds.resize(batchSize);
+    CK(xfthip_model_last_ids(s.model, s.deviceIds.data(), nullptr));
+    std::vector<int> ids(batchSize);
+    if (!hostSearch) {
+        ids = s.deviceIds;
+    } else {
+        s.fetch_logits();
+        if (s.repetitionPenalty != 1.0f) s.repetition_penalty(s.logitsHost.data());
+        if (!s.sampling) {
+            // first maximum wins (greedy_search.cpp:190-215)
+            for (int b = 0; b < batchSize; ++b) {
+                const float *p = s.logitsHost.data() + (size_t)b * s.vocab;
+                int best = 0;
+                for (int j = 1; j < s.vocab; ++j)
+                    if (p[j] > p[best]) best = j;
+                ids[b] = best;
+            }
+        } else {
+            const int k = std::min(s.topK, s.vocab);
+            std::vector<int> cand(k);
+            std::vector<float> probs(k);
+            std::uniform_real_distribution<float> dist(0.0f, 1.0f);
+            for (int b = 0; b < batchSize; ++b) {
+                const int n = xft_sample_candidates(s.logitsHost.data() + (size_t)b * s.vocab, s.vocab, s.topK, s.topP,
+                        1.0f / s.temperatureInv, cand.data(), probs.data());
+                ids[b] = xft_sample_pick(cand.data(), probs.data(), n, dist(s.rng));
+            }
+        }
+    }
+    s.finish_tokens(ids);
+    s.nextTokens = ids;
+    s.curLen++;
+    for (int b = 0; b < batchSize; ++b) s.output.insert(s.output.begin() + (size_t)(b + 1) * s.curLen - 1, ids[b]);
+    return std::vector<int32_t>(ids.begin(), ids.end());
+}
+
+std::vector<int32_t> Model::finalize() {
+    return impl->output;
+}
+
+void Model::setPrefix(std::vector<int32_t> &) {
+    unsupported("Prefix sharing");
+}
+void Model::unsetPrefix() {
+    unsupported("Prefix sharing");
+}
+bool Model::freeSeqs(std::vector<int> &) {
+    unsupported("The sequence-id interface (freeSeqs)");
+    return false;
+}
+std::vector<int> Model::set_input(std::vector<int32_t> &, int, SearcherConfig &, const std::vector<std::vector<int>> &) {
+    unsupported("The sequence-id interface (set_input)");
+    return {};
+}
+
+AutoModel::AutoModel(std::string modelPath, xft::DataType dataType, xft::DataType KVCacheDataType) : Model() {
+    const std::string configPath = modelPath + "/config.ini";
+    Ini ini(configPath);
+    if (!ini.ok || ini.sections.empty()) {
+        printf("Could not load model config.ini.\n");
+        exit(-1);
+    }
+    const std::string sec = *ini.sections.begin();
+    setVocabSize((int)ini.get_int(sec, "vocab_size", 0));
+
+    const std::string modelKey = sec + "-" + type_name(dataType) + "-" + type_name(KVCacheDataType);
+    int wkind = -1;
+    switch (dataType) {
+        case xft::DataType::bf16:
+        case xft::DataType::fp16:
+        case xft::DataType::int8:
+        case xft::DataType::w8a8:
+        case xft::DataType::int4:
+        case xft::DataType::nf4: wkind = kind_of(dataType); break;
+        default: break; // the mixed first-token / next-token types are not served
+    }
+    const bool kvOk = KVCacheDataType == xft::DataType::fp16 || KVCacheDataType == xft::DataType::int8;
+    if (Ini::lower(sec) != "llama" || wkind < 0 || !kvOk) {
+        printf("Unsupported data type or KV cache data type: %s\n", modelKey.c_str());
+        exit(-1);
+    }
+
+    ensure_init();
+    impl = new ModelImpl();
+    ModelImpl &s = *impl;
+    s.path = modelPath;
+    s.modelType = sec;
+    s.wkind = wkind;
+    s.kvDtype = KVCacheDataType == xft::DataType::int8 ? XFTHIP_INT8 : XFTHIP_FP16;
+    // the keys and defaults of CommonDecoder's constructor (common_decoder.h:176-212)
+    s.heads = (int)ini.get_int(sec, "head_num", 0);
+    s.kvHeads = (int)ini.get_int(sec, "kv_head_num", s.heads);
+    s.headSize = (int)ini.get_int(sec, "size_per_head", 0);
+    s.inter = (int)ini.get_int(sec, "inter_size", 0);
+    s.layers = (int)ini.get_int(sec, "num_layer", 0);
+    s.vocab = (int)ini.get_int(sec, "vocab_size", 0);
+    s.maxPosEmbed = (int)ini.get_int(sec, "max_pos_seq_len", 0);
+    s.maxPositions = (int)ini.get_int(sec, "model_max_length", s.maxPosEmbed);
+    s.maxSeqLength = (int)ini.get_int(sec, "seq_length", -1);
+    s.hidden = (int)ini.get_int(sec, "hidden_size", (long)s.heads * s.headSize);
+    s.eps = (float)ini.get_float(sec, "layernorm_eps", 1e-6);
+    s.ropeTheta = (float)ini.get_float(sec, "rope_theta", 10000.0);
+    s.startId = (int)ini.get_int(sec, "start_id", 0);
+    s.endId = (int)ini.get_int(sec, "end_id", s.startId);
+    if (s.heads <= 0 || s.headSize <= 0 || s.inter <= 0 || s.layers <= 0 || s.vocab <= 0 || s.hidden <= 0) {
+        printf("config.ini of %s lacks head_num / size_per_head / inter_size / num_layer / vocab_size.\n", modelPath.c_str());
+        exit(-1);
+    }
+    const std::string ropeType = ini.get(sec, "rope_scaling_type", "");
+    if (!ropeType.empty() && Ini::lower(ropeType) != "null" && Ini::lower(ropeType) != "none") {
+        printf("rope_scaling_type = %s is not supported by this build.\n", ropeType.c_str());
+        exit(-1);
+    }
+    std::string act = Ini::lower(ini.get(sec, "activation_type", "silu"));
+    if (act != "silu" && act != "swiglu") {
+        printf("activation_type = %s is not supported by this build.\n", act.c_str());
+        exit(-1);
+    }
+    // element type of the plain files (weight_util.h:37-67)
+    const std::string wt = ini.get(sec, "weight_data_type", "fp32");
+    if (wt.find("fp32") != std::string::npos) s.fileType = xft::DataType::fp32;
+    else if (wt.find("fp16") != std::string::npos) s.fileType = xft::DataType::fp16;
+    else if (wt.find("bf16") != std::string::npos) s.fileType = xft::DataType::bf16;
+    else {
+        printf("Invalid type %s. Use FP32 as default", wt.c_str());
+        s.fileType = xft::DataType::fp32;
+    }
+    // pre-quantised directories (common_decoder.h:214-233)
+    const std::string qt = ini.get(sec, "quant_qweight_data_type", "");
+    if (qt == "int8" || qt == "uint4") {
+        s.fileQuant = qt == "int8" ? XFTHIP_W_INT8 : XFTHIP_W_UINT4;
+        if (ini.get(sec, "quant_scales_data_type", "") != "fp32") {
+            printf("scales should be fp32 data type.\n");
+            exit(-1);
+        }
+        if (ini.get(sec, "quant_zeros_data_type", "") != "fp32") {
+            printf("zeros should be fp32 data type.\n");
+            exit(-1);
+        }
+        if (ini.get_int(sec, "quant_groupsize", -1) != -1) {
+            printf("Quantization with groupsize is not supported.\n");
+            exit(-1);
+        }
+    }
+    s.load();
+    maxSeqLen = s.maxSeqLength > 0 ? s.maxSeqLength : s.maxPositions;
+}
+
+} // namespace xft
+
+// ---- C entry points for language bindings (the role of the reference's Torch custom class,
+// src/pytorch/auto_model.h): one opaque handle per AutoModel ----------------------------------------
+extern "C" {
+
+static xft::DataType dtype_from_name(const char *name) {
+    static const char *names[] = {"fp32", "bf16", "fp16", "int8", "w8a8", "int4", "nf4", "bf16_fp16", "bf16_int8", "bf16_w8a8",
+            "bf16_int4", "bf16_nf4", "w8a8_int8", "w8a8_int4", "w8a8_nf4", "fp8_e4m3"};
+    for (int i = 0; i < 16; ++i)
+        if (strcmp(name, names[i]) == 0) return (xft::DataType)i;
+    return xft::DataType::unknown;
+}
+
+void *xft_automodel_create(const char *path, const char *dtype, const char *kv_dtype) {
+    return new xft::AutoModel(path, dtype_from_name(dtype), dtype_from_name(kv_dtype));
+}
+
+void xft_automodel_destroy(void *h) {
+    delete (xft::AutoModel *)h;
+}
+
+// stop words arrive flattened: n_words lengths, then the ids back to back
+void xft_automodel_config(void *h, int maxLen, int numBeams, int numBeamHypsToKeep, float lenPenalty, int doEarlyStopping,
+        int eosTokenId, int padTokenId, int doSample, float temperature, int topK, float topP, float repetitionPenalty,
+        const int *stop_lens, const int *stop_ids, int n_words) {
+    std::vector<std::vector<int>> words;
+    int off = 0;
+    for (int i = 0; i < n_words; ++i) {
+        words.emplace_back(stop_ids + off, stop_ids + off + stop_lens[i]);
+        off += stop_lens[i];
+    }
+    ((xft::AutoModel *)h)->config(maxLen, numBeams, numBeamHypsToKeep, lenPenalty, doEarlyStopping != 0, eosTokenId, padTokenId,
+            doSample != 0, temperature, topK, topP, repetitionPenalty, words);
+}
+
+void xft_automodel_input(void *h, const int *ids, int batch, int seq_len) {
+    std::vector<int32_t> v(ids, ids + (size_t)batch * seq_len);
+    ((xft::AutoModel *)h)->input(v, batch);
+}
+
+// one generation step; next_out holds batch ids
+int xft_automodel_generate(void *h, int *next_out) {
+    std::vector<int32_t> r = ((xft::AutoModel *)h)->generate();
+    memcpy(next_out, r.data(), r.size() * 4);
+    return (int)r.size();
+}
+
+int xft_automodel_is_done(void *h) {
+    return ((xft::AutoModel *)h)->isDone() ? 1 : 0;
+}
+
+// copies up to `capacity` ids of the [batch, length] result; returns how many there are
+int xft_automodel_finalize(void *h, int *out, int capacity) {
+    std::vector<int32_t> r = ((xft::AutoModel *)h)->finalize();
+    const int n = (int)r.size();
+    if (out) memcpy(out, r.data(), (size_t)std::min(n, capacity) * 4);
+    return n;
+}
+
+// logits of the prompt's next token, fp32 [batch, vocab] (Model::forward(false))
+int xft_automodel_forward(void *h, float *logits_out) {
+    auto t = ((xft::AutoModel *)h)->forward(false);
+    xft::AutoModel *m = (xft::AutoModel *)h;
+    memcpy(logits_out, std::get<0>(t), (size_t)m->getBatchSize() * std::get<2>(t) * 4);
+    return std::get<2>(t);
+}
+
+int xft_automodel_vocab_size(void *h) {
+    return ((xft::AutoModel *)h)->getVocabSize();
+}
+
+int xft_automodel_max_seq_len(void *h) {
+    return ((xft::AutoModel *)h)->getMaxSeqLen();
+}
+
+} // extern "C"

@@ -800,6 +800,17 @@ int xfthip_model_last_ids(xfthip_model_t m, int *ids_host, int *position) {
     return 0;
 }
 
+int xfthip_model_set_next_ids(xfthip_model_t m, const int *ids_host, xfthip_stream_t stream) {
+    XFT_REQUIRE(m && ids_host, "xfthip_model_set_next_ids: null argument");
+    XFT_REQUIRE(m->cur_B > 0, "xfthip_model_set_next_ids: call xfthip_model_prefill first");
+    for (int b = 0; b < m->cur_B; ++b)
+        XFT_REQUIRE(ids_host[b] >= 0 && ids_host[b] < m->cfg.vocab, "xfthip_model_set_next_ids: id %d of sequence %d outside the vocabulary",
+                ids_host[b], b);
+    XFT_CHECK_HIP(hipMemcpyAsync(m->ids, ids_host, (size_t)m->cur_B * 4, hipMemcpyHostToDevice, (hipStream_t)stream));
+    XFT_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return 0;
+}
+
 int xfthip_model_logits(xfthip_model_t m, const float **logits_dev) {
     XFT_REQUIRE(m && logits_dev && m->logits, "xfthip_model_logits: no logits");
     *logits_dev = m->logits;

@@ -4,12 +4,14 @@
 // Replaces MMHelper::compute* (reference src/utils/matmul_helper.h:565-1705) at large M, where
 // the reference switches to AMX (oneDNN) kernels.  MFMA-bound.
 //
-// A workgroup of 4 wavefronts computes a (4*WN*16 columns) x (WM*16 rows) output tile.  Each
+// A workgroup of 4 wavefronts computes a (4*WN*32 columns) x (WM*32 rows) output tile.  Each
 // wave owns WN column tiles and streams their packed codes from global memory straight into
-// registers (the same 1-KiB tile layout the M <= 32 kernel uses: one 128-bit load per lane is an
-// MFMA "A" operand after widening), so weights never pass through LDS.  The activation rows are
-// shared by the 4 waves: staged through a double-buffered, padded LDS tile and read back as
-// 128-bit "B" operands.  Widening cost (12 VALU ops per 16 codes) is amortised over WM MFMAs.
+// registers (the same 1-KiB tile layout the M <= 32 kernel uses: a 128-bit load per lane becomes
+// MFMA "B" operands after widening), so weights never pass through LDS.  The activation rows are
+// shared by the 4 waves: staged through three padded LDS tiles and read back as 128-bit "A"
+// operands.  The k loop is a three-stage pipeline (weights two tiles ahead in registers,
+// activations four tiles ahead in registers and two in LDS) whose memory instructions are spread
+// over the MFMAs of a step; the widening of each operand runs one MFMA group ahead of its use.
 // Scale / zero-point / bias / activation / residual are applied in the epilogue.
 #pragma once
 #include <type_traits>
@@ -55,7 +57,10 @@ template <int KIND>
 struct StepTraits;
 template <>
 struct StepTraits<XFTHIP_W_INT8> {
-    static constexpr int KTILE = 64, GROUPS = 4, SUB = 1, WREGS = 2; // 8 bytes per lane per k group
+    // a lane of half h takes the whole 16-byte chunks of k groups h and 2 + h (one 128-bit load each):
+    // the k index of an MFMA is only a summation index, so lane half h of micro-step (g, sb) stands for
+    // k = 32 g + 16 h + 8 sb .. + 7 in both operands
+    static constexpr int KTILE = 64, GROUPS = 2, SUB = 2, WREGS = 4;
 };
 template <>
 struct StepTraits<XFTHIP_W_UINT4> {
@@ -135,7 +140,7 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     for (int t = 0; t < WN; ++t) {
         int nt = (n32_0 + t) * 2 + (nl >> 4);
         nt = nt < p.NTILES ? nt : p.NTILES - 1;
-        wbase[t] = p.packed + (size_t)nt * p.KT * 1024 + (nl & 15) * 16 + (KIND == XFTHIP_W_INT8 ? 8 * h : 0);
+        wbase[t] = p.packed + (size_t)nt * p.KT * 1024 + (nl & 15) * 16;
     }
     constexpr int ROW_STEP = 256 / CHUNKS_PER_ROW;
     const int a_kc = threadIdx.x % CHUNKS_PER_ROW;
@@ -149,137 +154,217 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     }
 
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
-    uint32_t wreg[2][GROUPS][WN][WREGS];
-    u32x4 areg[ALOADS];
+    // Three-stage pipeline over k tiles.  At the start of step k: LDS buffers k % 3 and (k + 1) % 3 hold the
+    // activation tiles k and k + 1 (published by earlier barriers), the weight registers of sets k % 3
+    // and (k + 1) % 3 hold or await tiles k and k + 1, the activation registers await tile k + 2, and
+    // the first MFMA operands of tile k are already in registers.  Step k sends the loads of weight
+    // tile k + 2 and activation tile k + 3, moves activation tile k + 2 from registers into LDS buffer
+    // (k + 2) % 3 (last read two steps ago), computes tile k while reading each next operand set a
+    // micro-step ahead (the last one from tile k + 1's buffer), and ends in the barrier that publishes
+    // buffer (k + 2) % 3.  Every wait is for loads at least one full step old, and the MFMAs after a
+    // barrier never wait for an LDS read.
+    constexpr int MICRO = GROUPS * SUB;
+    uint32_t wreg[3][GROUPS][WN][WREGS];
+    u32x4 areg[3][ALOADS];
+    const int kt_n = (p.K + KTILE - 1) / KTILE;
 
-    auto load_w = [&](int buf, int kt) {
+    // weight codes of k group gq of tile kt_ into register set buf
+    auto load_w_part = [&](int buf, int kt_, int gq) {
+        const int kt = kt_ < kt_n ? kt_ : kt_n - 1; // past the end: a valid tile, never used
 #pragma unroll
-        for (int gq = 0; gq < GROUPS; ++gq)
-#pragma unroll
-            for (int t = 0; t < WN; ++t) {
-                if constexpr (KIND == XFTHIP_W_INT8) {
-                    const uint2 v = *(const uint2 *)(wbase[t] + (size_t)kt * 1024 + gq * 256);
-                    wreg[buf][gq][t][0] = v.x;
-                    wreg[buf][gq][t][1] = v.y;
-                } else if constexpr (KIND == XFTHIP_W_BF16) {
-                    // chunk g = 2 s + h holds k = 8 g .. 8 g + 7
-                    const u32x4 v = *(const u32x4 *)(wbase[t] + (size_t)kt * 1024 + (2 * gq + h) * 256);
-                    wreg[buf][gq][t][0] = v[0]; wreg[buf][gq][t][1] = v[1]; wreg[buf][gq][t][2] = v[2]; wreg[buf][gq][t][3] = v[3];
-                } else {
-                    const u32x4 v = *(const u32x4 *)(wbase[t] + (size_t)kt * 1024 + gq * 256);
-                    wreg[buf][gq][t][0] = v[0]; wreg[buf][gq][t][1] = v[1]; wreg[buf][gq][t][2] = v[2]; wreg[buf][gq][t][3] = v[3];
-                }
-            }
-    };
-    auto load_a = [&](int kt) {
-#pragma unroll
-        for (int i = 0; i < ALOADS; ++i) {
-            if constexpr (KTAIL) {
-                const int k = kt * KTILE + a_kc * 8;
-                const bool v = k < p.K;
-                const u32x4 a = *(const u32x4 *)(p.A + a_off[i] + (v ? (size_t)kt * KTILE : (size_t)0) - (v ? 0 : a_kc * 8));
-                areg[i] = v ? a : zero4;
+        for (int t = 0; t < WN; ++t) {
+            if constexpr (KIND == XFTHIP_W_INT8) {
+                const u32x4 v = *(const u32x4 *)(wbase[t] + (size_t)kt * 1024 + (2 * gq + h) * 256);
+                wreg[buf][gq][t][0] = v[0]; wreg[buf][gq][t][1] = v[1]; wreg[buf][gq][t][2] = v[2]; wreg[buf][gq][t][3] = v[3];
+            } else if constexpr (KIND == XFTHIP_W_BF16) {
+                // chunk g = 2 s + h holds k = 8 g .. 8 g + 7
+                const u32x4 v = *(const u32x4 *)(wbase[t] + (size_t)kt * 1024 + (2 * gq + h) * 256);
+                wreg[buf][gq][t][0] = v[0]; wreg[buf][gq][t][1] = v[1]; wreg[buf][gq][t][2] = v[2]; wreg[buf][gq][t][3] = v[3];
             } else {
-                areg[i] = *(const u32x4 *)(p.A + a_off[i] + (size_t)kt * KTILE);
+                const u32x4 v = *(const u32x4 *)(wbase[t] + (size_t)kt * 1024 + gq * 256);
+                wreg[buf][gq][t][0] = v[0]; wreg[buf][gq][t][1] = v[1]; wreg[buf][gq][t][2] = v[2]; wreg[buf][gq][t][3] = v[3];
             }
         }
     };
-    auto store_a = [&](int buf) {
-        unsigned char *dst = abuf_base + buf * (ROWS * ROWB);
+    auto load_w = [&](int buf, int kt_) {
 #pragma unroll
-        for (int i = 0; i < ALOADS; ++i) *(u32x4 *)(dst + (a_row0 + i * ROW_STEP) * ROWB + a_kc * 16) = areg[i];
+        for (int gq = 0; gq < GROUPS; ++gq) load_w_part(buf, kt_, gq);
     };
-    // one MFMA k step = 16 k: lane (row/col, h) holds k = kbase + 8 h .. + 8
-    auto compute = [&](int wb, int ab) {
-        const unsigned char *src = abuf_base + ab * (ROWS * ROWB) + nl * ROWB;
+    // 16-byte chunk i of this thread's share of activation tile kt_ into register set `set`
+    auto load_a_part = [&](int set, int kt_, int i) {
+        const int kt = kt_ < kt_n ? kt_ : kt_n - 1;
+        if constexpr (KTAIL) {
+            const int k = kt * KTILE + a_kc * 8;
+            const bool v = k < p.K;
+            const u32x4 a = *(const u32x4 *)(p.A + a_off[i] + (v ? (size_t)kt * KTILE : (size_t)0) - (v ? 0 : a_kc * 8));
+            areg[set][i] = v ? a : zero4;
+        } else {
+            areg[set][i] = *(const u32x4 *)(p.A + a_off[i] + (size_t)kt * KTILE);
+        }
+    };
+    auto load_a = [&](int set, int kt_) {
 #pragma unroll
-        for (int gq = 0; gq < GROUPS; ++gq) {
+        for (int i = 0; i < ALOADS; ++i) load_a_part(set, kt_, i);
+    };
+    auto store_a_part = [&](int set, int buf, int i) {
+        unsigned char *dst = abuf_base + buf * (ROWS * ROWB);
+        *(u32x4 *)(dst + (a_row0 + i * ROW_STEP) * ROWB + a_kc * 16) = areg[set][i];
+    };
+    auto store_a = [&](int set, int buf) {
 #pragma unroll
-            for (int sb = 0; sb < SUB; ++sb) {
-                // k offset of this step inside the tile
-                const int koff = (KIND == XFTHIP_W_INT8) ? 16 * gq + 8 * h
-                        : (KIND == XFTHIP_W_BF16)        ? 16 * gq + 8 * h
-                                                         : 32 * gq + 16 * sb + 8 * h;
-                MFrag a[WM];
+        for (int i = 0; i < ALOADS; ++i) store_a_part(set, buf, i);
+    };
+    // k offset (elements) of micro-step ms inside a tile: lane (row/col, h) holds k = koff .. koff + 7
+    auto koff_of = [&](int ms) {
+        const int gq = ms / SUB, sb = ms % SUB;
+        return KIND == XFTHIP_W_INT8 ? 32 * gq + 16 * h + 8 * sb : KIND == XFTHIP_W_BF16 ? 16 * gq + 8 * h : 32 * gq + 16 * sb + 8 * h;
+    };
+    MFrag afr[2][WM];
+    auto read_frags = [&](int slot, int ab, int ms) {
+        const unsigned char *src = abuf_base + ab * (ROWS * ROWB) + nl * ROWB + koff_of(ms) * 2;
 #pragma unroll
-                for (int m = 0; m < WM; ++m) a[m].q = *(const u32x4 *)(src + m * 32 * ROWB + koff * 2);
+        for (int m = 0; m < WM; ++m) afr[slot][m].q = *(const u32x4 *)(src + m * 32 * ROWB);
+    };
+    // one MFMA k step = 16 k.  Operands of micro-step ms sit in afr[ms & 1]; the next set (of the
+    // next tile's buffer after the last micro-step) is read while this one's MFMAs run.
+    // Besides the MFMAs of tile kt (weight set wb, LDS buffer ab), a step sends the loads of weight
+    // tile kt + 2 (into set wnext) and activation tile kt + 4 (into register set ab_next) and moves
+    // activation tile kt + 2 (register set wnext, loaded two steps ago) into LDS buffer
+    // wnext: one slice of each per micro-step, so that no wave ever queues a burst of memory
+    // instructions in front of its MFMAs (a wave issues in order; 4 waves sending 12 loads each right
+    // after a barrier kept the MFMA pipes waiting for the address path).
+    constexpr int A_EVERY = MICRO / ALOADS;
+    static_assert(MICRO % ALOADS == 0, "activation slices must spread evenly over the micro-steps");
+    // widened MFMA operands of (weight set wb, micro-step ms, column tile t)
+    auto widen = [&](int wb, int ms, int t, MFrag &whi, MFrag &wlo) {
+        const int gq = ms / SUB, sb = ms % SUB;
+        if constexpr (KIND == XFTHIP_W_INT8) {
+            const uint32_t x = wreg[wb][gq][t][2 * sb], y = wreg[wb][gq][t][2 * sb + 1];
+            whi.u[0] = pack_hi16_m((float)(int)(int8_t)(x), (float)(int)(int8_t)(x >> 8));
+            whi.u[1] = pack_hi16_m((float)(int)(int8_t)(x >> 16), (float)((int)x >> 24));
+            whi.u[2] = pack_hi16_m((float)(int)(int8_t)(y), (float)(int)(int8_t)(y >> 8));
+            whi.u[3] = pack_hi16_m((float)(int)(int8_t)(y >> 16), (float)((int)y >> 24));
+        } else if constexpr (KIND == XFTHIP_W_BF16) {
+            whi.u[0] = wreg[wb][gq][t][0]; whi.u[1] = wreg[wb][gq][t][1];
+            whi.u[2] = wreg[wb][gq][t][2]; whi.u[3] = wreg[wb][gq][t][3];
+        } else {
+            // codes 16 sb + 8 h .. + 8 of the lane's 32-code chunk = dword 2 sb + h
+            const uint32_t x0 = wreg[wb][gq][t][2 * sb], x1 = wreg[wb][gq][t][2 * sb + 1];
+            const uint32_t x = h ? x1 : x0;
+            if constexpr (KIND == XFTHIP_W_UINT4) {
+                whi.u[0] = (x & 0x000F000Fu) | 0x43004300u;
+                whi.u[1] = ((x >> 4) & 0x000F000Fu) | 0x43004300u;
+                whi.u[2] = ((x >> 8) & 0x000F000Fu) | 0x43004300u;
+                whi.u[3] = ((x >> 12) & 0x000F000Fu) | 0x43004300u;
+            } else {
+                const uint2 e0 = lut[x & 0xFF], e1 = lut[(x >> 8) & 0xFF], e2 = lut[(x >> 16) & 0xFF], e3 = lut[x >> 24];
+                whi.u[0] = e0.x; whi.u[1] = e1.x; whi.u[2] = e2.x; whi.u[3] = e3.x;
+                wlo.u[0] = e0.y; wlo.u[1] = e1.y; wlo.u[2] = e2.y; wlo.u[3] = e3.y;
+            }
+        }
+    };
+    // The operands of slot (ms, t) are widened while the MFMAs of the slot before run: wcur_* enter
+    // a step holding slot (0, 0) of its tile and leave it holding slot (0, 0) of the next tile.
+    MFrag wcur_hi, wcur_lo;
+    // the explicit interleave below pays for the BF16 kind (no widening work to hide: +5 %) and costs
+    // the INT8 kind 6 % on 128 x 128 tiles, where the compiler's own order is better
+    constexpr bool SGB = KIND == XFTHIP_W_BF16;
+    // VALU instructions one widening takes (a hint for the instruction interleave below)
+    constexpr int VW = KIND == XFTHIP_W_INT8 ? 12 : KIND == XFTHIP_W_UINT4 ? 9 : KIND == XFTHIP_W_NF4 ? 6 : 0;
+    constexpr int VPER = (VW + WM - 1) / WM;
+    auto compute = [&](int wb, int ab, int ab_next, int wnext, int kt_cur) {
 #pragma unroll
-                for (int t = 0; t < WN; ++t) {
-                    MFrag whi, wlo;
-                    if constexpr (KIND == XFTHIP_W_INT8) {
-                        const uint32_t x = wreg[wb][gq][t][0], y = wreg[wb][gq][t][1];
-                        whi.u[0] = pack_hi16_m((float)(int)(int8_t)(x), (float)(int)(int8_t)(x >> 8));
-                        whi.u[1] = pack_hi16_m((float)(int)(int8_t)(x >> 16), (float)((int)x >> 24));
-                        whi.u[2] = pack_hi16_m((float)(int)(int8_t)(y), (float)(int)(int8_t)(y >> 8));
-                        whi.u[3] = pack_hi16_m((float)(int)(int8_t)(y >> 16), (float)((int)y >> 24));
-                    } else if constexpr (KIND == XFTHIP_W_BF16) {
-                        whi.u[0] = wreg[wb][gq][t][0]; whi.u[1] = wreg[wb][gq][t][1];
-                        whi.u[2] = wreg[wb][gq][t][2]; whi.u[3] = wreg[wb][gq][t][3];
-                    } else {
-                        // codes 16 sb + 8 h .. + 8 of the lane's 32-code chunk = dword 2 sb + h
-                        const uint32_t x0 = wreg[wb][gq][t][2 * sb], x1 = wreg[wb][gq][t][2 * sb + 1];
-                        const uint32_t x = h ? x1 : x0;
-                        if constexpr (KIND == XFTHIP_W_UINT4) {
-                            whi.u[0] = (x & 0x000F000Fu) | 0x43004300u;
-                            whi.u[1] = ((x >> 4) & 0x000F000Fu) | 0x43004300u;
-                            whi.u[2] = ((x >> 8) & 0x000F000Fu) | 0x43004300u;
-                            whi.u[3] = ((x >> 12) & 0x000F000Fu) | 0x43004300u;
-                        } else {
-                            const uint2 e0 = lut[x & 0xFF], e1 = lut[(x >> 8) & 0xFF], e2 = lut[(x >> 16) & 0xFF], e3 = lut[x >> 24];
-                            whi.u[0] = e0.x; whi.u[1] = e1.x; whi.u[2] = e2.x; whi.u[3] = e3.x;
-                            wlo.u[0] = e0.y; wlo.u[1] = e1.y; wlo.u[2] = e2.y; wlo.u[3] = e3.y;
+        for (int ms = 0; ms < MICRO; ++ms) {
+            const int gq = ms / SUB, sb = ms % SUB;
+            if (sb == 0) load_w_part(wnext, kt_cur + 2, gq);
+            if (ms % A_EVERY == 0) {
+                load_a_part(ab_next, kt_cur + 4, ms / A_EVERY);
+                store_a_part(wnext, wnext, ms / A_EVERY);
+            }
+            if (ms + 1 < MICRO)
+                read_frags((ms + 1) & 1, ab, ms + 1);
+            else
+                read_frags((ms + 1) & 1, ab_next, 0);
+            const MFrag *a = afr[ms & 1];
+#pragma unroll
+            for (int t = 0; t < WN; ++t) {
+                MFrag nhi, nlo;
+                if (t + 1 < WN)
+                    widen(wb, ms, t + 1, nhi, nlo);
+                else if (ms + 1 < MICRO)
+                    widen(wb, ms + 1, 0, nhi, nlo);
+                else
+                    widen(ab_next, 0, 0, nhi, nlo); // the next tile's set: loaded during the step before this one
+#pragma unroll
+                for (int m = 0; m < WM; ++m) {
+                    if constexpr (KIND == XFTHIP_W_NF4)
+                        acc[t][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[m].v, wcur_lo.v, acc[t][m], 0, 0, 0);
+                    acc[t][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[m].v, wcur_hi.v, acc[t][m], 0, 0, 0);
+                }
+                if constexpr (NEED_SUM) {
+                    if (t + 1 == WN) {
+#pragma unroll
+                        for (int m = 0; m < WM; ++m) accS[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[m].v, ones.v, accS[m], 0, 0, 0);
+                    }
+                }
+                wcur_hi = nhi;
+                if constexpr (KIND == XFTHIP_W_NF4) wcur_lo = nlo;
+                if constexpr (SGB) {
+                    // order of the slot's instructions: its memory instructions first, then one MFMA at a
+                    // time with a share of the widening and (first column tile) one LDS read behind it
+                    if (t == 0) {
+                        if (sb == 0) {
+#pragma unroll
+                            for (int tt = 0; tt < WN; ++tt) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                        }
+                        if (ms % A_EVERY == 0) {
+                            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
                         }
                     }
 #pragma unroll
                     for (int m = 0; m < WM; ++m) {
-                        if constexpr (KIND == XFTHIP_W_NF4)
-                            acc[t][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[m].v, wlo.v, acc[t][m], 0, 0, 0);
-                        acc[t][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[m].v, whi.v, acc[t][m], 0, 0, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x008, KIND == XFTHIP_W_NF4 ? 2 : 1, 0);
+                        if (t == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                        if (VPER > 0) __builtin_amdgcn_sched_group_barrier(0x002, VPER, 0);
                     }
-                }
-                if constexpr (NEED_SUM) {
-#pragma unroll
-                    for (int m = 0; m < WM; ++m) accS[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[m].v, ones.v, accS[m], 0, 0, 0);
+                    if (NEED_SUM && t + 1 == WN) __builtin_amdgcn_sched_group_barrier(0x008, WM, 0);
                 }
             }
         }
     };
 
 #define XFT_FENCE() __builtin_amdgcn_sched_barrier(0)
-    const int kt_n = (p.K + KTILE - 1) / KTILE;
+    // prologue: tiles 0 and 1 in LDS, weight tiles 0 and 1 and activation tiles 2 and 3 under way
     load_w(0, 0);
-    load_a(0);
-    store_a(0);
+    load_a(0, 0);
+    load_w(1, 1);
+    load_a(1, 1);
+    load_a(2, 2);
+    XFT_FENCE();
+    store_a(0, 0);
+    XFT_FENCE();
+    load_a(0, 3);
+    XFT_FENCE();
+    store_a(1, 1);
     __syncthreads();
+    read_frags(0, 0, 0);
+    widen(0, 0, 0, wcur_hi, wcur_lo);
+    // step k with s = k % 3 (static): tile j lives in weight set, activation register set and LDS buffer j % 3
+#define XFT_STEP(s)                                        \
+    {                                                      \
+        compute((s), (s), ((s) + 1) % 3, ((s) + 2) % 3, kt); \
+        XFT_FENCE();                                       \
+        __syncthreads();                                   \
+        ++kt;                                              \
+    }
     int kt = 0;
-    for (; kt + 2 <= kt_n - 1; kt += 2) {
-        load_w(1, kt + 1);
-        load_a(kt + 1);
-        XFT_FENCE();
-        compute(0, 0);
-        XFT_FENCE();
-        store_a(1);
-        __syncthreads();
-        load_w(0, kt + 2);
-        load_a(kt + 2);
-        XFT_FENCE();
-        compute(1, 1);
-        XFT_FENCE();
-        store_a(0);
-        __syncthreads();
+    while (kt + 3 <= kt_n) {
+        XFT_STEP(0) XFT_STEP(1) XFT_STEP(2)
     }
-    if (kt + 1 < kt_n) {
-        load_w(1, kt + 1);
-        load_a(kt + 1);
-        XFT_FENCE();
-        compute(0, 0);
-        XFT_FENCE();
-        store_a(1);
-        __syncthreads();
-        compute(1, 1);
-    } else {
-        compute(0, 0);
-    }
+    if (kt < kt_n) XFT_STEP(0)
+    if (kt < kt_n) XFT_STEP(1)
+#undef XFT_STEP
 #undef XFT_FENCE
 
     // ---- epilogue: lane holds C[m0 + 32 mt + 8 (j/4) + 4 h + j%4][32 (n32_0 + t) + nl] ----
@@ -463,9 +548,15 @@ static int launch_big2(const SkinnyParams &p, hipStream_t stream) {
     const int nblocks_m = (p.M + ROWS - 1) / ROWS;
     const int nb8 = (nblocks_n + 7) / 8;
     const int blocks = nb8 * 8 * nblocks_m;
-    // the activation double buffer, reused after the k loop by the four waves' output patches
-    const size_t pipe = 2 * ROWS * ROWB, patches = 4 * 32 * (32 * WN * 4 + 32);
+    // the three activation buffers, reused after the k loop by the four waves' output patches
+    const size_t pipe = 3 * ROWS * ROWB, patches = 4 * 32 * (32 * WN * 4 + 32);
     const size_t smem = (pipe > patches ? pipe : patches) + (KIND == XFTHIP_W_NF4 ? 2048 : 0);
+    if (smem > 64 * 1024) {
+        // more dynamic LDS than the default limit: raise it once per instantiation
+        static const hipError_t attr = hipFuncSetAttribute((const void *)qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL>,
+                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        XFT_CHECK_HIP(attr);
+    }
     hipLaunchKernelGGL((qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL>), dim3(blocks), dim3(256), smem, stream, p, nblocks_n,
             nblocks_m);
     XFT_CHECK_HIP(hipGetLastError());
@@ -494,10 +585,10 @@ static int dispatch_big_tile(const SkinnyParams &p, hipStream_t stream) {
         if (t_mid >= cus) return launch_big<KIND, 1, 4, NEED_SUM>(p, stream);
         return launch_big<KIND, 1, 2, NEED_SUM>(p, stream);
     } else if constexpr (KIND == XFTHIP_W_INT8) {
-        if (p.M > 1024) {
-            if (t_large >= 2 * cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
-            if (t_mid >= cus) return launch_big<KIND, 1, 4, NEED_SUM>(p, stream);
-        }
+        // 128 x 128 tiles, two workgroups a CU: measured 745 / 888 / 821 / 786 / 814 TFLOP/s on N x K =
+        // 11008x4096 / 4096x4096 / 4096x11008 / 12288x4096 / 22016x4096 at 2048 rows; the 128 x 256 tile
+        // (one wave per SIMD, nothing to run while it waits) stays at 750-760 wherever it applies
+        if (p.M > 1024 && t_mid >= cus) return launch_big<KIND, 1, 4, NEED_SUM>(p, stream);
     } else {
         // 4-bit kinds: the 128 x 128 tile holds half the accumulators of the 128 x 256 one at the
         // same occupancy (LDS for the 128-deep k tile) and never won

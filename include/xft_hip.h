@@ -265,6 +265,32 @@ int xfthip_attention_static(xfthip_kvcache_t c, const void *q, int qStride, void
         int S, int qHeads, float scale, int past, const int *past_dev, xfthip_stream_t stream);
 
 
+/*
+ * Attention over a block-paged BF16 KV cache: the device side of xft::invokeAttention
+ * (include/layers_attention.h:22-59, src/kernels/attention_kernels.cpp:24-157).  Caches are
+ * [block_num][block_size][kv_heads][head_size] bf16 in device memory; slot = block * block_size + row.
+ * Decode: one new token per sequence.  key / value row b is stored at slot_mapping[b], then query row b
+ * attends to the context_lens[b] + 1 tokens that block_tables row b (table_stride entries a row)
+ * maps, new token included: fp32 scores, softmax(scale * s), fp32 P.V, bf16 out [batch, o_stride].
+ * max_context: the largest context_lens value (host copy); every table row must hold
+ * max_context / block_size + 1 valid entries.  All pointers but none of the integers are device memory.
+ * The reference reads query / key / value row 0 for every sequence and indexes the KV head with the
+ * query head (attention_kernels.cpp:51-61); this entry point uses row b and head hq / (q_heads / kv_heads),
+ * the same for batch 1 without grouped heads.
+ */
+int xfthip_paged_attention_decode(void *out, const void *q, const void *k, const void *v, int q_heads, int kv_heads,
+        int head_size, int q_stride, int kv_stride, int o_stride, float scale, int batch, void *kcache, void *vcache,
+        int block_num, int block_size, const int *block_tables, int table_stride, const int *context_lens,
+        const int *slot_mapping, int max_context, xfthip_stream_t stream);
+/*
+ * Prefill: sequences lie back to back in q / k / v (token_lens_host[b] rows each, host array); causal
+ * self-attention per sequence (the reference's selfAttention call, attention_kernels.cpp:141-151) and
+ * every token's key / value row stored at slot_mapping[token] (device int32, one entry per token).
+ */
+int xfthip_paged_attention_prefill(void *out, const void *q, const void *k, const void *v, int q_heads, int kv_heads,
+        int head_size, int q_stride, int kv_stride, int o_stride, float scale, int batch, const int *token_lens_host,
+        void *kcache, void *vcache, int block_num, int block_size, const int *slot_mapping, xfthip_stream_t stream);
+
 /* ---- decoder layers and the model driver -------------------------------------------- */
 typedef struct xfthip_model *xfthip_model_t;
 

@@ -499,3 +499,62 @@ def mixtral_mlp(x, ln, router, experts, logits_override=None, do_norm=True, roun
         wt = f32(w[rows, slot])
         lib.orc_scatter_add(p(out), out.shape[1], p(f32(eo)), out.shape[1], p(idx), p(wt), rows.size)
     return out, sel, w
+
+
+# ---- attention over a block-paged BF16 cache (xft::invokeAttention) ------------------------------
+# The reference's crossAttention (src/kernels/attention_kernels.cpp:24-112) per (sequence, head):
+# store the new key / value rows at slot_mapping[b], scores = q . K^T over context + 1 tokens through
+# the block table (fp32, xDNN small_sgemm_bf16bf16f32_b: closed source, textbook GEMM assumed),
+# small_softmax_f32(scores, scale, n) = softmax(scale * scores) in fp32, out = P . V in fp32
+# narrowed to bf16.  PARITY UNPINNED against the reference (no test of it there, xDNN kernels not in
+# the tree); pinned against float64 brute force in tests/test_oracle_pins.py.  Sequence b uses row b
+# of query / key / value and KV head hq // (q_heads // kv_heads): see include/layers_attention.h for
+# how that differs from the reference's text.
+def paged_attention_decode(q, k, v, kcache, vcache, block_tables, context_lens, slot_mapping, scale):
+    """q [B, qH, D], k / v [B, kvH, D] fp32 holding bf16 values; kcache / vcache
+    [blocks, block_size, kvH, D] fp32 holding bf16 values, updated in place.  Returns bf16-rounded
+    fp32 [B, qH, D]."""
+    B, qH, D = q.shape
+    kvH = k.shape[1]
+    bs = kcache.shape[1]
+    kflat, vflat = kcache.reshape(-1, kvH, D), vcache.reshape(-1, kvH, D)
+    out = np.zeros((B, qH, D), np.float32)
+    for b in range(B):
+        kflat[slot_mapping[b]] = k[b]
+        vflat[slot_mapping[b]] = v[b]
+    for b in range(B):
+        n = int(context_lens[b]) + 1
+        slots = [int(block_tables[b][t // bs]) * bs + t % bs for t in range(n)]
+        for h in range(qH):
+            kh = h // (qH // kvH)
+            K, V = f32(kflat[slots, kh]), f32(vflat[slots, kh])
+            s = (K @ f32(q[b, h])).astype(np.float32) * np.float32(scale)
+            e = np.exp(s - s.max()).astype(np.float32)
+            p = e / e.sum(dtype=np.float32)
+            out[b, h] = round_bf16((p @ V).astype(np.float32))
+    return out
+
+
+def paged_attention_prefill(q, k, v, token_lens, kcache, vcache, slot_mapping, scale):
+    """Causal self-attention per sequence over its own tokens (xft::selfAttention as invokeAttention
+    calls it, attention_kernels.cpp:141-151: bf16 inputs, fp32 softmax) and every token's key / value
+    row stored at its slot.  q [T, qH, D], k / v [T, kvH, D].  Returns bf16-rounded fp32 [T, qH, D]."""
+    T, qH, D = q.shape
+    kvH = k.shape[1]
+    kflat, vflat = kcache.reshape(-1, kvH, D), vcache.reshape(-1, kvH, D)
+    for t in range(T):
+        kflat[slot_mapping[t]] = k[t]
+        vflat[slot_mapping[t]] = v[t]
+    out = np.zeros((T, qH, D), np.float32)
+    first = 0
+    for L in token_lens:
+        for h in range(qH):
+            kh = h // (qH // kvH)
+            Q, K, V = f32(q[first:first + L, h]), f32(k[first:first + L, kh]), f32(v[first:first + L, kh])
+            s = (Q @ K.T).astype(np.float32) * np.float32(scale)
+            s = np.where(np.tril(np.ones((L, L), bool)), s, -np.inf)
+            e = np.exp(s - s.max(1, keepdims=True)).astype(np.float32)
+            p = e / e.sum(1, keepdims=True, dtype=np.float32)
+            out[first:first + L, h] = round_bf16((p @ V).astype(np.float32))
+        first += L
+    return out

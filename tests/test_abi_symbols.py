@@ -41,7 +41,7 @@ def test_c_abi_exports_every_declared_symbol():
 @pytest.mark.skipif(not os.path.exists(LIB_LAYERS), reason="host library not built")
 def test_host_layer_exports_reference_entry_points(tmp_path):
     out = subprocess.check_output(["nm", "-DC", "--defined-only", LIB_LAYERS], text=True)
-    for fn in ("xft::invokeLayerLLaMA(", "xft::invokeAttentionLLaMA(", "xft::invokeMLPLLaMA(", "xft::invokeGemm(",
+    for fn in ("xft::invokeLayerLLaMA(", "xft::invokeAttentionLLaMA(", "xft::invokeAttention(", "xft::invokeMLPLLaMA(", "xft::invokeGemm(",
                "xft::invokeRmsNorm(", "xft::invokeRotaryEmbedding("):
         assert fn in out, fn
     # the signatures are the reference's: a translation unit written against its headers links
@@ -61,6 +61,8 @@ def test_host_layer_exports_reference_entry_points(tmp_path):
                     nullptr, nullptr, nullptr, nullptr);
             xft::invokeMLPLLaMA(xft::DataType::bf16, xft::ActivationType::SILU, 1, 4096, 11008, nullptr, 4096, nullptr, 4096,
                     nullptr, nullptr, nullptr);
+            xft::invokeAttention(xft::DataType::bf16, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 4096, 1024, 0.088f, 1,
+                    nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, false, nullptr);
             xft::invokeGemm(xft::DataType::bf16, false, false, 1, 1, 8, 1.0f, nullptr, 8, nullptr, 0.0f, nullptr, 1);
             xft::invokeRmsNorm(xft::DataType::fp32, nullptr, nullptr, nullptr, 1, 8);
             xft::invokeRotaryEmbedding(xft::DataType::bf16, nullptr, nullptr, nullptr, nullptr, nullptr, 128, 128, 128, 1, 1,

@@ -677,3 +677,56 @@ def test_device_bf16_narrowing_exhaustive(tmp_path):
                            os.path.join(root, "oracle", "liboracle.so"), "-Wl,-rpath," + os.path.join(root, "oracle")])
     out = subprocess.run([exe], capture_output=True, text=True, timeout=600)
     assert out.returncode == 0 and "ref=0 sel=0" in out.stdout, out.stdout + out.stderr
+
+
+def test_paged_attention_oracle_vs_float64_dense_attention():
+    """The paged-cache oracle (block-table lookup, slot stores, grouped heads, causal prefill) against
+    dense float64 attention over the same tokens laid out contiguously."""
+    from oracle import pyoracle as orc
+    rng = np.random.default_rng(5)
+    qH, kvH, D, bs, blocks = 8, 2, 128, 4, 40
+    scale = 1 / np.sqrt(D)
+    ctx = np.asarray([0, 7, 8, 21], np.int32)
+    B = len(ctx)
+    need = [(c + 1 + bs - 1) // bs for c in ctx]
+    perm = rng.permutation(blocks)
+    tab = np.zeros((B, max(need)), np.int32)
+    at = 0
+    for b, n in enumerate(need):
+        tab[b, :n] = perm[at:at + n]
+        at += n
+    bf = lambda shape: orc.round_bf16(rng.standard_normal(shape).astype(np.float32))
+    kc, vc = bf((blocks, bs, kvH, D)), bf((blocks, bs, kvH, D))
+    before_k = kc.copy()
+    q, k, v = bf((B, qH, D)), bf((B, kvH, D)), bf((B, kvH, D))
+    slots = np.asarray([tab[b, ctx[b] // bs] * bs + ctx[b] % bs for b in range(B)], np.int32)
+    out = orc.paged_attention_decode(q, k, v, kc, vc, tab, ctx, slots, scale)
+    changed = np.argwhere(np.any(kc.reshape(-1, kvH * D) != before_k.reshape(-1, kvH * D), axis=1)).ravel()
+    assert sorted(changed) == sorted(slots)  # exactly the new rows were written
+    for b in range(B):
+        toks = [tab[b, t // bs] * bs + t % bs for t in range(ctx[b] + 1)]
+        K = kc.reshape(-1, kvH, D)[toks].astype(np.float64)
+        V = vc.reshape(-1, kvH, D)[toks].astype(np.float64)
+        assert np.array_equal(K[-1].astype(np.float32), k[b])
+        for h in range(qH):
+            s = K[:, h // 4] @ q[b, h].astype(np.float64) * scale
+            p = np.exp(s - s.max())
+            p /= p.sum()
+            assert np.abs(p @ V[:, h // 4] - out[b, h]).max() < 1.5e-2
+    # prefill: two sequences, causal within each, nothing across
+    lens = [5, 9]
+    T = sum(lens)
+    q, k, v = bf((T, qH, D)), bf((T, kvH, D)), bf((T, kvH, D))
+    slots = rng.permutation(blocks * bs)[:T].astype(np.int32)
+    out = orc.paged_attention_prefill(q, k, v, lens, kc, vc, slots, scale)
+    assert np.array_equal(kc.reshape(-1, kvH, D)[slots], k) and np.array_equal(vc.reshape(-1, kvH, D)[slots], v)
+    first = 0
+    for L in lens:
+        for t in range(L):
+            for h in range(qH):
+                K, V = k[first:first + t + 1, h // 4].astype(np.float64), v[first:first + t + 1, h // 4].astype(np.float64)
+                s = K @ q[first + t, h].astype(np.float64) * scale
+                p = np.exp(s - s.max())
+                p /= p.sum()
+                assert np.abs(p @ V - out[first + t, h]).max() < 1.5e-2
+        first += L

@@ -418,6 +418,22 @@ class Model:
             pass
 
 
+def paged_attention_decode(out_dev, q_dev, k_dev, v_dev, q_heads, kv_heads, head, q_stride, kv_stride, o_stride, scale, batch,
+                           kcache_dev, vcache_dev, block_num, block_size, tables_dev, table_stride, ctx_dev, slots_dev, max_context,
+                           stream=None):
+    check(lib.xfthip_paged_attention_decode(out_dev, q_dev, k_dev, v_dev, q_heads, kv_heads, head, q_stride, kv_stride, o_stride,
+                                            C.c_float(scale), batch, kcache_dev, vcache_dev, block_num, block_size, tables_dev,
+                                            table_stride, ctx_dev, slots_dev, max_context, stream))
+
+
+def paged_attention_prefill(out_dev, q_dev, k_dev, v_dev, q_heads, kv_heads, head, q_stride, kv_stride, o_stride, scale, token_lens,
+                            kcache_dev, vcache_dev, block_num, block_size, slots_dev, stream=None):
+    lens = np.ascontiguousarray(token_lens, np.int32)
+    check(lib.xfthip_paged_attention_prefill(out_dev, q_dev, k_dev, v_dev, q_heads, kv_heads, head, q_stride, kv_stride, o_stride,
+                                             C.c_float(scale), len(lens), _hp(lens), kcache_dev, vcache_dev, block_num, block_size,
+                                             slots_dev, stream))
+
+
 def argmax(logits_dev, rows, cols, stream=None):
     """First-maximum argmax of fp32 logits [rows, cols] in device memory; returns host int32 [rows]."""
     ids = DeviceBuffer(rows * 4)

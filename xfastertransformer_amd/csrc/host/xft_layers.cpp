@@ -183,6 +183,88 @@ void invokeLayerLLaMA(DataType dt, ActivationType at, NormType nt, int batchSize
     });
 }
 
+void invokeAttention(DataType dt, void *output, const void *query, const void *key, const void *value, int *query_shape,
+        int *kv_shape, const int q_stride, const int kv_stride, const float scale, const int batch_size,
+        const int *token_lens, const void *kcache, const void *vcache, int *kvcache_shape, int *block_tables,
+        int *block_nums, int *context_lens, int layer_id, bool is_prefill, int *slot_mapping) {
+    static std::mutex mutex;
+    std::lock_guard<std::mutex> lock(mutex);
+    (void)layer_id;
+    if (dt != DataType::bf16) {
+        printf("Error: data type (%d) is not supported yet!\n", dt);
+        exit(-1);
+    }
+    ensure_init();
+    const int total = query_shape[0], qHeads = query_shape[1], headSize = query_shape[2], kvHeads = kv_shape[1];
+    const int blockNum = kvcache_shape[0], blockSize = kvcache_shape[1];
+    if (kvcache_shape[2] != kvHeads || kvcache_shape[3] != headSize || batch_size <= 0 || total <= 0) {
+        printf("invokeAttention: kvcache_shape [%d, %d, %d, %d] does not match %d KV heads of size %d\n", kvcache_shape[0],
+                kvcache_shape[1], kvcache_shape[2], kvcache_shape[3], kvHeads, headSize);
+        exit(-1);
+    }
+    const size_t rowElems = (size_t)kvHeads * headSize, cacheBytes = (size_t)blockNum * blockSize * rowElems * 2;
+    // device copies of the caches, keyed by the host address
+    struct Mirror {
+        void *dev = nullptr;
+        size_t bytes = 0;
+    };
+    static std::unordered_map<const void *, Mirror> mirrors;
+    auto mirror_of = [&](const void *host) {
+        Mirror &m = mirrors[host];
+        if (m.bytes != cacheBytes) {
+            if (m.dev) xfthip_free(m.dev);
+            CK(xfthip_malloc(&m.dev, cacheBytes));
+            CK(xfthip_memcpy_h2d(m.dev, host, cacheBytes, nullptr));
+            m.bytes = cacheBytes;
+        }
+        return m.dev;
+    };
+    void *kc = mirror_of(kcache), *vc = mirror_of(vcache);
+
+    const int oStride = qHeads * headSize;
+    int rows = total;
+    if (!is_prefill) rows = batch_size;
+    static DevBuf dq, dk, dv, dout, dtab, dctx, dslot;
+    CK(xfthip_memcpy_h2d(dq.get((size_t)rows * q_stride * 2), query, ((size_t)(rows - 1) * q_stride + (size_t)qHeads * headSize) * 2, nullptr));
+    CK(xfthip_memcpy_h2d(dk.get((size_t)rows * kv_stride * 2), key, ((size_t)(rows - 1) * kv_stride + rowElems) * 2, nullptr));
+    CK(xfthip_memcpy_h2d(dv.get((size_t)rows * kv_stride * 2), value, ((size_t)(rows - 1) * kv_stride + rowElems) * 2, nullptr));
+    CK(xfthip_memcpy_h2d(dslot.get((size_t)rows * 4), slot_mapping, (size_t)rows * 4, nullptr));
+    dout.get((size_t)rows * oStride * 2);
+    if (!is_prefill) {
+        int maxCtx = 0, tableStride = 0;
+        for (int b = 0; b < batch_size; ++b) {
+            if (context_lens[b] > maxCtx) maxCtx = context_lens[b];
+            const int nb = block_nums ? block_nums[b] : context_lens[b] / blockSize + 1;
+            if (nb > tableStride) tableStride = nb;
+            if (nb * blockSize < context_lens[b] + 1) {
+                printf("invokeAttention: sequence %d has %d blocks of %d for %d + 1 tokens\n", b, nb, blockSize, context_lens[b]);
+                exit(-1);
+            }
+        }
+        CK(xfthip_memcpy_h2d(dtab.get((size_t)batch_size * tableStride * 4), block_tables, (size_t)batch_size * tableStride * 4, nullptr));
+        CK(xfthip_memcpy_h2d(dctx.get((size_t)batch_size * 4), context_lens, (size_t)batch_size * 4, nullptr));
+        CK(xfthip_paged_attention_decode(dout.p, dq.p, dk.p, dv.p, qHeads, kvHeads, headSize, q_stride, kv_stride, oStride, scale, batch_size,
+                kc, vc, blockNum, blockSize, (const int *)dtab.p, tableStride, (const int *)dctx.p, (const int *)dslot.p, maxCtx, nullptr));
+    } else {
+        int sum = 0;
+        for (int b = 0; b < batch_size; ++b) sum += token_lens[b];
+        if (sum != total) {
+            printf("invokeAttention: token_lens sum to %d, query_shape[0] is %d\n", sum, total);
+            exit(-1);
+        }
+        CK(xfthip_paged_attention_prefill(dout.p, dq.p, dk.p, dv.p, qHeads, kvHeads, headSize, q_stride, kv_stride, oStride, scale, batch_size,
+                token_lens, kc, vc, blockNum, blockSize, (const int *)dslot.p, nullptr));
+    }
+    CK(xfthip_memcpy_d2h(output, dout.p, (size_t)rows * oStride * 2, nullptr));
+    // the host copies of the caches get the new rows too
+    for (int r = 0; r < rows; ++r) {
+        const int slot = slot_mapping[r];
+        if (slot < 0 || slot >= blockNum * blockSize) continue;
+        memcpy((uint16_t *)const_cast<void *>(kcache) + (size_t)slot * rowElems, (const uint16_t *)key + (size_t)r * kv_stride, rowElems * 2);
+        memcpy((uint16_t *)const_cast<void *>(vcache) + (size_t)slot * rowElems, (const uint16_t *)value + (size_t)r * kv_stride, rowElems * 2);
+    }
+}
+
 void invokeAttentionLLaMA(DataType dt, int batchSize, int inputSeqLen, int attHeadDim, int attHeadNum, int kvHeadNum,
         int maxPositions, int maxPosEmbed, int pastSeqLen, int currentSeqLen, int step, int hiddenSize, void *output,
         int outputStride, const void *input, int inputStride, const void *queryWeight, const void *keyWeight,

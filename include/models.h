@@ -7,8 +7,8 @@
 // for Llama-family model directories (config.ini + .bin files as the reference's convert tools
 // write them, src/models/common_decoder.h:167-262, src/layers/decoder_block.h:205-343) on one
 // MI355X.  Greedy search and sampling (top-k / top-p / temperature, repetition penalty, stop
-// words) are served; beam search, prefix sharing and the sequence-id (continuous batching)
-// overloads print a message and exit(-1), the reference's style for an unsupported request.
+// words) and the sequence-id (continuous batching) interface are served; beam search and prefix
+// sharing print a message and exit(-1), the reference's style for an unsupported request.
 // The declarations follow intel/xFasterTransformer (Apache-2.0, Copyright (c) Intel Corporation).
 #pragma once
 
@@ -74,12 +74,24 @@ public:
 
     bool setStopWords(std::vector<std::vector<int>> stopWordsList);
 
+    // Continuous batching (models.cpp:278-410, 847-903): set_input with no sequence ids turns prompts of any
+    // lengths into new sequences and returns their ids; with ids it selects which live sequences the next
+    // generate() steps.  generate() runs the prompts (first call) or one decode step, greedy with optional
+    // repetition penalty, and marks a sequence done at EOS or at maxLen; finalize() returns the working
+    // sequences' tokens back to back and frees them; freeSeqs() frees sequences early.  Every live sequence
+    // holds one KV cache row of the device model (8 rows unless XFT_CB_ROWS says otherwise; the model can
+    // only grow while no sequence is alive).
+    std::vector<int> set_input(std::vector<int32_t> &inputIds_, int batchSize_, SearcherConfig &config_,
+            const std::vector<std::vector<int>> &stopWordsList_ = {});
+    std::vector<int> set_input(std::vector<std::vector<int32_t>> &inputIds_, SearcherConfig &config_,
+            const std::vector<std::vector<int>> &stopWordsList_ = {});
+    std::vector<int> set_input(std::vector<std::vector<int32_t>> &inputIds_, std::vector<int> seqIDs, SearcherConfig &config_,
+            const std::vector<std::vector<int>> &stopWordsList_ = {});
+    bool freeSeqs(std::vector<int> &seqIDs);
+
     // not served by this build (print + exit(-1))
     void setPrefix(std::vector<int32_t> &prefixIDs);
     void unsetPrefix();
-    bool freeSeqs(std::vector<int> &seqIDs);
-    std::vector<int> set_input(std::vector<int32_t> &inputIds_, int batchSize_, SearcherConfig &config_,
-            const std::vector<std::vector<int>> &stopWordsList_ = {});
 
 protected:
     ModelImpl *impl;

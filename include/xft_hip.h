@@ -377,6 +377,29 @@ int xfthip_model_prefill(xfthip_model_t m, const int *ids_host, int B, int S, fl
  * [steps, B] or NULL.  Must follow xfthip_model_prefill with the same B.
  */
 int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_stream_t stream);
+/*
+ * Continuous batching: every sequence lives in one of the model's max_batch cache rows, at its own
+ * position; sequences start, step and end independently.  Replaces what the reference's second
+ * Attention::forward overload (src/layers/attention.h:501-730) and its per-sequence KV manager
+ * (src/common/kvcache_mgr.h:37-194, src/common/sequence.h) give CommonDecoder::forward(seqs):
+ * prompts of different lengths in one batch and decode steps over any subset of the live sequences.
+ * The caller assigns rows (the host layer's Model class keeps the sequence-id -> row map).
+ *   _seq_prefill: the prompt of ONE sequence (ids_host int32 [S]) into `row`: its first token becomes the
+ *       row's next input, its position S; logits_host (fp32 [vocab]) may be NULL.
+ *   _seq_decode: one step for the listed rows (each must hold a sequence); every other row keeps its
+ *       token, position and cache.  ids_out_host int32 [n], in the order of rows_host.  All rows up to
+ *       the highest live one run through the kernels (the step is one graph over a dense batch);
+ *       the rows that sit out are masked when ids and positions are updated.
+ *   _seq_set_next_id / _seq_logits: the searcher's hooks (replace the token a row feeds next; read
+ *       the row's last logits).
+ *   _seq_release: frees the row.
+ * xfthip_model_prefill resets this state (all rows in lockstep again).
+ */
+int xfthip_model_seq_prefill(xfthip_model_t m, int row, const int *ids_host, int S, float *logits_host, xfthip_stream_t stream);
+int xfthip_model_seq_decode(xfthip_model_t m, const int *rows_host, int n, int *ids_out_host, xfthip_stream_t stream);
+int xfthip_model_seq_set_next_id(xfthip_model_t m, int row, int id);
+int xfthip_model_seq_logits(xfthip_model_t m, int row, float *logits_host);
+int xfthip_model_seq_release(xfthip_model_t m, int row);
 /* enable (default) or disable replaying the decode step as a captured HIP graph; with 0 every
  * step launches its kernels one by one (for per-kernel profiling) */
 int xfthip_model_use_graph(xfthip_model_t m, int enable);

@@ -31,6 +31,9 @@ _lib.xft_automodel_finalize.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
 _lib.xft_automodel_forward.argtypes = [C.c_void_p, C.c_void_p]
 _lib.xft_automodel_vocab_size.argtypes = [C.c_void_p]
 _lib.xft_automodel_max_seq_len.argtypes = [C.c_void_p]
+_lib.xft_automodel_set_input.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
+                                         C.c_float, C.c_void_p]
+_lib.xft_automodel_free_seqs.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
 _lib.xft_sample_candidates.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_float, C.c_void_p, C.c_void_p]
 _lib.xft_sample_pick.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_float]
 
@@ -122,6 +125,34 @@ class AutoModel:
         self._batch = a.shape[0]
         _lib.xft_automodel_input(self._h, a.ctypes.data, a.shape[0], a.shape[1])
 
+    def set_input_cb(self, input_ids=None, seq_ids=None, max_length=20, eos_token_id=-1, pad_token_id=-1, repetition_penalty=1.0):
+        """Continuous batching (automodel.py:41-69 of the reference): prompts of any lengths become new
+        sequences when seq_ids is None, else seq_ids names the live sequences the next forward_cb() steps.
+        Returns the sequence ids."""
+        if seq_ids is None:
+            prompts = [list(map(int, (p.tolist() if hasattr(p, "tolist") else p))) for p in input_ids]
+            given = np.zeros(0, np.int32)
+        else:
+            given = np.ascontiguousarray(seq_ids.tolist() if hasattr(seq_ids, "tolist") else seq_ids, np.int32)
+            prompts = [[0]] * len(given)
+        lens = np.asarray([len(p) for p in prompts], np.int32)
+        flat = np.asarray([t for p in prompts for t in p], np.int32)
+        out = np.zeros(len(prompts), np.int32)
+        n = _lib.xft_automodel_set_input(self._h, lens.ctypes.data, flat.ctypes.data, len(prompts), given.ctypes.data if len(given) else None,
+                                         len(given), int(max_length), int(eos_token_id), int(pad_token_id), float(repetition_penalty),
+                                         out.ctypes.data)
+        self._batch = n
+        self._torch_out = False
+        return out[:n].tolist()
+
+    def forward_cb(self):
+        """One step of the sequences chosen by set_input_cb: their next tokens, in that order."""
+        return self.forward().ravel().tolist()
+
+    def free_seqs(self, seq_ids):
+        ids = np.ascontiguousarray(seq_ids.tolist() if hasattr(seq_ids, "tolist") else seq_ids, np.int32)
+        return bool(_lib.xft_automodel_free_seqs(self._h, ids.ctypes.data, len(ids)))
+
     def _wrap(self, a):
         if self._torch_out:
             import torch
@@ -147,6 +178,8 @@ class AutoModel:
         n = _lib.xft_automodel_finalize(self._h, None, 0)
         out = np.zeros(n, np.int32)
         _lib.xft_automodel_finalize(self._h, out.ctypes.data, n)
+        if self._batch <= 0 or n % self._batch != 0:
+            return self._wrap(out)  # sequences of different lengths, back to back
         return self._wrap(out.reshape(self._batch, -1))
 
     def generate(self, input_ids=None, max_length=20, num_beams=1, num_return_sequences=1, length_penalty=1.0,

@@ -389,6 +389,29 @@ class Model:
     def decode_mode(self):
         return int(lib.xfthip_model_decode_mode(self.h))
 
+    def seq_prefill(self, row, ids, want_logits=False, stream=None):
+        ids = np.ascontiguousarray(ids, np.int32).ravel()
+        logits = np.empty(self.cfg.vocab, np.float32) if want_logits else None
+        check(lib.xfthip_model_seq_prefill(self.h, int(row), _hp(ids), len(ids), _hp(logits), stream))
+        return logits
+
+    def seq_decode(self, rows, stream=None):
+        rows = np.ascontiguousarray(rows, np.int32)
+        out = np.empty(len(rows), np.int32)
+        check(lib.xfthip_model_seq_decode(self.h, _hp(rows), len(rows), _hp(out), stream))
+        return out
+
+    def seq_logits(self, row):
+        out = np.empty(self.cfg.vocab, np.float32)
+        check(lib.xfthip_model_seq_logits(self.h, int(row), _hp(out)))
+        return out
+
+    def seq_set_next_id(self, row, tok):
+        check(lib.xfthip_model_seq_set_next_id(self.h, int(row), int(tok)))
+
+    def seq_release(self, row):
+        check(lib.xfthip_model_seq_release(self.h, int(row)))
+
     def set_next_ids(self, ids, stream=None):
         ids = np.ascontiguousarray(ids, np.int32)
         check(lib.xfthip_model_set_next_ids(self.h, _hp(ids), stream))

@@ -78,7 +78,12 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, cl = lane & 15;
-    const int past = p.past_dev ? p.past_dev[b] : p.past;
+    int past = p.past;
+    if (p.past_dev) {
+        // a position read from device memory is held inside the cache whatever it contains
+        past = p.past_dev[b];
+        past = past < 0 ? 0 : (past > p.kv.S - p.S ? p.kv.S - p.S : past);
+    }
 
     // this lane's column
     const int ncols = p.S * p.G;

@@ -253,6 +253,52 @@ struct ModelImpl {
     int step = 0, curLen = 0, batch = 0;
     std::mt19937_64 rng {std::random_device {}()};
 
+    // continuous batching (Model::set_input / generate / freeSeqs): the sequence pool and the
+    // sequence-id -> cache-row map, the roles of SequencePool and KVCacheMgr
+    // (src/common/sequence.h, src/common/kvcache_mgr.h:37-194)
+    struct Seq {
+        int id = 0, row = 0, step = 0;
+        bool done = false;
+        std::vector<int32_t> prompt, generated;
+        SearcherConfig cfg;
+        std::vector<int> cachedRepetVec;
+    };
+    std::map<int, Seq> pool;
+    std::vector<int> working; // ids of the sequences the next generate() call steps
+    int nextSeqId = 0;
+    bool cbMode = false;
+
+    int free_row() const {
+        std::vector<char> used(cfg.max_batch, 0);
+        for (auto &kv : pool) used[kv.second.row] = 1;
+        for (int r = 0; r < cfg.max_batch; ++r)
+            if (!used[r]) return r;
+        return -1;
+    }
+
+    // Room for `add` more sequences of up to maxLen tokens.  The device model (and with it every cache row)
+    // is rebuilt when it has to grow, which is only possible while no sequence is alive.
+    void fit_rows(int add, int maxLen, int longestPrompt) {
+        const int live = (int)pool.size();
+        int rows = 8;
+        if (const char *e = getenv("XFT_CB_ROWS")) rows = atoi(e) > 0 ? atoi(e) : rows;
+        const bool grow = model == nullptr || live + add > cfg.max_batch || maxLen + 1 > cfg.max_seq || longestPrompt > cfg.max_tokens;
+        if (!grow) return;
+        if (live > 0) {
+            printf("[ERROR] %d sequences are alive in %d cache rows of %d positions: no room for %d more of length %d.\n", live, cfg.max_batch,
+                    cfg.max_seq, add, maxLen);
+            exit(-1);
+        }
+        if (model) CK(xfthip_model_destroy(model)); // rebuilt below with the larger limits
+        model = nullptr;
+        cfg.max_batch = std::max(std::max(cfg.max_batch, rows), add);
+        fit(cfg.max_batch, std::max(longestPrompt, 1), maxLen + 1);
+        if (cfg.max_tokens < longestPrompt) {
+            printf("[ERROR] internal: token capacity %d below the prompt length %d.\n", cfg.max_tokens, longestPrompt);
+            exit(-1);
+        }
+    }
+
     ModelImpl() {
         // the reference seeds its sampler from std::random_device on every step (sample_search.cpp:229-231);
         // XFT_SEED makes a run repeatable
@@ -531,6 +577,11 @@ Model::~Model() {
 }
 
 void Model::input(std::vector<int32_t> &inputIds_, int batchSize_) {
+    if (impl->cbMode && !impl->pool.empty()) {
+        printf("Model::input: %zu sequences of the sequence-id interface are still alive; free them first.\n", impl->pool.size());
+        exit(-1);
+    }
+    impl->cbMode = false;
     if (batchSize_ <= 0 || inputIds_.empty() || inputIds_.size() % (size_t)batchSize_ != 0) {
         printf("Model::input: %zu ids do not form %d sequences of equal length.\n", inputIds_.size(), batchSize_);
         exit(-1);
@@ -600,6 +651,11 @@ bool Model::setStopWords(std::vector<std::vector<int>> stopWordsList) {
 
 bool Model::isDone() {
     ModelImpl &s = *impl;
+    if (s.cbMode) {
+        for (int id : s.working)
+            if (!s.pool.at(id).done) return false;
+        return true;
+    }
     if (!s.haveSearcher || inputIds.empty()) {
         printf("Please set input and config first.\n");
         exit(-1);
@@ -623,8 +679,81 @@ std::tuple<float *, int, int> Model::forward(bool logitsAll) {
     return std::make_tuple(s.logitsHost.data(), 0, s.vocab);
 }
 
+// models.cpp:847-903: one step of the working sequences, all prompts or all decodes
+static std::vector<int32_t> generate_cb(ModelImpl &s) {
+    if (s.working.empty()) {
+        printf("Please set input tokens by model.set_input().\n");
+        exit(-1);
+    }
+    const int n = (int)s.working.size();
+    std::vector<ModelImpl::Seq *> seqs;
+    for (int id : s.working) seqs.push_back(&s.pool.at(id));
+    const bool prompts = seqs[0]->step == 0;
+    for (auto *q : seqs)
+        if ((q->step == 0) != prompts) {
+            printf("[ERROR] The sequences of one step must be all prompts or all decodes.\n");
+            exit(-1);
+        }
+    std::vector<int> ids(n);
+    if (prompts) {
+        std::vector<int> all(s.cfg.max_batch);
+        for (int i = 0; i < n; ++i) {
+            CK(xfthip_model_seq_prefill(s.model, seqs[i]->row, seqs[i]->prompt.data(), (int)seqs[i]->prompt.size(), nullptr, nullptr));
+            CK(xfthip_model_last_ids(s.model, all.data(), nullptr));
+            ids[i] = all[seqs[i]->row];
+        }
+    } else {
+        std::vector<int> rows(n);
+        for (int i = 0; i < n; ++i) rows[i] = seqs[i]->row;
+        CK(xfthip_model_seq_decode(s.model, rows.data(), n, ids.data(), nullptr));
+    }
+    // repetition penalty (search_utils.cpp:103-171) then first-maximum arg-max on the host
+    std::vector<float> lg;
+    for (int i = 0; i < n; ++i) {
+        ModelImpl::Seq &q = *seqs[i];
+        if (q.cfg.repetitionPenalty == 1.0f) continue;
+        auto &v = q.cachedRepetVec;
+        if (q.step == 0) {
+            v = std::vector<int>(q.prompt.begin(), q.prompt.end());
+            std::sort(v.begin(), v.end());
+            v.erase(std::unique(v.begin(), v.end()), v.end());
+        } else {
+            const int last = q.generated.back();
+            auto it = std::lower_bound(v.begin(), v.end(), last);
+            if (it == v.end() || *it != last) v.insert(it, last);
+        }
+        lg.resize(s.vocab);
+        CK(xfthip_model_seq_logits(s.model, q.row, lg.data()));
+        for (int idx : v) {
+            if (idx < 0 || idx >= s.vocab) continue;
+            lg[idx] = lg[idx] < 0 ? lg[idx] * q.cfg.repetitionPenalty : lg[idx] / q.cfg.repetitionPenalty;
+        }
+        int best = 0;
+        for (int j = 1; j < s.vocab; ++j)
+            if (lg[j] > lg[best]) best = j;
+        ids[i] = best;
+    }
+    // stopCheck (sampling.cpp:134-154), then every sequence steps forward with its token
+    for (int i = 0; i < n; ++i) {
+        ModelImpl::Seq &q = *seqs[i];
+        if (q.done) {
+            ids[i] = q.cfg.eosTokenId;
+        } else if (ids[i] == q.cfg.eosTokenId) {
+            q.done = true;
+        } else if ((int)(q.prompt.size() + q.generated.size()) + 1 >= q.cfg.maxLen) {
+            q.done = true;
+        }
+        q.generated.push_back(ids[i]);
+        q.step++;
+        // the row feeds what the searcher settled on
+        if (ids[i] >= 0 && ids[i] < s.vocab) CK(xfthip_model_seq_set_next_id(s.model, q.row, ids[i]));
+    }
+    return std::vector<int32_t>(ids.begin(), ids.end());
+}
+
 std::vector<int32_t> Model::generate() {
     ModelImpl &s = *impl;
+    if (s.cbMode) return generate_cb(s);
     if (!s.haveSearcher) {
         printf("Please set the generation config by model.config().\n");
         exit(-1);
@@ -691,7 +820,19 @@ std::vector<int32_t> Model::generate() {
 }
 
 std::vector<int32_t> Model::finalize() {
-    return impl->output;
+    ModelImpl &s = *impl;
+    if (!s.cbMode) return s.output;
+    // models.cpp:738-756: prompt + generated tokens of the working sequences, back to back; their cache
+    // rows are released
+    std::vector<int32_t> result;
+    std::vector<int> ids = s.working;
+    for (int id : ids) {
+        ModelImpl::Seq &q = s.pool.at(id);
+        result.insert(result.end(), q.prompt.begin(), q.prompt.end());
+        result.insert(result.end(), q.generated.begin(), q.generated.end());
+    }
+    freeSeqs(ids);
+    return result;
 }
 
 void Model::setPrefix(std::vector<int32_t> &) {
@@ -700,13 +841,102 @@ void Model::setPrefix(std::vector<int32_t> &) {
 void Model::unsetPrefix() {
     unsupported("Prefix sharing");
 }
-bool Model::freeSeqs(std::vector<int> &) {
-    unsupported("The sequence-id interface (freeSeqs)");
-    return false;
+bool Model::freeSeqs(std::vector<int> &seqIDs) {
+    ModelImpl &s = *impl;
+    bool all = true;
+    for (int id : seqIDs) {
+        auto it = s.pool.find(id);
+        if (it == s.pool.end()) {
+            all = false;
+            continue;
+        }
+        CK(xfthip_model_seq_release(s.model, it->second.row));
+        s.pool.erase(it);
+        s.working.erase(std::remove(s.working.begin(), s.working.end(), id), s.working.end());
+    }
+    return all;
 }
-std::vector<int> Model::set_input(std::vector<int32_t> &, int, SearcherConfig &, const std::vector<std::vector<int>> &) {
-    unsupported("The sequence-id interface (set_input)");
-    return {};
+
+// models.cpp:278-349: new sequences (prompts of any lengths), one pool entry and one cache row each
+std::vector<int> Model::set_input(std::vector<std::vector<int32_t>> &inputIds_, SearcherConfig &config_,
+        const std::vector<std::vector<int>> &stopWordsList_) {
+    std::vector<int> none;
+    return set_input(inputIds_, none, config_, stopWordsList_);
+}
+
+std::vector<int> Model::set_input(std::vector<int32_t> &inputIds_, int batchSize_, SearcherConfig &config_,
+        const std::vector<std::vector<int>> &stopWordsList_) {
+    if (batchSize_ <= 0 || inputIds_.size() % (size_t)batchSize_ != 0) {
+        printf("Model::set_input: %zu ids do not form %d sequences of equal length.\n", inputIds_.size(), batchSize_);
+        exit(-1);
+    }
+    const size_t len = inputIds_.size() / (size_t)batchSize_;
+    std::vector<std::vector<int32_t>> rows;
+    for (int b = 0; b < batchSize_; ++b) rows.emplace_back(inputIds_.begin() + b * len, inputIds_.begin() + (b + 1) * len);
+    std::vector<int> none;
+    return set_input(rows, none, config_, stopWordsList_);
+}
+
+// models.cpp:351-410: with no ids, the prompts become new sequences; with ids, those live sequences form
+// the batch of the next generate() call (their inputs are the tokens they produced last)
+std::vector<int> Model::set_input(std::vector<std::vector<int32_t>> &inputIds_, std::vector<int> seqIDs, SearcherConfig &config_,
+        const std::vector<std::vector<int>> &stopWordsList_) {
+    ModelImpl &s = *impl;
+    if (!stopWordsList_.empty()) printf("Model::set_input: stop words are not checked on this path (as in the reference).\n");
+    if (config_.numBeams != 1) unsupported("Beam search (numBeams != 1)");
+    if (config_.doSample) unsupported("Sampling with sequence ids (the reference throws here as well)");
+    if (config_.repetitionPenalty <= 0) {
+        printf("`repetitionPenalty` has to be a strictly positive float, but is %f.\n", config_.repetitionPenalty);
+        exit(-1);
+    }
+    if (config_.eosTokenId == -1) config_.eosTokenId = s.endId;
+    if (config_.padTokenId == -1) config_.padTokenId = config_.eosTokenId;
+    if (config_.maxLen < 0) config_.maxLen = maxSeqLen;
+    config_.maxLen = std::min(config_.maxLen, maxSeqLen);
+    configuration = config_;
+    batchSize = (int)inputIds_.size();
+    s.cbMode = true;
+    s.working.clear();
+    if (seqIDs.empty()) {
+        int maxLen = config_.maxLen, longest = 0;
+        for (auto &ids : inputIds_) {
+            if (ids.empty()) {
+                printf("[ERROR] Empty prompt.\n");
+                exit(-1);
+            }
+            maxLen = std::max(maxLen, (int)ids.size());
+            longest = std::max(longest, (int)ids.size());
+        }
+        s.fit_rows(batchSize, maxLen, longest);
+        for (auto &ids : inputIds_) {
+            ModelImpl::Seq q;
+            q.id = s.nextSeqId++;
+            q.prompt = ids;
+            q.cfg = config_;
+            q.cfg.maxLen = maxLen;
+            q.row = s.free_row();
+            if (q.row < 0) {
+                printf("[ERROR] No free KV cache row.\n");
+                exit(-1);
+            }
+            s.pool[q.id] = q;
+            s.working.push_back(q.id);
+            seqIDs.push_back(q.id);
+        }
+    } else {
+        if (inputIds_.size() != seqIDs.size()) {
+            printf("[ERROR] Input size and seqIDs size mismatch.\n");
+            exit(-1);
+        }
+        for (int id : seqIDs) {
+            if (!s.pool.count(id)) {
+                printf("[ERROR] Sequence ID %d not found.\n", id);
+                exit(-1);
+            }
+            s.working.push_back(id);
+        }
+    }
+    return seqIDs;
 }
 
 AutoModel::AutoModel(std::string modelPath, xft::DataType dataType, xft::DataType KVCacheDataType) : Model() {
@@ -854,11 +1084,17 @@ int xft_automodel_is_done(void *h) {
     return ((xft::AutoModel *)h)->isDone() ? 1 : 0;
 }
 
-// copies up to `capacity` ids of the [batch, length] result; returns how many there are
+// Two-call protocol: out = NULL finalizes (which also frees continuously batched sequences) and returns
+// the number of ids; the next call with a buffer copies them out.
 int xft_automodel_finalize(void *h, int *out, int capacity) {
-    std::vector<int32_t> r = ((xft::AutoModel *)h)->finalize();
+    static std::map<void *, std::vector<int32_t>> pending;
+    if (out == nullptr || !pending.count(h)) pending[h] = ((xft::AutoModel *)h)->finalize();
+    std::vector<int32_t> &r = pending[h];
     const int n = (int)r.size();
-    if (out) memcpy(out, r.data(), (size_t)std::min(n, capacity) * 4);
+    if (out) {
+        memcpy(out, r.data(), (size_t)std::min(n, capacity) * 4);
+        pending.erase(h);
+    }
     return n;
 }
 
@@ -868,6 +1104,28 @@ int xft_automodel_forward(void *h, float *logits_out) {
     xft::AutoModel *m = (xft::AutoModel *)h;
     memcpy(logits_out, std::get<0>(t), (size_t)m->getBatchSize() * std::get<2>(t) * 4);
     return std::get<2>(t);
+}
+
+// Continuous batching.  Prompts arrive flattened (n lengths, then the ids back to back); seq_ids may be
+// NULL (n_ids = 0: new sequences).  Returns the number of sequence ids written to ids_out.
+int xft_automodel_set_input(void *h, const int *lens, const int *ids, int n, const int *seq_ids, int n_ids, int maxLen, int eosTokenId,
+        int padTokenId, float repetitionPenalty, int *ids_out) {
+    std::vector<std::vector<int32_t>> prompts;
+    int off = 0;
+    for (int i = 0; i < n; ++i) {
+        prompts.emplace_back(ids + off, ids + off + lens[i]);
+        off += lens[i];
+    }
+    SearcherConfig cfg(maxLen, 1, 1, 1.0f, false, eosTokenId, padTokenId, false, 1.0f, 50, 1.0f, repetitionPenalty);
+    std::vector<int> given(seq_ids, seq_ids + n_ids);
+    std::vector<int> out = ((xft::AutoModel *)h)->set_input(prompts, given, cfg, {});
+    memcpy(ids_out, out.data(), out.size() * 4);
+    return (int)out.size();
+}
+
+int xft_automodel_free_seqs(void *h, const int *seq_ids, int n) {
+    std::vector<int> v(seq_ids, seq_ids + n);
+    return ((xft::AutoModel *)h)->freeSeqs(v) ? 1 : 0;
 }
 
 int xft_automodel_vocab_size(void *h) {

@@ -49,8 +49,10 @@ __global__ void gather_last_kernel(const float *__restrict__ x, float *__restric
 // across threads
 // advance_pos / advance_step (may be null): the decode step's position and step counters, bumped
 // here so that the step needs no launches of its own for them
+// active: optional per-row flags; a row whose flag is 0 keeps its id and its position (a sequence
+// that sits out this step of a continuously batched decode)
 __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ logits, int cols, int *__restrict__ ids,
-        int *advance_pos, int *advance_step) {
+        int *advance_pos, int *advance_step, const int *__restrict__ active) {
     __shared__ float sv[1024];
     __shared__ int si[1024];
     const float *p = logits + (size_t)blockIdx.x * cols;
@@ -86,8 +88,9 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ 
         __syncthreads();
     }
     if (threadIdx.x == 0) {
-        ids[blockIdx.x] = si[0];
-        if (advance_pos) advance_pos[blockIdx.x] += 1;
+        const bool on = active == nullptr || active[blockIdx.x] != 0;
+        if (on) ids[blockIdx.x] = si[0];
+        if (advance_pos && on) advance_pos[blockIdx.x] += 1;
         if (advance_step && blockIdx.x == 0) advance_step[0] += 1;
     }
 }
@@ -139,6 +142,12 @@ struct xfthip_model {
     xfthip_weight_t lm_head = nullptr;
     // decode state
     int cur_B = 0, cur_pos = 0;
+    // continuous batching: sequences live in cache rows of their own, each at its own position
+    int row0 = 0; // cache row of the first sequence of the forward call in flight
+    bool ragged = false; // rows may differ in position or sit out a step (set by the xfthip_model_seq_* calls)
+    int *active = nullptr; // device [max_batch]: rows taking part in the next decode call
+    int *prompt_ids = nullptr; // device [max_tokens]: prompt of a single-sequence prefill
+    std::vector<int> row_pos; // host copy of every row's position (-1 = free row)
     hipGraphExec_t graph = nullptr;
     int graph_B = 0;
     int graph_nsplit = 0; // attention split count the captured step was built with
@@ -317,6 +326,17 @@ static int attention_block(xfthip_model *m, int idx, const float *x_in, int in_s
     const int qcols = c.q_heads * c.head_size, kvcols = c.kv_heads * c.head_size;
     const int qkv_cols = qcols + 2 * kvcols;
     int rc;
+    // the B sequences of this call live in cache rows row0 .. row0 + B - 1
+    auto rows_of = [&](xfthip_kvcache_t full) {
+        xfthip_kvcache v = *full;
+        const size_t per_row = (size_t)v.kv.H * v.kv.S * v.kv.D;
+        v.kv.k = (char *)v.kv.k + (size_t)m->row0 * per_row * (v.kv.int8 ? 1 : 2);
+        v.kv.v = (char *)v.kv.v + (size_t)m->row0 * per_row * (v.kv.int8 ? 1 : 2);
+        if (v.kv.kscale) v.kv.kscale += (size_t)m->row0 * v.kv.H * v.kv.S, v.kv.vscale += (size_t)m->row0 * v.kv.H * v.kv.S;
+        v.kv.B = full->kv.B - m->row0;
+        return v;
+    };
+    xfthip_kvcache layer_cache = rows_of(m->caches[idx]);
     // Decode step (one new token per sequence, a handful of rows): the norm runs as the QKV
     // GEMV's prologue and the rotation + cache append as its epilogue, which takes two launches
     // (and their gaps) out of every layer.
@@ -348,7 +368,7 @@ static int attention_block(xfthip_model *m, int idx, const float *x_in, int in_s
         }
         if (fuse_rope) {
             sp.rope = 1, sp.cosT = m->cosT, sp.sinT = m->sinT, sp.pos_dev = past_dev, sp.pos_host = past;
-            sp.qH = c.q_heads, sp.kvH = c.kv_heads, sp.kv = m->caches[idx]->kv;
+            sp.qH = c.q_heads, sp.kvH = c.kv_heads, sp.kv = layer_cache.kv;
         }
         if ((rc = qgemm_skinny(wq, sp, st))) return rc;
     } else {
@@ -357,14 +377,16 @@ static int attention_block(xfthip_model *m, int idx, const float *x_in, int in_s
             return rc;
     }
     if (!fuse_rope)
-        if ((rc = xfthip_rope_kvstore(m->caches[idx], m->qkv, XFTHIP_BF16, qkv_cols, B, S, c.q_heads, m->cosT, m->sinT, past, past_dev, st)))
+        if ((rc = xfthip_rope_kvstore(&layer_cache, m->qkv, XFTHIP_BF16, qkv_cols, B, S, c.q_heads, m->cosT, m->sinT, past, past_dev, st)))
             return rc;
-    xfthip_kvcache_t attend = m->caches[idx];
+    xfthip_kvcache_t attend = &layer_cache;
+    xfthip_kvcache first_pass;
     if (c.kv_dtype == XFTHIP_INT8 && S > 1 && past == 0 && past_dev == nullptr) {
-        if ((rc = rope_kvstore_impl(m->prefill_cache, m->qkv, XFTHIP_BF16, qkv_cols, B, S, c.q_heads, m->cosT, m->sinT, 0, nullptr,
+        first_pass = rows_of(m->prefill_cache);
+        if ((rc = rope_kvstore_impl(&first_pass, m->qkv, XFTHIP_BF16, qkv_cols, B, S, c.q_heads, m->cosT, m->sinT, 0, nullptr,
                      false, st)))
             return rc;
-        attend = m->prefill_cache;
+        attend = &first_pass;
     }
     if ((rc = attention_launch(attend, m->qkv, qkv_cols, m->att, qcols, XFTHIP_BF16, B, S, c.q_heads, 1.0f / sqrtf((float)c.head_size), past,
                  past_dev, past_dev ? m->len_hint : 0, st, &m->attn_ws)))
@@ -425,14 +447,15 @@ static int layer_forward(xfthip_model *m, int idx, const float *x_in, int in_str
 static int head_forward(xfthip_model *m, const float *xrows, int B, bool advance, hipStream_t st) {
     const xfthip_model_config &c = m->cfg;
     int rc;
+    const int r0 = m->row0; // logits, ids and positions of row r0 + b
     // (the norm stays a kernel of its own here: as a prologue of the 2000-tile lm_head GEMV it cost
     // 3 us more than it saved)
     if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, xrows, XFTHIP_F32, m->final_norm, B, c.hidden, c.hidden, c.hidden, c.rms_eps, st))) return rc;
-    if ((rc = xfthip_gemm(m->lm_head, B, m->xn, c.hidden, m->logits, c.vocab, XFTHIP_F32, XFTHIP_EPI_NONE, nullptr, nullptr, 0, XFTHIP_F32,
-                 1.0f, st)))
+    if ((rc = xfthip_gemm(m->lm_head, B, m->xn, c.hidden, m->logits + (size_t)r0 * c.vocab, c.vocab, XFTHIP_F32, XFTHIP_EPI_NONE, nullptr,
+                 nullptr, 0, XFTHIP_F32, 1.0f, st)))
         return rc;
-    hipLaunchKernelGGL(argmax_kernel, dim3(B), dim3(1024), 0, st, m->logits, c.vocab, m->ids, advance ? m->pos : nullptr,
-            advance ? m->step : nullptr);
+    hipLaunchKernelGGL(argmax_kernel, dim3(B), dim3(1024), 0, st, m->logits + (size_t)r0 * c.vocab, c.vocab, m->ids + r0,
+            advance ? m->pos + r0 : nullptr, advance ? m->step : nullptr, (advance && m->ragged) ? m->active + r0 : nullptr);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }
@@ -450,7 +473,8 @@ extern "C" {
 
 int xfthip_argmax(const float *logits, int rows, int cols, int *ids_dev, xfthip_stream_t stream) {
     XFT_REQUIRE(logits && ids_dev && rows > 0 && cols > 0, "xfthip_argmax: bad argument");
-    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, logits, cols, ids_dev, (int *)nullptr, (int *)nullptr);
+    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, logits, cols, ids_dev, (int *)nullptr, (int *)nullptr,
+            (const int *)nullptr);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }
@@ -478,7 +502,9 @@ int xfthip_model_create(const xfthip_model_config *cfg, xfthip_model_t *out) {
     if (int rc = attention_workspace_create(&m->attn_ws, kWsSlots)) return fail(rc);
     if (c.kv_dtype == XFTHIP_INT8)
         if (int rc = xfthip_kvcache_create(XFTHIP_FP16, c.max_batch, c.kv_heads, c.max_seq, c.head_size, &m->prefill_cache)) return fail(rc);
-    if (int rc = xfthip_rope_tables_create(c.head_size, c.max_pos_embed, c.rope_base, 1.0f, &m->cosT, &m->sinT)) return fail(rc);
+    // (the tables cover the cache rows up to their padded length: a clamped device position stays inside both)
+    const int table_rows = c.max_pos_embed > (c.max_seq + 31) / 32 * 32 ? c.max_pos_embed : (c.max_seq + 31) / 32 * 32;
+    if (int rc = xfthip_rope_tables_create(c.head_size, table_rows, c.rope_base, 1.0f, &m->cosT, &m->sinT)) return fail(rc);
     const size_t T = c.max_tokens;
     const size_t qkv_cols = (size_t)(c.q_heads + 2 * c.kv_heads) * c.head_size;
     bool ok = hipMalloc((void **)&m->xn, T * (c.hidden > c.intermediate ? c.hidden : c.intermediate) * 2) == hipSuccess
@@ -493,6 +519,12 @@ int xfthip_model_create(const xfthip_model_config *cfg, xfthip_model_t *out) {
     if (ok && c.vocab > 0) ok = hipMalloc((void **)&m->logits, (size_t)c.max_batch * c.vocab * 4) == hipSuccess;
     if (!ok) {
         set_error("xfthip_model_create: scratch allocation failed");
+        return fail(1);
+    }
+    // every row starts at position 0 with token 0: a decode step may run over rows that hold no sequence
+    if (hipMemset(m->ids, 0, (size_t)(T > 64 ? T : 64) * 4) != hipSuccess || hipMemset(m->pos, 0, (size_t)c.max_batch * 4) != hipSuccess
+            || hipMemset(m->step, 0, 64) != hipSuccess) {
+        set_error("xfthip_model_create: clearing the position buffers failed");
         return fail(1);
     }
     m->idlog_cap = c.max_seq + 1;
@@ -517,7 +549,7 @@ int xfthip_model_destroy(xfthip_model_t m) {
         if (L.o_bias) (void)hipFree(L.o_bias);
     }
     void *bufs[] = {m->w8a8_qa, m->w8a8_stat, m->gu, m->mega_trace, m->mega_layers, m->mega_ws, m->mega_sync, m->cosT, m->sinT, m->xn, m->qkv, m->att, m->h, m->x, m->xlast, m->logits, m->ids, m->pos, m->step, m->idlog,
-            m->embedding, m->final_norm};
+            m->embedding, m->final_norm, m->active, m->prompt_ids};
     for (void *b : bufs)
         if (b) (void)hipFree(b);
     delete m;
@@ -647,6 +679,10 @@ int xfthip_model_prefill(xfthip_model_t m, const int *ids_host, int B, int S, fl
     XFT_REQUIRE(B > 0 && B <= c.max_batch && S > 0 && B * S <= c.max_tokens && S <= c.max_seq,
             "xfthip_model_prefill: B=%d S=%d exceed the model limits", B, S);
     hipStream_t st = (hipStream_t)stream;
+    m->row0 = 0;
+    m->ragged = false;
+    m->row_pos.assign(c.max_batch, -1);
+    for (int b = 0; b < B; ++b) m->row_pos[b] = S;
     XFT_CHECK_HIP(hipMemcpyAsync(m->ids, ids_host, (size_t)B * S * 4, hipMemcpyHostToDevice, st));
     hipLaunchKernelGGL(embed_kernel, dim3(B * S), dim3(256), 0, st, m->embedding, m->ids, m->x, c.hidden, c.vocab);
     for (int l = 0; l < c.layers; ++l)
@@ -679,7 +715,7 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
     m->len_hint = ((m->cur_pos + steps + 127) / 128) * 128;
     const int nsplit = attention_split_count(m->len_hint < c.max_seq ? m->len_hint : c.max_seq, B * c.kv_heads);
     bool persistent = false;
-    if (m->use_persistent && B <= 4 && (size_t)B * c.kv_heads <= (size_t)kWsSlots) {
+    if (m->use_persistent && !m->ragged && B <= 4 && (size_t)B * c.kv_heads <= (size_t)kWsSlots) {
         if (m->mega_state == 0)
             if (int rc = mega_prepare(m)) return rc;
         if (m->mega_state == 1)
@@ -745,6 +781,115 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
         XFT_CHECK_HIP(hipMemcpy(ids_out_host + (size_t)(steps - 1) * B, m->ids, (size_t)B * 4, hipMemcpyDeviceToHost));
     }
     m->cur_pos += steps;
+    for (int b = 0; b < B && b < (int)m->row_pos.size(); ++b)
+        if (m->row_pos[b] >= 0 && !m->ragged) m->row_pos[b] += steps;
+    return 0;
+}
+
+// ---- continuous batching: sequences come and go, each in a cache row of its own ------------------
+int xfthip_model_seq_prefill(xfthip_model_t m, int row, const int *ids_host, int S, float *logits_host, xfthip_stream_t stream) {
+    XFT_REQUIRE(m && ids_host, "xfthip_model_seq_prefill: null argument");
+    const xfthip_model_config &c = m->cfg;
+    XFT_REQUIRE(m->embedding && m->lm_head, "xfthip_model_seq_prefill: embedding / lm_head not set");
+    XFT_REQUIRE(row >= 0 && row < c.max_batch, "xfthip_model_seq_prefill: row %d outside the %d cache rows", row, c.max_batch);
+    XFT_REQUIRE(S > 0 && S <= c.max_tokens && S < c.max_seq, "xfthip_model_seq_prefill: %d tokens exceed max_tokens %d / max_seq %d", S,
+            c.max_tokens, c.max_seq);
+    hipStream_t st = (hipStream_t)stream;
+    if ((int)m->row_pos.size() != c.max_batch) m->row_pos.assign(c.max_batch, -1);
+    if (!m->active) {
+        XFT_CHECK_HIP(hipMalloc((void **)&m->active, (size_t)c.max_batch * 4));
+        XFT_CHECK_HIP(hipMemset(m->active, 0, (size_t)c.max_batch * 4));
+    }
+    if (!m->prompt_ids) XFT_CHECK_HIP(hipMalloc((void **)&m->prompt_ids, (size_t)c.max_tokens * 4));
+    if (!m->ragged) {
+        // leaving lockstep mode: no row holds a sequence, all sit at position 0 with token 0
+        XFT_CHECK_HIP(hipDeviceSynchronize());
+        XFT_CHECK_HIP(hipMemset(m->pos, 0, (size_t)c.max_batch * 4));
+        XFT_CHECK_HIP(hipMemset(m->ids, 0, (size_t)c.max_batch * 4));
+        m->row_pos.assign(c.max_batch, -1);
+        m->cur_B = 0;
+    }
+    m->ragged = true;
+    XFT_CHECK_HIP(hipMemcpyAsync(m->prompt_ids, ids_host, (size_t)S * 4, hipMemcpyHostToDevice, st));
+    hipLaunchKernelGGL(embed_kernel, dim3(S), dim3(256), 0, st, m->embedding, m->prompt_ids, m->x, c.hidden, c.vocab);
+    m->row0 = row;
+    int rc = 0;
+    for (int l = 0; l < c.layers && rc == 0; ++l) rc = layer_forward(m, l, m->x, c.hidden, m->x, c.hidden, 1, S, 0, nullptr, st);
+    if (rc == 0) {
+        hipLaunchKernelGGL(gather_last_kernel, dim3(1), dim3(256), 0, st, m->x, m->xlast, S, c.hidden);
+        rc = head_forward(m, m->xlast, 1, false, st);
+    }
+    m->row0 = 0;
+    if (rc) return rc;
+    hipLaunchKernelGGL(fill_int_kernel, dim3(1), dim3(64), 0, st, m->pos + row, 1, S);
+    XFT_CHECK_HIP(hipGetLastError());
+    XFT_CHECK_HIP(hipStreamSynchronize(st));
+    if (logits_host) XFT_CHECK_HIP(hipMemcpy(logits_host, m->logits + (size_t)row * c.vocab, (size_t)c.vocab * 4, hipMemcpyDeviceToHost));
+    m->row_pos[row] = S;
+    if (row + 1 > m->cur_B) m->cur_B = row + 1;
+    return 0;
+}
+
+int xfthip_model_seq_release(xfthip_model_t m, int row) {
+    XFT_REQUIRE(m && row >= 0 && row < m->cfg.max_batch, "xfthip_model_seq_release: bad row");
+    if ((int)m->row_pos.size() != m->cfg.max_batch) m->row_pos.assign(m->cfg.max_batch, -1);
+    m->row_pos[row] = -1;
+    // a free row keeps decoding along (at position 0, results dropped) until the rows above it are free too
+    XFT_CHECK_HIP(hipDeviceSynchronize());
+    int zero = 0;
+    if (m->pos) XFT_CHECK_HIP(hipMemcpy(m->pos + row, &zero, 4, hipMemcpyHostToDevice));
+    if (m->ids) XFT_CHECK_HIP(hipMemcpy(m->ids + row, &zero, 4, hipMemcpyHostToDevice));
+    int top = 0;
+    for (int r = 0; r < m->cfg.max_batch; ++r)
+        if (m->row_pos[r] >= 0) top = r + 1;
+    m->cur_B = top;
+    return 0;
+}
+
+int xfthip_model_seq_decode(xfthip_model_t m, const int *rows_host, int n, int *ids_out_host, xfthip_stream_t stream) {
+    XFT_REQUIRE(m && rows_host && n > 0, "xfthip_model_seq_decode: bad argument");
+    const xfthip_model_config &c = m->cfg;
+    XFT_REQUIRE(m->ragged && m->active, "xfthip_model_seq_decode: no sequence was started with xfthip_model_seq_prefill");
+    std::vector<int> act(c.max_batch, 0);
+    int top = 0, deepest = 0;
+    for (int i = 0; i < n; ++i) {
+        const int r = rows_host[i];
+        XFT_REQUIRE(r >= 0 && r < c.max_batch && m->row_pos[r] >= 0, "xfthip_model_seq_decode: row %d holds no sequence", r);
+        XFT_REQUIRE(m->row_pos[r] + 1 <= c.max_seq, "xfthip_model_seq_decode: row %d is at position %d of %d", r, m->row_pos[r], c.max_seq);
+        XFT_REQUIRE(act[r] == 0, "xfthip_model_seq_decode: row %d listed twice", r);
+        act[r] = 1;
+    }
+    for (int r = 0; r < c.max_batch; ++r)
+        if (m->row_pos[r] >= 0) {
+            top = r + 1;
+            if (m->row_pos[r] > deepest) deepest = m->row_pos[r];
+        }
+    hipStream_t st = (hipStream_t)stream;
+    XFT_CHECK_HIP(hipMemcpyAsync(m->active, act.data(), (size_t)c.max_batch * 4, hipMemcpyHostToDevice, st));
+    XFT_CHECK_HIP(hipStreamSynchronize(st));
+    // one step over rows 0 .. top - 1; the split count of the attention follows the deepest row
+    m->cur_B = top;
+    m->cur_pos = deepest;
+    if (int rc = xfthip_model_decode(m, 1, nullptr, stream)) return rc;
+    for (int i = 0; i < n; ++i) m->row_pos[rows_host[i]] += 1;
+    if (ids_out_host) {
+        std::vector<int> all(top);
+        XFT_CHECK_HIP(hipMemcpy(all.data(), m->ids, (size_t)top * 4, hipMemcpyDeviceToHost));
+        for (int i = 0; i < n; ++i) ids_out_host[i] = all[rows_host[i]];
+    }
+    return 0;
+}
+
+int xfthip_model_seq_set_next_id(xfthip_model_t m, int row, int id) {
+    XFT_REQUIRE(m && row >= 0 && row < m->cfg.max_batch && m->ids, "xfthip_model_seq_set_next_id: bad row");
+    XFT_REQUIRE(id >= 0 && id < m->cfg.vocab, "xfthip_model_seq_set_next_id: id %d outside the vocabulary", id);
+    XFT_CHECK_HIP(hipMemcpy(m->ids + row, &id, 4, hipMemcpyHostToDevice));
+    return 0;
+}
+
+int xfthip_model_seq_logits(xfthip_model_t m, int row, float *logits_host) {
+    XFT_REQUIRE(m && logits_host && row >= 0 && row < m->cfg.max_batch && m->logits, "xfthip_model_seq_logits: bad argument");
+    XFT_CHECK_HIP(hipMemcpy(logits_host, m->logits + (size_t)row * m->cfg.vocab, (size_t)m->cfg.vocab * 4, hipMemcpyDeviceToHost));
     return 0;
 }
 

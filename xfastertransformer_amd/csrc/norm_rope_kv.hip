@@ -144,7 +144,13 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(RopeKvParams p) {
     const int tok = blockIdx.y;
     const int b = tok / p.S, s = tok % p.S;
     const int half = p.D / 2;
-    const int past = p.past_dev ? p.past_dev[b] : p.past;
+    int past = p.past;
+    if (p.past_dev) {
+        // a position read from device memory is held inside the cache whatever it contains
+        past = p.past_dev[b];
+        past = past < 0 ? 0 : past;
+        if (p.kv.k && past > p.kv.S - p.S) past = p.kv.S - p.S;
+    }
     const int pos = p.positions ? p.positions[tok] : past + s;
     const bool isq = head < p.qHeads;
     if (isq && p.skip_q) return;

@@ -409,7 +409,9 @@ __global__ __launch_bounds__(512) void qgemm_skinny_kernel(SkinnyParams p) {
                     // the projection's output is bf16 in the reference (the rotation reads it back)
                     const float lo = bf16_to_f32(f32_to_bf16_ref(column_value(m, c, sumA)));
                     const float hi = bf16_to_f32(f32_to_bf16_ref(column_value(m, 16 + c, sumA)));
-                    const int i = jj * 16 + c, pos = p.pos_dev ? p.pos_dev[m] : p.pos_host;
+                    int pos = p.pos_dev ? p.pos_dev[m] : p.pos_host;
+                    pos = pos < 0 ? 0 : (pos >= p.kv.S ? p.kv.S - 1 : pos); // held inside the cache whatever the device value is
+                    const int i = jj * 16 + c;
                     const float cs = p.cosT[(size_t)pos * 64 + i], sn = p.sinT[(size_t)pos * 64 + i];
                     // reference: fmsub(q, cos, qHalf*sin) ; fmadd(qHalf, cos, q*sin)
                     const float nlo = fmaf(lo, cs, -(hi * sn)), nhi = fmaf(hi, cs, lo * sn);
@@ -430,7 +432,8 @@ __global__ __launch_bounds__(512) void qgemm_skinny_kernel(SkinnyParams p) {
                     const int vt = 2 * (it - rope_pairs) + (cc >> 4);
                     const float sumA = need_sum ? total_sum(m) : 0.0f;
                     const float val = bf16_to_f32(f32_to_bf16_ref(column_value(m, cc, sumA)));
-                    const int pos = p.pos_dev ? p.pos_dev[m] : p.pos_host;
+                    int pos = p.pos_dev ? p.pos_dev[m] : p.pos_host;
+                    pos = pos < 0 ? 0 : (pos >= p.kv.S ? p.kv.S - 1 : pos);
                     if (pos < p.kv.S) {
                         const size_t bh = (size_t)m * p.kv.H + (vt >> 3);
                         const int d = (vt & 7) * 16 + (cc & 15);

@@ -91,14 +91,20 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     const int h = lane >> 5, nl = lane & 31;
 
     // block -> (column block, row block): blocks that share a column block sit on the same XCD
-    // (block ids round-robin over the 8 XCDs), so their weight reads hit that XCD's L2
+    // (block ids round-robin over the 8 XCDs), so their weight reads hit that XCD's L2.  Row blocks are
+    // walked in bands of 8: all column blocks of a band before the next band, so that the band's
+    // activation rows stay cached while the weights stream past them.
     int nb, mb;
     {
+        constexpr int BAND = 8;
         const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
         const int nb8 = (nblocks_n + 7) >> 3;
-        nb = (slot / nblocks_m) + xcd * nb8;
-        mb = slot % nblocks_m;
-        if (slot / nblocks_m >= nb8 || nb >= nblocks_n) return;
+        if (slot >= nb8 * nblocks_m) return;
+        const int band = slot / (nb8 * BAND), rem = slot - band * (nb8 * BAND);
+        const int left = nblocks_m - band * BAND, rows_in_band = left < BAND ? left : BAND;
+        nb = rem / rows_in_band + xcd * nb8;
+        mb = band * BAND + rem % rows_in_band;
+        if (nb >= nblocks_n) return;
     }
     const int n32_0 = (nb * 4 + wave) * WN; // first 32-column tile of this wave
     const int m0 = mb * ROWS;

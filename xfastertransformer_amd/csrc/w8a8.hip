@@ -18,37 +18,97 @@ namespace xfthip {
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 
-// ---- activation quantisation: one wave per row ---------------------------------------------
+// ---- activation quantisation: one 256-thread workgroup per row -------------------------------
 // zero = (min+max)/2, scale = max(|max-zero|, |zero-min|)/127, q = rne(fma(x, 1/scale, -zero/scale)),
-// sum = (sum q) * scale + K * zero   (matmul_helper.h:2810-2853)
-__global__ __launch_bounds__(64) void w8a8_quantize_kernel(const void *__restrict__ A, int a_dtype, int K, int lda,
+// sum = (sum q) * scale + K * zero   (matmul_helper.h:2810-2853).  min / max and the integer sum do not
+// depend on the order of the reduction, so the result is the one of a sequential pass.  A thread moves
+// 8 values at a time (16-byte loads, 8-byte stores) where the row pitches allow it.
+__device__ inline void w8a8_load8(const void *A, int a_dtype, size_t at, bool wide, float v[8]) {
+    if (wide) {
+        if (a_dtype == XFTHIP_F32) {
+            const f32x4 a = *(const f32x4 *)((const float *)A + at), b = *(const f32x4 *)((const float *)A + at + 4);
+            v[0] = a[0], v[1] = a[1], v[2] = a[2], v[3] = a[3], v[4] = b[0], v[5] = b[1], v[6] = b[2], v[7] = b[3];
+        } else {
+            const i32x4 a = *(const i32x4 *)((const uint16_t *)A + at);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[2 * e] = bf16_to_f32((uint16_t)((uint32_t)a[e] & 0xFFFFu));
+                v[2 * e + 1] = bf16_to_f32((uint16_t)((uint32_t)a[e] >> 16));
+            }
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = load_as_f32(A, a_dtype, at + e);
+    }
+}
+
+__global__ __launch_bounds__(256) void w8a8_quantize_kernel(const void *__restrict__ A, int a_dtype, int K, int lda,
         int8_t *__restrict__ qa, int ldq, float *__restrict__ scale, float *__restrict__ zero, float *__restrict__ sum) {
-    const int row = blockIdx.x, lane = threadIdx.x;
+    __shared__ float s_mx[4], s_mn[4];
+    __shared__ int s_sum[4];
+    const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const size_t base = (size_t)row * lda;
+    const int esz = a_dtype == XFTHIP_F32 ? 4 : 2;
+    const bool wide = (((size_t)A | ((size_t)lda * esz)) & 15) == 0;
+    const bool qwide = (((size_t)qa | (size_t)ldq) & 7) == 0;
+    const int nchunk = K >> 3;
     float mx = -INFINITY, mn = INFINITY;
-    for (int k = lane; k < K; k += 64) {
+    for (int c = tid; c < nchunk; c += 256) {
+        float v[8];
+        w8a8_load8(A, a_dtype, base + 8 * (size_t)c, wide, v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) mx = fmaxf(mx, v[e]), mn = fminf(mn, v[e]);
+    }
+    for (int k = 8 * nchunk + tid; k < K; k += 256) {
         const float x = load_as_f32(A, a_dtype, base + k);
-        mx = fmaxf(mx, x);
-        mn = fminf(mn, x);
+        mx = fmaxf(mx, x), mn = fminf(mn, x);
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         mx = fmaxf(mx, __shfl_xor(mx, off, 64));
         mn = fminf(mn, __shfl_xor(mn, off, 64));
     }
+    if (lane == 0) s_mx[wave] = mx, s_mn[wave] = mn;
+    __syncthreads();
+    mx = fmaxf(fmaxf(s_mx[0], s_mx[1]), fmaxf(s_mx[2], s_mx[3]));
+    mn = fminf(fminf(s_mn[0], s_mn[1]), fminf(s_mn[2], s_mn[3]));
     const float fzero = (mn + mx) / 2.0f;
     const float fscale = fmaxf(fabsf(mx - fzero), fabsf(fzero - mn)) / 127.0f;
     const float vs = 1.0f / fscale, vz = -fzero / fscale;
     int isum = 0;
-    for (int k = lane; k < K; k += 64) {
-        const float x = load_as_f32(A, a_dtype, base + k);
-        const int q = __float2int_rn(fmaf(x, vs, vz));
+    int8_t *qrow = qa + (size_t)row * ldq;
+    for (int c = tid; c < nchunk; c += 256) {
+        float v[8];
+        w8a8_load8(A, a_dtype, base + 8 * (size_t)c, wide, v);
+        uint32_t w0 = 0, w1 = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int q = __float2int_rn(fmaf(v[e], vs, vz));
+            isum += q;
+            const uint32_t b = (uint32_t)(uint8_t)(int8_t)q;
+            if (e < 4)
+                w0 |= b << (8 * e);
+            else
+                w1 |= b << (8 * (e - 4));
+        }
+        if (qwide) {
+            *(uint2 *)(qrow + 8 * (size_t)c) = make_uint2(w0, w1);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qrow[8 * (size_t)c + e] = (int8_t)((e < 4 ? w0 >> (8 * e) : w1 >> (8 * (e - 4))) & 0xFFu);
+        }
+    }
+    for (int k = 8 * nchunk + tid; k < K; k += 256) {
+        const int q = __float2int_rn(fmaf(load_as_f32(A, a_dtype, base + k), vs, vz));
         isum += q;
-        qa[(size_t)row * ldq + k] = (int8_t)q;
+        qrow[k] = (int8_t)q;
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) isum += __shfl_xor(isum, off, 64);
-    if (lane == 0) {
+    if (lane == 0) s_sum[wave] = isum;
+    __syncthreads();
+    if (tid == 0) {
+        isum = (s_sum[0] + s_sum[1]) + (s_sum[2] + s_sum[3]);
         scale[row] = fscale;
         zero[row] = fzero;
         const float qs = (float)isum * fscale, kz = (float)K * fzero;
@@ -225,22 +285,46 @@ static int launch_w8a8(const W8A8Params &p, hipStream_t stream) {
 // same expression, evaluated in the same order, as in the M <= 32 kernel: bit-identical results.
 typedef int i32x16 __attribute__((ext_vector_type(16)));
 
+// the epilogue of one output value; x is the dequantised sum
+__device__ inline float w8a8_epilogue(int epi, float x, float bias, bool has_bias, float r, float gamma) {
+    switch (epi) {
+        case XFTHIP_EPI_BIAS: return x + bias;
+        case XFTHIP_EPI_SILU: return x / (1.0f + fast_exp(-x));
+        case XFTHIP_EPI_GELU: {
+            const float e = fast_exp(1.702f * x);
+            return e / (e + 1.0f) * x;
+        }
+        case XFTHIP_EPI_RESMUL: return x * r;
+        case XFTHIP_EPI_RESIDENTIAL: return (has_bias ? x + bias : x) + r;
+        case XFTHIP_EPI_RESEXT: return fmaf(gamma, r, has_bias ? x + bias : x);
+        default: return x;
+    }
+}
+
 template <int WN, int WM>
 __global__ __launch_bounds__(256) void w8a8_mfma_kernel(W8A8Params p, int nblocks_n, int nblocks_m) {
     constexpr int ROWS = 32 * WM, ROWB = 64 + 16; // padded LDS row pitch in bytes
     constexpr int CHUNKS = ROWS * 4; // 16-byte chunks of an activation tile
-    constexpr int ALOADS = (CHUNKS + 255) / 256;
+    constexpr int ALOADS = CHUNKS / 256;
+    static_assert(CHUNKS % 256 == 0, "an activation tile must split evenly over the workgroup");
+    constexpr int OPITCH = 32 * WN * 4 + 32; // row pitch in bytes of a wave's result patch
+    constexpr int STAT_OFF = 3 * ROWS * ROWB > 4 * 32 * OPITCH ? 3 * ROWS * ROWB : 4 * 32 * OPITCH;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_a[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = lane >> 5, nl = lane & 31;
-    // block -> (column block, row block): blocks that share a column block sit on the same XCD
+    // block -> (column block, row block): blocks that share a column block sit on the same XCD; row
+    // blocks are walked in bands of 8, all column blocks of a band before the next band
     int nb, mb;
     {
+        constexpr int BAND = 8;
         const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
         const int nb8 = (nblocks_n + 7) >> 3;
-        nb = (slot / nblocks_m) + xcd * nb8;
-        mb = slot % nblocks_m;
-        if (slot / nblocks_m >= nb8 || nb >= nblocks_n) return;
+        if (slot >= nb8 * nblocks_m) return;
+        const int band = slot / (nb8 * BAND), rem = slot - band * (nb8 * BAND);
+        const int left = nblocks_m - band * BAND, rows_in_band = left < BAND ? left : BAND;
+        nb = rem / rows_in_band + xcd * nb8;
+        mb = band * BAND + rem % rows_in_band;
+        if (nb >= nblocks_n) return;
     }
     const int n32_0 = (nb * 4 + wave) * WN;
     const int m0 = mb * ROWS;
@@ -269,116 +353,198 @@ __global__ __launch_bounds__(256) void w8a8_mfma_kernel(W8A8Params p, int nblock
         a_src[i] = p.qa + (size_t)row * p.ldq + a_kc * 16;
     }
     const i32x4 zero4 = {0, 0, 0, 0};
-    i32x4 wreg[2][2][WN], areg[ALOADS];
-    auto load_w = [&](int buf, int kt) {
+    // Six k tiles in flight in registers, three activation tiles in LDS.  At step T the registers of slot
+    // T % 6 hold weight tile T, LDS buffers T % 3 and (T + 1) % 3 hold activation tiles T and T + 1 (published by
+    // the barriers that ended steps T - 2 and T - 1), and the first operand half of tile T is already in
+    // registers.  The step reads the second half, multiplies the first, reads the first half of tile T + 1,
+    // multiplies the second, moves activation tile T + 2 from its registers into buffer (T + 2) % 3 (last read in
+    // step T - 1), and sends the loads of tile T + 6 into the slot it has just used: no MFMA waits for an LDS
+    // read issued in front of it and every global load is four to six steps old when it is needed.  The tile
+    // count is rounded up to whole rounds of six steps; tiles past the last one are all zero on the activation
+    // side (their weight loads re-read the last tile).
+    constexpr int SLOTS = 6, TILEB = ROWS * ROWB;
+    i32x4 wreg[SLOTS][2][WN], areg[SLOTS][ALOADS];
+    bool aval[SLOTS];
+    const int kt_n = (p.K + 63) / 64;
+    auto load_w = [&](int slot, int kt_raw) {
+        const int kt = kt_raw < kt_n ? kt_raw : kt_n - 1;
 #pragma unroll
         for (int s = 0; s < 2; ++s)
 #pragma unroll
-            for (int t = 0; t < WN; ++t) wreg[buf][s][t] = *(const i32x4 *)(wbase[t] + (size_t)kt * 1024 + s * 512);
+            for (int t = 0; t < WN; ++t) wreg[slot][s][t] = *(const i32x4 *)(wbase[t] + (size_t)kt * 1024 + s * 512);
     };
-    auto load_a = [&](int kt) {
-        // chunk inside the row iff kt * 64 + 16 a_kc + 16 <= K (K % 16 == 0); otherwise the row start is read and dropped
+    auto load_a = [&](int slot, int kt) {
+        // chunk inside the row iff kt * 64 + 16 a_kc + 16 <= K (K % 16 == 0); otherwise the row start is read and
+        // replaced by zeros on its way to LDS (there, not here: the loaded value is not touched before its step)
         const bool v = kt * 64 + a_kc * 16 + 16 <= p.K;
+        aval[slot] = v;
 #pragma unroll
-        for (int i = 0; i < ALOADS; ++i) {
-            const i32x4 a = *(const i32x4 *)(a_src[i] + (v ? kt * 64 : -a_kc * 16));
-            areg[i] = v ? a : zero4;
-        }
+        for (int i = 0; i < ALOADS; ++i) areg[slot][i] = *(const i32x4 *)(a_src[i] + (v ? kt * 64 : -a_kc * 16));
     };
-    auto store_a = [&](int buf) {
-        unsigned char *dst = lds_a + buf * (ROWS * ROWB);
+    auto store_a = [&](int slot, int buf) {
+        unsigned char *dst = lds_a + buf * TILEB;
 #pragma unroll
-        for (int i = 0; i < ALOADS; ++i)
-            if (a_row0 + 64 * i < ROWS) *(i32x4 *)(dst + (a_row0 + 64 * i) * ROWB + a_kc * 16) = areg[i];
+        for (int i = 0; i < ALOADS; ++i) *(i32x4 *)(dst + (a_row0 + 64 * i) * ROWB + a_kc * 16) = aval[slot] ? areg[slot][i] : zero4;
     };
-    auto compute = [&](int wb, int ab) {
-        const unsigned char *src = lds_a + ab * (ROWS * ROWB) + nl * ROWB + 16 * h;
+    const unsigned char *opnd = lds_a + nl * ROWB + 16 * h;
+    i32x4 a0[WM], a1[WM];
+    auto read_half = [&](i32x4 (&a)[WM], int buf, int s) {
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            i32x4 a[WM];
-#pragma unroll
-            for (int m = 0; m < WM; ++m) a[m] = *(const i32x4 *)(src + m * 32 * ROWB + 32 * s);
-#pragma unroll
-            for (int t = 0; t < WN; ++t)
-#pragma unroll
-                for (int m = 0; m < WM; ++m) acc[t][m] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[m], wreg[wb][s][t], acc[t][m], 0, 0, 0);
-        }
+        for (int m = 0; m < WM; ++m) a[m] = *(const i32x4 *)(opnd + buf * TILEB + m * 32 * ROWB + 32 * s);
     };
-#define XFT_FENCE() __builtin_amdgcn_sched_barrier(0)
-    const int kt_n = (p.K + 63) / 64;
-    load_w(0, 0);
-    load_a(0);
-    store_a(0);
+    auto mul_half = [&](const i32x4 (&a)[WM], int slot, int s) {
+#pragma unroll
+        for (int t = 0; t < WN; ++t)
+#pragma unroll
+            for (int m = 0; m < WM; ++m) acc[t][m] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[m], wreg[slot][s][t], acc[t][m], 0, 0, 0);
+    };
+    // per-row statistics of this row block, kept behind the tiles / result patches for the epilogue
+    float *rowstat = (float *)(lds_a + STAT_OFF);
+    if (threadIdx.x < ROWS) {
+        int row = m0 + threadIdx.x;
+        row = row < p.M ? row : p.M - 1;
+        rowstat[threadIdx.x] = p.sA[row];
+        rowstat[ROWS + threadIdx.x] = p.zA[row];
+        rowstat[2 * ROWS + threadIdx.x] = p.sumA[row];
+    }
+#pragma unroll
+    for (int d = 0; d < SLOTS; ++d) {
+        load_w(d, d);
+        load_a(d, d);
+    }
+    store_a(0, 0);
+    store_a(1, 1);
     __syncthreads();
-    int kt = 0;
-    for (; kt + 2 <= kt_n - 1; kt += 2) {
-        load_w(1, kt + 1);
-        load_a(kt + 1);
-        XFT_FENCE();
-        compute(0, 0);
-        XFT_FENCE();
-        store_a(1);
-        __syncthreads();
-        load_w(0, kt + 2);
-        load_a(kt + 2);
-        XFT_FENCE();
-        compute(1, 1);
-        XFT_FENCE();
-        store_a(0);
-        __syncthreads();
+    read_half(a0, 0, 0);
+#define XFT_FENCE() __builtin_amdgcn_sched_barrier(0)
+#define XFT_W8_STEP(S)                                  \
+    {                                                   \
+        read_half(a1, (S) % 3, 1);                      \
+        XFT_FENCE();                                    \
+        mul_half(a0, (S), 0);                           \
+        XFT_FENCE();                                    \
+        read_half(a0, ((S) + 1) % 3, 0);                \
+        XFT_FENCE();                                    \
+        mul_half(a1, (S), 1);                           \
+        XFT_FENCE();                                    \
+        store_a(((S) + 2) % SLOTS, ((S) + 2) % 3);      \
+        load_w((S), kt + (S) + SLOTS);                  \
+        load_a((S), kt + (S) + SLOTS);                  \
+        __syncthreads();                                \
+        XFT_FENCE();                                    \
     }
-    if (kt + 1 < kt_n) {
-        load_w(1, kt + 1);
-        load_a(kt + 1);
-        XFT_FENCE();
-        compute(0, 0);
-        XFT_FENCE();
-        store_a(1);
-        __syncthreads();
-        compute(1, 1);
-    } else {
-        compute(0, 0);
+    for (int kt = 0; kt < kt_n; kt += SLOTS) {
+        XFT_W8_STEP(0)
+        XFT_W8_STEP(1)
+        XFT_W8_STEP(2)
+        XFT_W8_STEP(3)
+        XFT_W8_STEP(4)
+        XFT_W8_STEP(5)
     }
+#undef XFT_W8_STEP
 #undef XFT_FENCE
 
     // ---- epilogue: lane holds C[m0 + 32 m + 8 (j / 4) + 4 h + j % 4][32 (n32_0 + t) + nl] ----------
+    // Each wave drops one 32-row block of its int32 sums at a time into an LDS patch of its own (constant
+    // offsets, so the accumulators stay in registers), then walks the patch in 8-column chunks, consecutive
+    // lanes along a row: dequantisation, the epilogue of the call and 16-byte stores run in that short loop.
+    __syncthreads(); // every wave is past its last read of the activation tiles
+    unsigned char *obuf = lds_a + wave * (32 * OPITCH);
+    const int epi = p.epi;
+    const bool with_res = epi == XFTHIP_EPI_RESMUL || epi == XFTHIP_EPI_RESIDENTIAL || epi == XFTHIP_EPI_RESEXT;
+    const bool c_wide = (((size_t)p.C | ((size_t)p.ldc * (p.c_dtype == XFTHIP_F32 ? 4 : 2))) & 15) == 0;
+    const bool res_wide = with_res && (((size_t)p.res | ((size_t)p.ldres * (p.res_dtype == XFTHIP_F32 ? 4 : 2))) & 15) == 0;
+    int *put_base = (int *)(obuf + 4 * h * OPITCH) + nl;
+    constexpr int CPR = 4 * WN; // 8-column chunks a row
+    constexpr int ITERS = 32 * CPR / 64, RSTEP = 64 / CPR;
+    // a lane keeps the same 8 columns in every pass over the patch: their constants are fetched once
+    const int ch = lane % CPR, r0 = lane / CPR;
+    const int c = n32_0 * 32 + 8 * ch;
+    const bool full = c + 8 <= p.N;
+    float sB[8], zB[8], sumBsB[8], bias[8];
 #pragma unroll
-    for (int t = 0; t < WN; ++t) {
-        const int np = (n32_0 + t) * 32 + nl;
-        if (np >= p.N) continue;
-        const float sB = p.scaleB[np], zB = p.zeroB ? p.zeroB[np] : 0.0f, sumB = p.sumB[np];
-        const float bias = p.bias ? p.bias[np] : 0.0f;
+    for (int e = 0; e < 8; ++e) {
+        const int np = c + e < p.N ? c + e : (c < p.N ? c : 0);
+        sB[e] = p.scaleB[np];
+        zB[e] = p.zeroB ? p.zeroB[np] : 0.0f;
+        sumBsB[e] = p.sumB[np] * sB[e];
+        bias[e] = p.bias ? p.bias[np] : 0.0f;
+    }
+    const bool has_bias = p.bias != nullptr;
 #pragma unroll
-        for (int m = 0; m < WM; ++m) {
+    for (int m = 0; m < WM; ++m) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                const int row = m0 + 32 * m + 8 * (j >> 2) + 4 * h + (j & 3);
-                if (row >= p.M) continue;
-                // C = s32*sA*sB + sumB*sB*zA + sumA*zB, evaluated left to right without contraction
-                const float t0 = ((float)acc[t][m][j] * p.sA[row]) * sB;
-                const float t1 = (sumB * sB) * p.zA[row];
-                const float t2 = p.sumA[row] * zB;
-                float x = (t0 + t1) + t2;
-                switch (p.epi) {
-                    case XFTHIP_EPI_BIAS: x += bias; break;
-                    case XFTHIP_EPI_SILU: x = x / (1.0f + fast_exp(-x)); break;
-                    case XFTHIP_EPI_GELU: {
-                        float e = fast_exp(1.702f * x);
-                        x = e / (e + 1.0f) * x;
-                        break;
+        for (int t = 0; t < WN; ++t)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) put_base[(8 * (j >> 2) + (j & 3)) * (OPITCH / 4) + 32 * t] = acc[t][m][j];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll 1
+        for (int it = 0; it < ITERS; ++it) {
+            const int r = r0 + RSTEP * it;
+            const int row = m0 + 32 * m + r;
+            if (row >= p.M || c >= p.N) continue;
+            const int *src = (const int *)(obuf + r * OPITCH) + 8 * ch;
+            const i32x4 lo = *(const i32x4 *)src, hi = *(const i32x4 *)(src + 4);
+            const int s32[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            const float sA = rowstat[32 * m + r], zA = rowstat[ROWS + 32 * m + r], sumA = rowstat[2 * ROWS + 32 * m + r];
+            float res[8];
+            if (with_res) {
+                const size_t ri = (size_t)row * p.ldres + c;
+                if (full && res_wide) {
+                    if (p.res_dtype == XFTHIP_F32) {
+                        const f32x4 a = *(const f32x4 *)((const float *)p.res + ri), b = *(const f32x4 *)((const float *)p.res + ri + 4);
+                        res[0] = a[0], res[1] = a[1], res[2] = a[2], res[3] = a[3], res[4] = b[0], res[5] = b[1], res[6] = b[2], res[7] = b[3];
+                    } else {
+                        const i32x4 a = *(const i32x4 *)((const uint16_t *)p.res + ri);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint16_t b0 = (uint16_t)((uint32_t)a[e] & 0xFFFFu), b1 = (uint16_t)((uint32_t)a[e] >> 16);
+                            res[2 * e] = p.res_dtype == XFTHIP_BF16 ? bf16_to_f32(b0) : fp16_bits_to_f32(b0);
+                            res[2 * e + 1] = p.res_dtype == XFTHIP_BF16 ? bf16_to_f32(b1) : fp16_bits_to_f32(b1);
+                        }
                     }
-                    case XFTHIP_EPI_RESMUL: x *= load_as_f32(p.res, p.res_dtype, (size_t)row * p.ldres + np); break;
-                    case XFTHIP_EPI_RESIDENTIAL:
-                        if (p.bias) x += bias;
-                        x += load_as_f32(p.res, p.res_dtype, (size_t)row * p.ldres + np);
-                        break;
-                    case XFTHIP_EPI_RESEXT:
-                        if (p.bias) x += bias;
-                        x = fmaf(p.gamma, load_as_f32(p.res, p.res_dtype, (size_t)row * p.ldres + np), x);
-                        break;
-                    default: break;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) res[e] = c + e < p.N ? load_as_f32(p.res, p.res_dtype, ri + e) : 0.0f;
                 }
-                store_from_f32(p.C, p.c_dtype, (size_t)row * p.ldc + np, x);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) res[e] = 0.0f;
+            }
+            float v[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                // C = s32*sA*sB + sumB*sB*zA + sumA*zB, evaluated left to right without contraction
+                const float t0 = ((float)s32[e] * sA) * sB[e];
+                const float t1 = sumBsB[e] * zA;
+                const float t2 = sumA * zB[e];
+                v[e] = w8a8_epilogue(epi, (t0 + t1) + t2, bias[e], has_bias, res[e], p.gamma);
+            }
+            const size_t ci = (size_t)row * p.ldc + c;
+            if (full && c_wide) {
+                if (p.c_dtype == XFTHIP_F32) {
+                    const f32x4 o0 = {v[0], v[1], v[2], v[3]}, o1 = {v[4], v[5], v[6], v[7]};
+                    *(f32x4 *)((float *)p.C + ci) = o0;
+                    *(f32x4 *)((float *)p.C + ci + 4) = o1;
+                } else {
+                    i32x4 o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t b0 = p.c_dtype == XFTHIP_BF16 ? f32_to_bf16_ref(v[2 * e]) : f32_to_fp16_bits(v[2 * e]);
+                        const uint32_t b1 = p.c_dtype == XFTHIP_BF16 ? f32_to_bf16_ref(v[2 * e + 1]) : f32_to_fp16_bits(v[2 * e + 1]);
+                        o[e] = (int)(b0 | (b1 << 16));
+                    }
+                    *(i32x4 *)((uint16_t *)p.C + ci) = o;
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (c + e < p.N) store_from_f32(p.C, p.c_dtype, ci + e, v[e]);
             }
         }
     }
@@ -390,7 +556,9 @@ static int launch_w8a8_mfma(const W8A8Params &p, hipStream_t stream) {
     const int nblocks_n = (n32 + 4 * WN - 1) / (4 * WN);
     const int nblocks_m = (p.M + 32 * WM - 1) / (32 * WM);
     const int blocks = ((nblocks_n + 7) / 8) * 8 * nblocks_m;
-    const size_t smem = 2 * (size_t)(32 * WM) * (64 + 16);
+    const size_t tiles = 3 * (size_t)(32 * WM) * (64 + 16), patches = 4 * 32 * (size_t)(32 * WN * 4 + 32);
+    // the result patches reuse the activation tiles; the per-row statistics sit behind both
+    const size_t smem = (tiles > patches ? tiles : patches) + 3 * (size_t)(32 * WM) * sizeof(float);
     hipLaunchKernelGGL((w8a8_mfma_kernel<WN, WM>), dim3(blocks), dim3(256), smem, stream, p, nblocks_n, nblocks_m);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
@@ -412,7 +580,7 @@ int xfthip_w8a8_quantize_rows(const void *A, int a_dtype, int M, int K, int lda,
     XFT_REQUIRE(A && qa && scale && zero && sum, "xfthip_w8a8_quantize_rows: null argument");
     XFT_REQUIRE(M > 0 && K > 0 && lda >= K && ldq >= K, "xfthip_w8a8_quantize_rows: bad shape");
     XFT_REQUIRE(a_dtype == XFTHIP_F32 || a_dtype == XFTHIP_BF16, "xfthip_w8a8_quantize_rows: dtype must be f32 or bf16");
-    hipLaunchKernelGGL(w8a8_quantize_kernel, dim3(M), dim3(64), 0, (hipStream_t)stream, A, a_dtype, K, lda, qa, ldq, scale, zero, sum);
+    hipLaunchKernelGGL(w8a8_quantize_kernel, dim3(M), dim3(256), 0, (hipStream_t)stream, A, a_dtype, K, lda, qa, ldq, scale, zero, sum);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }

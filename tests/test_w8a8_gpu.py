@@ -117,3 +117,37 @@ def test_w8a8_model_shape_rows_2048(xh, orc):
     rows = np.array([0, 1, 31, 32, 127, 128, 1000, 2046, 2047])
     exp = orc.qgemm(w, A[rows])
     assert np.array_equal(got[rows].view(np.uint32), exp.view(np.uint32))
+
+
+def test_w8a8_256_row_blocks_bit_exact(xh, orc):
+    """Enough 256 x 256 blocks to fill the chip twice: eight waves a workgroup, two stacked over the rows.  Ragged M
+    and N, sampled rows against the oracle (rows are independent), plain and residual epilogues, bf16 output."""
+    M, K, N = 3000, 512, 11024
+    rng = np.random.default_rng(77)
+    w = orc.quantize(orc.W_W8A8, (rng.standard_normal((K, N)) * 0.02).astype(np.float32))
+    w.zero = (rng.standard_normal(N) * 0.002).astype(np.float32)
+    A = orc.round_bf16(rng.standard_normal((M, K)) + 0.1)
+    dw = xh.Weight(xh.W_W8A8, K, N, w.q, w.scale, w.zero)
+    ad = xh.DeviceBuffer.from_numpy(orc.to_bf16(A))
+    cd = xh.DeviceBuffer(M * N * 4)
+    xh.gemm(dw, ad.ptr, M, K, cd.ptr, N, xh.F32)
+    xh.synchronize()
+    got = cd.to_numpy(np.float32, (M, N))
+    assert np.isfinite(got).all()
+    rows = np.array([0, 1, 31, 32, 127, 128, 129, 255, 256, 257, 383, 384, 511, 512, 1000, 1279, 1280, 2047, 2048, 2815, 2816, 2998, 2999])
+    exp = orc.qgemm(w, A[rows])
+    assert np.array_equal(got[rows].view(np.uint32), exp.view(np.uint32)), np.abs(got[rows] - exp).max()
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    qa, s, z, sm, ldq = xh.w8a8_quantize_rows(ad.ptr, xh.BF16, M, K, K)
+    rd, bd = xh.DeviceBuffer.from_numpy(res), xh.DeviceBuffer.from_numpy(bias)
+    xh.gemm_w8a8(dw, M, qa, ldq, s, z, sm, cd.ptr, N, xh.F32, xh.EPI_RESIDENTIAL, bd.ptr, rd.ptr, N)
+    xh.synchronize()
+    e2 = orc.qgemm(w, A[rows], orc.EPI_RESIDENTIAL, bias=bias, res=res[rows])
+    assert np.abs(cd.to_numpy(np.float32, (M, N))[rows] - e2).max() < 2e-4
+    c16 = xh.DeviceBuffer(M * N * 2)
+    xh.gemm(dw, ad.ptr, M, K, c16.ptr, N, xh.BF16)
+    xh.synchronize()
+    got16 = c16.to_numpy(np.uint16, (M, N))
+    assert np.array_equal(got16[rows], orc.to_bf16(exp))
+    dw.free()

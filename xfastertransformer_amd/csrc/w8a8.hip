@@ -301,14 +301,16 @@ __device__ inline float w8a8_epilogue(int epi, float x, float bias, bool has_bia
     }
 }
 
-template <int WN, int WM>
-__global__ __launch_bounds__(256) void w8a8_mfma_kernel(W8A8Params p, int nblocks_n, int nblocks_m) {
-    constexpr int ROWS = 32 * WM, ROWB = 64 + 16; // padded LDS row pitch in bytes
-    constexpr int CHUNKS = ROWS * 4; // 16-byte chunks of an activation tile
-    constexpr int ALOADS = CHUNKS / 256;
-    static_assert(CHUNKS % 256 == 0, "an activation tile must split evenly over the workgroup");
+// A workgroup is 4 x WR waves: four side by side over 4 * WN * 32 columns, WR on top of each other over
+// WR * WM * 32 rows; a wave owns WN x WM accumulator tiles of 32 x 32.
+template <int WN, int WM, int WR>
+__global__ __launch_bounds__(256 * WR) void w8a8_mfma_kernel(W8A8Params p, int nblocks_n, int nblocks_m) {
+    constexpr int ROWS = 32 * WM, BROWS = ROWS * WR, ROWB = 64 + 16; // rows of a wave / of the block, padded LDS row pitch in bytes
+    constexpr int CHUNKS = BROWS * 4; // 16-byte chunks of an activation tile
+    constexpr int ALOADS = CHUNKS / (256 * WR);
+    static_assert(CHUNKS % (256 * WR) == 0, "an activation tile must split evenly over the workgroup");
     constexpr int OPITCH = 32 * WN * 4 + 32; // row pitch in bytes of a wave's result patch
-    constexpr int STAT_OFF = 3 * ROWS * ROWB > 4 * 32 * OPITCH ? 3 * ROWS * ROWB : 4 * 32 * OPITCH;
+    constexpr int STAT_OFF = 3 * BROWS * ROWB > 4 * WR * 32 * OPITCH ? 3 * BROWS * ROWB : 4 * WR * 32 * OPITCH;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_a[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = lane >> 5, nl = lane & 31;
@@ -326,8 +328,9 @@ __global__ __launch_bounds__(256) void w8a8_mfma_kernel(W8A8Params p, int nblock
         mb = band * BAND + rem % rows_in_band;
         if (nb >= nblocks_n) return;
     }
-    const int n32_0 = (nb * 4 + wave) * WN;
-    const int m0 = mb * ROWS;
+    const int wave_c = wave & 3, wave_r = wave >> 2;
+    const int n32_0 = (nb * 4 + wave_c) * WN;
+    const int m0 = mb * BROWS, mw = wave_r * ROWS; // first row of the block, of this wave inside the block
 
     i32x16 acc[WN][WM];
 #pragma unroll
@@ -348,7 +351,7 @@ __global__ __launch_bounds__(256) void w8a8_mfma_kernel(W8A8Params p, int nblock
     const int8_t *a_src[ALOADS];
 #pragma unroll
     for (int i = 0; i < ALOADS; ++i) {
-        int row = m0 + a_row0 + 64 * i;
+        int row = m0 + a_row0 + 64 * WR * i;
         row = row < p.M ? row : p.M - 1;
         a_src[i] = p.qa + (size_t)row * p.ldq + a_kc * 16;
     }
@@ -362,7 +365,7 @@ __global__ __launch_bounds__(256) void w8a8_mfma_kernel(W8A8Params p, int nblock
     // read issued in front of it and every global load is four to six steps old when it is needed.  The tile
     // count is rounded up to whole rounds of six steps; tiles past the last one are all zero on the activation
     // side (their weight loads re-read the last tile).
-    constexpr int SLOTS = 6, TILEB = ROWS * ROWB;
+    constexpr int SLOTS = WR == 1 ? 6 : 3, TILEB = BROWS * ROWB; // two waves a SIMD share its registers: fewer tiles in flight
     i32x4 wreg[SLOTS][2][WN], areg[SLOTS][ALOADS];
     bool aval[SLOTS];
     const int kt_n = (p.K + 63) / 64;
@@ -384,9 +387,9 @@ __global__ __launch_bounds__(256) void w8a8_mfma_kernel(W8A8Params p, int nblock
     auto store_a = [&](int slot, int buf) {
         unsigned char *dst = lds_a + buf * TILEB;
 #pragma unroll
-        for (int i = 0; i < ALOADS; ++i) *(i32x4 *)(dst + (a_row0 + 64 * i) * ROWB + a_kc * 16) = aval[slot] ? areg[slot][i] : zero4;
+        for (int i = 0; i < ALOADS; ++i) *(i32x4 *)(dst + (a_row0 + 64 * WR * i) * ROWB + a_kc * 16) = aval[slot] ? areg[slot][i] : zero4;
     };
-    const unsigned char *opnd = lds_a + nl * ROWB + 16 * h;
+    const unsigned char *opnd = lds_a + (mw + nl) * ROWB + 16 * h;
     i32x4 a0[WM], a1[WM];
     auto read_half = [&](i32x4 (&a)[WM], int buf, int s) {
 #pragma unroll
@@ -400,12 +403,12 @@ __global__ __launch_bounds__(256) void w8a8_mfma_kernel(W8A8Params p, int nblock
     };
     // per-row statistics of this row block, kept behind the tiles / result patches for the epilogue
     float *rowstat = (float *)(lds_a + STAT_OFF);
-    if (threadIdx.x < ROWS) {
+    if (threadIdx.x < BROWS) {
         int row = m0 + threadIdx.x;
         row = row < p.M ? row : p.M - 1;
         rowstat[threadIdx.x] = p.sA[row];
-        rowstat[ROWS + threadIdx.x] = p.zA[row];
-        rowstat[2 * ROWS + threadIdx.x] = p.sumA[row];
+        rowstat[BROWS + threadIdx.x] = p.zA[row];
+        rowstat[2 * BROWS + threadIdx.x] = p.sumA[row];
     }
 #pragma unroll
     for (int d = 0; d < SLOTS; ++d) {
@@ -437,9 +440,11 @@ __global__ __launch_bounds__(256) void w8a8_mfma_kernel(W8A8Params p, int nblock
         XFT_W8_STEP(0)
         XFT_W8_STEP(1)
         XFT_W8_STEP(2)
-        XFT_W8_STEP(3)
-        XFT_W8_STEP(4)
-        XFT_W8_STEP(5)
+        if constexpr (SLOTS == 6) {
+            XFT_W8_STEP(3)
+            XFT_W8_STEP(4)
+            XFT_W8_STEP(5)
+        }
     }
 #undef XFT_W8_STEP
 #undef XFT_FENCE
@@ -486,12 +491,12 @@ __global__ __launch_bounds__(256) void w8a8_mfma_kernel(W8A8Params p, int nblock
 #pragma unroll 1
         for (int it = 0; it < ITERS; ++it) {
             const int r = r0 + RSTEP * it;
-            const int row = m0 + 32 * m + r;
+            const int row = m0 + mw + 32 * m + r;
             if (row >= p.M || c >= p.N) continue;
             const int *src = (const int *)(obuf + r * OPITCH) + 8 * ch;
             const i32x4 lo = *(const i32x4 *)src, hi = *(const i32x4 *)(src + 4);
             const int s32[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            const float sA = rowstat[32 * m + r], zA = rowstat[ROWS + 32 * m + r], sumA = rowstat[2 * ROWS + 32 * m + r];
+            const float sA = rowstat[mw + 32 * m + r], zA = rowstat[BROWS + mw + 32 * m + r], sumA = rowstat[2 * BROWS + mw + 32 * m + r];
             float res[8];
             if (with_res) {
                 const size_t ri = (size_t)row * p.ldres + c;
@@ -550,16 +555,22 @@ __global__ __launch_bounds__(256) void w8a8_mfma_kernel(W8A8Params p, int nblock
     }
 }
 
-template <int WN, int WM>
+template <int WN, int WM, int WR>
 static int launch_w8a8_mfma(const W8A8Params &p, hipStream_t stream) {
     const int n32 = (p.NTILES + 1) / 2;
+    const int brows = 32 * WM * WR;
     const int nblocks_n = (n32 + 4 * WN - 1) / (4 * WN);
-    const int nblocks_m = (p.M + 32 * WM - 1) / (32 * WM);
+    const int nblocks_m = (p.M + brows - 1) / brows;
     const int blocks = ((nblocks_n + 7) / 8) * 8 * nblocks_m;
-    const size_t tiles = 3 * (size_t)(32 * WM) * (64 + 16), patches = 4 * 32 * (size_t)(32 * WN * 4 + 32);
+    const size_t tiles = 3 * (size_t)brows * (64 + 16), patches = 4 * WR * 32 * (size_t)(32 * WN * 4 + 32);
     // the result patches reuse the activation tiles; the per-row statistics sit behind both
-    const size_t smem = (tiles > patches ? tiles : patches) + 3 * (size_t)(32 * WM) * sizeof(float);
-    hipLaunchKernelGGL((w8a8_mfma_kernel<WN, WM>), dim3(blocks), dim3(256), smem, stream, p, nblocks_n, nblocks_m);
+    const size_t smem = (tiles > patches ? tiles : patches) + 3 * (size_t)brows * sizeof(float);
+    if (smem > 64 * 1024) {
+        static const hipError_t attr = hipFuncSetAttribute((const void *)w8a8_mfma_kernel<WN, WM, WR>,
+                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        XFT_CHECK_HIP(attr);
+    }
+    hipLaunchKernelGGL((w8a8_mfma_kernel<WN, WM, WR>), dim3(blocks), dim3(256 * WR), smem, stream, p, nblocks_n, nblocks_m);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }
@@ -611,8 +622,10 @@ int xfthip_gemm_w8a8(xfthip_weight_t w, int M, const int8_t *qa, int ldq, const 
         p.res = res, p.ldres = ldres, p.res_dtype = res_dtype, p.gamma = gamma;
         const int n32 = (pw.NTILES + 1) / 2;
         const long t_large = (long)((n32 + 7) / 8) * ((M + 127) / 128);
-        if (t_large >= cus) return launch_w8a8_mfma<2, 4>(p, (hipStream_t)stream);
-        return launch_w8a8_mfma<1, 2>(p, (hipStream_t)stream);
+        const long t_huge = (long)((n32 + 7) / 8) * ((M + 255) / 256);
+        if (t_huge >= 2 * cus) return launch_w8a8_mfma<2, 4, 2>(p, (hipStream_t)stream);
+        if (t_large >= cus) return launch_w8a8_mfma<2, 4, 1>(p, (hipStream_t)stream);
+        return launch_w8a8_mfma<1, 2, 1>(p, (hipStream_t)stream);
     }
     for (int m0 = 0; m0 < M; m0 += 32) {
         W8A8Params p = {};

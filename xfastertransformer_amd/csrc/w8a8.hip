@@ -12,6 +12,7 @@
 // into fused multiply-adds anywhere in this file (plain operators, not the __fmul_rn family,
 // whose bodies live in a header compiled with the default contraction); the one fused operation
 // of the reference (the activation quantiser) is an explicit fmaf.
+#include <type_traits>
 #pragma clang fp contract(off)
 
 namespace xfthip {
@@ -455,10 +456,8 @@ __global__ __launch_bounds__(256 * WR) void w8a8_mfma_kernel(W8A8Params p, int n
     // lanes along a row: dequantisation, the epilogue of the call and 16-byte stores run in that short loop.
     __syncthreads(); // every wave is past its last read of the activation tiles
     unsigned char *obuf = lds_a + wave * (32 * OPITCH);
-    const int epi = p.epi;
-    const bool with_res = epi == XFTHIP_EPI_RESMUL || epi == XFTHIP_EPI_RESIDENTIAL || epi == XFTHIP_EPI_RESEXT;
     const bool c_wide = (((size_t)p.C | ((size_t)p.ldc * (p.c_dtype == XFTHIP_F32 ? 4 : 2))) & 15) == 0;
-    const bool res_wide = with_res && (((size_t)p.res | ((size_t)p.ldres * (p.res_dtype == XFTHIP_F32 ? 4 : 2))) & 15) == 0;
+    const bool res_wide = p.res && (((size_t)p.res | ((size_t)p.ldres * (p.res_dtype == XFTHIP_F32 ? 4 : 2))) & 15) == 0;
     int *put_base = (int *)(obuf + 4 * h * OPITCH) + nl;
     constexpr int CPR = 4 * WN; // 8-column chunks a row
     constexpr int ITERS = 32 * CPR / 64, RSTEP = 64 / CPR;
@@ -476,82 +475,106 @@ __global__ __launch_bounds__(256 * WR) void w8a8_mfma_kernel(W8A8Params p, int n
         bias[e] = p.bias ? p.bias[np] : 0.0f;
     }
     const bool has_bias = p.bias != nullptr;
+    // the epilogue of the call is a compile-time constant inside the loops (one copy of them per epilogue)
+    auto run = [&](auto epi_tag) {
+        constexpr int EPI = decltype(epi_tag)::value;
+        constexpr bool HAS_RES = EPI == XFTHIP_EPI_RESMUL || EPI == XFTHIP_EPI_RESIDENTIAL || EPI == XFTHIP_EPI_RESEXT;
 #pragma unroll
-    for (int m = 0; m < WM; ++m) {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        for (int m = 0; m < WM; ++m) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-        for (int t = 0; t < WN; ++t)
+            for (int t = 0; t < WN; ++t)
 #pragma unroll
-            for (int j = 0; j < 16; ++j) put_base[(8 * (j >> 2) + (j & 3)) * (OPITCH / 4) + 32 * t] = acc[t][m][j];
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                for (int j = 0; j < 16; ++j) put_base[(8 * (j >> 2) + (j & 3)) * (OPITCH / 4) + 32 * t] = acc[t][m][j];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll 1
-        for (int it = 0; it < ITERS; ++it) {
-            const int r = r0 + RSTEP * it;
-            const int row = m0 + mw + 32 * m + r;
-            if (row >= p.M || c >= p.N) continue;
-            const int *src = (const int *)(obuf + r * OPITCH) + 8 * ch;
-            const i32x4 lo = *(const i32x4 *)src, hi = *(const i32x4 *)(src + 4);
-            const int s32[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            const float sA = rowstat[mw + 32 * m + r], zA = rowstat[BROWS + mw + 32 * m + r], sumA = rowstat[2 * BROWS + mw + 32 * m + r];
-            float res[8];
-            if (with_res) {
-                const size_t ri = (size_t)row * p.ldres + c;
-                if (full && res_wide) {
-                    if (p.res_dtype == XFTHIP_F32) {
-                        const f32x4 a = *(const f32x4 *)((const float *)p.res + ri), b = *(const f32x4 *)((const float *)p.res + ri + 4);
-                        res[0] = a[0], res[1] = a[1], res[2] = a[2], res[3] = a[3], res[4] = b[0], res[5] = b[1], res[6] = b[2], res[7] = b[3];
+            for (int it = 0; it < ITERS; ++it) {
+                const int r = r0 + RSTEP * it;
+                const int row = m0 + mw + 32 * m + r;
+                if (row >= p.M || c >= p.N) continue;
+                const int *src = (const int *)(obuf + r * OPITCH) + 8 * ch;
+                const i32x4 lo = *(const i32x4 *)src, hi = *(const i32x4 *)(src + 4);
+                const int s32[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                const float sA = rowstat[mw + 32 * m + r], zA = rowstat[BROWS + mw + 32 * m + r], sumA = rowstat[2 * BROWS + mw + 32 * m + r];
+                float res[8];
+                if constexpr (HAS_RES) {
+                    const size_t ri = (size_t)row * p.ldres + c;
+                    if (full && res_wide) {
+                        if (p.res_dtype == XFTHIP_F32) {
+                            const f32x4 a = *(const f32x4 *)((const float *)p.res + ri), b = *(const f32x4 *)((const float *)p.res + ri + 4);
+                            res[0] = a[0], res[1] = a[1], res[2] = a[2], res[3] = a[3], res[4] = b[0], res[5] = b[1], res[6] = b[2], res[7] = b[3];
+                        } else {
+                            const i32x4 a = *(const i32x4 *)((const uint16_t *)p.res + ri);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const uint16_t b0 = (uint16_t)((uint32_t)a[e] & 0xFFFFu), b1 = (uint16_t)((uint32_t)a[e] >> 16);
+                                res[2 * e] = p.res_dtype == XFTHIP_BF16 ? bf16_to_f32(b0) : fp16_bits_to_f32(b0);
+                                res[2 * e + 1] = p.res_dtype == XFTHIP_BF16 ? bf16_to_f32(b1) : fp16_bits_to_f32(b1);
+                            }
+                        }
                     } else {
-                        const i32x4 a = *(const i32x4 *)((const uint16_t *)p.res + ri);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) res[e] = c + e < p.N ? load_as_f32(p.res, p.res_dtype, ri + e) : 0.0f;
+                    }
+                }
+                float v[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    // C = s32*sA*sB + sumB*sB*zA + sumA*zB, evaluated left to right without contraction
+                    const float t0 = ((float)s32[e] * sA) * sB[e];
+                    const float t1 = sumBsB[e] * zA;
+                    const float t2 = sumA * zB[e];
+                    float x = (t0 + t1) + t2;
+                    if constexpr (EPI == XFTHIP_EPI_BIAS) x = x + bias[e];
+                    if constexpr (EPI == XFTHIP_EPI_SILU) x = x / (1.0f + fast_exp(-x));
+                    if constexpr (EPI == XFTHIP_EPI_GELU) {
+                        const float ex = fast_exp(1.702f * x);
+                        x = ex / (ex + 1.0f) * x;
+                    }
+                    if constexpr (EPI == XFTHIP_EPI_RESMUL) x = x * res[e];
+                    if constexpr (EPI == XFTHIP_EPI_RESIDENTIAL) x = (has_bias ? x + bias[e] : x) + res[e];
+                    if constexpr (EPI == XFTHIP_EPI_RESEXT) x = fmaf(p.gamma, res[e], has_bias ? x + bias[e] : x);
+                    v[e] = x;
+                }
+                const size_t ci = (size_t)row * p.ldc + c;
+                if (full && c_wide) {
+                    if (p.c_dtype == XFTHIP_F32) {
+                        const f32x4 o0 = {v[0], v[1], v[2], v[3]}, o1 = {v[4], v[5], v[6], v[7]};
+                        *(f32x4 *)((float *)p.C + ci) = o0;
+                        *(f32x4 *)((float *)p.C + ci + 4) = o1;
+                    } else {
+                        i32x4 o;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            const uint16_t b0 = (uint16_t)((uint32_t)a[e] & 0xFFFFu), b1 = (uint16_t)((uint32_t)a[e] >> 16);
-                            res[2 * e] = p.res_dtype == XFTHIP_BF16 ? bf16_to_f32(b0) : fp16_bits_to_f32(b0);
-                            res[2 * e + 1] = p.res_dtype == XFTHIP_BF16 ? bf16_to_f32(b1) : fp16_bits_to_f32(b1);
+                            const uint32_t b0 = p.c_dtype == XFTHIP_BF16 ? f32_bits_to_bf16_sel(f2u(v[2 * e])) : f32_to_fp16_bits(v[2 * e]);
+                            const uint32_t b1 = p.c_dtype == XFTHIP_BF16 ? f32_bits_to_bf16_sel(f2u(v[2 * e + 1])) : f32_to_fp16_bits(v[2 * e + 1]);
+                            o[e] = (int)(b0 | (b1 << 16));
                         }
+                        *(i32x4 *)((uint16_t *)p.C + ci) = o;
                     }
                 } else {
+                    // ragged or unaligned rows: through the patch again, one value at a time
+                    float *back = (float *)(obuf + r * OPITCH) + 8 * ch;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) res[e] = c + e < p.N ? load_as_f32(p.res, p.res_dtype, ri + e) : 0.0f;
+                    for (int e = 0; e < 8; ++e) back[e] = v[e];
+#pragma unroll 1
+                    for (int e = 0; e < 8 && c + e < p.N; ++e) store_from_f32(p.C, p.c_dtype, ci + e, back[e]);
                 }
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) res[e] = 0.0f;
-            }
-            float v[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                // C = s32*sA*sB + sumB*sB*zA + sumA*zB, evaluated left to right without contraction
-                const float t0 = ((float)s32[e] * sA) * sB[e];
-                const float t1 = sumBsB[e] * zA;
-                const float t2 = sumA * zB[e];
-                v[e] = w8a8_epilogue(epi, (t0 + t1) + t2, bias[e], has_bias, res[e], p.gamma);
-            }
-            const size_t ci = (size_t)row * p.ldc + c;
-            if (full && c_wide) {
-                if (p.c_dtype == XFTHIP_F32) {
-                    const f32x4 o0 = {v[0], v[1], v[2], v[3]}, o1 = {v[4], v[5], v[6], v[7]};
-                    *(f32x4 *)((float *)p.C + ci) = o0;
-                    *(f32x4 *)((float *)p.C + ci + 4) = o1;
-                } else {
-                    i32x4 o;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const uint32_t b0 = p.c_dtype == XFTHIP_BF16 ? f32_to_bf16_ref(v[2 * e]) : f32_to_fp16_bits(v[2 * e]);
-                        const uint32_t b1 = p.c_dtype == XFTHIP_BF16 ? f32_to_bf16_ref(v[2 * e + 1]) : f32_to_fp16_bits(v[2 * e + 1]);
-                        o[e] = (int)(b0 | (b1 << 16));
-                    }
-                    *(i32x4 *)((uint16_t *)p.C + ci) = o;
-                }
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (c + e < p.N) store_from_f32(p.C, p.c_dtype, ci + e, v[e]);
             }
         }
+    };
+    switch (p.epi) {
+        case XFTHIP_EPI_BIAS: run(std::integral_constant<int, XFTHIP_EPI_BIAS> {}); break;
+        case XFTHIP_EPI_SILU: run(std::integral_constant<int, XFTHIP_EPI_SILU> {}); break;
+        case XFTHIP_EPI_GELU: run(std::integral_constant<int, XFTHIP_EPI_GELU> {}); break;
+        case XFTHIP_EPI_RESMUL: run(std::integral_constant<int, XFTHIP_EPI_RESMUL> {}); break;
+        case XFTHIP_EPI_RESIDENTIAL: run(std::integral_constant<int, XFTHIP_EPI_RESIDENTIAL> {}); break;
+        case XFTHIP_EPI_RESEXT: run(std::integral_constant<int, XFTHIP_EPI_RESEXT> {}); break;
+        default: run(std::integral_constant<int, XFTHIP_EPI_NONE> {}); break;
     }
 }
 

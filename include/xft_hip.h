@@ -392,6 +392,11 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
  *       the rows that sit out are masked when ids and positions are updated.
  *   _seq_set_next_id / _seq_logits: the searcher's hooks (replace the token a row feeds next; read
  *       the row's last logits).
+ *   _seq_reorder: cache row dst_rows_host[i] becomes a copy of row src_rows_host[i] over the positions
+ *       [pos0, pos1) (whole 32-token blocks), with its position and next token: the beam searcher's
+ *       KVCacheTensor::expandAllSequence (pos0 = 0, beams filled from the row that ran the prompt) and
+ *       ::reorder (pos0 = prompt length; src/common/kvcache_tensor.h:147-286).  A row may be source and
+ *       destination at once: everything is read before anything is written.
  *   _seq_release: frees the row.
  * xfthip_model_prefill resets this state (all rows in lockstep again).
  */
@@ -399,6 +404,8 @@ int xfthip_model_seq_prefill(xfthip_model_t m, int row, const int *ids_host, int
 int xfthip_model_seq_decode(xfthip_model_t m, const int *rows_host, int n, int *ids_out_host, xfthip_stream_t stream);
 int xfthip_model_seq_set_next_id(xfthip_model_t m, int row, int id);
 int xfthip_model_seq_logits(xfthip_model_t m, int row, float *logits_host);
+int xfthip_model_seq_reorder(xfthip_model_t m, const int *dst_rows_host, const int *src_rows_host, int n, int pos0, int pos1,
+        xfthip_stream_t stream);
 int xfthip_model_seq_release(xfthip_model_t m, int row);
 /* enable (default) or disable replaying the decode step as a captured HIP graph; with 0 every
  * step launches its kernels one by one (for per-kernel profiling) */

@@ -104,3 +104,57 @@ def test_sequences_come_and_go(xh, orc, kind, kv):
     # the lockstep API still works afterwards and resets the rows
     first, _ = model.prefill(np.asarray(prompts["b"], np.int32)[None, :])
     assert int(first[0]) == alone["b"][0][0]
+
+
+@pytest.mark.parametrize("kv", ["fp16", "int8"])
+def test_cache_rows_copied_and_reordered_for_beams(xh, orc, kv):
+    """xfthip_model_seq_reorder, the device half of KVCacheTensor::expandAllSequence / ::reorder
+    (src/common/kvcache_tensor.h:147-286): three prompts run in rows 0, 2, 4, every row is copied to its
+    neighbour (two beams), forced tokens are fed to all six rows, and three times the rows are re-mapped
+    the way a beam searcher does (a row may be read and overwritten in the same call).  Every row must then
+    produce the logits of its own token history run alone."""
+    from test_layer_model_gpu import make_layer_weights, to_device_weights
+    layers, hidden, inter, qh, kvh, D, vocab, rows, max_seq = 2, 512, 1408, 4, 2, 128, 1000, 6, 96
+    rng = np.random.default_rng(123)
+    model = xh.Model(layers, hidden, inter, qh, kvh, D, vocab=vocab, max_batch=rows, max_seq=max_seq, max_tokens=rows * max_seq,
+                     kv_dtype=xh.INT8 if kv == "int8" else xh.FP16)
+    for l in range(layers):
+        ws = make_layer_weights(orc, rng, 0, hidden, inter, qh, kvh, D)
+        model.set_layer(l, *to_device_weights(xh, ws, 0), rng.uniform(0.8, 1.2, hidden).astype(np.float32),
+                        rng.uniform(0.8, 1.2, hidden).astype(np.float32))
+    lm = orc.round_bf16(rng.standard_normal((hidden, vocab)) * 0.05)
+    model.set_head(orc.to_fp16(rng.standard_normal((vocab, hidden)) * 0.5), rng.uniform(0.8, 1.2, hidden).astype(np.float32),
+                   xh.Weight(xh.W_BF16, hidden, vocab, orc.to_bf16(lm)))
+    S, steps = 20, 18  # the generated part crosses the 32-token block boundary
+    prompts = [rng.integers(0, vocab, S).tolist() for _ in range(3)]
+    toks = rng.integers(0, vocab, (steps, rows))
+    remaps = {3: [1, 1, 2, 3, 5, 4], 9: [0, 0, 3, 2, 5, 5], 14: [1, 0, 2, 2, 4, 5]}
+    # the plan on the host: which history every row ends with
+    hist = [list(prompts[r // 2]) for r in range(rows)]
+    for k in range(steps):
+        if k in remaps:
+            hist = [list(hist[s]) for s in remaps[k]]
+        for r in range(rows):
+            hist[r].append(int(toks[k, r]))
+    want = []
+    for r in range(rows):  # each history alone, lockstep interface
+        model.prefill(np.asarray(hist[r][:S], np.int32)[None, :])
+        for t in hist[r][S:]:
+            model.set_next_ids([t])
+            model.decode(1, 1)
+        want.append(model.logits(1)[0].copy())
+    # the same through cache rows
+    for b in range(3):
+        model.seq_prefill(2 * b, prompts[b])
+    model.seq_reorder([1, 3, 5], [0, 2, 4], 0, S)
+    for k in range(steps):
+        if k in remaps:
+            model.seq_reorder(list(range(rows)), remaps[k], S, S + k)
+        for r in range(rows):
+            model.seq_set_next_id(r, int(toks[k, r]))
+        model.seq_decode(list(range(rows)))
+    for r in range(rows):
+        got = model.seq_logits(r)
+        err = float(np.abs(got - want[r]).max())
+        assert err < 2e-2, (r, err)
+    print(f"six rows agree with their solo runs after three re-mappings ({kv=})", flush=True)

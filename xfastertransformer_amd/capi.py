@@ -412,6 +412,13 @@ class Model:
     def seq_release(self, row):
         check(lib.xfthip_model_seq_release(self.h, int(row)))
 
+    def seq_reorder(self, dst_rows, src_rows, pos0, pos1, stream=None):
+        """Cache row dst_rows[i] becomes a copy of row src_rows[i] over positions [pos0, pos1)."""
+        d = np.ascontiguousarray(dst_rows, np.int32)
+        s_ = np.ascontiguousarray(src_rows, np.int32)
+        assert d.size == s_.size
+        check(lib.xfthip_model_seq_reorder(self.h, _hp(d), _hp(s_), int(d.size), int(pos0), int(pos1), stream))
+
     def set_next_ids(self, ids, stream=None):
         ids = np.ascontiguousarray(ids, np.int32)
         check(lib.xfthip_model_set_next_ids(self.h, _hp(ids), stream))

@@ -106,6 +106,43 @@ __global__ void decode_begin_kernel(const uint16_t *__restrict__ table, const in
     for (int c = threadIdx.x; c < hidden; c += blockDim.x) x[(size_t)b * hidden + c] = fp16_bits_to_f32(row[c]);
 }
 
+// Cache rows copied through a staging buffer (beam search: KVCacheTensor::expandAllSequence and ::reorder,
+// reference src/common/kvcache_tensor.h:147-286).  Entry i moves the 32-token blocks [blk0, blk0 + nblk) of
+// every head of cache row rows[i]: TO_STAGE reads them into stage[i], otherwise stage[i] is written over them.
+// Keys [B][H][S][D] and values [B][H][S/32][D][32] keep a token block at the same offset of a head's
+// segment, so one index serves both.  grid (16-byte chunks / 256, heads, 2 * entries), 256 threads.
+template <bool TO_STAGE>
+__global__ __launch_bounds__(256) void kv_rows_move_kernel(KvView kv, const int *__restrict__ rows, int blk0, int nblk,
+        unsigned char *__restrict__ stage) {
+    const int esz = kv.int8 ? 1 : 2;
+    const size_t seg = (size_t)nblk * 32 * kv.D * esz; // bytes of a head's blocks
+    const size_t at = ((size_t)blockIdx.x * 256 + threadIdx.x) * 16;
+    if (at >= seg) return;
+    const int head = blockIdx.y, i = blockIdx.z >> 1, which = blockIdx.z & 1;
+    const int row = rows[i];
+    unsigned char *cache = (unsigned char *)(which ? kv.v : kv.k) + (((size_t)row * kv.H + head) * kv.S + (size_t)blk0 * 32) * kv.D * esz + at;
+    unsigned char *st = stage + (((size_t)i * 2 + which) * kv.H + head) * seg + at;
+    if (TO_STAGE)
+        *(uint4 *)st = *(const uint4 *)cache;
+    else
+        *(uint4 *)cache = *(const uint4 *)st;
+}
+
+// the per-token scales of an INT8 cache, same staging scheme; grid (ceil(nblk * 32 / 256), heads, 2 * entries)
+template <bool TO_STAGE>
+__global__ __launch_bounds__(256) void kv_scales_move_kernel(KvView kv, const int *__restrict__ rows, int blk0, int nblk,
+        float *__restrict__ stage) {
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= nblk * 32) return;
+    const int head = blockIdx.y, i = blockIdx.z >> 1, which = blockIdx.z & 1;
+    float *cache = (which ? kv.vscale : kv.kscale) + ((size_t)rows[i] * kv.H + head) * kv.S + (size_t)blk0 * 32 + t;
+    float *st = stage + (((size_t)i * 2 + which) * kv.H + head) * ((size_t)nblk * 32) + t;
+    if (TO_STAGE)
+        *st = *cache;
+    else
+        *cache = *st;
+}
+
 __global__ void fill_int_kernel(int *p, int n, int v) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = v;
@@ -148,6 +185,9 @@ struct xfthip_model {
     int *active = nullptr; // device [max_batch]: rows taking part in the next decode call
     int *prompt_ids = nullptr; // device [max_tokens]: prompt of a single-sequence prefill
     std::vector<int> row_pos; // host copy of every row's position (-1 = free row)
+    unsigned char *kv_stage = nullptr; // staging buffer of xfthip_model_seq_reorder (grown on demand)
+    size_t kv_stage_bytes = 0;
+    int *reorder_rows = nullptr; // device [2 * max_batch]: source rows, destination rows
     hipGraphExec_t graph = nullptr;
     int graph_B = 0;
     int graph_nsplit = 0; // attention split count the captured step was built with
@@ -549,7 +589,7 @@ int xfthip_model_destroy(xfthip_model_t m) {
         if (L.o_bias) (void)hipFree(L.o_bias);
     }
     void *bufs[] = {m->w8a8_qa, m->w8a8_stat, m->gu, m->mega_trace, m->mega_layers, m->mega_ws, m->mega_sync, m->cosT, m->sinT, m->xn, m->qkv, m->att, m->h, m->x, m->xlast, m->logits, m->ids, m->pos, m->step, m->idlog,
-            m->embedding, m->final_norm, m->active, m->prompt_ids};
+            m->embedding, m->final_norm, m->active, m->prompt_ids, m->kv_stage, m->reorder_rows};
     for (void *b : bufs)
         if (b) (void)hipFree(b);
     delete m;
@@ -877,6 +917,69 @@ int xfthip_model_seq_decode(xfthip_model_t m, const int *rows_host, int n, int *
         XFT_CHECK_HIP(hipMemcpy(all.data(), m->ids, (size_t)top * 4, hipMemcpyDeviceToHost));
         for (int i = 0; i < n; ++i) ids_out_host[i] = all[rows_host[i]];
     }
+    return 0;
+}
+
+int xfthip_model_seq_reorder(xfthip_model_t m, const int *dst_rows_host, const int *src_rows_host, int n, int pos0, int pos1,
+        xfthip_stream_t stream) {
+    XFT_REQUIRE(m && dst_rows_host && src_rows_host && n > 0, "xfthip_model_seq_reorder: bad argument");
+    const xfthip_model_config &c = m->cfg;
+    XFT_REQUIRE(m->ragged && n <= c.max_batch, "xfthip_model_seq_reorder: needs sequences started with xfthip_model_seq_prefill, at most %d entries",
+            c.max_batch);
+    XFT_REQUIRE(pos0 >= 0 && pos0 <= pos1 && pos1 <= c.max_seq, "xfthip_model_seq_reorder: positions [%d, %d) outside the cache (%d)", pos0, pos1,
+            c.max_seq);
+    std::vector<char> seen(c.max_batch, 0);
+    bool identity = true;
+    for (int i = 0; i < n; ++i) {
+        const int d = dst_rows_host[i], s = src_rows_host[i];
+        XFT_REQUIRE(d >= 0 && d < c.max_batch && s >= 0 && s < c.max_batch, "xfthip_model_seq_reorder: row outside the %d cache rows", c.max_batch);
+        XFT_REQUIRE(m->row_pos[s] >= 0, "xfthip_model_seq_reorder: source row %d holds no sequence", s);
+        XFT_REQUIRE(!seen[d], "xfthip_model_seq_reorder: destination row %d listed twice", d);
+        seen[d] = 1;
+        identity = identity && d == s;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    // every destination takes over its source's position and next token
+    std::vector<int> pos_new(n), ids_all(c.max_batch), ids_new(n);
+    for (int i = 0; i < n; ++i) pos_new[i] = m->row_pos[src_rows_host[i]];
+    XFT_CHECK_HIP(hipStreamSynchronize(st));
+    XFT_CHECK_HIP(hipMemcpy(ids_all.data(), m->ids, (size_t)c.max_batch * 4, hipMemcpyDeviceToHost));
+    for (int i = 0; i < n; ++i) ids_new[i] = ids_all[src_rows_host[i]];
+    for (int i = 0; i < n; ++i) {
+        const int d = dst_rows_host[i];
+        m->row_pos[d] = pos_new[i];
+        XFT_CHECK_HIP(hipMemcpy(m->pos + d, &pos_new[i], 4, hipMemcpyHostToDevice));
+        XFT_CHECK_HIP(hipMemcpy(m->ids + d, &ids_new[i], 4, hipMemcpyHostToDevice));
+        if (d + 1 > m->cur_B) m->cur_B = d + 1;
+    }
+    if (identity || pos1 == pos0) return 0;
+    const int blk0 = pos0 / 32, nblk = (pos1 + 31) / 32 - blk0;
+    const KvView &k0 = m->caches[0]->kv;
+    const int esz = k0.int8 ? 1 : 2;
+    const size_t seg = (size_t)nblk * 32 * k0.D * esz;
+    const size_t need = (size_t)n * 2 * k0.H * seg + (k0.int8 ? (size_t)n * 2 * k0.H * nblk * 32 * sizeof(float) : 0);
+    XFT_REQUIRE((size_t)(blk0 + nblk) * 32 <= (size_t)k0.S, "xfthip_model_seq_reorder: blocks past the cache rows");
+    if (need > m->kv_stage_bytes) {
+        if (m->kv_stage) (void)hipFree(m->kv_stage);
+        m->kv_stage = nullptr, m->kv_stage_bytes = 0;
+        XFT_CHECK_HIP(hipMalloc((void **)&m->kv_stage, need));
+        m->kv_stage_bytes = need;
+    }
+    if (!m->reorder_rows) XFT_CHECK_HIP(hipMalloc((void **)&m->reorder_rows, (size_t)2 * c.max_batch * 4));
+    XFT_CHECK_HIP(hipMemcpy(m->reorder_rows, src_rows_host, (size_t)n * 4, hipMemcpyHostToDevice));
+    XFT_CHECK_HIP(hipMemcpy(m->reorder_rows + c.max_batch, dst_rows_host, (size_t)n * 4, hipMemcpyHostToDevice));
+    float *stage_scales = (float *)(m->kv_stage + (size_t)n * 2 * k0.H * seg);
+    const dim3 grid((unsigned)((seg / 16 + 255) / 256), k0.H, 2 * n), sgrid((nblk * 32 + 255) / 256, k0.H, 2 * n);
+    for (int l = 0; l < c.layers; ++l) {
+        const KvView &kv = m->caches[l]->kv;
+        hipLaunchKernelGGL(kv_rows_move_kernel<true>, grid, dim3(256), 0, st, kv, m->reorder_rows, blk0, nblk, m->kv_stage);
+        if (kv.int8) hipLaunchKernelGGL(kv_scales_move_kernel<true>, sgrid, dim3(256), 0, st, kv, m->reorder_rows, blk0, nblk, stage_scales);
+        hipLaunchKernelGGL(kv_rows_move_kernel<false>, grid, dim3(256), 0, st, kv, m->reorder_rows + c.max_batch, blk0, nblk, m->kv_stage);
+        if (kv.int8)
+            hipLaunchKernelGGL(kv_scales_move_kernel<false>, sgrid, dim3(256), 0, st, kv, m->reorder_rows + c.max_batch, blk0, nblk, stage_scales);
+    }
+    XFT_CHECK_HIP(hipGetLastError());
+    XFT_CHECK_HIP(hipStreamSynchronize(st));
     return 0;
 }
 

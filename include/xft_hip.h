@@ -218,6 +218,12 @@ int xfthip_rotary_embedding_full(int dtype, const int *positions, void *query, v
  */
 int xfthip_kvcache_create(int dtype, int batch, int kvHeads, int maxSeq, int headSize, xfthip_kvcache_t *out);
 int xfthip_kvcache_destroy(xfthip_kvcache_t c);
+/* Rows of one cache copied / re-mapped (beam search; KVCacheTensor::reorder, reference
+ * src/common/kvcache_tensor.h:196-286, and ::expandAllSequence, :147-173): row dst_rows_host[i] becomes a
+ * copy of row src_rows_host[i] over the positions [pos0, pos1), widened to whole 32-token blocks.  A row
+ * may be source and destination at once. */
+int xfthip_kvcache_reorder(xfthip_kvcache_t cache, const int *dst_rows_host, const int *src_rows_host, int n, int pos0, int pos1,
+        xfthip_stream_t stream);
 /* which: 0 = keys, 1 = values.  data_dev: fp16 bits or int8 [B][H][maxSeq][D]; scales_dev fp32 [B][H][maxSeq] (INT8 only, may be NULL for FP16) */
 int xfthip_kvcache_export(xfthip_kvcache_t c, int which, void *data_dev, float *scales_dev, xfthip_stream_t stream);
 int xfthip_kvcache_import(xfthip_kvcache_t c, int which, const void *data_dev, const float *scales_dev,

@@ -558,3 +558,120 @@ def paged_attention_prefill(q, k, v, token_lens, kcache, vcache, slot_mapping, s
             out[first:first + L, h] = round_bf16((p @ V).astype(np.float32))
         first += L
     return out
+
+
+# ---- beam search (src/searchers/beam_search.cpp) ----------------------------------------------------
+# Plain-Python restatement of BeamSearch::searchTopK / beam_search, BeamSearchScorer::process / finalize
+# and BeamHypotheses.  Pinned in tests/test_oracle_pins.py by brute force: with enough beams to keep every
+# prefix alive the best hypothesis must be the best of all vocab ** steps continuations.  The reference's
+# log-softmax uses a vectorised polynomial exp (bert_util.h); float32 numpy exp / log here: scores agree to
+# rounding, which can only matter at exact near-ties.
+class BeamSearchOracle:
+    def __init__(self, prompts, num_beams, max_len, eos, pad, vocab, keep=1, len_penalty=1.0, early=False):
+        prompts = np.asarray(prompts, np.int64)
+        self.batch, self.seq_len = prompts.shape
+        self.nb, self.keep, self.max_len, self.eos, self.pad, self.vocab = num_beams, keep, max_len, eos, pad, vocab
+        self.len_penalty, self.early = float(len_penalty), bool(early)
+        self.k = 2 * num_beams  # :284 kVal
+        self.rows = [list(prompts[b]) for b in range(self.batch) for _ in range(num_beams)]  # :285-291
+        self.scores = np.full(self.batch * num_beams, -1e9, np.float32)  # :296-300
+        self.scores[::num_beams] = 0.0
+        self.tokens = [0] * (self.batch * num_beams)
+        self.indices = [0] * (self.batch * num_beams)
+        self.hyps = [[] for _ in range(self.batch)]  # (score, ids)
+        self.worst = [1e9] * self.batch
+        self.done = [False] * self.batch
+        self.steps = 0
+
+    def _add(self, b, ids, sum_logprobs):  # BeamHypotheses::add :89-104
+        score = np.float32(sum_logprobs) / np.float32(float(len(ids)) ** self.len_penalty)
+        if len(self.hyps[b]) < self.nb or score > self.worst[b]:
+            self.hyps[b].append((float(score), list(ids)))
+            if len(self.hyps[b]) > self.nb:
+                self.hyps[b].sort(key=lambda h: h[0])
+                self.hyps[b].pop(0)
+                self.worst[b] = self.hyps[b][0][0]
+            else:
+                self.worst[b] = min(float(score), self.worst[b])
+
+    def _hyps_done(self, b, best_sum, cur_len):  # :106-116
+        if len(self.hyps[b]) < self.nb:
+            return False
+        if self.early:
+            return True
+        return self.worst[b] >= float(np.float32(best_sum) / np.float32(float(cur_len) ** self.len_penalty))
+
+    def step(self, logits):
+        """logits [batch * num_beams, vocab] of the rows' next token.  Returns (tokens, source rows)."""
+        lg = f32(logits).reshape(self.batch * self.nb, self.vocab)
+        mx = lg.max(axis=1, keepdims=True)
+        logp = lg - (mx + np.log(np.exp(lg - mx, dtype=np.float32).sum(axis=1, keepdims=True, dtype=np.float32)))  # :27-66
+        cur_len = len(self.rows[0])
+        next_scores, next_tokens, next_indices = [], [], []
+        for b in range(self.batch):
+            el = []
+            for j in range(self.nb):
+                row = b * self.nb + j
+                # the kVal largest under std::greater<pair<float, int>>: value, then the larger index (:470-481)
+                order = sorted(range(self.vocab), key=lambda t: (-float(logp[row, t]), -t))[:self.k]
+                el += [(np.float32(logp[row, t] + self.scores[row]), t, j) for t in order]
+            el.sort(key=lambda e: (-float(e[0]), e[2]))  # tupleCompare :69-77 (stable where it leaves the order open)
+            uniq = []
+            for e in el:  # std::unique with uniqueCompare :79-81: adjacent equal (score, token)
+                if uniq and uniq[-1][0] == e[0] and uniq[-1][1] == e[1]:
+                    continue
+                uniq.append(e)
+            uniq += el[len(uniq):]  # what std::unique leaves behind its new end is read as it lies; pad the same way
+            for e in uniq[:self.k]:
+                next_scores.append(e[0]), next_tokens.append(e[1]), next_indices.append(e[2])
+        new_scores = np.zeros(self.batch * self.nb, np.float32)
+        new_tokens = [self.pad] * (self.batch * self.nb)
+        new_indices = [0] * (self.batch * self.nb)
+        for b in range(self.batch):  # BeamSearchScorer::process :137-193
+            if self.done[b]:
+                continue
+            beam = 0
+            for rank in range(self.k):
+                tok, sc = next_tokens[b * self.k + rank], next_scores[b * self.k + rank]
+                row = b * self.nb + next_indices[b * self.k + rank]
+                if self.eos != -1 and tok == self.eos:
+                    if rank >= self.nb:
+                        continue
+                    self._add(b, self.rows[row], sc)
+                else:
+                    new_scores[b * self.nb + beam], new_tokens[b * self.nb + beam], new_indices[b * self.nb + beam] = sc, tok, row
+                    beam += 1
+                    if beam == self.nb:
+                        break
+            assert beam == self.nb, "At most tokens can be equal to `eosTokenId`"
+            # :187-190 reads nextScores with a stride of numBeams although a user sequence owns kVal entries
+            best = max(float(x) for x in next_scores[b * self.nb:(b + 1) * self.nb])
+            self.done[b] = self.done[b] or self._hyps_done(b, best, cur_len)
+        self.scores, self.tokens, self.indices = new_scores, new_tokens, new_indices
+        self.rows = [list(self.rows[self.indices[i]]) + [self.tokens[i]] for i in range(self.batch * self.nb)]  # :553-563
+        self.steps += 1
+        return list(self.tokens), list(self.indices)
+
+    def is_done(self):  # :330-332
+        return self.steps != 0 and (all(self.done) or len(self.rows[0]) >= self.max_len)
+
+    def finalize(self):  # BeamSearchScorer::finalize :195-263
+        for b in range(self.batch):
+            if self.done[b]:
+                continue
+            for j in range(self.nb):
+                self._add(b, self.rows[b * self.nb + j], self.scores[b * self.nb + j])
+        best = []
+        for b in range(self.batch):
+            hs = sorted(self.hyps[b], key=lambda h: h[0])
+            for _ in range(self.keep):
+                best.append(hs.pop()[1])
+        out_len = min(max(len(h) for h in best) + 1, self.max_len)
+        out = np.full((len(best), out_len), self.pad, np.int32)
+        for i, h in enumerate(best):
+            if len(h) < self.max_len:
+                out[i, :len(h)] = h
+                out[i, len(h)] = self.eos
+            else:
+                out[i, :] = h[:self.max_len]
+        return out

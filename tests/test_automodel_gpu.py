@@ -287,3 +287,49 @@ def test_continuous_batching_through_the_model_class(am, tmp_path):
     assert out[b[0]][:5] == pen[1][len(prompts[1]):len(prompts[1]) + 5].tolist() and all(t == never for t in out[b[0]][5:])
     assert len(out[b[1]]) == 13 and out[b[1]][:12] == pen[2][len(prompts[2]):len(prompts[2]) + 12].tolist()
     model.free()
+
+
+@pytest.mark.parametrize("kv", ["fp16", "int8"])
+def test_beam_search_through_the_model_class(xh, orc, am, tmp_path, kv):
+    """numBeams > 1 (BeamSearch, src/searchers/beam_search.cpp): every step's tokens and the final hypotheses must
+    be those of the pinned restatement of the searcher fed with the logits the directly built device model has
+    for each beam row's token history (recomputed from scratch - the prompt, then one decode step per generated
+    token, so the cache copies and re-mappings behind Model::generate are what is under test).  The EOS id is the first sequence's most likely first token, so a
+    hypothesis closes in the first step; two hypotheses are returned per sequence."""
+    import make_llama_fixture as fx
+    held = fx.write_model_dir(str(tmp_path / "model"), None, 11)
+    B, S, nb, keep, max_len = 2, 6, 3, 2, 15
+    V = held["cfg"]["vocab"]
+    ids = np.random.default_rng(12).integers(0, V, (B, S)).astype(np.int32)
+    direct, _ = _direct(xh, orc, held, "int8", kv, B * nb, max_len, with_oracle=False)
+    _, lg0 = direct.prefill(np.repeat(ids, nb, 0), want_logits=True)
+    eos, pad = int(lg0[0].argmax()), 1
+    model = am.AutoModel.from_pretrained(str(tmp_path / "model"), dtype="int8", kv_cache_dtype=kv)
+    model.config(max_length=max_len, num_beams=nb, num_return_sequences=keep, eos_token_id=eos, pad_token_id=pad)
+    model.input(ids)
+    ref = orc.BeamSearchOracle(ids, nb, max_len, eos, pad, V, keep=keep)
+    steps = 0
+    while not ref.is_done():
+        assert not model.is_done()
+        hist = np.asarray(ref.rows, np.int32)
+        _, lg = direct.prefill(hist[:, :S], want_logits=True)
+        for t in range(S, hist.shape[1]):
+            direct.set_next_ids(hist[:, t])
+            direct.decode(1, B * nb)
+            lg = direct.logits(B * nb)
+        want, _ = ref.step(lg)
+        got = model.forward().ravel().tolist()
+        assert got == want, (steps, got, want)
+        steps += 1
+    assert model.is_done() and steps >= 3
+    out = model.finalize()
+    exp = ref.finalize()
+    assert out.shape == exp.shape == (B * keep, exp.shape[1]) and np.array_equal(out, exp)
+    assert len(ref.hyps[0]) >= 1 and ref.hyps[0][0][1] == ids[0].tolist() or any(h[1] == ids[0].tolist() for h in ref.hyps[0])
+    # the one-call form gives the same
+    again = model.generate(ids, max_length=max_len, num_beams=nb, num_return_sequences=keep, eos_token_id=eos, pad_token_id=pad)
+    assert np.array_equal(again, exp)
+    # and greedy search still works on the same object afterwards
+    g = model.generate(ids, max_length=S + 4, eos_token_id=V + 3)
+    assert g.shape == (B, S + 4)
+    model.free()

@@ -157,6 +157,53 @@ def test_kv_import_export_roundtrip(xh, orc, int8):
             assert np.array_equal(s, scales)
 
 
+# index vectors of the reference's own reorder test (tests/ut/kv_reorder_test.cpp:64-124): the fixed ones of
+# reorder4 / reorder6, samples of reorder8 (beam size 4, two user sequences) and of reorder6More
+REORDER_CASES = [
+    [0, 2, 1, 3], [0, 0, 0, 0], [1, 1, 0, 0], [1, 0, 2, 1], [0, 1, 0, 1],
+    [0, 2, 1, 4, 3, 3], [1, 2, 3, 4, 5, 0], [1, 3, 2, 4, 3, 5], [2, 1, 0, 4, 5, 0], [2, 0, 1, 5, 5, 4],
+    [3, 0, 0, 2, 5, 7, 7, 4], [1, 1, 3, 2, 6, 6, 4, 5], [2, 3, 0, 1, 7, 4, 5, 6],
+    [0, 0, 0, 0, 5, 4], [3, 2, 1, 0, 5, 4], [1, 3, 3, 1, 5, 4],
+]
+
+
+@pytest.mark.parametrize("int8", [0, 1])
+def test_kv_reorder_reference_cases(xh, orc, int8):
+    """Every (position, row, head) holds a value of its own (the reference test's fill, :29-40); after
+    reorder(idx) row b must hold what row idx[b] held (:44-55), for keys, values and INT8 scales alike.
+    Positions outside [pos0, pos1) rounded to 32-token blocks stay what they were."""
+    H, S, D = 4, 70, 128
+    for case, idx in enumerate(REORDER_CASES):
+        B = len(idx)
+        cache = xh.KVCache(xh.INT8 if int8 else xh.FP16, B, H, S, D)
+        seq, row, head = np.meshgrid(np.arange(S), np.arange(B), np.arange(H), indexing="ij")
+        val = (seq * B + row) + 0.01 * head  # [S][B][H]
+        val = np.transpose(val, (1, 2, 0))  # [B][H][S]
+        if int8:
+            data = np.broadcast_to(((seq * B + row) % 251 - 125).transpose(1, 2, 0)[..., None], (B, H, S, D)).astype(np.int8)
+            scales = (0.001 * (1 + val)).astype(np.float32)
+        else:
+            data = orc.to_fp16(np.broadcast_to(val[..., None], (B, H, S, D)))
+            scales = np.zeros((B, H, S), np.float32)
+        for which in (0, 1):
+            cache.load(which, data + (which if int8 else 0), scales * (1 + which))
+        pos0, pos1 = (0, S) if case % 2 == 0 else (33, 64)  # whole cache / the second 32-token block only
+        cache.reorder(list(range(B)), idx, pos0, pos1)
+        lo, hi = pos0 // 32 * 32, min(S, (pos1 + 31) // 32 * 32)
+        for which in (0, 1):
+            d, sc = cache.export(which)
+            want_d = (data + (which if int8 else 0)).copy()
+            want_s = (scales * (1 + which)).copy()
+            src_d, src_s = want_d.copy(), want_s.copy()
+            for b in range(B):
+                want_d[b, :, lo:hi] = src_d[idx[b], :, lo:hi]
+                want_s[b, :, lo:hi] = src_s[idx[b], :, lo:hi]
+            assert np.array_equal(d[:, :, :S], want_d), (case, which)
+            if int8:
+                assert np.array_equal(sc[:, :, :S], want_s), (case, which)
+        cache.free()
+
+
 def test_kvstore_rejects_overflow(xh):
     cache = xh.KVCache(xh.FP16, 1, 2, 16, 128)
     dev = xh.DeviceBuffer(4 * (8 + 4) * 128 * 2)

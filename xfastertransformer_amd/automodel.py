@@ -36,6 +36,14 @@ _lib.xft_automodel_set_input.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c
 _lib.xft_automodel_free_seqs.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
 _lib.xft_sample_candidates.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_float, C.c_void_p, C.c_void_p]
 _lib.xft_sample_pick.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_float]
+_lib.xft_beam_create.restype = C.c_void_p
+_lib.xft_beam_create.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_int, C.c_int, C.c_int, C.c_int]
+_lib.xft_beam_step.restype = None
+_lib.xft_beam_step.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+_lib.xft_beam_is_done.argtypes = [C.c_void_p]
+_lib.xft_beam_finalize.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
+_lib.xft_beam_destroy.restype = None
+_lib.xft_beam_destroy.argtypes = [C.c_void_p]
 
 # the types this build serves out of the reference's list (automodel.py:21-39)
 _DTYPES = ["fp16", "bf16", "int8", "w8a8", "int4", "nf4"]
@@ -76,6 +84,43 @@ def sample_pick(ids, probs, u):
     return int(_lib.xft_sample_pick(ids.ctypes.data, probs.ctypes.data, len(ids), float(u)))
 
 
+class BeamSearcher:
+    """The beam searcher's host half on its own: feed it the logits of every beam row, read the token and the
+    source row it chose for each (what Model.generate does between two device steps)."""
+
+    def __init__(self, prompts, num_beams, max_length, eos_token_id, pad_token_id, vocab_size, num_return_sequences=1,
+                 length_penalty=1.0, early_stopping=False):
+        a = _ids_array(prompts)
+        self.rows, self.vocab, self.keep, self.max_length = a.shape[0] * num_beams, vocab_size, num_return_sequences, max_length
+        self.batch = a.shape[0]
+        self._h = _lib.xft_beam_create(a.ctypes.data, a.shape[0], a.shape[1], int(num_beams), int(num_return_sequences), int(max_length),
+                                       float(length_penalty), int(bool(early_stopping)), int(eos_token_id), int(pad_token_id),
+                                       int(vocab_size))
+
+    def step(self, logits):
+        lg = np.array(logits, dtype=np.float32, order="C").reshape(self.rows, self.vocab)
+        tokens, indices, scores = np.zeros(self.rows, np.int32), np.zeros(self.rows, np.int32), np.zeros(self.rows, np.float32)
+        _lib.xft_beam_step(self._h, lg.ctypes.data, tokens.ctypes.data, indices.ctypes.data, scores.ctypes.data)
+        return tokens.tolist(), indices.tolist(), scores
+
+    def is_done(self):
+        return bool(_lib.xft_beam_is_done(self._h))
+
+    def finalize(self):
+        cap = self.batch * self.keep * (self.max_length + 1)
+        out = np.zeros(cap, np.int32)
+        n = _lib.xft_beam_finalize(self._h, out.ctypes.data, cap)
+        return out[:n].reshape(self.batch * self.keep, -1)
+
+    def __del__(self):
+        try:
+            if self._h:
+                _lib.xft_beam_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
 class AutoModel:
     def __init__(self, path, dtype: str = "fp16", kv_cache_dtype: str = "fp16"):
         if dtype not in _REFERENCE_DTYPES:
@@ -89,6 +134,7 @@ class AutoModel:
         self._h = _lib.xft_automodel_create(os.fsencode(path), dtype.encode(), kv_cache_dtype.encode())
         self._torch_out = False
         self._batch = 0
+        self._beams, self._keep = 1, 1
 
     @classmethod
     def from_pretrained(cls, path, dtype: str = "fp16", kv_cache_dtype: str = "fp16"):
@@ -109,8 +155,7 @@ class AutoModel:
     def config(self, max_length=20, num_beams=1, num_return_sequences=1, length_penalty=1.0, early_stopping=False,
                eos_token_id=-1, pad_token_id=-1, do_sample=False, temperature=1.0, top_k=50, top_p=1.0,
                repetition_penalty=1.0, stop_words_ids=None, **kwargs):
-        if num_beams != 1:
-            raise NotImplementedError("beam search is not served by this build")
+        self._beams, self._keep = int(num_beams), int(num_return_sequences)
         words = [list(w) for w in (stop_words_ids or [])]
         lens = np.asarray([len(w) for w in words], np.int32)
         flat = np.asarray([t for w in words for t in w], np.int32)
@@ -142,6 +187,7 @@ class AutoModel:
                                          len(given), int(max_length), int(eos_token_id), int(pad_token_id), float(repetition_penalty),
                                          out.ctypes.data)
         self._batch = n
+        self._beams = 1
         self._torch_out = False
         return out[:n].tolist()
 
@@ -160,10 +206,10 @@ class AutoModel:
         return a
 
     def forward(self):
-        """One generation step: the next token of every sequence, [batch, 1]."""
-        out = np.zeros(self._batch, np.int32)
-        _lib.xft_automodel_generate(self._h, out.ctypes.data)
-        return self._wrap(out[:, None])
+        """One generation step: the next token of every sequence (of every beam row under beam search), [rows, 1]."""
+        out = np.zeros(self._batch * self._beams, np.int32)
+        n = _lib.xft_automodel_generate(self._h, out.ctypes.data)
+        return self._wrap(out[:n, None])
 
     def logits(self):
         """fp32 [batch, vocab] logits of the prompt's next token (Model::forward(false))."""
@@ -178,9 +224,10 @@ class AutoModel:
         n = _lib.xft_automodel_finalize(self._h, None, 0)
         out = np.zeros(n, np.int32)
         _lib.xft_automodel_finalize(self._h, out.ctypes.data, n)
-        if self._batch <= 0 or n % self._batch != 0:
+        rows = self._batch * (self._keep if self._beams > 1 else 1)
+        if rows <= 0 or n % rows != 0:
             return self._wrap(out)  # sequences of different lengths, back to back
-        return self._wrap(out.reshape(self._batch, -1))
+        return self._wrap(out.reshape(rows, -1))
 
     def generate(self, input_ids=None, max_length=20, num_beams=1, num_return_sequences=1, length_penalty=1.0,
                  early_stopping=False, eos_token_id=-1, pad_token_id=-1, do_sample=False, temperature=1.0, top_k=50,

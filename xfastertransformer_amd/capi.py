@@ -275,6 +275,13 @@ class KVCache:
         check(lib.xfthip_kvcache_import(self.h, which, d.ptr, None if s is None else s.ptr, None))
         synchronize()
 
+    def reorder(self, dst_rows, src_rows, pos0, pos1, stream=None):
+        """Row dst_rows[i] becomes a copy of row src_rows[i] over positions [pos0, pos1) (32-token blocks)."""
+        d = np.ascontiguousarray(dst_rows, np.int32)
+        s_ = np.ascontiguousarray(src_rows, np.int32)
+        assert d.size == s_.size
+        check(lib.xfthip_kvcache_reorder(self.h, _hp(d), _hp(s_), int(d.size), int(pos0), int(pos1), stream))
+
     def free(self):
         if self.h is not None:
             lib.xfthip_kvcache_destroy(self.h)

@@ -21,7 +21,9 @@
 #include <map>
 #include <random>
 #include <set>
+#include <limits>
 #include <string>
+#include <tuple>
 #include <vector>
 
 #include "../../../include/models.h"
@@ -219,6 +221,207 @@ HostMatrix hcat(const std::vector<const HostMatrix *> &parts) {
 
 namespace xft {
 
+// ---- beam search: the host half (reference src/searchers/beam_search.cpp) --------------------------
+// One object holds what BeamSearch, BeamSearchScorer and BeamHypotheses hold there.  The device supplies
+// the logits of every beam row and copies cache rows; everything else is integer / float bookkeeping.
+struct BeamSearcher {
+    struct Hyps { // BeamHypotheses (:86-116)
+        std::vector<std::pair<float, std::vector<int32_t>>> beams;
+        float worst = 1e9f;
+    };
+    int batch = 0, numBeams = 0, keep = 1, maxLen = 0, kVal = 0, vocab = 0, eos = -1, pad = -1;
+    float lenPenalty = 1.0f;
+    bool early = false;
+    std::vector<Hyps> hyps;
+    std::vector<char> done;
+    std::vector<int32_t> inputIds; // [batch * numBeams][len]
+    int len = 0; // tokens of a row of inputIds
+    std::vector<float> beamScores;
+    std::vector<int> beamTokens, beamIndices;
+    int steps = 0;
+
+    int rows() const { return batch * numBeams; }
+
+    void start(const int32_t *ids, int batch_, int seqLen, int numBeams_, int keep_, int maxLen_, float lenPenalty_, bool early_, int eos_,
+            int pad_, int vocab_) {
+        batch = batch_, numBeams = numBeams_, keep = keep_, maxLen = maxLen_, lenPenalty = lenPenalty_, early = early_;
+        eos = eos_, pad = pad_, vocab = vocab_, kVal = 2 * numBeams_, steps = 0;
+        if (numBeams <= 1) {
+            printf("numBeams has to be an integer strictly greater than 1\n");
+            exit(-1);
+        }
+        hyps.assign(batch, Hyps());
+        done.assign(batch, 0);
+        len = seqLen;
+        inputIds.resize((size_t)rows() * seqLen);
+        for (int b = 0; b < batch; ++b)
+            for (int j = 0; j < numBeams; ++j)
+                std::copy(ids + (size_t)b * seqLen, ids + (size_t)(b + 1) * seqLen, inputIds.begin() + ((size_t)b * numBeams + j) * seqLen);
+        // all candidates of the first step come from beam 0 (:296-300)
+        beamScores.assign(rows(), -1e9f);
+        for (int b = 0; b < batch; ++b) beamScores[(size_t)b * numBeams] = 0.0f;
+        beamTokens.assign(rows(), 0);
+        beamIndices.assign(rows(), 0);
+    }
+
+    void add_hyp(Hyps &h, std::vector<int32_t> hyp, float sumLogProbs) const { // :89-104
+        const float score = sumLogProbs / std::pow((float)hyp.size(), lenPenalty);
+        if ((int)h.beams.size() < numBeams || score > h.worst) {
+            h.beams.emplace_back(score, std::move(hyp));
+            if ((int)h.beams.size() > numBeams) {
+                std::sort(h.beams.begin(), h.beams.end(), [](const auto &a, const auto &b) { return a.first < b.first; });
+                h.beams.erase(h.beams.begin());
+                h.worst = h.beams[0].first;
+            } else {
+                h.worst = std::min(score, h.worst);
+            }
+        }
+    }
+
+    bool hyps_done(const Hyps &h, float bestSumLogProbs, int curLen) const { // :106-116
+        if ((int)h.beams.size() < numBeams) return false;
+        if (early) return true;
+        return h.worst >= bestSumLogProbs / std::pow((float)curLen, lenPenalty);
+    }
+
+    bool all_done() const {
+        for (char f : done)
+            if (!f) return false;
+        return true;
+    }
+
+    // logits: fp32 [rows][vocab], overwritten by their log-softmax.  Chooses the next token and the
+    // source row of every beam row (searchTopK + BeamSearchScorer::process + the inputIds update).
+    void step(float *logits) {
+        const int R = rows();
+        std::vector<float> topVals((size_t)R * kVal);
+        std::vector<int> topIds((size_t)R * kVal);
+        for (int i = 0; i < R; ++i) {
+            float *p = logits + (size_t)i * vocab;
+            float mx = std::numeric_limits<float>::lowest();
+            for (int j = 0; j < vocab; ++j) mx = std::max(mx, p[j]);
+            float sum = 0.0f;
+            for (int j = 0; j < vocab; ++j) sum += std::exp(p[j] - mx);
+            const float sub = mx + std::log(sum);
+            for (int j = 0; j < vocab; ++j) p[j] -= sub;
+            // the kVal largest in the order of std::greater<std::pair<float, int>> (:470-481)
+            std::vector<std::pair<float, int>> best;
+            best.reserve(kVal + 1);
+            for (int j = 0; j < vocab; ++j) {
+                const std::pair<float, int> e(p[j], j);
+                if ((int)best.size() == kVal && !(e > best.back())) continue;
+                best.insert(std::upper_bound(best.begin(), best.end(), e, std::greater<std::pair<float, int>>()), e);
+                if ((int)best.size() > kVal) best.pop_back();
+            }
+            for (int j = 0; j < kVal; ++j) {
+                topVals[(size_t)i * kVal + j] = best[j].first + beamScores[i];
+                topIds[(size_t)i * kVal + j] = best[j].second;
+            }
+        }
+        // per user sequence: the kVal best of its beams' candidates, equal (score, token) pairs once (:528-547)
+        std::vector<float> nextScores((size_t)batch * kVal);
+        std::vector<int> nextTokens((size_t)batch * kVal), nextIndices((size_t)batch * kVal);
+        for (int b = 0; b < batch; ++b) {
+            std::vector<std::tuple<float, int, int>> el((size_t)numBeams * kVal);
+            for (int j = 0; j < numBeams; ++j)
+                for (int k = 0; k < kVal; ++k) {
+                    const size_t at = ((size_t)b * numBeams + j) * kVal + k;
+                    el[(size_t)j * kVal + k] = std::make_tuple(topVals[at], topIds[at], j);
+                }
+            std::stable_sort(el.begin(), el.end(), [](const auto &x, const auto &y) {
+                if (std::get<0>(x) > std::get<0>(y)) return true;
+                return std::get<0>(x) == std::get<0>(y) && std::get<2>(x) < std::get<2>(y);
+            });
+            (void)std::unique(el.begin(), el.end(),
+                    [](const auto &x, const auto &y) { return std::get<0>(x) == std::get<0>(y) && std::get<1>(x) == std::get<1>(y); });
+            for (int k = 0; k < kVal; ++k) {
+                nextScores[(size_t)b * kVal + k] = std::get<0>(el[k]);
+                nextTokens[(size_t)b * kVal + k] = std::get<1>(el[k]);
+                nextIndices[(size_t)b * kVal + k] = std::get<2>(el[k]);
+            }
+        }
+        // BeamSearchScorer::process (:137-193): len is still the length before this step's token
+        std::vector<float> newScores(R, 0.0f);
+        std::vector<int> newTokens(R, pad), newIndices(R, 0);
+        for (int b = 0; b < batch; ++b) {
+            if (done[b]) continue; // its rows are fed the pad token from row 0
+            int beamIdx = 0;
+            for (int rank = 0; rank < kVal; ++rank) {
+                const int tok = nextTokens[(size_t)b * kVal + rank];
+                const float sc = nextScores[(size_t)b * kVal + rank];
+                const int row = b * numBeams + nextIndices[(size_t)b * kVal + rank];
+                if (eos != -1 && tok == eos) {
+                    if (rank >= numBeams) continue;
+                    add_hyp(hyps[b], std::vector<int32_t>(inputIds.begin() + (size_t)row * len, inputIds.begin() + (size_t)(row + 1) * len), sc);
+                } else {
+                    newScores[(size_t)b * numBeams + beamIdx] = sc;
+                    newTokens[(size_t)b * numBeams + beamIdx] = tok;
+                    newIndices[(size_t)b * numBeams + beamIdx] = row;
+                    if (++beamIdx == numBeams) break;
+                }
+            }
+            if (beamIdx < numBeams) {
+                printf("At most tokens can be equal to `eosTokenId`\n");
+                exit(-1);
+            }
+            // the reference takes this maximum over nextScores[b * numBeams .. (b + 1) * numBeams), although a
+            // user sequence owns kVal = 2 * numBeams entries (:187-190); kept as it is
+            const float best = *std::max_element(nextScores.begin() + (size_t)b * numBeams, nextScores.begin() + (size_t)(b + 1) * numBeams);
+            done[b] = done[b] || hyps_done(hyps[b], best, len);
+        }
+        beamScores = newScores, beamTokens = newTokens, beamIndices = newIndices;
+        // every row continues the history of its source row (:553-563)
+        std::vector<int32_t> grown((size_t)R * (len + 1));
+        for (int i = 0; i < R; ++i) {
+            std::copy(inputIds.begin() + (size_t)beamIndices[i] * len, inputIds.begin() + (size_t)(beamIndices[i] + 1) * len,
+                    grown.begin() + (size_t)i * (len + 1));
+            grown[(size_t)(i + 1) * (len + 1) - 1] = beamTokens[i];
+        }
+        inputIds.swap(grown);
+        ++len;
+        ++steps;
+    }
+
+    bool is_done() const { return steps != 0 && (all_done() || len >= maxLen); } // :330-332
+
+    std::vector<int32_t> finalize() { // BeamSearchScorer::finalize (:195-263)
+        for (int b = 0; b < batch; ++b) {
+            if (done[b]) continue;
+            for (int j = 0; j < numBeams; ++j) {
+                const size_t row = (size_t)b * numBeams + j;
+                add_hyp(hyps[b], std::vector<int32_t>(inputIds.begin() + row * len, inputIds.begin() + (row + 1) * len), beamScores[row]);
+            }
+        }
+        std::vector<std::vector<int32_t>> best;
+        std::vector<int> lens;
+        for (int b = 0; b < batch; ++b) {
+            auto sorted = hyps[b].beams;
+            std::sort(sorted.begin(), sorted.end(), [](const auto &x, const auto &y) { return x.first < y.first; });
+            for (int j = 0; j < keep; ++j) {
+                if (sorted.empty()) {
+                    printf("numBeamHypsToKeep (%d) exceeds the hypotheses kept for a sequence.\n", keep);
+                    exit(-1);
+                }
+                best.push_back(sorted.back().second);
+                lens.push_back((int)sorted.back().second.size());
+                sorted.pop_back();
+            }
+        }
+        const int longest = *std::max_element(lens.begin(), lens.end());
+        const int outLen = std::min(longest + 1, maxLen);
+        std::vector<int32_t> decoded((size_t)best.size() * outLen, pad);
+        for (size_t i = 0; i < best.size(); ++i) {
+            if (lens[i] < maxLen) {
+                std::copy(best[i].begin(), best[i].end(), decoded.begin() + i * outLen);
+                decoded[i * outLen + lens[i]] = eos;
+            } else {
+                std::copy(best[i].begin(), best[i].begin() + maxLen, decoded.begin() + i * outLen);
+            }
+        }
+        return decoded;
+    }
+};
+
 struct ModelImpl {
     std::string path, modelType;
     xft::DataType fileType = xft::DataType::fp32;
@@ -252,6 +455,11 @@ struct ModelImpl {
     std::vector<float> logitsHost;
     int step = 0, curLen = 0, batch = 0;
     std::mt19937_64 rng {std::random_device {}()};
+    bool beam = false; // numBeams > 1: BeamSearch instead of Greedy / SampleSearch
+    int numBeams = 1, numBeamHypsToKeep = 1;
+    float lenPenalty = 1.0f;
+    bool doEarlyStopping = false;
+    BeamSearcher beams;
 
     // continuous batching (Model::set_input / generate / freeSeqs): the sequence pool and the
     // sequence-id -> cache-row map, the roles of SequencePool and KVCacheMgr
@@ -615,8 +823,18 @@ void Model::config(SearcherConfig &config_, const std::vector<std::vector<int>> 
     configuration = config_;
     ModelImpl &s = *impl;
     // getGenerationMode: one beam = greedy or sampling, more = beam search (searcher.h)
-    if (config_.numBeams != 1) unsupported("Beam search (numBeams != 1)");
-    s.sampling = config_.doSample;
+    if (config_.numBeams < 1) {
+        printf("numBeams has to be an integer greater than 0\n");
+        exit(-1);
+    }
+    s.beam = config_.numBeams > 1;
+    s.numBeams = config_.numBeams;
+    s.numBeamHypsToKeep = config_.numBeamHypsToKeep;
+    s.lenPenalty = config_.lenPenalty;
+    s.doEarlyStopping = config_.doEarlyStopping;
+    if (s.beam && config_.repetitionPenalty != 1.0f)
+        printf("[Warning] BeamSearch doesn't support repetition penalty now and repetition penalty is %f.\n", config_.repetitionPenalty);
+    s.sampling = config_.doSample && !s.beam;
     s.maxLen = config_.maxLen;
     s.eosTokenId = config_.eosTokenId == -1 ? s.endId : config_.eosTokenId;
     s.padTokenId = config_.padTokenId == -1 ? s.eosTokenId : config_.padTokenId;
@@ -642,6 +860,11 @@ void Model::config(SearcherConfig &config_, const std::vector<std::vector<int>> 
 
 bool Model::setStopWords(std::vector<std::vector<int>> stopWordsList) {
     ModelImpl &s = *impl;
+    if (s.beam) { // beam_search.cpp:334-337
+        if (!stopWordsList.empty()) printf("[Warning] BeamSearch is not supporting stop words yet.\n");
+        s.stopWordsList.clear();
+        return false;
+    }
     // a stop word that is only the EOS token is dropped (greedy_search.cpp:140-146)
     s.stopWordsList.clear();
     for (auto &w : stopWordsList)
@@ -661,6 +884,7 @@ bool Model::isDone() {
         exit(-1);
     }
     if (isNewInput) return false;
+    if (s.beam) return s.beams.is_done();
     if (s.step == 0) return false;
     if (s.curLen >= s.maxLen) return true;
     for (int f : s.doneBatch)
@@ -751,9 +975,59 @@ static std::vector<int32_t> generate_cb(ModelImpl &s) {
     return std::vector<int32_t>(ids.begin(), ids.end());
 }
 
+// BeamSearch::getNextToken (beam_search.cpp:268-324): the prompt runs once per user sequence, in the cache
+// row of its first beam; the other beams' rows are filled from it.  Later steps re-map the generated part of
+// the cache rows to the beams the scorer kept, feed every row its token and read all rows' logits.
+static std::vector<int32_t> generate_beam(ModelImpl &s, const std::vector<int32_t> &inputIds, int batchSize, int seqLen, bool first) {
+    const int nb = s.numBeams, rows = batchSize * nb;
+    std::vector<int> all(rows);
+    for (int i = 0; i < rows; ++i) all[i] = i;
+    s.logitsHost.resize((size_t)rows * s.vocab);
+    if (first) {
+        s.batch = batchSize;
+        s.fit(rows, seqLen, std::max(seqLen + 1, s.maxLen) + 1);
+        for (int r = 0; r < s.cfg.max_batch; ++r) CK(xfthip_model_seq_release(s.model, r));
+        s.beams.start(inputIds.data(), batchSize, seqLen, nb, s.numBeamHypsToKeep, s.maxLen, s.lenPenalty, s.doEarlyStopping, s.eosTokenId,
+                s.padTokenId, s.vocab);
+        std::vector<int> dst, src;
+        for (int b = 0; b < batchSize; ++b) {
+            float *lg = s.logitsHost.data() + (size_t)b * nb * s.vocab;
+            CK(xfthip_model_seq_prefill(s.model, b * nb, inputIds.data() + (size_t)b * seqLen, seqLen, lg, nullptr));
+            for (int j = 1; j < nb; ++j) {
+                std::copy(lg, lg + s.vocab, lg + (size_t)j * s.vocab);
+                dst.push_back(b * nb + j);
+                src.push_back(b * nb);
+            }
+        }
+        CK(xfthip_model_seq_reorder(s.model, dst.data(), src.data(), (int)dst.size(), 0, seqLen, nullptr));
+    } else {
+        const int cached = s.beams.len - 1; // tokens in every cache row: all but the one about to be fed
+        CK(xfthip_model_seq_reorder(s.model, all.data(), s.beams.beamIndices.data(), rows, seqLen, cached, nullptr));
+        for (int i = 0; i < rows; ++i) CK(xfthip_model_seq_set_next_id(s.model, i, s.beams.beamTokens[i]));
+        CK(xfthip_model_seq_decode(s.model, all.data(), rows, nullptr, nullptr));
+        const float *dev = nullptr;
+        CK(xfthip_model_logits(s.model, &dev));
+        CK(xfthip_memcpy_d2h(s.logitsHost.data(), dev, s.logitsHost.size() * 4, nullptr));
+    }
+    s.beams.step(s.logitsHost.data());
+    s.step++;
+    s.curLen = s.beams.len;
+    return std::vector<int32_t>(s.beams.beamTokens.begin(), s.beams.beamTokens.end());
+}
+
 std::vector<int32_t> Model::generate() {
     ModelImpl &s = *impl;
     if (s.cbMode) return generate_cb(s);
+    if (s.beam) {
+        if (!s.haveSearcher || inputIds.empty()) {
+            printf("Please set input and config first.\n");
+            exit(-1);
+        }
+        const bool first = isNewInput;
+        isNewInput = false;
+        if (first) s.step = 0;
+        return generate_beam(s, inputIds, batchSize, seqLen, first);
+    }
     if (!s.haveSearcher) {
         printf("Please set the generation config by model.config().\n");
         exit(-1);
@@ -821,6 +1095,7 @@ std::vector<int32_t> Model::generate() {
 
 std::vector<int32_t> Model::finalize() {
     ModelImpl &s = *impl;
+    if (!s.cbMode && s.beam) return s.beams.finalize();
     if (!s.cbMode) return s.output;
     // models.cpp:738-756: prompt + generated tokens of the working sequences, back to back; their cache
     // rows are released
@@ -1126,6 +1401,34 @@ int xft_automodel_set_input(void *h, const int *lens, const int *ids, int n, con
 int xft_automodel_free_seqs(void *h, const int *seq_ids, int n) {
     std::vector<int> v(seq_ids, seq_ids + n);
     return ((xft::AutoModel *)h)->freeSeqs(v) ? 1 : 0;
+}
+
+// The beam searcher's host half on its own (no device): a test feeds it logits and reads its choices.
+void *xft_beam_create(const int *prompt_ids, int batch, int seq_len, int num_beams, int keep, int max_len, float len_penalty, int early,
+        int eos, int pad, int vocab) {
+    xft::BeamSearcher *b = new xft::BeamSearcher();
+    b->start(prompt_ids, batch, seq_len, num_beams, keep, max_len, len_penalty, early != 0, eos, pad, vocab);
+    return b;
+}
+// logits fp32 [batch * num_beams, vocab] (overwritten); tokens_out / indices_out int32 [batch * num_beams]
+void xft_beam_step(void *h, float *logits, int *tokens_out, int *indices_out, float *scores_out) {
+    xft::BeamSearcher *b = (xft::BeamSearcher *)h;
+    b->step(logits);
+    memcpy(tokens_out, b->beamTokens.data(), b->beamTokens.size() * 4);
+    memcpy(indices_out, b->beamIndices.data(), b->beamIndices.size() * 4);
+    if (scores_out) memcpy(scores_out, b->beamScores.data(), b->beamScores.size() * 4);
+}
+int xft_beam_is_done(void *h) {
+    return ((xft::BeamSearcher *)h)->is_done() ? 1 : 0;
+}
+// returns the number of ids (batch * keep * row length); copies at most `capacity`; call once
+int xft_beam_finalize(void *h, int *out, int capacity) {
+    std::vector<int32_t> r = ((xft::BeamSearcher *)h)->finalize();
+    memcpy(out, r.data(), (size_t)std::min((int)r.size(), capacity) * 4);
+    return (int)r.size();
+}
+void xft_beam_destroy(void *h) {
+    delete (xft::BeamSearcher *)h;
 }
 
 int xft_automodel_vocab_size(void *h) {

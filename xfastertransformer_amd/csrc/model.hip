@@ -920,6 +920,52 @@ int xfthip_model_seq_decode(xfthip_model_t m, const int *rows_host, int n, int *
     return 0;
 }
 
+// One cache on its own: row dst_rows_host[i] becomes a copy of row src_rows_host[i] over positions
+// [pos0, pos1) (whole 32-token blocks); everything is read before anything is written.  The staging
+// buffer lives for the call (not a hot path: the model driver keeps its own).
+int xfthip_kvcache_reorder(xfthip_kvcache_t cache, const int *dst_rows_host, const int *src_rows_host, int n, int pos0, int pos1,
+        xfthip_stream_t stream) {
+    XFT_REQUIRE(cache && dst_rows_host && src_rows_host && n > 0, "xfthip_kvcache_reorder: bad argument");
+    const KvView &kv = cache->kv;
+    XFT_REQUIRE(pos0 >= 0 && pos0 <= pos1 && pos1 <= cache->maxSeq, "xfthip_kvcache_reorder: positions [%d, %d) outside the cache (%d)", pos0, pos1,
+            cache->maxSeq);
+    std::vector<char> seen(kv.B, 0);
+    for (int i = 0; i < n; ++i) {
+        const int d = dst_rows_host[i], s = src_rows_host[i];
+        XFT_REQUIRE(d >= 0 && d < kv.B && s >= 0 && s < kv.B, "xfthip_kvcache_reorder: row outside the %d cache rows", kv.B);
+        XFT_REQUIRE(!seen[d], "xfthip_kvcache_reorder: destination row %d listed twice", d);
+        seen[d] = 1;
+    }
+    if (pos1 == pos0) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    const int blk0 = pos0 / 32, nblk = (pos1 + 31) / 32 - blk0;
+    const int esz = kv.int8 ? 1 : 2;
+    const size_t seg = (size_t)nblk * 32 * kv.D * esz;
+    const size_t need = (size_t)n * 2 * kv.H * seg + (kv.int8 ? (size_t)n * 2 * kv.H * nblk * 32 * sizeof(float) : 0);
+    unsigned char *stage = nullptr;
+    int *rows = nullptr;
+    XFT_CHECK_HIP(hipMalloc((void **)&stage, need));
+    if (hipMalloc((void **)&rows, (size_t)2 * n * 4) != hipSuccess) {
+        (void)hipFree(stage);
+        XFT_REQUIRE(false, "xfthip_kvcache_reorder: out of device memory");
+    }
+    bool ok = hipMemcpy(rows, src_rows_host, (size_t)n * 4, hipMemcpyHostToDevice) == hipSuccess
+            && hipMemcpy(rows + n, dst_rows_host, (size_t)n * 4, hipMemcpyHostToDevice) == hipSuccess;
+    if (ok) {
+        float *stage_scales = (float *)(stage + (size_t)n * 2 * kv.H * seg);
+        const dim3 grid((unsigned)((seg / 16 + 255) / 256), kv.H, 2 * n), sgrid((nblk * 32 + 255) / 256, kv.H, 2 * n);
+        hipLaunchKernelGGL(kv_rows_move_kernel<true>, grid, dim3(256), 0, st, kv, rows, blk0, nblk, stage);
+        if (kv.int8) hipLaunchKernelGGL(kv_scales_move_kernel<true>, sgrid, dim3(256), 0, st, kv, rows, blk0, nblk, stage_scales);
+        hipLaunchKernelGGL(kv_rows_move_kernel<false>, grid, dim3(256), 0, st, kv, rows + n, blk0, nblk, stage);
+        if (kv.int8) hipLaunchKernelGGL(kv_scales_move_kernel<false>, sgrid, dim3(256), 0, st, kv, rows + n, blk0, nblk, stage_scales);
+        ok = hipGetLastError() == hipSuccess && hipStreamSynchronize(st) == hipSuccess;
+    }
+    (void)hipFree(stage);
+    (void)hipFree(rows);
+    XFT_REQUIRE(ok, "xfthip_kvcache_reorder: device error");
+    return 0;
+}
+
 int xfthip_model_seq_reorder(xfthip_model_t m, const int *dst_rows_host, const int *src_rows_host, int n, int pos0, int pos1,
         xfthip_stream_t stream) {
     XFT_REQUIRE(m && dst_rows_host && src_rows_host && n > 0, "xfthip_model_seq_reorder: bad argument");

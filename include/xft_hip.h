@@ -339,6 +339,12 @@ int xfthip_model_set_layer(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthi
 int xfthip_model_set_attention(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthip_weight_t o, const float *ln1_host,
         const float *qkv_bias_host, const float *o_bias_host);
 int xfthip_model_set_mlp(xfthip_model_t m, int idx, xfthip_weight_t gateup, xfthip_weight_t down, const float *ln2_host);
+/* A second weight set for layer idx that only the prompt pass (xfthip_model_prefill / _seq_prefill) uses; the
+ * decode steps keep the layer's own set.  The reference's HybridModel (src/models/hybrid_model.h:25-84: one
+ * model per weight type sharing context and KV cache, behind the "bf16_int8"-style type names).  Shapes as in
+ * xfthip_model_set_layer, which must have been called for the layer; four NULLs drop the second set. */
+int xfthip_model_set_first_token_weights(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthip_weight_t o, xfthip_weight_t gateup,
+        xfthip_weight_t down);
 /*
  * Embedding table (host fp16 bit patterns [vocab, hidden], the reference keeps it in FP16:
  * src/layers/token_embedding.h:49-52), final RMSNorm weight (host fp32 [hidden]) and the

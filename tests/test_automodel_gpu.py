@@ -333,3 +333,44 @@ def test_beam_search_through_the_model_class(xh, orc, am, tmp_path, kv):
     g = model.generate(ids, max_length=S + 4, eos_token_id=V + 3)
     assert g.shape == (B, S + 4)
     model.free()
+
+
+def _layer_sets(xh, orc, held, kind):
+    sets = []
+    for lay in held["layers"]:
+        sets.append([_device_weight(xh, orc, lay["qkv"], kind)[0], _device_weight(xh, orc, lay["o"], kind)[0],
+                     _device_weight(xh, orc, _cat(lay["gate"], lay["up"]), kind, 0 if kind == xh.W_W8A8 else xh.WF_GATEUP)[0],
+                     _device_weight(xh, orc, lay["down"], kind)[0]])
+    return sets
+
+
+@pytest.mark.parametrize("dtype", ["bf16_int8", "w8a8_int4", "bf16_nf4"])
+def test_first_token_and_next_token_weight_types(xh, orc, am, tmp_path, dtype):
+    """The mixed types (HybridModel, src/models/hybrid_model.h:25-84): the prompt runs on the first type's
+    weights, every later token on the second type's, over one KV cache.  Checked against a model that is
+    switched by hand: built with the first type, prompt run, then its layers replaced by the second type's
+    weights (the cache stays) and decoded; the prompt's logits must be the first type's own."""
+    import make_llama_fixture as fx
+    held = fx.write_model_dir(str(tmp_path / "model"), None, 21)
+    first, nxt = dtype.split("_")
+    B, S, max_len = 2, 9, 20
+    V = held["cfg"]["vocab"]
+    ids = np.random.default_rng(22).integers(0, V, (B, S)).astype(np.int32)
+    model = am.AutoModel.from_pretrained(str(tmp_path / "model"), dtype=dtype)
+    out = model.generate(ids, max_length=max_len, eos_token_id=V + 5)
+    model.input(ids)
+    prompt_logits = model.logits()
+    # by hand
+    hand, _ = _direct(xh, orc, held, first, "fp16", B, max_len, with_oracle=False)
+    tok0, lg0 = hand.prefill(ids, want_logits=True)
+    assert np.array_equal(prompt_logits, lg0)
+    for l, ws in enumerate(_layer_sets(xh, orc, held, KIND[nxt])):
+        hand.set_layer(l, *ws, held["layers"][l]["ln1"], held["layers"][l]["ln2"])
+    rest = hand.decode(max_len - S - 1, B)
+    expect = np.concatenate([ids, tok0.reshape(B, 1), rest.T], 1)
+    assert np.array_equal(out, expect)
+    # and it differs from both pure types somewhere (the test would not notice a silent single-type model otherwise)
+    pure = [am.AutoModel.from_pretrained(str(tmp_path / "model"), dtype=t).generate(ids, max_length=max_len, eos_token_id=V + 5)
+            for t in (first, nxt)]
+    print(f"{dtype}: equal to pure {first}: {np.array_equal(out, pure[0])}, to pure {nxt}: {np.array_equal(out, pure[1])}", flush=True)
+    model.free()

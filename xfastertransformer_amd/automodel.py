@@ -46,9 +46,9 @@ _lib.xft_beam_destroy.restype = None
 _lib.xft_beam_destroy.argtypes = [C.c_void_p]
 
 # the types this build serves out of the reference's list (automodel.py:21-39)
-_DTYPES = ["fp16", "bf16", "int8", "w8a8", "int4", "nf4"]
-_REFERENCE_DTYPES = _DTYPES + ["bf16_fp16", "bf16_int8", "bf16_w8a8", "bf16_int4", "bf16_nf4", "w8a8_int8", "w8a8_int4",
-                               "w8a8_nf4", "fp8_e4m3"]
+_DTYPES = ["fp16", "bf16", "int8", "w8a8", "int4", "nf4", "bf16_fp16", "bf16_int8", "bf16_w8a8", "bf16_int4", "bf16_nf4", "w8a8_int8",
+           "w8a8_int4", "w8a8_nf4"]
+_REFERENCE_DTYPES = _DTYPES + ["fp8_e4m3"]
 _KV_DTYPES = ["fp16", "int8"]
 
 
@@ -126,7 +126,7 @@ class AutoModel:
         if dtype not in _REFERENCE_DTYPES:
             raise Exception(f"{self.__class__.__name__} don't support {dtype}.")
         if dtype not in _DTYPES:
-            raise Exception(f"{self.__class__.__name__} of this build don't support the mixed / fp8 type {dtype}.")
+            raise Exception(f"{self.__class__.__name__} of this build don't support the type {dtype}.")
         if kv_cache_dtype not in _KV_DTYPES:
             raise Exception(f"{self.__class__.__name__} don't support KV cache data type: {kv_cache_dtype}.")
         if not os.path.exists(os.path.join(path, "config.ini")):

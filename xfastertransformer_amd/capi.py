@@ -349,6 +349,12 @@ class Model:
         check(lib.xfthip_model_set_layer(self.h, idx, qkv.h, o.h, gateup.h, down.h, _hp(ln1), _hp(ln2), _hp(qkv_bias),
                                          _hp(o_bias)))
 
+    def set_first_token_weights(self, idx, qkv, o, gateup, down):
+        """A second weight set of layer idx for the prompt pass only (None x 4 drops it)."""
+        ws = [qkv, o, gateup, down]
+        self._keep += [w for w in ws if w is not None]
+        check(lib.xfthip_model_set_first_token_weights(self.h, idx, *[None if w is None else w.h for w in ws]))
+
     def set_head(self, embedding_fp16, final_norm, lm_head):
         self._keep.append(lm_head)
         e = np.ascontiguousarray(embedding_fp16, np.uint16)

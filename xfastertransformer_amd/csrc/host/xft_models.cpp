@@ -427,6 +427,7 @@ struct ModelImpl {
     xft::DataType fileType = xft::DataType::fp32;
     int fileQuant = -1; // weight kind of pre-quantised files or -1
     int wkind = XFTHIP_W_BF16;
+    int firstKind = -1; // weight kind of the prompt pass when it differs (the mixed "first_next" types), else -1
     int kvDtype = XFTHIP_FP16;
     int layers = 0, hidden = 0, inter = 0, heads = 0, kvHeads = 0, headSize = 0, vocab = 0;
     int maxPosEmbed = 0, maxPositions = 0, maxSeqLength = -1, startId = 0, endId = 0;
@@ -434,6 +435,7 @@ struct ModelImpl {
 
     struct Layer {
         xfthip_weight_t qkv = nullptr, o = nullptr, gateup = nullptr, down = nullptr;
+        xfthip_weight_t firstQkv = nullptr, firstO = nullptr, firstGateup = nullptr, firstDown = nullptr;
         std::vector<float> ln1, ln2, qkvBias, oBias;
     };
     std::vector<Layer> L;
@@ -516,7 +518,7 @@ struct ModelImpl {
     ~ModelImpl() {
         if (model) xfthip_model_destroy(model);
         for (auto &l : L)
-            for (xfthip_weight_t w : {l.qkv, l.o, l.gateup, l.down})
+            for (xfthip_weight_t w : {l.qkv, l.o, l.gateup, l.down, l.firstQkv, l.firstO, l.firstGateup, l.firstDown})
                 if (w) xfthip_weight_destroy(w);
         if (lmHead) xfthip_weight_destroy(lmHead);
     }
@@ -540,7 +542,8 @@ struct ModelImpl {
     // Pre-quantised codes go to the device as they are when the requested type is the files' own
     // (MMHelper::convertWeight's INT8->INT8 / UINT4->UINT4 copies, matmul_helper.h:284-315);
     // anything else is dequantised (w = scale * q + zero) and converted like a plain matrix.
-    xfthip_weight_t to_device(HostMatrix &m, int flags) {
+    xfthip_weight_t to_device(HostMatrix &m, int flags, int kind = -1) {
+        const int wkind = kind >= 0 ? kind : this->wkind;
         xfthip_weight_t h = nullptr;
         if (m.qkind >= 0 && m.qkind == wkind) {
             CK(xfthip_weight_create(wkind, m.K, m.N, m.q.data(), m.scale.data(), m.zero.data(), flags, &h));
@@ -570,10 +573,13 @@ struct ModelImpl {
         L.resize(layers);
         for (int l = 0; l < layers; ++l) {
             Layer &y = L[l];
+            const bool mixed = firstKind >= 0 && firstKind != wkind;
             HostMatrix qkv = load_matrix(l, "attention.query_key_value", hidden, qkvCols);
             y.qkv = to_device(qkv, XFTHIP_WF_NONE);
+            if (mixed) y.firstQkv = to_device(qkv, XFTHIP_WF_NONE, firstKind);
             HostMatrix o = load_matrix(l, "attention.dense", qCols, hidden);
             y.o = to_device(o, XFTHIP_WF_NONE);
+            if (mixed) y.firstO = to_device(o, XFTHIP_WF_NONE, firstKind);
             if (file_exists(layer_file(l, fileQuant >= 0 ? "mlp.dense_h_to_4h.qweight.0.bin" : "mlp.dense_h_to_4h.weight.0.bin"))) {
                 printf("The model directory holds a two-matrix MLP (dense_h_to_4h); only gate/up/down MLPs are served.\n");
                 exit(-1);
@@ -584,9 +590,11 @@ struct ModelImpl {
                 HostMatrix gu = hcat({&gate, &up});
                 // the W8A8 path runs gate/up as one plain GEMM followed by silu(gate) * up
                 y.gateup = to_device(gu, wkind == XFTHIP_W_W8A8 ? XFTHIP_WF_NONE : XFTHIP_WF_GATEUP);
+                if (mixed) y.firstGateup = to_device(gu, firstKind == XFTHIP_W_W8A8 ? XFTHIP_WF_NONE : XFTHIP_WF_GATEUP, firstKind);
             }
             HostMatrix down = load_matrix(l, "mlp.down_proj", inter, hidden);
             y.down = to_device(down, XFTHIP_WF_NONE);
+            if (mixed) y.firstDown = to_device(down, XFTHIP_WF_NONE, firstKind);
             y.ln1 = read_floats(layer_file(l, "input_layernorm.weight.bin"), hidden, fileType);
             y.ln2 = read_floats(layer_file(l, "post_attention_layernorm.weight.bin"), hidden, fileType);
             y.qkvBias = read_floats(layer_file(l, "attention.query_key_value.bias.0.bin"), qkvCols, fileType, false);
@@ -636,6 +644,7 @@ struct ModelImpl {
             Layer &y = L[l];
             CK(xfthip_model_set_layer(model, l, y.qkv, y.o, y.gateup, y.down, y.ln1.data(), y.ln2.data(),
                     y.qkvBias.empty() ? nullptr : y.qkvBias.data(), y.oBias.empty() ? nullptr : y.oBias.data()));
+            if (y.firstQkv) CK(xfthip_model_set_first_token_weights(model, l, y.firstQkv, y.firstO, y.firstGateup, y.firstDown));
         }
         CK(xfthip_model_set_head(model, embedding.data(), finalNorm.data(), lmHead));
     }
@@ -1225,7 +1234,9 @@ AutoModel::AutoModel(std::string modelPath, xft::DataType dataType, xft::DataTyp
     setVocabSize((int)ini.get_int(sec, "vocab_size", 0));
 
     const std::string modelKey = sec + "-" + type_name(dataType) + "-" + type_name(KVCacheDataType);
-    int wkind = -1;
+    // one weight type, or FirstTokenDtype_NextTokenDtype (HybridModel, models.cpp:1014-1035 with the
+    // registry keys of src/models/*.cpp)
+    int wkind = -1, firstKind = -1;
     switch (dataType) {
         case xft::DataType::bf16:
         case xft::DataType::fp16:
@@ -1233,7 +1244,15 @@ AutoModel::AutoModel(std::string modelPath, xft::DataType dataType, xft::DataTyp
         case xft::DataType::w8a8:
         case xft::DataType::int4:
         case xft::DataType::nf4: wkind = kind_of(dataType); break;
-        default: break; // the mixed first-token / next-token types are not served
+        case xft::DataType::bf16_fp16: firstKind = kind_of(xft::DataType::bf16), wkind = kind_of(xft::DataType::fp16); break;
+        case xft::DataType::bf16_int8: firstKind = kind_of(xft::DataType::bf16), wkind = kind_of(xft::DataType::int8); break;
+        case xft::DataType::bf16_w8a8: firstKind = kind_of(xft::DataType::bf16), wkind = kind_of(xft::DataType::w8a8); break;
+        case xft::DataType::bf16_int4: firstKind = kind_of(xft::DataType::bf16), wkind = kind_of(xft::DataType::int4); break;
+        case xft::DataType::bf16_nf4: firstKind = kind_of(xft::DataType::bf16), wkind = kind_of(xft::DataType::nf4); break;
+        case xft::DataType::w8a8_int8: firstKind = kind_of(xft::DataType::w8a8), wkind = kind_of(xft::DataType::int8); break;
+        case xft::DataType::w8a8_int4: firstKind = kind_of(xft::DataType::w8a8), wkind = kind_of(xft::DataType::int4); break;
+        case xft::DataType::w8a8_nf4: firstKind = kind_of(xft::DataType::w8a8), wkind = kind_of(xft::DataType::nf4); break;
+        default: break; // fp8_e4m3 and unknown
     }
     const bool kvOk = KVCacheDataType == xft::DataType::fp16 || KVCacheDataType == xft::DataType::int8;
     if (Ini::lower(sec) != "llama" || wkind < 0 || !kvOk) {
@@ -1247,6 +1266,7 @@ AutoModel::AutoModel(std::string modelPath, xft::DataType dataType, xft::DataTyp
     s.path = modelPath;
     s.modelType = sec;
     s.wkind = wkind;
+    s.firstKind = firstKind;
     s.kvDtype = KVCacheDataType == xft::DataType::int8 ? XFTHIP_INT8 : XFTHIP_FP16;
     // the keys and defaults of CommonDecoder's constructor (common_decoder.h:176-212)
     s.heads = (int)ini.get_int(sec, "head_num", 0);

@@ -15,6 +15,7 @@
 //   x   = h * Wdown + x                    fp32
 #include <string.h>
 
+#include <utility>
 #include <vector>
 
 #include "attention_dev.h"
@@ -26,6 +27,9 @@ namespace xfthip {
 
 struct LayerW {
     xfthip_weight_t qkv = nullptr, o = nullptr, gateup = nullptr, down = nullptr;
+    // optional second set used by the prompt pass only (the reference's HybridModel: one weight type for the
+    // first token, another for the following ones, src/models/hybrid_model.h:25-84)
+    xfthip_weight_t first_qkv = nullptr, first_o = nullptr, first_gateup = nullptr, first_down = nullptr;
     float *ln1 = nullptr, *ln2 = nullptr, *qkv_bias = nullptr, *o_bias = nullptr;
 };
 
@@ -206,6 +210,22 @@ struct xfthip_model {
     int mega_pitch = 0;
     unsigned long long *mega_trace = nullptr;
     int mega_trace_cap = 0;
+};
+
+// While one of these lives, the layers that hold first-token weights run with them.
+struct FirstTokenWeights {
+    xfthip_model *m;
+    explicit FirstTokenWeights(xfthip_model *model) : m(model) { swap_all(); }
+    ~FirstTokenWeights() { swap_all(); }
+    FirstTokenWeights(const FirstTokenWeights &) = delete;
+    FirstTokenWeights &operator=(const FirstTokenWeights &) = delete;
+    void swap_all() {
+        for (LayerW &L : m->layers) {
+            if (!L.first_qkv) continue;
+            std::swap(L.qkv, L.first_qkv), std::swap(L.o, L.first_o);
+            std::swap(L.gateup, L.first_gateup), std::swap(L.down, L.first_down);
+        }
+    }
 };
 
 static void mega_invalidate(xfthip_model *m) {
@@ -657,6 +677,31 @@ int xfthip_model_set_layer(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthi
     return xfthip_model_set_mlp(m, idx, gateup, down, ln2_host);
 }
 
+int xfthip_model_set_first_token_weights(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthip_weight_t o, xfthip_weight_t gateup,
+        xfthip_weight_t down) {
+    XFT_REQUIRE(m && idx >= 0 && idx < m->cfg.layers, "xfthip_model_set_first_token_weights: bad model or layer");
+    LayerW &L = m->layers[idx];
+    if (!qkv && !o && !gateup && !down) { // back to one weight set
+        L.first_qkv = L.first_o = L.first_gateup = L.first_down = nullptr;
+        return 0;
+    }
+    XFT_REQUIRE(qkv && o && gateup && down, "xfthip_model_set_first_token_weights: all four weights or none");
+    XFT_REQUIRE(L.qkv && L.o && L.gateup && L.down, "xfthip_model_set_first_token_weights: set the layer's own weights first");
+    const xfthip_model_config &c = m->cfg;
+    const bool gu_w8a8 = gateup->pw.kind == XFTHIP_W_W8A8;
+    XFT_REQUIRE(qkv->pw.K == L.qkv->pw.K && qkv->pw.N == L.qkv->pw.N && o->pw.K == L.o->pw.K && o->pw.N == L.o->pw.N
+                    && gateup->pw.K == c.hidden && gateup->pw.N == 2 * c.intermediate && down->pw.K == c.intermediate && down->pw.N == c.hidden,
+            "xfthip_model_set_first_token_weights: shapes differ from the layer's own weights");
+    XFT_REQUIRE(gu_w8a8 ? !(gateup->pw.flags & XFTHIP_WF_GATEUP) : (gateup->pw.flags & XFTHIP_WF_GATEUP) != 0,
+            "xfthip_model_set_first_token_weights: gate/up weight must be created with XFTHIP_WF_GATEUP (W8A8: without it)");
+    if (int rc = w8a8_reserve(m, qkv->pw, false)) return rc;
+    if (int rc = w8a8_reserve(m, o->pw, false)) return rc;
+    if (int rc = w8a8_reserve(m, gateup->pw, true)) return rc;
+    if (int rc = w8a8_reserve(m, down->pw, false)) return rc;
+    L.first_qkv = qkv, L.first_o = o, L.first_gateup = gateup, L.first_down = down;
+    return 0;
+}
+
 int xfthip_model_set_head(xfthip_model_t m, const uint16_t *embedding_fp16_host, const float *final_norm_host,
         xfthip_weight_t lm_head) {
     XFT_REQUIRE(m && embedding_fp16_host && final_norm_host && lm_head, "xfthip_model_set_head: null argument");
@@ -719,6 +764,7 @@ int xfthip_model_prefill(xfthip_model_t m, const int *ids_host, int B, int S, fl
     XFT_REQUIRE(B > 0 && B <= c.max_batch && S > 0 && B * S <= c.max_tokens && S <= c.max_seq,
             "xfthip_model_prefill: B=%d S=%d exceed the model limits", B, S);
     hipStream_t st = (hipStream_t)stream;
+    FirstTokenWeights first_token(m);
     m->row0 = 0;
     m->ragged = false;
     m->row_pos.assign(c.max_batch, -1);
@@ -850,6 +896,7 @@ int xfthip_model_seq_prefill(xfthip_model_t m, int row, const int *ids_host, int
         m->cur_B = 0;
     }
     m->ragged = true;
+    FirstTokenWeights first_token(m);
     XFT_CHECK_HIP(hipMemcpyAsync(m->prompt_ids, ids_host, (size_t)S * 4, hipMemcpyHostToDevice, st));
     hipLaunchKernelGGL(embed_kernel, dim3(S), dim3(256), 0, st, m->embedding, m->prompt_ids, m->x, c.hidden, c.vocab);
     m->row0 = row;

@@ -540,6 +540,7 @@ int xfthip_argmax(const float *logits, int rows, int cols, int *ids_dev, xfthip_
 }
 
 int xfthip_model_create(const xfthip_model_config *cfg, xfthip_model_t *out) {
+    if (int rc = qgemm_split_reserve()) return rc; // decode steps at more than 32 rows are captured into graphs: no allocation there
     XFT_REQUIRE(cfg && out, "xfthip_model_create: null argument");
     const xfthip_model_config &c = *cfg;
     XFT_REQUIRE(c.layers > 0 && c.hidden > 0 && c.intermediate > 0, "xfthip_model_create: bad sizes");

@@ -60,38 +60,81 @@ __global__ void top2_kernel(const float *__restrict__ logits, int M, int E, int 
     w[2 * t + 1] = e2 / (e1 + e2);
 }
 
-// per-expert token lists in ascending token order: thread e scans all tokens
-__global__ void build_lists_kernel(const int *__restrict__ sel, const float *__restrict__ w, int M, int E,
-        int *__restrict__ counts, int *__restrict__ idx, float *__restrict__ wts) {
-    const int e = threadIdx.x;
-    if (e >= E) return;
+// Per-expert token lists in ascending token order, in one workgroup: wave e collects expert e's tokens 64 at
+// a time (ballot + prefix count), then the lists are laid back to back (expert 0's rows first) and every
+// (token, choice) learns the row of the gathered matrix that holds its copy:
+//   counts[e], offsets[e] (first row of expert e), row_token[g] / row_weight[g] for the 2 M gathered rows,
+//   slot_row[2 t + s] = row of token t's s-th choice.
+// blockDim.x = 64 * E; rank[] is scratch of 2 M ints.
+__global__ __launch_bounds__(512) void build_lists_kernel(const int *__restrict__ sel, const float *__restrict__ w, int M, int E,
+        int *__restrict__ counts, int *__restrict__ offsets, int *__restrict__ row_token, float *__restrict__ row_weight,
+        int *__restrict__ slot_row, int *__restrict__ rank) {
+    __shared__ int s_count[8], s_off[8];
+    const int e = threadIdx.x >> 6, lane = threadIdx.x & 63;
     int n = 0;
-    for (int t = 0; t < M; ++t) {
-        for (int s = 0; s < 2; ++s) {
-            if (sel[2 * t + s] == e) {
-                idx[(size_t)e * M + n] = t;
-                wts[(size_t)e * M + n] = w[2 * t + s];
-                ++n;
-            }
+    for (int t0 = 0; t0 < M; t0 += 64) {
+        const int t = t0 + lane;
+        int slot = -1;
+        if (t < M) slot = sel[2 * t] == e ? 0 : (sel[2 * t + 1] == e ? 1 : -1);
+        const unsigned long long mask = __ballot(slot >= 0);
+        if (slot >= 0) rank[2 * t + slot] = n + __popcll(mask & ((1ull << lane) - 1ull));
+        n += __popcll(mask);
+    }
+    if (lane == 0) s_count[e] = n;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int acc = 0;
+        for (int i = 0; i < E; ++i) {
+            s_off[i] = acc;
+            counts[i] = s_count[i];
+            offsets[i] = acc;
+            acc += s_count[i];
         }
     }
-    counts[e] = n;
+    __syncthreads();
+    for (int i = threadIdx.x; i < 2 * M; i += blockDim.x) {
+        const int t = i >> 1, g = s_off[sel[i]] + rank[i];
+        slot_row[i] = g;
+        row_token[g] = t;
+        row_weight[g] = w[i];
+    }
 }
 
-__global__ void gather_rows_kernel(const uint16_t *__restrict__ xn, int ld, const int *__restrict__ idx, uint16_t *__restrict__ out,
-        int hidden) {
+// gathered[g] = xn[row_token[g]], 16 bytes a thread; grid = rows
+__global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t *__restrict__ xn, int ld, const int *__restrict__ row_token,
+        uint16_t *__restrict__ out, int hidden) {
     const int r = blockIdx.x;
-    const uint16_t *src = xn + (size_t)idx[r] * ld;
-    for (int c = threadIdx.x; c < hidden; c += blockDim.x) out[(size_t)r * hidden + c] = src[c];
+    const uint4 *src = (const uint4 *)(xn + (size_t)row_token[r] * ld);
+    uint4 *dst = (uint4 *)(out + (size_t)r * hidden);
+    for (int c = threadIdx.x; c < hidden / 8; c += blockDim.x) dst[c] = src[c];
 }
 
-// out[idx[r]] += expert_out[r] * w[r]   (xft::addto: one fused multiply-add per element)
-__global__ void scatter_add_kernel(float *__restrict__ out, int ld, const float *__restrict__ eo, const int *__restrict__ idx,
-        const float *__restrict__ wts, int hidden) {
-    const int r = blockIdx.x;
-    float *dst = out + (size_t)idx[r] * ld;
-    const float wv = wts[r];
-    for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = fmaf(eo[(size_t)r * hidden + c], wv, dst[c]);
+// out[t] += eo[row of choice] * weight, the lower expert index first: the order in which the reference's
+// loop over the experts adds a token's two contributions (xft::addto: one fused multiply-add per element).
+// grid = tokens
+__global__ __launch_bounds__(256) void combine_kernel(float *__restrict__ out, int ld, const float *__restrict__ eo, const int *__restrict__ sel,
+        const int *__restrict__ slot_row, const float *__restrict__ w, int hidden, int wide) {
+    const int t = blockIdx.x;
+    const int first = sel[2 * t] < sel[2 * t + 1] ? 0 : 1;
+    const int ga = slot_row[2 * t + first], gb = slot_row[2 * t + 1 - first];
+    const float wa = w[2 * t + first], wb = w[2 * t + 1 - first];
+    if (wide) { // rows of out start on 16-byte boundaries
+        const float4 *ea = (const float4 *)(eo + (size_t)ga * hidden), *eb = (const float4 *)(eo + (size_t)gb * hidden);
+        float4 *dst = (float4 *)(out + (size_t)t * ld);
+        for (int c = threadIdx.x; c < hidden / 4; c += blockDim.x) {
+            float4 o = dst[c];
+            const float4 a = ea[c], b = eb[c];
+            o.x = fmaf(b.x, wb, fmaf(a.x, wa, o.x));
+            o.y = fmaf(b.y, wb, fmaf(a.y, wa, o.y));
+            o.z = fmaf(b.z, wb, fmaf(a.z, wa, o.z));
+            o.w = fmaf(b.w, wb, fmaf(a.w, wa, o.w));
+            dst[c] = o;
+        }
+    } else {
+        const float *ea = eo + (size_t)ga * hidden, *eb = eo + (size_t)gb * hidden;
+        float *dst = out + (size_t)t * ld;
+        for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = fmaf(eb[c], wb, fmaf(ea[c], wa, dst[c]));
+    }
 }
 
 __global__ void copy_rows_kernel(const float *__restrict__ in, int in_ld, float *__restrict__ out, int out_ld, int hidden) {
@@ -114,8 +157,8 @@ struct xfthip_moe {
     float *router = nullptr, *ln = nullptr;
     std::vector<xfthip_weight_t> gateup, down;
     uint16_t *xn = nullptr, *xg = nullptr, *h = nullptr;
-    float *eo = nullptr, *logits = nullptr, *w = nullptr, *wts = nullptr;
-    int *sel = nullptr, *counts = nullptr, *idx = nullptr;
+    float *eo = nullptr, *logits = nullptr, *w = nullptr, *row_weight = nullptr;
+    int *sel = nullptr, *counts = nullptr, *row_token = nullptr, *slot_row = nullptr, *rank = nullptr; // counts: [E] counts, [E] offsets
 };
 
 extern "C" {
@@ -140,12 +183,14 @@ int xfthip_moe_create(int hidden, int intermediate, int experts, int max_tokens,
     m->gateup.assign(experts, nullptr);
     m->down.assign(experts, nullptr);
     const size_t T = max_tokens;
+    // every token is gathered twice (its two experts): 2 T rows of activations and of expert outputs
     bool ok = hipMalloc((void **)&m->router, (size_t)hidden * experts * 4) == hipSuccess
-            && hipMalloc((void **)&m->xn, T * hidden * 2) == hipSuccess && hipMalloc((void **)&m->xg, T * hidden * 2) == hipSuccess
-            && hipMalloc((void **)&m->h, T * intermediate * 2) == hipSuccess && hipMalloc((void **)&m->eo, T * hidden * 4) == hipSuccess
+            && hipMalloc((void **)&m->xn, T * hidden * 2) == hipSuccess && hipMalloc((void **)&m->xg, 2 * T * hidden * 2) == hipSuccess
+            && hipMalloc((void **)&m->h, T * intermediate * 2) == hipSuccess && hipMalloc((void **)&m->eo, 2 * T * hidden * 4) == hipSuccess
             && hipMalloc((void **)&m->logits, T * experts * 4) == hipSuccess && hipMalloc((void **)&m->w, T * 2 * 4) == hipSuccess
-            && hipMalloc((void **)&m->sel, T * 2 * 4) == hipSuccess && hipMalloc((void **)&m->counts, 64) == hipSuccess
-            && hipMalloc((void **)&m->idx, T * experts * 4) == hipSuccess && hipMalloc((void **)&m->wts, T * experts * 4) == hipSuccess;
+            && hipMalloc((void **)&m->sel, T * 2 * 4) == hipSuccess && hipMalloc((void **)&m->counts, 2 * 64) == hipSuccess
+            && hipMalloc((void **)&m->row_token, 2 * T * 4) == hipSuccess && hipMalloc((void **)&m->row_weight, 2 * T * 4) == hipSuccess
+            && hipMalloc((void **)&m->slot_row, 2 * T * 4) == hipSuccess && hipMalloc((void **)&m->rank, 2 * T * 4) == hipSuccess;
     if (ok && ln_host) ok = hipMalloc((void **)&m->ln, (size_t)hidden * 4) == hipSuccess
             && hipMemcpy(m->ln, ln_host, (size_t)hidden * 4, hipMemcpyHostToDevice) == hipSuccess;
     if (ok) ok = hipMemcpy(m->router, router_host, (size_t)hidden * experts * 4, hipMemcpyHostToDevice) == hipSuccess;
@@ -160,7 +205,7 @@ int xfthip_moe_create(int hidden, int intermediate, int experts, int max_tokens,
 
 int xfthip_moe_destroy(xfthip_moe_t m) {
     if (!m) return 0;
-    void *bufs[] = {m->router, m->ln, m->xn, m->xg, m->h, m->eo, m->logits, m->w, m->wts, m->sel, m->counts, m->idx};
+    void *bufs[] = {m->router, m->ln, m->xn, m->xg, m->h, m->eo, m->logits, m->w, m->row_weight, m->sel, m->counts, m->row_token, m->slot_row, m->rank};
     for (void *b : bufs)
         if (b) (void)hipFree(b);
     delete m;
@@ -200,24 +245,28 @@ int xfthip_moe_forward(xfthip_moe_t m, const float *x_in, int in_stride, float *
         logits = m->logits;
     }
     if (int rc = xfthip_moe_top2(logits, T, m->E, m->sel, m->w, st)) return rc;
-    hipLaunchKernelGGL(build_lists_kernel, dim3(1), dim3(64), 0, st, m->sel, m->w, T, m->E, m->counts, m->idx, m->wts);
+    hipLaunchKernelGGL(build_lists_kernel, dim3(1), dim3(64 * m->E), 0, st, m->sel, m->w, T, m->E, m->counts, m->counts + m->E, m->row_token,
+            m->row_weight, m->slot_row, m->rank);
+    hipLaunchKernelGGL(gather_rows_kernel, dim3(2 * T), dim3(256), 0, st, m->xn, H, m->row_token, m->xg, H);
     XFT_CHECK_HIP(hipGetLastError());
     int counts[64];
     XFT_CHECK_HIP(hipMemcpyAsync(counts, m->counts, m->E * sizeof(int), hipMemcpyDeviceToHost, st));
     XFT_CHECK_HIP(hipStreamSynchronize(st)); // the per-expert row counts size the GEMMs below
     if (sel_host_out) XFT_CHECK_HIP(hipMemcpy(sel_host_out, m->sel, (size_t)T * 2 * 4, hipMemcpyDeviceToHost));
     if (w_host_out) XFT_CHECK_HIP(hipMemcpy(w_host_out, m->w, (size_t)T * 2 * 4, hipMemcpyDeviceToHost));
+    int off = 0;
     for (int e = 0; e < m->E; ++e) {
         const int n = counts[e];
         if (n == 0) continue;
-        const int *idx = m->idx + (size_t)e * T;
-        hipLaunchKernelGGL(gather_rows_kernel, dim3(n), dim3(256), 0, st, m->xn, H, idx, m->xg, H);
-        if (int rc = xfthip_gemm_gateup_silu(m->gateup[e], n, m->xg, H, m->h, m->inter, XFTHIP_BF16, st)) return rc;
-        if (int rc = xfthip_gemm(m->down[e], n, m->h, m->inter, m->eo, H, XFTHIP_F32, XFTHIP_EPI_NONE, nullptr, nullptr, 0, XFTHIP_F32,
-                    1.0f, st))
+        // expert e owns rows [off, off + n) of the gathered activations and of the expert outputs
+        if (int rc = xfthip_gemm_gateup_silu(m->gateup[e], n, m->xg + (size_t)off * H, H, m->h, m->inter, XFTHIP_BF16, st)) return rc;
+        if (int rc = xfthip_gemm(m->down[e], n, m->h, m->inter, m->eo + (size_t)off * H, H, XFTHIP_F32, XFTHIP_EPI_NONE, nullptr, nullptr, 0,
+                    XFTHIP_F32, 1.0f, st))
             return rc;
-        hipLaunchKernelGGL(scatter_add_kernel, dim3(n), dim3(256), 0, st, x_out, out_stride, m->eo, idx, m->wts + (size_t)e * T, H);
+        off += n;
     }
+    const int wide = (((size_t)x_out | ((size_t)out_stride * 4)) & 15) == 0;
+    hipLaunchKernelGGL(combine_kernel, dim3(T), dim3(256), 0, st, x_out, out_stride, m->eo, m->sel, m->slot_row, m->w, H, wide);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }

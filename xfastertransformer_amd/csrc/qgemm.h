@@ -21,6 +21,11 @@ struct SkinnyParams {
     float gamma;
     int gateup; // 1: combine tile pairs as silu(gate)*up, N counts cat columns
     int nblocks; // column blocks of the launch (set by the launcher)
+    // K split of the M > 32 kernel (few rows against few columns and a deep K): workgroup row blockIdx.y
+    // multiplies k tiles [y * split_ktiles, (y + 1) * split_ktiles) and writes its scaled partial result as
+    // fp32 [M][N] into split_part + y * M * N; a second kernel adds the parts in order and applies the epilogue
+    int ksplit, split_ktiles;
+    float *split_part;
 
     // ---- fusions of the decode step (M <= 4, skinny kernel only) ----
     // RMSNorm prologue: when norm_x is set, A is ignored and every workgroup normalises the M rows
@@ -45,6 +50,7 @@ struct SkinnyParams {
 int qgemm_skinny(const PackedWeight &pw, const SkinnyParams &p, hipStream_t stream); // M <= 32
 bool skinny_can_fuse_norm(const PackedWeight &pw, int M); // may SkinnyParams::norm_x be used
 int qgemm_mfma(const PackedWeight &pw, const SkinnyParams &p, hipStream_t stream); // any M, built for M > 32
+int qgemm_split_reserve(); // allocates the K-split workspace of qgemm_mfma now (before a stream capture, say)
 
 int gemm_w8a8_from_bf16(xfthip_weight_t w, int M, const void *A, int lda, void *C, int ldc, int c_dtype, int epilogue,
         const float *bias, const void *res, int ldres, int res_dtype, float gamma, hipStream_t stream);

@@ -89,6 +89,18 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = lane >> 5, nl = lane & 31;
+    if (p.ksplit > 1) {
+        // this row of workgroups owns a range of k tiles: shift the operands to it, the result goes to its part
+        const int kt0 = blockIdx.y * p.split_ktiles;
+        const int k_left = p.K - kt0 * KTILE, k_span = p.split_ktiles * KTILE;
+        p.packed += (size_t)kt0 * 1024;
+        p.A += (size_t)kt0 * KTILE;
+        p.K = k_left < k_span ? k_left : k_span;
+        p.C = p.split_part + (size_t)blockIdx.y * p.M * p.N;
+        p.ldc = p.N;
+        p.c_dtype = XFTHIP_F32;
+        p.epi = XFTHIP_EPI_NONE;
+    }
 
     // block -> (column block, row block): blocks that share a column block sit on the same XCD
     // (block ids round-robin over the 8 XCDs), so their weight reads hit that XCD's L2.  Row blocks are
@@ -563,8 +575,8 @@ static int launch_big2(const SkinnyParams &p, hipStream_t stream) {
                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         XFT_CHECK_HIP(attr);
     }
-    hipLaunchKernelGGL((qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL>), dim3(blocks), dim3(256), smem, stream, p, nblocks_n,
-            nblocks_m);
+    hipLaunchKernelGGL((qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL>), dim3(blocks, p.ksplit > 1 ? p.ksplit : 1), dim3(256), smem, stream,
+            p, nblocks_n, nblocks_m);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }

@@ -19,6 +19,7 @@
 // gemm_kernel_ext2.cpp:75-91).
 #include <mutex>
 
+
 #include "attention_dev.h"
 
 namespace xfthip {
@@ -31,7 +32,7 @@ __global__ __launch_bounds__(256) void attn_kernel(AttnParams p) {
 
 // prefill form: 4 waves = 4 neighbouring groups of 16 CT columns of one (sequence, KV head)
 template <bool INT8, int CT>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnParams p) {
     // the column groups that see the longest history are dispatched first (the causal triangle's long rows
     // would otherwise start last and finish alone)
     attn_prefill_unit<INT8, CT>(p, blockIdx.y, (gridDim.x - 1 - blockIdx.x) * 4 + (threadIdx.x >> 6), blockIdx.z);
@@ -39,7 +40,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnParams p) {
 
 // FP16 cache, K / V blocks shared through LDS: a workgroup = 64 CT neighbouring columns of one (sequence, KV head)
 template <int CT>
-__global__ __launch_bounds__(256) void attn_prefill_lds_kernel(AttnParams p) {
+// launch bounds: three workgroups a CU with one column tile a wave (140 registers), two with two (216)
+__global__ __launch_bounds__(256, (CT == 1 ? 3 : 2)) void attn_prefill_lds_kernel(AttnParams p) {
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kPfBufBytes];
     attn_prefill_lds_unit<CT>(p, blockIdx.y, gridDim.x - 1 - blockIdx.x, blockIdx.z, lds); // longest history first
 }
@@ -136,30 +138,23 @@ int xfthip::attention_launch(xfthip_kvcache_t c, const void *q, int qStride, voi
     p.past = past;
     p.past_dev = past_dev;
     p.CG = (S * p.G + 15) / 16;
-    // Many columns per KV head (prefill, long chunks): the form in which a wave keeps a K / V block for 16 or
-    // 32 columns and walks the whole visible sequence, taken once it fills the device by itself.
+    // Many columns per KV head (prefill, long chunks): the forms in which a wave walks the whole visible
+    // sequence for its 16 (or 32) columns, taken once they fill the device by themselves.  Occupancy decides
+    // here: with one column tile a wave the FP16 form runs three workgroups a CU, with two tiles two; measured
+    // (4 x 2048 and 8 x 1024 GQA, 1 x 512 / 1 x 2048 / 32 x 512 MHA) one tile wins or ties except for long
+    // sequences of a model without grouped heads, where a workgroup's 64 columns are 64 tokens.
     {
         const long waves1 = (long)B * c->kv.H * p.CG; // waves with one column tile each
         if (S > 1 && waves1 >= 4L * device_cu_count()) {
-            const int ct = waves1 >= 16L * device_cu_count() ? 2 : 1;
             p.nsplit = 1;
             if (!c->kv.int8) {
-                // 4 column tiles a wave once that still leaves two workgroups for every CU
-                const int ctl = waves1 >= 32L * device_cu_count() ? 4 : ct;
+                const int ctl = (p.G == 1 && waves1 >= 16L * device_cu_count()) ? 2 : 1;
                 dim3 grid((p.CG + 4 * ctl - 1) / (4 * ctl), c->kv.H, B);
-                if (ctl == 4) hipLaunchKernelGGL(attn_prefill_lds_kernel<4>, grid, dim3(256), 0, stream, p);
-                else if (ctl == 2) hipLaunchKernelGGL(attn_prefill_lds_kernel<2>, grid, dim3(256), 0, stream, p);
+                if (ctl == 2) hipLaunchKernelGGL(attn_prefill_lds_kernel<2>, grid, dim3(256), 0, stream, p);
                 else hipLaunchKernelGGL(attn_prefill_lds_kernel<1>, grid, dim3(256), 0, stream, p);
-                XFT_CHECK_HIP(hipGetLastError());
-                return 0;
-            }
-            dim3 grid((p.CG + 4 * ct - 1) / (4 * ct), c->kv.H, B);
-            if (c->kv.int8) {
-                if (ct == 2) hipLaunchKernelGGL((attn_prefill_kernel<true, 2>), grid, dim3(256), 0, stream, p);
-                else hipLaunchKernelGGL((attn_prefill_kernel<true, 1>), grid, dim3(256), 0, stream, p);
             } else {
-                if (ct == 2) hipLaunchKernelGGL((attn_prefill_kernel<false, 2>), grid, dim3(256), 0, stream, p);
-                else hipLaunchKernelGGL((attn_prefill_kernel<false, 1>), grid, dim3(256), 0, stream, p);
+                dim3 grid((p.CG + 3) / 4, c->kv.H, B);
+                hipLaunchKernelGGL((attn_prefill_kernel<true, 1>), grid, dim3(256), 0, stream, p);
             }
             XFT_CHECK_HIP(hipGetLastError());
             return 0;

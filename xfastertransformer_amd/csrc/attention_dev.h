@@ -739,17 +739,29 @@ __device__ inline void attn_prefill_lds_unit(const AttnParams &p, const int kvh,
         for (int a = 0; a < 2; ++a)
 #pragma unroll
             for (int s = 0; s < 4; ++s) kf[a][s].q = *(const u32x4 *)(kb + (16 * a + cl) * kPfKPitch + (8 * g + 32 * s) * 2);
+        // all score tiles first, k step by k step over the 2 CT independent accumulators: no MFMA waits for the
+        // one before it, and the scores of the later column tiles are ready while the earlier ones go through
+        // the softmax arithmetic (their P.V products then run behind that arithmetic instead of in front of it)
+        f32x4 sc_all[CT][2];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+            for (int a = 0; a < 2; ++a) sc_all[ct][a] = f32x4 {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                for (int a = 0; a < 2; ++a)
+                    sc_all[ct][a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[a][s].v, qf[ct][s].v, sc_all[ct][a], 0, 0, 0);
+        // the value operands are read only now (the fence keeps the compiler from hoisting the reads): they reuse
+        // the registers of the key operands, and their LDS latency passes behind the softmax arithmetic
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int dt = 0; dt < 8; ++dt) vf[dt].q = *(const u32x4 *)(vb + (16 * dt + cl) * kPfVPitch + 8 * g * 2);
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
-            f32x4 sc[2];
-#pragma unroll
-            for (int a = 0; a < 2; ++a) {
-                sc[a] = f32x4 {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int s = 0; s < 4; ++s) sc[a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[a][s].v, qf[ct][s].v, sc[a], 0, 0, 0);
-            }
+            f32x4 sc[2] = {sc_all[ct][0], sc_all[ct][1]};
             float bmax = kNegBig;
             const bool masked = t0 + 32 > lim_min[ct]; // wave-uniform
 #pragma unroll

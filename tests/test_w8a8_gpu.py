@@ -119,9 +119,9 @@ def test_w8a8_model_shape_rows_2048(xh, orc):
     assert np.array_equal(got[rows].view(np.uint32), exp.view(np.uint32))
 
 
-def test_w8a8_256_row_blocks_bit_exact(xh, orc):
-    """Enough 256 x 256 blocks to fill the chip twice: eight waves a workgroup, two stacked over the rows.  Ragged M
-    and N, sampled rows against the oracle (rows are independent), plain and residual epilogues, bf16 output."""
+def test_w8a8_many_tiles_bit_exact(xh, orc):
+    """Enough 128 x 128 tiles for three workgroups on every CU (the tile taken then).  Ragged M and N, sampled rows
+    against the oracle (rows are independent), plain and residual epilogues, bf16 output."""
     M, K, N = 3000, 512, 11024
     rng = np.random.default_rng(77)
     w = orc.quantize(orc.W_W8A8, (rng.standard_normal((K, N)) * 0.02).astype(np.float32))

@@ -303,7 +303,8 @@ __device__ inline float w8a8_epilogue(int epi, float x, float bias, bool has_bia
 }
 
 // A workgroup is 4 x WR waves: four side by side over 4 * WN * 32 columns, WR on top of each other over
-// WR * WM * 32 rows; a wave owns WN x WM accumulator tiles of 32 x 32.
+// WR * WM * 32 rows; a wave owns WN x WM accumulator tiles of 32 x 32.  (WR = 2, eight waves on 256 x 256, was
+// measured and is no better than 128 x 128 tiles at three workgroups a CU: every dispatch uses WR = 1.)
 template <int WN, int WM, int WR>
 __global__ __launch_bounds__(256 * WR) void w8a8_mfma_kernel(W8A8Params p, int nblocks_n, int nblocks_m) {
     constexpr int ROWS = 32 * WM, BROWS = ROWS * WR, ROWB = 64 + 16; // rows of a wave / of the block, padded LDS row pitch in bytes
@@ -366,7 +367,7 @@ __global__ __launch_bounds__(256 * WR) void w8a8_mfma_kernel(W8A8Params p, int n
     // read issued in front of it and every global load is four to six steps old when it is needed.  The tile
     // count is rounded up to whole rounds of six steps; tiles past the last one are all zero on the activation
     // side (their weight loads re-read the last tile).
-    constexpr int SLOTS = WR == 1 ? 6 : 3, TILEB = BROWS * ROWB; // two waves a SIMD share its registers: fewer tiles in flight
+    constexpr int SLOTS = (WR == 1 && WN == 2) ? 6 : 3, TILEB = BROWS * ROWB; // several waves a SIMD share its registers: fewer tiles in flight each
     i32x4 wreg[SLOTS][2][WN], areg[SLOTS][ALOADS];
     bool aval[SLOTS];
     const int kt_n = (p.K + 63) / 64;
@@ -644,9 +645,12 @@ int xfthip_gemm_w8a8(xfthip_weight_t w, int M, const int8_t *qa, int ldq, const 
         p.C = C, p.ldc = ldc, p.c_dtype = c_dtype, p.epi = epilogue, p.bias = bias;
         p.res = res, p.ldres = ldres, p.res_dtype = res_dtype, p.gamma = gamma;
         const int n32 = (pw.NTILES + 1) / 2;
+        // 128 x 128 tiles once they give every CU its three resident workgroups (registers allow three), else
+        // 128 x 256 with one (measured at 2048 / 8192 rows: 64 / 165 / 148 us and 225 / 554 / 510 us on
+        // 4096x4096 / 11008x4096 / 4096x11008; eight-wave 256 x 256 blocks were no better anywhere)
         const long t_large = (long)((n32 + 7) / 8) * ((M + 127) / 128);
-        const long t_huge = (long)((n32 + 7) / 8) * ((M + 255) / 256);
-        if (t_huge >= 2 * cus) return launch_w8a8_mfma<2, 4, 2>(p, (hipStream_t)stream);
+        const long t_mid = (long)((n32 + 3) / 4) * ((M + 127) / 128);
+        if (t_mid >= 3 * cus) return launch_w8a8_mfma<1, 4, 1>(p, (hipStream_t)stream);
         if (t_large >= cus) return launch_w8a8_mfma<2, 4, 1>(p, (hipStream_t)stream);
         return launch_w8a8_mfma<1, 2, 1>(p, (hipStream_t)stream);
     }

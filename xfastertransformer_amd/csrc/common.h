@@ -81,6 +81,14 @@ __host__ __device__ inline int logical_col(int np, int inter) {
     return (r >= 16) ? j + inter : j;
 }
 
+// NormalFloat4 code values (QLoRA, Dettmers et al. 2023, appendix E): the one copy the device tables of the
+// pack / unpack kernels and of both GEMM kernels are initialised from
+#define XFTHIP_NF4_CODE_VALUES                                                                              \
+    {-1.0f, -0.6961928009986877f, -0.5250730514526367f, -0.39491748809814453f, -0.28444138169288635f,       \
+            -0.18477343022823334f, -0.09105003625154495f, 0.0f, 0.07958029955625534f, 0.16093020141124725f, \
+            0.24611230194568634f, 0.33791524171829224f, 0.44070982933044434f, 0.5626170039176941f,          \
+            0.7229568362236023f, 1.0f}
+
 // ---- numeric helpers -----------------------------------------------------------------
 __device__ inline uint32_t f2u(float f) { return __float_as_uint(f); }
 __device__ inline float u2f(uint32_t u) { return __uint_as_float(u); }

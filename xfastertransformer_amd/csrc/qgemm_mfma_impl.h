@@ -36,10 +36,7 @@ __device__ inline uint32_t pack_hi16_m(float lo, float hi) {
     return __builtin_amdgcn_perm(f2u(hi), f2u(lo), 0x07060302u);
 }
 
-__constant__ float c_nf4_big[16] = {-1.0f, -0.6961928009986877f, -0.5250730514526367f, -0.39491748809814453f,
-        -0.28444138169288635f, -0.18477343022823334f, -0.09105003625154495f, 0.0f, 0.07958029955625534f,
-        0.16093020141124725f, 0.24611230194568634f, 0.33791524171829224f, 0.44070982933044434f,
-        0.5626170039176941f, 0.7229568362236023f, 1.0f};
+__constant__ float c_nf4_big[16] = XFTHIP_NF4_CODE_VALUES;
 
 __device__ inline float silu_big(float x) {
     return x / (1.0f + fast_exp(-x));

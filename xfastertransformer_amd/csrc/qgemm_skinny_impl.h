@@ -102,10 +102,7 @@ __device__ inline float silu_f(float x) {
 }
 
 // NF4 code values (QLoRA appendix E), split into bf16 hi + lo parts for the MFMA
-__constant__ float c_nf4_gemm[16] = {-1.0f, -0.6961928009986877f, -0.5250730514526367f, -0.39491748809814453f,
-        -0.28444138169288635f, -0.18477343022823334f, -0.09105003625154495f, 0.0f, 0.07958029955625534f,
-        0.16093020141124725f, 0.24611230194568634f, 0.33791524171829224f, 0.44070982933044434f,
-        0.5626170039176941f, 0.7229568362236023f, 1.0f};
+__constant__ float c_nf4_gemm[16] = XFTHIP_NF4_CODE_VALUES;
 
 // KIND: weight kind; NT: column tiles per wave; MT: 16-row activation tiles (1 or 2);
 // U: k tiles per load batch (the packed K extent is padded to whole batches);

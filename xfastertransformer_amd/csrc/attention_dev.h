@@ -321,13 +321,26 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
     float *s_linv = s_f + 64 * 16;
     float *s_pm = s_linv + 16, *s_pl = s_pm + 64 * 16; // [nsplit][16] partial maxima and sums
     // one load per thread (independent round trips), then the per-column arithmetic from LDS
-    for (int v = threadIdx.x; v < p.nsplit * 32; v += 64 * NW) {
-        const int s = v >> 5, e = v & 31;
-        const float x = ws_ld(&base[(size_t)s * kSlotFloats + e]);
-        if (e < 16)
-            s_pm[s * 16 + e] = x;
-        else
-            s_pl[s * 16 + e - 16] = x;
+    // (up to 8 a thread at 64 splits: all sent before the first is used)
+    {
+        constexpr int PER = 64 * 32 / (64 * NW) > 0 ? 64 * 32 / (64 * NW) : 1;
+        float x[PER];
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int v = threadIdx.x + i * 64 * NW;
+            x[i] = v < p.nsplit * 32 ? ws_ld(&base[(size_t)(v >> 5) * kSlotFloats + (v & 31)]) : 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int v = threadIdx.x + i * 64 * NW;
+            if (v < p.nsplit * 32) {
+                const int s = v >> 5, e = v & 31;
+                if (e < 16)
+                    s_pm[s * 16 + e] = x[i];
+                else
+                    s_pl[s * 16 + e - 16] = x[i];
+            }
+        }
     }
     wg_sync();
     if (threadIdx.x < 16) {
@@ -348,12 +361,13 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
         const int cc = cg * 16 + col;
         if (cc >= ncols) continue;
         float acc = 0.0f;
-        for (int s0 = 0; s0 < p.nsplit; s0 += 4) {
-            float t[4];
+        // 32 partials in flight a thread (4 made the merge of 64 splits a chain of 16 round trips per output)
+        for (int s0 = 0; s0 < p.nsplit; s0 += 32) {
+            float t[32];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) t[u] = s0 + u < p.nsplit ? ws_ld(&base[(size_t)(s0 + u) * kSlotFloats + 32 + col * D + d]) : 0.0f;
+            for (int u = 0; u < 32; ++u) t[u] = s0 + u < p.nsplit ? ws_ld(&base[(size_t)(s0 + u) * kSlotFloats + 32 + col * D + d]) : 0.0f;
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
+            for (int u = 0; u < 32; ++u)
                 if (s0 + u < p.nsplit) acc = fmaf(t[u], s_f[(s0 + u) * 16 + col], acc);
         }
         const int s_tok = cc / p.G, j = cc % p.G;

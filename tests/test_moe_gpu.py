@@ -123,3 +123,50 @@ def test_mixtral_shape_full_size_spot_check(xh, orc):
             ref = ref + ew[t, s] * orc.qgemm(dn, h)
         assert np.abs(got[t] - ref[0]).max() < 2e-2 * max(1.0, np.abs(ref).max()), t
         assert _cos(got[t], ref[0]) >= 0.9999
+
+
+def test_layer_without_routing_output_is_capturable(xh, orc):
+    """Asked for no routing output, the layer never waits for the device (the per-expert row counts stay in
+    device memory), so it can be recorded into a graph: every replay, on fresh inputs and with eager work
+    between the replays, must give the eager call's result bit for bit."""
+    hidden, inter, E, tokens = 1024, 3584, 8, 96
+    rng = np.random.default_rng(11)
+    experts = _experts(orc, rng, 0, hidden, inter, E)
+    router = (rng.standard_normal((hidden, E)) * 0.05).astype(np.float32)
+    ln = rng.uniform(0.8, 1.2, hidden).astype(np.float32)
+    moe = xh.MoE(hidden, inter, E, tokens, router, ln)
+    for e, (gu, dn) in enumerate(experts):
+        moe.set_expert(e, xh.Weight(0, gu.K, gu.N, gu.q, gu.scale, gu.zero, flags=xh.WF_GATEUP),
+                       xh.Weight(0, dn.K, dn.N, dn.q, dn.scale, dn.zero))
+    xs = [orc.round_bf16(rng.standard_normal((tokens, hidden))) for _ in range(3)]
+    los = [rng.standard_normal((tokens, E)).astype(np.float32) for _ in range(3)]
+    # the third input sends every token to experts 0 and 1 only: six experts get no rows at all
+    los[2][:, 0], los[2][:, 1], los[2][:, 2:] = 9.0, 8.0, -5.0
+    xd, lod = xh.DeviceBuffer.from_numpy(xs[0]), xh.DeviceBuffer.from_numpy(los[0])
+    od = xh.DeviceBuffer(xs[0].nbytes)
+    eager = []
+    for x, lo in zip(xs, los):
+        xd.upload(x)
+        lod.upload(lo)
+        od.zero()
+        sel, w = moe.forward(xd.ptr, od.ptr, tokens, True, lod.ptr)
+        xh.synchronize()
+        eager.append(od.to_numpy(np.float32, x.shape).copy())
+        exp, esel, _ = orc.mixtral_mlp(x, ln, router, experts, lo, rounding="bf16")
+        assert np.array_equal(sel, esel) and np.abs(eager[-1] - exp).max() < 2e-2
+    assert set(np.unique(orc.moe_top2(los[2])[0])) == {0, 1}
+    side = xh.Stream()
+    xh.synchronize()
+    with xh.Graph(side) as graph:
+        got = moe.forward(xd.ptr, od.ptr, tokens, True, lod.ptr, stream=side.h, want_routing=False)
+    assert got == (None, None)
+    for i in (2, 0, 1, 2):
+        xd.upload(xs[i])
+        lod.upload(los[i])
+        od.zero()
+        xh.synchronize()
+        graph.launch()
+        side.synchronize()
+        assert np.array_equal(od.to_numpy(np.float32, xs[i].shape), eager[i]), i
+    graph.free()
+    side.free()

@@ -58,6 +58,61 @@ def synchronize():
     check(lib.xfthip_device_synchronize())
 
 
+class Stream:
+    """A stream of default priority; pass `.h` wherever a call takes a stream."""
+
+    def __init__(self):
+        self.h = C.c_void_p()
+        check(lib.xfthip_stream_create(C.byref(self.h)))
+
+    def synchronize(self):
+        check(lib.xfthip_stream_synchronize(self.h))
+
+    def free(self):
+        if self.h is not None:
+            lib.xfthip_stream_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Graph:
+    """Records the calls made on `stream` inside the `with` block and replays them with launch()."""
+
+    def __init__(self, stream):
+        self.stream, self.h = stream, None
+
+    def __enter__(self):
+        check(lib.xfthip_graph_begin(self.stream.h))
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        g = C.c_void_p()
+        rc = lib.xfthip_graph_end(self.stream.h, C.byref(g))
+        if exc_type is None:
+            check(rc)
+            self.h = g
+        return False
+
+    def launch(self, stream=None):
+        check(lib.xfthip_graph_launch(self.h, (stream or self.stream).h))
+
+    def free(self):
+        if self.h is not None:
+            lib.xfthip_graph_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
 def _hp(a):
     return None if a is None else a.ctypes.data_as(C.c_void_p)
 
@@ -516,7 +571,13 @@ class MoE:
         self._keep += [gateup, down]
         check(lib.xfthip_moe_set_expert(self.h, e, gateup.h, down.h))
 
-    def forward(self, x_in_dev, x_out_dev, tokens, do_norm=True, logits_override_dev=None, stream=None):
+    def forward(self, x_in_dev, x_out_dev, tokens, do_norm=True, logits_override_dev=None, stream=None, want_routing=True):
+        """Returns the chosen experts and their weights (which costs a wait for the stream); with
+        want_routing=False nothing is copied back, the call only enqueues work and may be captured into a graph."""
+        if not want_routing:
+            check(lib.xfthip_moe_forward(self.h, x_in_dev, self.hidden, x_out_dev, self.hidden, tokens, int(do_norm),
+                                         logits_override_dev, None, None, stream))
+            return None, None
         sel = np.empty((tokens, 2), np.int32)
         w = np.empty((tokens, 2), np.float32)
         check(lib.xfthip_moe_forward(self.h, x_in_dev, self.hidden, x_out_dev, self.hidden, tokens, int(do_norm),

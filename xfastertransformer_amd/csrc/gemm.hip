@@ -13,6 +13,33 @@ static int check_common(const char *fn, xfthip_weight_t w, int M, const void *A,
     return 0;
 }
 
+namespace xfthip {
+
+int gemm_rows_dev(xfthip_weight_t w, int m_max, int m_hint, const int *rows_dev, const void *A, int lda, void *C, int ldc, int c_dtype,
+        hipStream_t stream) {
+    if (int rc = check_common("gemm_rows_dev", w, m_max, A, lda, C, ldc)) return rc;
+    const PackedWeight &pw = w->pw;
+    XFT_REQUIRE(rows_dev != nullptr && pw.kind != XFTHIP_W_W8A8, "gemm_rows_dev: needs a device row record and a weight-only kind");
+    XFT_REQUIRE(c_dtype == XFTHIP_F32 || c_dtype == XFTHIP_BF16, "gemm_rows_dev: c_dtype must be f32 or bf16");
+    const int gateup = (pw.flags & XFTHIP_WF_GATEUP) ? 1 : 0;
+    XFT_REQUIRE(ldc >= (gateup ? pw.N / 2 : pw.N), "gemm_rows_dev: ldc=%d too small", ldc);
+    SkinnyParams p = {};
+    p.M = m_max;
+    p.A = (const uint16_t *)A;
+    p.lda = lda;
+    p.C = C;
+    p.ldc = ldc;
+    p.c_dtype = c_dtype;
+    p.epi = XFTHIP_EPI_NONE;
+    p.gateup = gateup;
+    p.rows_dev = rows_dev;
+    p.m_hint = m_hint;
+    if (m_max <= 32) return qgemm_skinny(pw, p, stream);
+    return qgemm_mfma(pw, p, stream);
+}
+
+} // namespace xfthip
+
 extern "C" {
 
 int xfthip_gemm(xfthip_weight_t w, int M, const void *A, int lda, void *C, int ldc, int c_dtype, int epilogue,

@@ -6,6 +6,7 @@
 #include <vector>
 
 #include "common.h"
+#include "qgemm.h"
 
 namespace xfthip {
 
@@ -64,11 +65,11 @@ __global__ void top2_kernel(const float *__restrict__ logits, int M, int E, int 
 // a time (ballot + prefix count), then the lists are laid back to back (expert 0's rows first) and every
 // (token, choice) learns the row of the gathered matrix that holds its copy:
 //   counts[e], offsets[e] (first row of expert e), row_token[g] / row_weight[g] for the 2 M gathered rows,
-//   slot_row[2 t + s] = row of token t's s-th choice.
+//   slot_row[2 t + s] = row of token t's s-th choice, gemm_rows[6 e ..] = the row records of expert e's GEMMs.
 // blockDim.x = 64 * E; rank[] is scratch of 2 M ints.
 __global__ __launch_bounds__(512) void build_lists_kernel(const int *__restrict__ sel, const float *__restrict__ w, int M, int E,
         int *__restrict__ counts, int *__restrict__ offsets, int *__restrict__ row_token, float *__restrict__ row_weight,
-        int *__restrict__ slot_row, int *__restrict__ rank) {
+        int *__restrict__ slot_row, int *__restrict__ rank, int *__restrict__ gemm_rows) {
     __shared__ int s_count[8], s_off[8];
     const int e = threadIdx.x >> 6, lane = threadIdx.x & 63;
     int n = 0;
@@ -88,6 +89,11 @@ __global__ __launch_bounds__(512) void build_lists_kernel(const int *__restrict_
             s_off[i] = acc;
             counts[i] = s_count[i];
             offsets[i] = acc;
+            // what the two GEMMs of expert i read instead of a host-side row count: {rows, first row of A, first
+            // row of C}: gate/up reads its gathered rows and writes the shared hidden buffer from row 0, down
+            // reads that buffer and writes the expert-output rows
+            gemm_rows[6 * i + 0] = s_count[i], gemm_rows[6 * i + 1] = acc, gemm_rows[6 * i + 2] = 0;
+            gemm_rows[6 * i + 3] = s_count[i], gemm_rows[6 * i + 4] = 0, gemm_rows[6 * i + 5] = acc;
             acc += s_count[i];
         }
     }
@@ -158,7 +164,7 @@ struct xfthip_moe {
     std::vector<xfthip_weight_t> gateup, down;
     uint16_t *xn = nullptr, *xg = nullptr, *h = nullptr;
     float *eo = nullptr, *logits = nullptr, *w = nullptr, *row_weight = nullptr;
-    int *sel = nullptr, *counts = nullptr, *row_token = nullptr, *slot_row = nullptr, *rank = nullptr; // counts: [E] counts, [E] offsets
+    int *sel = nullptr, *counts = nullptr, *row_token = nullptr, *slot_row = nullptr, *rank = nullptr; // counts: [E] counts, [E] offsets, [6 E] GEMM row records
 };
 
 extern "C" {
@@ -175,6 +181,7 @@ int xfthip_moe_create(int hidden, int intermediate, int experts, int max_tokens,
     XFT_REQUIRE(out && router_host, "xfthip_moe_create: null argument");
     XFT_REQUIRE(experts == 8, "xfthip_moe_create: %d experts unsupported (the router kernel is built for 8)", experts);
     XFT_REQUIRE(hidden > 0 && hidden % 8 == 0 && intermediate % 16 == 0 && max_tokens > 0, "xfthip_moe_create: bad sizes");
+    if (int rc = qgemm_split_reserve()) return rc; // the down projections split K: have the workspace before any capture
     xfthip_moe *m = new xfthip_moe();
     m->hidden = hidden;
     m->inter = intermediate;
@@ -188,7 +195,7 @@ int xfthip_moe_create(int hidden, int intermediate, int experts, int max_tokens,
             && hipMalloc((void **)&m->xn, T * hidden * 2) == hipSuccess && hipMalloc((void **)&m->xg, 2 * T * hidden * 2) == hipSuccess
             && hipMalloc((void **)&m->h, T * intermediate * 2) == hipSuccess && hipMalloc((void **)&m->eo, 2 * T * hidden * 4) == hipSuccess
             && hipMalloc((void **)&m->logits, T * experts * 4) == hipSuccess && hipMalloc((void **)&m->w, T * 2 * 4) == hipSuccess
-            && hipMalloc((void **)&m->sel, T * 2 * 4) == hipSuccess && hipMalloc((void **)&m->counts, 2 * 64) == hipSuccess
+            && hipMalloc((void **)&m->sel, T * 2 * 4) == hipSuccess && hipMalloc((void **)&m->counts, (2 + 6) * 64) == hipSuccess
             && hipMalloc((void **)&m->row_token, 2 * T * 4) == hipSuccess && hipMalloc((void **)&m->row_weight, 2 * T * 4) == hipSuccess
             && hipMalloc((void **)&m->slot_row, 2 * T * 4) == hipSuccess && hipMalloc((void **)&m->rank, 2 * T * 4) == hipSuccess;
     if (ok && ln_host) ok = hipMalloc((void **)&m->ln, (size_t)hidden * 4) == hipSuccess
@@ -245,25 +252,24 @@ int xfthip_moe_forward(xfthip_moe_t m, const float *x_in, int in_stride, float *
         logits = m->logits;
     }
     if (int rc = xfthip_moe_top2(logits, T, m->E, m->sel, m->w, st)) return rc;
+    int *gemm_rows = m->counts + 2 * m->E;
     hipLaunchKernelGGL(build_lists_kernel, dim3(1), dim3(64 * m->E), 0, st, m->sel, m->w, T, m->E, m->counts, m->counts + m->E, m->row_token,
-            m->row_weight, m->slot_row, m->rank);
+            m->row_weight, m->slot_row, m->rank, gemm_rows);
     hipLaunchKernelGGL(gather_rows_kernel, dim3(2 * T), dim3(256), 0, st, m->xn, H, m->row_token, m->xg, H);
     XFT_CHECK_HIP(hipGetLastError());
-    int counts[64];
-    XFT_CHECK_HIP(hipMemcpyAsync(counts, m->counts, m->E * sizeof(int), hipMemcpyDeviceToHost, st));
-    XFT_CHECK_HIP(hipStreamSynchronize(st)); // the per-expert row counts size the GEMMs below
-    if (sel_host_out) XFT_CHECK_HIP(hipMemcpy(sel_host_out, m->sel, (size_t)T * 2 * 4, hipMemcpyDeviceToHost));
-    if (w_host_out) XFT_CHECK_HIP(hipMemcpy(w_host_out, m->w, (size_t)T * 2 * 4, hipMemcpyDeviceToHost));
-    int off = 0;
+    if (sel_host_out || w_host_out) {
+        XFT_CHECK_HIP(hipStreamSynchronize(st));
+        if (sel_host_out) XFT_CHECK_HIP(hipMemcpy(sel_host_out, m->sel, (size_t)T * 2 * 4, hipMemcpyDeviceToHost));
+        if (w_host_out) XFT_CHECK_HIP(hipMemcpy(w_host_out, m->w, (size_t)T * 2 * 4, hipMemcpyDeviceToHost));
+    }
+    // The host never learns how many rows an expert got: every expert's two GEMMs are launched for up to T
+    // rows and read their row count and row offsets from the record build_lists_kernel left in device memory
+    // (workgroups past the count leave at once).  The forms are chosen for the 2 T / E rows an expert gets on
+    // average.  Nothing here synchronises, so the layer can be captured into a graph.
+    const int hint = (2 * T + m->E - 1) / m->E;
     for (int e = 0; e < m->E; ++e) {
-        const int n = counts[e];
-        if (n == 0) continue;
-        // expert e owns rows [off, off + n) of the gathered activations and of the expert outputs
-        if (int rc = xfthip_gemm_gateup_silu(m->gateup[e], n, m->xg + (size_t)off * H, H, m->h, m->inter, XFTHIP_BF16, st)) return rc;
-        if (int rc = xfthip_gemm(m->down[e], n, m->h, m->inter, m->eo + (size_t)off * H, H, XFTHIP_F32, XFTHIP_EPI_NONE, nullptr, nullptr, 0,
-                    XFTHIP_F32, 1.0f, st))
-            return rc;
-        off += n;
+        if (int rc = gemm_rows_dev(m->gateup[e], T, hint, gemm_rows + 6 * e, m->xg, H, m->h, m->inter, XFTHIP_BF16, st)) return rc;
+        if (int rc = gemm_rows_dev(m->down[e], T, hint, gemm_rows + 6 * e + 3, m->h, m->inter, m->eo, H, XFTHIP_F32, st)) return rc;
     }
     const int wide = (((size_t)x_out | ((size_t)out_stride * 4)) & 15) == 0;
     hipLaunchKernelGGL(combine_kernel, dim3(T), dim3(256), 0, st, x_out, out_stride, m->eo, m->sel, m->slot_row, m->w, H, wide);

@@ -26,6 +26,11 @@ struct SkinnyParams {
     // fp32 [M][N] into split_part + y * M * N; a second kernel adds the parts in order and applies the epilogue
     int ksplit, split_ktiles;
     float *split_part;
+    // Row count known on the device only (the experts of a sparse MLP): when rows_dev is set the kernels read
+    // {rows, first row of A, first row of C} from it, M is only the upper bound that sizes the grid, and m_hint
+    // (0 = M) is the row count the host expects, used where it chooses between forms.  No residual epilogues.
+    const int *rows_dev;
+    int m_hint;
 
     // ---- fusions of the decode step (M <= 4, skinny kernel only) ----
     // RMSNorm prologue: when norm_x is set, A is ignored and every workgroup normalises the M rows
@@ -51,6 +56,10 @@ int qgemm_skinny(const PackedWeight &pw, const SkinnyParams &p, hipStream_t stre
 bool skinny_can_fuse_norm(const PackedWeight &pw, int M); // may SkinnyParams::norm_x be used
 int qgemm_mfma(const PackedWeight &pw, const SkinnyParams &p, hipStream_t stream); // any M, built for M > 32
 int qgemm_split_reserve(); // allocates the K-split workspace of qgemm_mfma now (before a stream capture, say)
+// xfthip_gemm / xfthip_gemm_gateup_silu (by the weight's flag) with the row count in device memory: rows_dev =
+// {rows, first row of A, first row of C}, at most m_max rows, about m_hint expected; plain epilogue only
+int gemm_rows_dev(xfthip_weight_t w, int m_max, int m_hint, const int *rows_dev, const void *A, int lda, void *C, int ldc, int c_dtype,
+        hipStream_t stream);
 
 int gemm_w8a8_from_bf16(xfthip_weight_t w, int M, const void *A, int lda, void *C, int ldc, int c_dtype, int epilogue,
         const float *bias, const void *res, int ldres, int res_dtype, float gamma, hipStream_t stream);

@@ -26,6 +26,11 @@ __global__ __launch_bounds__(256) void qgemm_split_finish_kernel(SkinnyParams p)
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (size_t)p.M * p.N) return;
     const int m = (int)(idx / p.N), n = (int)(idx - (size_t)m * p.N);
+    int row_out = m;
+    if (p.rows_dev) {
+        if (m >= p.rows_dev[0]) return;
+        row_out = m + p.rows_dev[2];
+    }
     float x = 0.0f;
     for (int s = 0; s < p.ksplit; ++s) x += p.split_part[((size_t)s * p.M + m) * p.N + n];
     switch (p.epi) {
@@ -47,7 +52,7 @@ __global__ __launch_bounds__(256) void qgemm_split_finish_kernel(SkinnyParams p)
             break;
         default: break;
     }
-    store_from_f32(p.C, p.c_dtype, (size_t)m * p.ldc + n, x);
+    store_from_f32(p.C, p.c_dtype, (size_t)row_out * p.ldc + n, x);
 }
 
 // Partial results of the K split: one buffer per process and device, allocated once at its upper bound (a
@@ -83,7 +88,8 @@ int qgemm_mfma(const PackedWeight &pw, const SkinnyParams &p0, hipStream_t strea
     // few dozen sequences): the 32-row tiles would not even give every CU a workgroup, so K is split as well.
     const int ktile = ktile_of(pw.kind), kt_n = (pw.K + ktile - 1) / ktile;
     const int cus = device_cu_count(), n32 = (pw.NTILES + 1) / 2;
-    const long tiles = (long)((n32 + 3) / 4) * ((p.M + 31) / 32);
+    const int rows_expected = (p.rows_dev && p.m_hint > 0) ? p.m_hint : p.M;
+    const long tiles = (long)((n32 + 3) / 4) * ((rows_expected + 31) / 32);
     if (!p.gateup && 2 * tiles <= cus && kt_n >= 16) {
         long want = (2L * cus) / tiles;
         want = want < kt_n / 8 ? want : kt_n / 8;

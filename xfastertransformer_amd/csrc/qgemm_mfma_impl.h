@@ -86,37 +86,53 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = lane >> 5, nl = lane & 31;
-    if (p.ksplit > 1) {
-        // this row of workgroups owns a range of k tiles: shift the operands to it, the result goes to its part
-        const int kt0 = blockIdx.y * p.split_ktiles;
-        const int k_left = p.K - kt0 * KTILE, k_span = p.split_ktiles * KTILE;
-        p.packed += (size_t)kt0 * 1024;
-        p.A += (size_t)kt0 * KTILE;
-        p.K = k_left < k_span ? k_left : k_span;
-        p.C = p.split_part + (size_t)blockIdx.y * p.M * p.N;
-        p.ldc = p.N;
-        p.c_dtype = XFTHIP_F32;
-        p.epi = XFTHIP_EPI_NONE;
+    const int part_rows = p.M; // rows of a K part: the host's bound, also when the device knows fewer
+    if (p.rows_dev) {
+        p.M = p.rows_dev[0] < part_rows ? p.rows_dev[0] : part_rows;
+        p.A += (size_t)p.rows_dev[1] * p.lda;
+        p.C = (char *)p.C + (size_t)p.rows_dev[2] * p.ldc * (p.c_dtype == XFTHIP_F32 ? 4 : 2);
     }
-
-    // block -> (column block, row block): blocks that share a column block sit on the same XCD
-    // (block ids round-robin over the 8 XCDs), so their weight reads hit that XCD's L2.  Row blocks are
-    // walked in bands of 8: all column blocks of a band before the next band, so that the band's
-    // activation rows stay cached while the weights stream past them.
-    int nb, mb;
+    // workgroup -> (K part, column block, row block): workgroups that share a column block sit on the same XCD
+    // (workgroup ids round-robin over the 8 XCDs in launch order), so their weight reads hit that XCD's L2.  Row
+    // blocks are walked in bands of 8: all K parts and column blocks of a band before the next band, so that the
+    // band's activation rows stay cached while the weights stream past them.
+    int nb, mb, part;
     {
-        constexpr int BAND = 8;
-        const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
+        // With a device-side row count the band is only as tall as the rows the host expects: the workgroups
+        // that do work then come first in the launch order and spread over the CUs; the ones past the count
+        // (which leave at once) follow them instead of sitting between them.
+        int BAND = 8;
+        if (p.rows_dev) {
+            const int want = (p.m_hint + ROWS - 1) / ROWS;
+            BAND = want < 1 ? 1 : want < 8 ? want : 8;
+        }
+        const int parts = p.ksplit > 1 ? p.ksplit : 1;
+        const int id = blockIdx.y * gridDim.x + blockIdx.x, xcd = id & 7, slot = id >> 3; // gridDim.x is a multiple of 8
         const int nb8 = (nblocks_n + 7) >> 3;
-        if (slot >= nb8 * nblocks_m) return;
-        const int band = slot / (nb8 * BAND), rem = slot - band * (nb8 * BAND);
+        if (slot >= nb8 * nblocks_m * parts) return;
+        const int band = slot / (nb8 * BAND * parts), rem_band = slot - band * (nb8 * BAND * parts);
         const int left = nblocks_m - band * BAND, rows_in_band = left < BAND ? left : BAND;
+        part = rem_band / (nb8 * rows_in_band);
+        const int rem = rem_band - part * (nb8 * rows_in_band);
         nb = rem / rows_in_band + xcd * nb8;
         mb = band * BAND + rem % rows_in_band;
         if (nb >= nblocks_n) return;
     }
+    if (p.ksplit > 1) {
+        // this workgroup owns a range of k tiles: shift the operands to it, the result goes to its part
+        const int kt0 = part * p.split_ktiles;
+        const int k_left = p.K - kt0 * KTILE, k_span = p.split_ktiles * KTILE;
+        p.packed += (size_t)kt0 * 1024;
+        p.A += (size_t)kt0 * KTILE;
+        p.K = k_left < k_span ? k_left : k_span;
+        p.C = p.split_part + (size_t)part * part_rows * p.N;
+        p.ldc = p.N;
+        p.c_dtype = XFTHIP_F32;
+        p.epi = XFTHIP_EPI_NONE;
+    }
     const int n32_0 = (nb * 4 + wave) * WN; // first 32-column tile of this wave
     const int m0 = mb * ROWS;
+    if (m0 >= p.M) return; // fewer rows than the grid was sized for (the whole workgroup leaves)
 
     uint2 *lut = nullptr;
     unsigned char *abuf_base = lds;
@@ -592,9 +608,11 @@ static int dispatch_big_tile(const SkinnyParams &p, hipStream_t stream) {
     // pay once there are many row blocks to share a weight tile's trip through L2; below that,
     // more and smaller workgroups per CU (whose k loops overlap) win by up to 1.5x.
     const int n32 = (p.NTILES + 1) / 2;
-    const long t_large = (long)((n32 + 7) / 8) * ((p.M + 127) / 128);
-    const long t_mid = (long)((n32 + 3) / 4) * ((p.M + 127) / 128);
-    const long t_small = (long)((n32 + 3) / 4) * ((p.M + 63) / 64);
+    // the tile is chosen for the rows the host expects; with a device-side row count p.M is only the bound
+    const int rows = (p.rows_dev && p.m_hint > 0) ? p.m_hint : p.M;
+    const long t_large = (long)((n32 + 7) / 8) * ((rows + 127) / 128);
+    const long t_mid = (long)((n32 + 3) / 4) * ((rows + 127) / 128);
+    const long t_small = (long)((n32 + 3) / 4) * ((rows + 63) / 64);
     if constexpr (KIND == XFTHIP_W_BF16) {
         if (t_large >= cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
         if (t_mid >= cus) return launch_big<KIND, 1, 4, NEED_SUM>(p, stream);
@@ -603,11 +621,11 @@ static int dispatch_big_tile(const SkinnyParams &p, hipStream_t stream) {
         // 128 x 128 tiles, two workgroups a CU: measured 745 / 888 / 821 / 786 / 814 TFLOP/s on N x K =
         // 11008x4096 / 4096x4096 / 4096x11008 / 12288x4096 / 22016x4096 at 2048 rows; the 128 x 256 tile
         // (one wave per SIMD, nothing to run while it waits) stays at 750-760 wherever it applies
-        if (p.M > 1024 && t_mid >= cus) return launch_big<KIND, 1, 4, NEED_SUM>(p, stream);
+        if (rows > 1024 && t_mid >= cus) return launch_big<KIND, 1, 4, NEED_SUM>(p, stream);
     } else {
         // 4-bit kinds: the 128 x 128 tile holds half the accumulators of the 128 x 256 one at the
         // same occupancy (LDS for the 128-deep k tile) and never won
-        if (p.M > 512 && t_large >= cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
+        if (rows > 512 && t_large >= cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
     }
     if constexpr (KIND != XFTHIP_W_BF16) {
         // Few rows against a deep K (512 tokens x 4096 columns): 64-row tiles would leave one

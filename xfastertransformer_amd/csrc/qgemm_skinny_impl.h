@@ -124,6 +124,12 @@ __global__ __launch_bounds__(512) void qgemm_skinny_kernel(SkinnyParams p) {
     const int nwaves = blockDim.x >> 6;
     const int g = lane >> 4, ml = lane & 15;
     constexpr bool need_sum = NEED_SUM;
+    if (p.rows_dev) {
+        if (p.rows_dev[0] <= 0) return; // uniform: the whole workgroup leaves
+        p.M = p.rows_dev[0] < p.M ? p.rows_dev[0] : p.M;
+        p.A += (size_t)p.rows_dev[1] * p.lda;
+        p.C = (char *)p.C + (size_t)p.rows_dev[2] * p.ldc * (p.c_dtype == XFTHIP_F32 ? 4 : 2);
+    }
 
     uint2 *lut = nullptr;
     if constexpr (KIND == XFTHIP_W_NF4) {

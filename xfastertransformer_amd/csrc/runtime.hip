@@ -150,6 +150,35 @@ int xfthip_device_synchronize(void) {
     return 0;
 }
 
+int xfthip_graph_begin(xfthip_stream_t stream) {
+    XFT_REQUIRE(stream != nullptr, "xfthip_graph_begin: capture needs a stream of its own, not the null stream");
+    XFT_CHECK_HIP(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+    return 0;
+}
+
+int xfthip_graph_end(xfthip_stream_t stream, xfthip_graph_t *graph) {
+    XFT_REQUIRE(stream != nullptr && graph != nullptr, "xfthip_graph_end: null argument");
+    hipGraph_t g = nullptr;
+    XFT_CHECK_HIP(hipStreamEndCapture((hipStream_t)stream, &g));
+    hipGraphExec_t exec = nullptr;
+    const hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    XFT_CHECK_HIP(e);
+    *graph = (xfthip_graph_t)exec;
+    return 0;
+}
+
+int xfthip_graph_launch(xfthip_graph_t graph, xfthip_stream_t stream) {
+    XFT_REQUIRE(graph != nullptr, "xfthip_graph_launch: null graph");
+    XFT_CHECK_HIP(hipGraphLaunch((hipGraphExec_t)graph, (hipStream_t)stream));
+    return 0;
+}
+
+int xfthip_graph_destroy(xfthip_graph_t graph) {
+    if (graph) XFT_CHECK_HIP(hipGraphExecDestroy((hipGraphExec_t)graph));
+    return 0;
+}
+
 int xfthip_event_create(xfthip_event_t *ev) {
     hipEvent_t e;
     XFT_CHECK_HIP(hipEventCreate(&e));

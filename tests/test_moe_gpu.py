@@ -84,6 +84,34 @@ def test_mixtral_mlp_vs_oracle(xh, orc, tokens, override):
         assert _cos(got, e32) >= 0.9999
 
 
+@pytest.mark.parametrize("kind", [1, 2])
+@pytest.mark.parametrize("tokens", [9, 150])
+def test_mixtral_mlp_four_bit_experts(xh, orc, kind, tokens):
+    """UINT4 and NF4 experts, through the per-expert launches (18 gathered rows) and through the launch
+    that serves all experts at once (300 gathered rows), with two experts that get no token."""
+    hidden, inter, E = 1024, 3584, 8
+    rng = np.random.default_rng(100 * kind + tokens)
+    experts = _experts(orc, rng, kind, hidden, inter, E)
+    router = np.zeros((hidden, E), np.float32)
+    ln = rng.uniform(0.8, 1.2, hidden).astype(np.float32)
+    x = orc.round_bf16(rng.standard_normal((tokens, hidden)))
+    lo = rng.standard_normal((tokens, E)).astype(np.float32)
+    lo[:, 3] = lo[:, 6] = -20.0
+    moe = xh.MoE(hidden, inter, E, tokens, router, ln)
+    for e, (gu, dn) in enumerate(experts):
+        moe.set_expert(e, xh.Weight(kind, gu.K, gu.N, gu.q, gu.scale, gu.zero, flags=xh.WF_GATEUP),
+                       xh.Weight(kind, dn.K, dn.N, dn.q, dn.scale, dn.zero))
+    xd, lod = xh.DeviceBuffer.from_numpy(x), xh.DeviceBuffer.from_numpy(lo)
+    od = xh.DeviceBuffer(x.nbytes)
+    sel, w = moe.forward(xd.ptr, od.ptr, tokens, True, lod.ptr)
+    xh.synchronize()
+    got = od.to_numpy(np.float32, x.shape)
+    exp, esel, ew = orc.mixtral_mlp(x, ln, router, experts, lo, rounding="bf16")
+    assert np.array_equal(sel, esel) and not np.isin(sel, (3, 6)).any()
+    assert np.abs(w - ew).max() < 1e-6
+    assert np.abs(got - exp).max() < 2e-2 and _cos(got, exp) >= 0.9999
+
+
 def test_mixtral_shape_full_size_spot_check(xh, orc):
     """Mixtral-8x7B shape (hidden 4096, FFN 14336, 8 INT8 experts, 256 tokens, overridden N(0,1)
     logits): routing must equal the oracle's, and a handful of tokens are recomputed by the oracle."""

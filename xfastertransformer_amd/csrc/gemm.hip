@@ -38,6 +38,38 @@ int gemm_rows_dev(xfthip_weight_t w, int m_max, int m_hint, const int *rows_dev,
     return qgemm_mfma(pw, p, stream);
 }
 
+int gemm_grouped_rows_dev(const xfthip_weight_t *w, int n_group, const GroupWeight *table_dev, int rows_max, const int *rows_dev,
+        int rows_stride, const void *A, int lda, void *C, int ldc, int c_dtype, hipStream_t stream) {
+    XFT_REQUIRE(w && n_group >= 1 && table_dev && rows_dev && rows_stride >= 3, "gemm_grouped_rows_dev: bad group arguments");
+    if (int rc = check_common("gemm_grouped_rows_dev", w[0], rows_max, A, lda, C, ldc)) return rc;
+    XFT_REQUIRE(rows_max > 32, "gemm_grouped_rows_dev: needs more than 32 rows in all (the few-row kernel has no grouped form)");
+    const PackedWeight &pw = w[0]->pw;
+    XFT_REQUIRE(pw.kind != XFTHIP_W_W8A8, "gemm_grouped_rows_dev: needs a weight-only kind");
+    for (int e = 1; e < n_group; ++e) {
+        XFT_REQUIRE(w[e] != nullptr, "gemm_grouped_rows_dev: weight %d is null", e);
+        const PackedWeight &o = w[e]->pw;
+        XFT_REQUIRE(o.kind == pw.kind && o.K == pw.K && o.N == pw.N && o.flags == pw.flags && (o.zero != nullptr) == (pw.zero != nullptr),
+                "gemm_grouped_rows_dev: weight %d differs from weight 0 in kind, shape or layout", e);
+    }
+    XFT_REQUIRE(c_dtype == XFTHIP_F32 || c_dtype == XFTHIP_BF16, "gemm_grouped_rows_dev: c_dtype must be f32 or bf16");
+    const int gateup = (pw.flags & XFTHIP_WF_GATEUP) ? 1 : 0;
+    XFT_REQUIRE(ldc >= (gateup ? pw.N / 2 : pw.N), "gemm_grouped_rows_dev: ldc=%d too small", ldc);
+    SkinnyParams p = {};
+    p.M = rows_max;
+    p.A = (const uint16_t *)A;
+    p.lda = lda;
+    p.C = C;
+    p.ldc = ldc;
+    p.c_dtype = c_dtype;
+    p.epi = XFTHIP_EPI_NONE;
+    p.gateup = gateup;
+    p.rows_dev = rows_dev;
+    p.group = table_dev;
+    p.group_n = n_group;
+    p.rows_stride = rows_stride;
+    return qgemm_mfma(pw, p, stream);
+}
+
 } // namespace xfthip
 
 extern "C" {

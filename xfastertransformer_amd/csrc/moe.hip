@@ -65,7 +65,7 @@ __global__ void top2_kernel(const float *__restrict__ logits, int M, int E, int 
 // a time (ballot + prefix count), then the lists are laid back to back (expert 0's rows first) and every
 // (token, choice) learns the row of the gathered matrix that holds its copy:
 //   counts[e], offsets[e] (first row of expert e), row_token[g] / row_weight[g] for the 2 M gathered rows,
-//   slot_row[2 t + s] = row of token t's s-th choice, gemm_rows[6 e ..] = the row records of expert e's GEMMs.
+//   slot_row[2 t + s] = row of token t's s-th choice, gemm_rows[9 e ..] = the row records of expert e's GEMMs.
 // blockDim.x = 64 * E; rank[] is scratch of 2 M ints.
 __global__ __launch_bounds__(512) void build_lists_kernel(const int *__restrict__ sel, const float *__restrict__ w, int M, int E,
         int *__restrict__ counts, int *__restrict__ offsets, int *__restrict__ row_token, float *__restrict__ row_weight,
@@ -92,8 +92,10 @@ __global__ __launch_bounds__(512) void build_lists_kernel(const int *__restrict_
             // what the two GEMMs of expert i read instead of a host-side row count: {rows, first row of A, first
             // row of C}: gate/up reads its gathered rows and writes the shared hidden buffer from row 0, down
             // reads that buffer and writes the expert-output rows
-            gemm_rows[6 * i + 0] = s_count[i], gemm_rows[6 * i + 1] = acc, gemm_rows[6 * i + 2] = 0;
-            gemm_rows[6 * i + 3] = s_count[i], gemm_rows[6 * i + 4] = 0, gemm_rows[6 * i + 5] = acc;
+            // (the launch that serves all experts at once keeps every expert's hidden rows: {rows, first, first})
+            gemm_rows[9 * i + 0] = s_count[i], gemm_rows[9 * i + 1] = acc, gemm_rows[9 * i + 2] = 0;
+            gemm_rows[9 * i + 3] = s_count[i], gemm_rows[9 * i + 4] = 0, gemm_rows[9 * i + 5] = acc;
+            gemm_rows[9 * i + 6] = s_count[i], gemm_rows[9 * i + 7] = acc, gemm_rows[9 * i + 8] = acc;
             acc += s_count[i];
         }
     }
@@ -164,7 +166,8 @@ struct xfthip_moe {
     std::vector<xfthip_weight_t> gateup, down;
     uint16_t *xn = nullptr, *xg = nullptr, *h = nullptr;
     float *eo = nullptr, *logits = nullptr, *w = nullptr, *row_weight = nullptr;
-    int *sel = nullptr, *counts = nullptr, *row_token = nullptr, *slot_row = nullptr, *rank = nullptr; // counts: [E] counts, [E] offsets, [6 E] GEMM row records
+    GroupWeight *group = nullptr; // device pointers of the experts' weights: [E] gate/up, [E] down
+    int *sel = nullptr, *counts = nullptr, *row_token = nullptr, *slot_row = nullptr, *rank = nullptr; // counts: [E] counts, [E] offsets, [9 E] GEMM row records
 };
 
 extern "C" {
@@ -193,9 +196,9 @@ int xfthip_moe_create(int hidden, int intermediate, int experts, int max_tokens,
     // every token is gathered twice (its two experts): 2 T rows of activations and of expert outputs
     bool ok = hipMalloc((void **)&m->router, (size_t)hidden * experts * 4) == hipSuccess
             && hipMalloc((void **)&m->xn, T * hidden * 2) == hipSuccess && hipMalloc((void **)&m->xg, 2 * T * hidden * 2) == hipSuccess
-            && hipMalloc((void **)&m->h, T * intermediate * 2) == hipSuccess && hipMalloc((void **)&m->eo, 2 * T * hidden * 4) == hipSuccess
+            && hipMalloc((void **)&m->h, 2 * T * intermediate * 2) == hipSuccess && hipMalloc((void **)&m->eo, 2 * T * hidden * 4) == hipSuccess
             && hipMalloc((void **)&m->logits, T * experts * 4) == hipSuccess && hipMalloc((void **)&m->w, T * 2 * 4) == hipSuccess
-            && hipMalloc((void **)&m->sel, T * 2 * 4) == hipSuccess && hipMalloc((void **)&m->counts, (2 + 6) * 64) == hipSuccess
+            && hipMalloc((void **)&m->sel, T * 2 * 4) == hipSuccess && hipMalloc((void **)&m->counts, (2 + 9) * 64) == hipSuccess && hipMalloc((void **)&m->group, 2 * 64 * sizeof(GroupWeight)) == hipSuccess
             && hipMalloc((void **)&m->row_token, 2 * T * 4) == hipSuccess && hipMalloc((void **)&m->row_weight, 2 * T * 4) == hipSuccess
             && hipMalloc((void **)&m->slot_row, 2 * T * 4) == hipSuccess && hipMalloc((void **)&m->rank, 2 * T * 4) == hipSuccess;
     if (ok && ln_host) ok = hipMalloc((void **)&m->ln, (size_t)hidden * 4) == hipSuccess
@@ -212,7 +215,7 @@ int xfthip_moe_create(int hidden, int intermediate, int experts, int max_tokens,
 
 int xfthip_moe_destroy(xfthip_moe_t m) {
     if (!m) return 0;
-    void *bufs[] = {m->router, m->ln, m->xn, m->xg, m->h, m->eo, m->logits, m->w, m->row_weight, m->sel, m->counts, m->row_token, m->slot_row, m->rank};
+    void *bufs[] = {m->router, m->ln, m->xn, m->xg, m->h, m->eo, m->logits, m->w, m->row_weight, m->sel, m->counts, m->row_token, m->slot_row, m->rank, m->group};
     for (void *b : bufs)
         if (b) (void)hipFree(b);
     delete m;
@@ -226,6 +229,9 @@ int xfthip_moe_set_expert(xfthip_moe_t m, int e, xfthip_weight_t gateup, xfthip_
     XFT_REQUIRE(down->pw.K == m->inter && down->pw.N == m->hidden, "xfthip_moe_set_expert: down weight must be [%d,%d]", m->inter, m->hidden);
     m->gateup[e] = gateup;
     m->down[e] = down;
+    const GroupWeight g = {gateup->pw.packed, gateup->pw.scale, gateup->pw.zero}, d = {down->pw.packed, down->pw.scale, down->pw.zero};
+    XFT_CHECK_HIP(hipMemcpy(m->group + e, &g, sizeof(g), hipMemcpyHostToDevice));
+    XFT_CHECK_HIP(hipMemcpy(m->group + m->E + e, &d, sizeof(d), hipMemcpyHostToDevice));
     return 0;
 }
 
@@ -262,14 +268,29 @@ int xfthip_moe_forward(xfthip_moe_t m, const float *x_in, int in_stride, float *
         if (sel_host_out) XFT_CHECK_HIP(hipMemcpy(sel_host_out, m->sel, (size_t)T * 2 * 4, hipMemcpyDeviceToHost));
         if (w_host_out) XFT_CHECK_HIP(hipMemcpy(w_host_out, m->w, (size_t)T * 2 * 4, hipMemcpyDeviceToHost));
     }
-    // The host never learns how many rows an expert got: every expert's two GEMMs are launched for up to T
-    // rows and read their row count and row offsets from the record build_lists_kernel left in device memory
-    // (workgroups past the count leave at once).  The forms are chosen for the 2 T / E rows an expert gets on
-    // average.  Nothing here synchronises, so the layer can be captured into a graph.
-    const int hint = (2 * T + m->E - 1) / m->E;
-    for (int e = 0; e < m->E; ++e) {
-        if (int rc = gemm_rows_dev(m->gateup[e], T, hint, gemm_rows + 6 * e, m->xg, H, m->h, m->inter, XFTHIP_BF16, st)) return rc;
-        if (int rc = gemm_rows_dev(m->down[e], T, hint, gemm_rows + 6 * e + 3, m->h, m->inter, m->eo, H, XFTHIP_F32, st)) return rc;
+    // The host never learns how many rows an expert got: the GEMMs read row counts and row offsets from the
+    // records build_lists_kernel left in device memory, and nothing here synchronises, so the layer can be
+    // captured into a graph.  With more than 32 gathered rows and experts of one kind, one launch serves the gate/up
+    // projections of all experts and one their down projections (their workgroups run side by side instead of
+    // one expert after another); otherwise every expert's two GEMMs are launched for up to T rows, in the form
+    // for the 2 T / E rows an expert gets on average, and workgroups past the count leave at once.
+    bool uniform = 2 * T > 32;
+    for (int e = 1; e < m->E && uniform; ++e) {
+        const PackedWeight &g0 = m->gateup[0]->pw, &g = m->gateup[e]->pw, &d0 = m->down[0]->pw, &d = m->down[e]->pw;
+        uniform = g.kind == g0.kind && g.flags == g0.flags && (g.zero != nullptr) == (g0.zero != nullptr) && d.kind == d0.kind
+                && d.flags == d0.flags && (d.zero != nullptr) == (d0.zero != nullptr);
+    }
+    if (uniform && m->gateup[0]->pw.kind != XFTHIP_W_W8A8 && m->down[0]->pw.kind != XFTHIP_W_W8A8) {
+        if (int rc = gemm_grouped_rows_dev(m->gateup.data(), m->E, m->group, 2 * T, gemm_rows + 6, 9, m->xg, H, m->h, m->inter, XFTHIP_BF16, st))
+            return rc;
+        if (int rc = gemm_grouped_rows_dev(m->down.data(), m->E, m->group + m->E, 2 * T, gemm_rows + 6, 9, m->h, m->inter, m->eo, H, XFTHIP_F32, st))
+            return rc;
+    } else {
+        const int hint = (2 * T + m->E - 1) / m->E;
+        for (int e = 0; e < m->E; ++e) {
+            if (int rc = gemm_rows_dev(m->gateup[e], T, hint, gemm_rows + 9 * e, m->xg, H, m->h, m->inter, XFTHIP_BF16, st)) return rc;
+            if (int rc = gemm_rows_dev(m->down[e], T, hint, gemm_rows + 9 * e + 3, m->h, m->inter, m->eo, H, XFTHIP_F32, st)) return rc;
+        }
     }
     const int wide = (((size_t)x_out | ((size_t)out_stride * 4)) & 15) == 0;
     hipLaunchKernelGGL(combine_kernel, dim3(T), dim3(256), 0, st, x_out, out_stride, m->eo, m->sel, m->slot_row, m->w, H, wide);

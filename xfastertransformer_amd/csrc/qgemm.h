@@ -5,6 +5,12 @@
 
 namespace xfthip {
 
+struct GroupWeight { // one weight of a grouped launch, in device memory
+    const uint8_t *packed;
+    const float *scale;
+    const float *zero;
+};
+
 struct SkinnyParams {
     const uint8_t *packed;
     const float *scale;
@@ -31,6 +37,11 @@ struct SkinnyParams {
     // (0 = M) is the row count the host expects, used where it chooses between forms.  No residual epilogues.
     const int *rows_dev;
     int m_hint;
+    // Several weights of one shape and kind behind one launch (M > 32 kernel only): weight e multiplies the rows
+    // that record e of rows_dev (records rows_stride ints apart) names; M bounds the sum of their rows, and their
+    // rows of C must tile [0, sum of rows) without gaps.
+    const GroupWeight *group;
+    int group_n, rows_stride;
 
     // ---- fusions of the decode step (M <= 4, skinny kernel only) ----
     // RMSNorm prologue: when norm_x is set, A is ignored and every workgroup normalises the M rows
@@ -60,6 +71,12 @@ int qgemm_split_reserve(); // allocates the K-split workspace of qgemm_mfma now 
 // {rows, first row of A, first row of C}, at most m_max rows, about m_hint expected; plain epilogue only
 int gemm_rows_dev(xfthip_weight_t w, int m_max, int m_hint, const int *rows_dev, const void *A, int lda, void *C, int ldc, int c_dtype,
         hipStream_t stream);
+
+// The same for n_group weights of one shape behind one launch: table_dev holds their device pointers, record e
+// of rows_dev (rows_stride ints apart) the rows of weight e; rows_max bounds the sum of the rows (and must be
+// above 32: the few-row kernel has no grouped form); the weights' rows of C tile [0, sum of rows).
+int gemm_grouped_rows_dev(const xfthip_weight_t *w, int n_group, const GroupWeight *table_dev, int rows_max, const int *rows_dev,
+        int rows_stride, const void *A, int lda, void *C, int ldc, int c_dtype, hipStream_t stream);
 
 int gemm_w8a8_from_bf16(xfthip_weight_t w, int M, const void *A, int lda, void *C, int ldc, int c_dtype, int epilogue,
         const float *bias, const void *res, int ldres, int res_dtype, float gamma, hipStream_t stream);

@@ -87,11 +87,6 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = lane >> 5, nl = lane & 31;
     const int part_rows = p.M; // rows of a K part: the host's bound, also when the device knows fewer
-    if (p.rows_dev) {
-        p.M = p.rows_dev[0] < part_rows ? p.rows_dev[0] : part_rows;
-        p.A += (size_t)p.rows_dev[1] * p.lda;
-        p.C = (char *)p.C + (size_t)p.rows_dev[2] * p.ldc * (p.c_dtype == XFTHIP_F32 ? 4 : 2);
-    }
     // workgroup -> (K part, column block, row block): workgroups that share a column block sit on the same XCD
     // (workgroup ids round-robin over the 8 XCDs in launch order), so their weight reads hit that XCD's L2.  Row
     // blocks are walked in bands of 8: all K parts and column blocks of a band before the next band, so that the
@@ -102,7 +97,7 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
         // that do work then come first in the launch order and spread over the CUs; the ones past the count
         // (which leave at once) follow them instead of sitting between them.
         int BAND = 8;
-        if (p.rows_dev) {
+        if (p.rows_dev && !p.group) {
             const int want = (p.m_hint + ROWS - 1) / ROWS;
             BAND = want < 1 ? 1 : want < 8 ? want : 8;
         }
@@ -118,6 +113,31 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
         mb = band * BAND + rem % rows_in_band;
         if (nb >= nblocks_n) return;
     }
+    int c_row = 0, part_row = 0; // first row of this GEMM in C and in a K part
+    if (p.group) {
+        // several weights of one shape behind one launch: the row blocks of all of them are numbered in a
+        // row, weight after weight, by their device-side row counts; blocks past the last one leave
+        int e = 0, first = 0;
+        for (; e < p.group_n; ++e) {
+            const int nblk = (p.rows_dev[e * p.rows_stride] + ROWS - 1) / ROWS;
+            if (mb < first + nblk) break;
+            first += nblk;
+        }
+        if (e == p.group_n) return;
+        mb -= first;
+        const int *rec = p.rows_dev + e * p.rows_stride;
+        p.M = rec[0];
+        p.A += (size_t)rec[1] * p.lda;
+        c_row = part_row = rec[2];
+        p.packed = p.group[e].packed;
+        p.scale = p.group[e].scale;
+        p.zero = p.group[e].zero;
+    } else if (p.rows_dev) {
+        p.M = p.rows_dev[0] < part_rows ? p.rows_dev[0] : part_rows;
+        p.A += (size_t)p.rows_dev[1] * p.lda;
+        c_row = p.rows_dev[2]; // the K parts hold local rows, the kernel that adds them shifts
+    }
+    p.C = (char *)p.C + (size_t)c_row * p.ldc * (p.c_dtype == XFTHIP_F32 ? 4 : 2);
     if (p.ksplit > 1) {
         // this workgroup owns a range of k tiles: shift the operands to it, the result goes to its part
         const int kt0 = part * p.split_ktiles;
@@ -125,7 +145,7 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
         p.packed += (size_t)kt0 * 1024;
         p.A += (size_t)kt0 * KTILE;
         p.K = k_left < k_span ? k_left : k_span;
-        p.C = p.split_part + (size_t)part * part_rows * p.N;
+        p.C = p.split_part + ((size_t)part * part_rows + part_row) * p.N;
         p.ldc = p.N;
         p.c_dtype = XFTHIP_F32;
         p.epi = XFTHIP_EPI_NONE;
@@ -576,7 +596,8 @@ static int launch_big2(const SkinnyParams &p, hipStream_t stream) {
     constexpr int ROWS = 32 * WM, ROWB = T::KTILE * 2 + 16;
     const int n32 = (p.NTILES + 1) / 2;
     const int nblocks_n = (n32 + 4 * WN - 1) / (4 * WN);
-    const int nblocks_m = (p.M + ROWS - 1) / ROWS;
+    // a group's row blocks: every weight may end in a partly filled one
+    const int nblocks_m = (p.M + ROWS - 1) / ROWS + (p.group ? p.group_n : 0);
     const int nb8 = (nblocks_n + 7) / 8;
     const int blocks = nb8 * 8 * nblocks_m;
     // the three activation buffers, reused after the k loop by the four waves' output patches
@@ -609,7 +630,7 @@ static int dispatch_big_tile(const SkinnyParams &p, hipStream_t stream) {
     // more and smaller workgroups per CU (whose k loops overlap) win by up to 1.5x.
     const int n32 = (p.NTILES + 1) / 2;
     // the tile is chosen for the rows the host expects; with a device-side row count p.M is only the bound
-    const int rows = (p.rows_dev && p.m_hint > 0) ? p.m_hint : p.M;
+    const int rows = (p.rows_dev && !p.group && p.m_hint > 0) ? p.m_hint : p.M;
     const long t_large = (long)((n32 + 7) / 8) * ((rows + 127) / 128);
     const long t_mid = (long)((n32 + 3) / 4) * ((rows + 127) / 128);
     const long t_small = (long)((n32 + 3) / 4) * ((rows + 63) / 64);
@@ -631,7 +652,9 @@ static int dispatch_big_tile(const SkinnyParams &p, hipStream_t stream) {
         // Few rows against a deep K (512 tokens x 4096 columns): 64-row tiles would leave one
         // workgroup per CU, whose k loop is then a chain of load latencies; 32-row tiles put two
         // on a CU.
-        if (t_small < 2 * cus) return launch_big<KIND, 1, 1, NEED_SUM>(p, stream);
+        // (a group's weights with more than 32 rows each keep 64-row tiles: the 32-row ones read every weight
+        // tile twice, and with all the weights' workgroups side by side there is no CU left to fill)
+        if (t_small < 2 * cus && !(p.group && p.M > 32 * p.group_n)) return launch_big<KIND, 1, 1, NEED_SUM>(p, stream);
         return launch_big<KIND, 1, 2, NEED_SUM>(p, stream);
     }
 }

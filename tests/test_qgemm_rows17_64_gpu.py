@@ -115,6 +115,48 @@ def test_rows17_64_gateup_silu_vs_oracle(xh, orc, kind, M, K, I):
     dw.free()
 
 
+@pytest.mark.parametrize("kind", ["int8", "int8_asym", "uint4", "nf4"])
+@pytest.mark.parametrize("M,K,N", [(32, 1024, 12288), (20, 1024, 16400), (17, 576, 13000)])
+def test_rows17_32_wide_column_blocks(xh, orc, kind, M, K, N):
+    """At 17 .. 32 rows and more than two column tiles a CU, a workgroup takes 3 or 4 column tiles (one round over
+    the CUs): the 768 tiles of a 7B QKV projection, a ragged tile count whose last block is mostly past N, a
+    ragged K."""
+    print(f"case kind={kind} M={M} K={K} N={N}", flush=True)
+    k = {"int8": 0, "int8_asym": 0, "uint4": 1, "nf4": 2}[kind]
+    w = _weights(orc, k, K, N, 350 + M, asym_int8=(kind == "int8_asym"))
+    rng = np.random.default_rng(351 + M)
+    A = orc.round_bf16(rng.standard_normal((M, K)))
+    dw = xh.Weight(k, K, N, w.q, w.scale, w.zero)
+    exp = orc.qgemm(w, A)
+    got32 = _gemm(xh, orc, dw, A, M, K, N, xh.F32, lda=K + 8, ldc=N + 3)
+    assert np.abs(got32 - exp).max() < 2e-3, np.abs(got32 - exp).max()
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    exp_r = orc.qgemm(w, A, orc.EPI_RESIDENTIAL, res=res)
+    got_r = _gemm(xh, orc, dw, A, M, K, N, xh.F32, orc.EPI_RESIDENTIAL, None, res)
+    assert np.abs(got_r - exp_r).max() < 2e-3
+    dw.free()
+
+
+@pytest.mark.parametrize("kind", ["int8", "uint4", "nf4"])
+@pytest.mark.parametrize("M,K,I", [(32, 1024, 11008), (24, 1024, 6000), (18, 512, 4112)])
+def test_rows17_32_gateup_wide_column_blocks(xh, orc, kind, M, K, I):
+    """SwiGLU pairs at 17 .. 32 rows with 6 (1376 tiles, the 7B gate/up) and 4 column tiles a workgroup."""
+    print(f"case kind={kind} M={M} K={K} I={I}", flush=True)
+    k = {"int8": 0, "uint4": 1, "nf4": 2}[kind]
+    w = _weights(orc, k, K, 2 * I, 360)
+    rng = np.random.default_rng(361 + M)
+    A = orc.round_bf16(rng.standard_normal((M, K)))
+    dw = xh.Weight(k, K, 2 * I, w.q, w.scale, w.zero, flags=xh.WF_GATEUP)
+    a_dev = xh.DeviceBuffer.from_numpy(orc.to_bf16(A))
+    o_dev = xh.DeviceBuffer(M * I * 4)
+    xh.gemm_gateup_silu(dw, a_dev.ptr, M, K, o_dev.ptr, I, xh.F32)
+    xh.synchronize()
+    got = o_dev.to_numpy(np.float32, (M, I))
+    exp = orc.silu_sum(orc.qgemm(w, A))
+    assert np.abs(got - exp).max() < 2e-3 + 2e-4 * np.abs(exp).max()
+    dw.free()
+
+
 def test_rows17_64_bf16_weights_and_repeatability(xh, orc):
     """BF16 weights at 17 .. 64 rows; the summation order is fixed, so two runs agree to the bit."""
     rng = np.random.default_rng(340)

@@ -111,6 +111,8 @@ __constant__ float c_nf4_gemm[16] = XFTHIP_NF4_CODE_VALUES;
 // RMSNorm prologue in LDS (M <= 4, MT == 1, no K tail).  blockDim.x = 64 * (K slices).
 // ROPE: the RoPE + cache-append epilogue of the QKV projection with its paired column tiles
 // (a template flag, so that the plain kernels keep their affine tile addressing).
+// 8 waves (K slices) a workgroup; 16 for the one-tile blocks at 17 .. 32 rows, whose time is the chain of load
+// round trips over a wave's K slice
 template <int KIND, int NT, int MT, int U, bool NEED_SUM, bool KTAIL, bool NORM, bool ROPE>
 __global__ __launch_bounds__(512) void qgemm_skinny_kernel(SkinnyParams p) {
     static_assert(!NORM || (MT == 1 && !KTAIL), "the norm prologue covers M <= 4 without a K tail");
@@ -447,10 +449,13 @@ __global__ __launch_bounds__(512) void qgemm_skinny_kernel(SkinnyParams p) {
             }
             (void)qcols;
         } else if (!p.gateup) {
-            for (int v = threadIdx.x; v < ROWS * COLS; v += blockDim.x) {
-                const int m = v / COLS, c = v % COLS;
+            // up to two tiles: all lanes along the block's rows at once; more: tile by tile (a static index into
+            // the per-tile scales), 16 lanes along a row
+            constexpr int PASSES = NT <= 2 ? 1 : NT, PCOLS = NT <= 2 ? COLS : 16;
+            auto finish = [&](int t, int v) {
+                const int m = v / PCOLS, c = t * 16 + v % PCOLS;
                 const int np = nt0 * 16 + c;
-                if (m >= p.M || np >= p.N) continue;
+                if (m >= p.M || np >= p.N) return;
                 const float sumA = need_sum ? total_sum(m) : 0.0f;
                 float x = column_value(m, c, sumA);
                 switch (p.epi) {
@@ -473,13 +478,24 @@ __global__ __launch_bounds__(512) void qgemm_skinny_kernel(SkinnyParams p) {
                     default: break;
                 }
                 store_from_f32(p.C, p.c_dtype, (size_t)m * p.ldc + np, x);
+            };
+            if constexpr (PASSES == 1) {
+                for (int v = threadIdx.x; v < ROWS * COLS; v += blockDim.x) finish(0, v);
+            } else {
+#pragma unroll
+                for (int t = 0; t < PASSES; ++t) {
+#pragma unroll 1
+                    for (int v = threadIdx.x; v < ROWS * 16; v += blockDim.x) finish(t, v);
+                }
             }
         } else if constexpr (NT >= 2) {
             // tile pairs (2j, 2j+1) hold gate / up columns [16 j', 16 j' + 16)
             constexpr int PAIRS = NT / 2;
-            for (int v = threadIdx.x; v < ROWS * PAIRS * 16; v += blockDim.x) {
-                const int m = v / (PAIRS * 16), rr = v % (PAIRS * 16);
-                const int pr = rr >> 4, c = rr & 15;
+#pragma unroll
+            for (int pr = 0; pr < PAIRS; ++pr)
+#pragma unroll 1
+            for (int v = threadIdx.x; v < ROWS * 16; v += blockDim.x) {
+                const int m = v >> 4, c = v & 15;
                 const int out_col = (blk * PAIRS + pr) * 16 + c;
                 if (m >= p.M || out_col >= p.N / 2) continue;
                 const float sumA = need_sum ? total_sum(m) : 0.0f;
@@ -502,8 +518,9 @@ __global__ __launch_bounds__(512) void qgemm_skinny_kernel(SkinnyParams p) {
 
 // k tiles per load batch, sized so that two batches of weight + activation fragments stay in
 // registers (256 VGPRs per lane at 8 waves per block)
-template <int KIND, int MT>
+template <int KIND, int MT, int NT = 1>
 constexpr int batch_tiles() {
+    if (MT == 2 && NT >= 4) return 1; // wide column blocks: the weight registers of one k tile are a batch already
     if (KIND == XFTHIP_W_INT8) return MT == 1 ? 4 : 2;
     if (KIND == XFTHIP_W_BF16) return MT == 1 ? 4 : 2;
     return MT == 1 ? 2 : 1;
@@ -528,6 +545,12 @@ static int launch(const SkinnyParams &p, int kslices, hipStream_t stream) {
         const int cus = device_cu_count() * 2;
         blocks = blocks < cus ? blocks : cus;
     }
+    if (smem > 64 * 1024) {
+        // more dynamic LDS than the default limit (wide column blocks at 17 .. 32 rows): raise it once per instantiation
+        static const hipError_t attr = hipFuncSetAttribute((const void *)qgemm_skinny_kernel<KIND, NT, MT, U, NEED_SUM, KTAIL, NORM, ROPE>,
+                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        XFT_CHECK_HIP(attr);
+    }
     hipLaunchKernelGGL((qgemm_skinny_kernel<KIND, NT, MT, U, NEED_SUM, KTAIL, NORM, ROPE>), dim3(blocks), dim3(64 * kslices), smem,
             stream, q);
     XFT_CHECK_HIP(hipGetLastError());
@@ -536,7 +559,7 @@ static int launch(const SkinnyParams &p, int kslices, hipStream_t stream) {
 
 template <int KIND, int NT, int MT, bool NEED_SUM>
 static int dispatch_tail(const SkinnyParams &p, int kslices, hipStream_t stream) {
-    constexpr int U = batch_tiles<KIND, MT>();
+    constexpr int U = batch_tiles<KIND, MT, NT>();
     if (p.KT * KindTraits<KIND>::KTILE != p.K) {
         if (p.norm_x || p.rope) {
             set_error("qgemm_skinny: the fused prologue / epilogue needs K to be a whole number of weight tiles");
@@ -603,6 +626,18 @@ static int dispatch_shape(const SkinnyParams &p, hipStream_t stream) {
         if (wide) return dispatch_sum<KIND, 2, 1>(p, kslices, stream);
         return dispatch_sum<KIND, 1, 1>(p, kslices, stream);
     }
+    // 17 .. 32 rows: the kernel holds one workgroup a CU and a column block costs about the same time whether it
+    // is 16 or 96 columns wide (a chain of load round trips over the wave's K slice), so the blocks are made wide
+    // enough for one round over the CUs where the registers allow it: 3 tiles for the 768 of a 7B QKV projection
+    // (384 two-tile blocks took two rounds: 23.2 us), 6 for the 1376 of its gate/up
+    const int per_cu = (p.NTILES + cus - 1) / cus;
+    if (p.gateup) {
+        if (per_cu > 4) return dispatch_sum<KIND, 6, 2>(p, kslices, stream);
+        if (per_cu > 2) return dispatch_sum<KIND, 4, 2>(p, kslices, stream);
+        return dispatch_sum<KIND, 2, 2>(p, kslices, stream);
+    }
+    if (per_cu > 3) return dispatch_sum<KIND, 4, 2>(p, kslices, stream);
+    if (per_cu > 2) return dispatch_sum<KIND, 3, 2>(p, kslices, stream);
     if (wide) return dispatch_sum<KIND, 2, 2>(p, kslices, stream);
     return dispatch_sum<KIND, 1, 2>(p, kslices, stream);
 }

@@ -113,10 +113,16 @@ __constant__ float c_nf4_gemm[16] = XFTHIP_NF4_CODE_VALUES;
 // (a template flag, so that the plain kernels keep their affine tile addressing).
 // 8 waves (K slices) a workgroup; 16 for the one-tile blocks at 17 .. 32 rows, whose time is the chain of load
 // round trips over a wave's K slice
-template <int KIND, int NT, int MT, int U, bool NEED_SUM, bool KTAIL, bool NORM, bool ROPE>
-__global__ __launch_bounds__(512) void qgemm_skinny_kernel(SkinnyParams p) {
+// STAGE: activation rows are loaded as whole 128-byte runs (8 or 16 adjacent lanes along a row) and turned into
+// MFMA fragments through a wave-private LDS patch.  Loaded straight in fragment order a wave-load is 16 rows x
+// four 16-byte pieces, which the memory pipeline serves at a third of the rate of contiguous runs (37 against
+// 125 GB/s a CU from L2, measured): with more than a few rows those loads, not the weights, set the time.
+template <int KIND, int NT, int MT, int U, bool NEED_SUM, bool KTAIL, bool NORM, bool ROPE, bool STAGE = false>
+__global__ __launch_bounds__(512, (STAGE && MT == 1 && NT == 1) ? 4 : 1) void qgemm_skinny_kernel(SkinnyParams p) {
+    // (the one-tile staged form is held to 128 registers, two workgroups a CU like its unstaged twin)
     static_assert(!NORM || (MT == 1 && !KTAIL), "the norm prologue covers M <= 4 without a K tail");
     static_assert(!ROPE || (NT == 2 && MT == 1 && !KTAIL), "the RoPE epilogue works on tile pairs of up to 16 rows");
+    static_assert(!STAGE || (!NORM && !ROPE), "staged activation loads belong to the plain kernels");
     using T = KindTraits<KIND>;
     constexpr int MPT = T::MPT, KL = T::KL, KTILE = T::KTILE;
     extern __shared__ float smem[];
@@ -147,6 +153,12 @@ __global__ __launch_bounds__(512) void qgemm_skinny_kernel(SkinnyParams p) {
         __syncthreads();
     }
     float *red = smem + (KIND == XFTHIP_W_NF4 ? 512 : 0);
+    // STAGE: this wave's patch, [U][16 MT rows][KTILE bf16 + 16 bytes] (the pad keeps the fragment reads off each
+    // other's banks); it shares its LDS with the reduction area, which is used only after the K loop
+    constexpr int LPR = KTILE / 8, RPI = 64 / LPR; // lanes along a row, rows a wave-load
+    constexpr int SPITCH = KTILE * 2 + 16, STILE = 16 * MT * SPITCH;
+    unsigned char *stage = (unsigned char *)red + (size_t)wave * (U * STILE);
+    const int s_row = lane / LPR, s_kc = lane % LPR;
 
     // K slice of this wave: balanced split of the KT / U load batches
     const int nbatch = p.KT / U;
@@ -205,6 +217,15 @@ __global__ __launch_bounds__(512) void qgemm_skinny_kernel(SkinnyParams p) {
             abase[m] = p.A + (size_t)row * p.lda + g * KL;
         }
 
+        // STAGE: element offset of wave-load j of a k tile (row j * RPI + s_row, clamped) without the k part
+        uint32_t s_off[MT * MPT];
+#pragma unroll
+        for (int j = 0; j < MT * MPT; ++j) {
+            int row = j * RPI + s_row;
+            row = row < p.M ? row : p.M - 1;
+            s_off[j] = (uint32_t)row * (uint32_t)p.lda;
+        }
+
         const u32x4 zero4 = {0u, 0u, 0u, 0u};
         u32x4 abuf[2][U][MT][MPT];
 
@@ -216,6 +237,20 @@ __global__ __launch_bounds__(512) void qgemm_skinny_kernel(SkinnyParams p) {
                 for (int t = 0; t < NT; ++t)
                     wbuf[buf][u][t] = __builtin_nontemporal_load((const u32x4 *)(wbase[t] + (size_t)kt * 1024));
                 if constexpr (NORM) continue; // activations are read from LDS in compute()
+                if constexpr (STAGE) {
+#pragma unroll
+                    for (int j = 0; j < MT * MPT; ++j) {
+                        const int koff = kt * KTILE + s_kc * 8;
+                        if constexpr (KTAIL) {
+                            const bool v = koff + 8 <= p.K;
+                            const u32x4 a = *(const u32x4 *)(p.A + s_off[j] + (v ? koff : 0));
+                            abuf[buf][u][j / MPT][j % MPT] = v ? a : zero4;
+                        } else {
+                            abuf[buf][u][j / MPT][j % MPT] = *(const u32x4 *)(p.A + s_off[j] + koff);
+                        }
+                    }
+                    continue;
+                }
 #pragma unroll
                 for (int m = 0; m < MT; ++m) {
 #pragma unroll
@@ -236,6 +271,14 @@ __global__ __launch_bounds__(512) void qgemm_skinny_kernel(SkinnyParams p) {
         };
         auto compute = [&](int buf, int batch) {
             (void)batch;
+            if constexpr (STAGE) {
+                // rows as loaded into the patch; the fragments are read back below (same wave, in order)
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+#pragma unroll
+                    for (int j = 0; j < MT * MPT; ++j)
+                        *(u32x4 *)(stage + u * STILE + (j * RPI + s_row) * SPITCH + s_kc * 16) = abuf[buf][u][j / MPT][j % MPT];
+            }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
 #pragma unroll
@@ -245,6 +288,8 @@ __global__ __launch_bounds__(512) void qgemm_skinny_kernel(SkinnyParams p) {
                     for (int m = 0; m < MT; ++m) {
                         if constexpr (NORM)
                             a[m].q = *(const u32x4 *)(xn + xn_row + (batch * U + u) * KTILE + g * KL + 8 * i);
+                        else if constexpr (STAGE)
+                            a[m].q = *(const u32x4 *)(stage + u * STILE + (m * 16 + ml) * SPITCH + (g * KL + 8 * i) * 2);
                         else
                             a[m].q = abuf[buf][u][m][i];
                     }
@@ -361,6 +406,7 @@ __global__ __launch_bounds__(512) void qgemm_skinny_kernel(SkinnyParams p) {
 
         // ---- cross-wave reduction through LDS: red[wave][m][n] -------------------------------
         constexpr int ROWS = 16 * MT, COLS = 16 * NT, LD = COLS + 1;
+        if constexpr (STAGE) __syncthreads(); // the reduction area lies over the other waves' activation patches
         float *mine = red + (size_t)wave * (ROWS * LD + ROWS);
 #pragma unroll
         for (int t = 0; t < NT; ++t)
@@ -526,10 +572,15 @@ constexpr int batch_tiles() {
     return MT == 1 ? 2 : 1;
 }
 
-template <int KIND, int NT, int MT, int U, bool NEED_SUM, bool KTAIL, bool NORM, bool ROPE = false>
+template <int KIND, int NT, int MT, int U, bool NEED_SUM, bool KTAIL, bool NORM, bool ROPE = false, bool STAGE = false>
 static int launch(const SkinnyParams &p, int kslices, hipStream_t stream) {
     constexpr int ROWS = 16 * MT, COLS = 16 * NT;
-    size_t smem = (size_t)kslices * (ROWS * (COLS + 1) + ROWS) * sizeof(float) + (KIND == XFTHIP_W_NF4 ? 2048 : 0);
+    size_t smem = (size_t)kslices * (ROWS * (COLS + 1) + ROWS) * sizeof(float);
+    if (STAGE) {
+        const size_t patches = (size_t)kslices * U * ROWS * (KindTraits<KIND>::KTILE * 2 + 16);
+        smem = smem > patches ? smem : patches;
+    }
+    smem += (KIND == XFTHIP_W_NF4 ? 2048 : 0);
     if (NORM) smem += 64 + skinny_norm_lds_bytes(p.M, p.K);
     int blocks = (p.NTILES + NT - 1) / NT;
     if (ROPE) blocks = (p.qH + 2 * p.kvH) * 4; // rotation pairs of the query and key heads, then value tile pairs
@@ -547,11 +598,11 @@ static int launch(const SkinnyParams &p, int kslices, hipStream_t stream) {
     }
     if (smem > 64 * 1024) {
         // more dynamic LDS than the default limit (wide column blocks at 17 .. 32 rows): raise it once per instantiation
-        static const hipError_t attr = hipFuncSetAttribute((const void *)qgemm_skinny_kernel<KIND, NT, MT, U, NEED_SUM, KTAIL, NORM, ROPE>,
+        static const hipError_t attr = hipFuncSetAttribute((const void *)qgemm_skinny_kernel<KIND, NT, MT, U, NEED_SUM, KTAIL, NORM, ROPE, STAGE>,
                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         XFT_CHECK_HIP(attr);
     }
-    hipLaunchKernelGGL((qgemm_skinny_kernel<KIND, NT, MT, U, NEED_SUM, KTAIL, NORM, ROPE>), dim3(blocks), dim3(64 * kslices), smem,
+    hipLaunchKernelGGL((qgemm_skinny_kernel<KIND, NT, MT, U, NEED_SUM, KTAIL, NORM, ROPE, STAGE>), dim3(blocks), dim3(64 * kslices), smem,
             stream, q);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
@@ -565,7 +616,8 @@ static int dispatch_tail(const SkinnyParams &p, int kslices, hipStream_t stream)
             set_error("qgemm_skinny: the fused prologue / epilogue needs K to be a whole number of weight tiles");
             return 2;
         }
-        return launch<KIND, NT, MT, U, NEED_SUM, true, false>(p, kslices, stream);
+        if (MT == 2 || p.M > 4) return launch<KIND, NT, MT, U, NEED_SUM, true, false, false, true>(p, kslices, stream);
+        if constexpr (MT == 1) return launch<KIND, NT, MT, U, NEED_SUM, true, false>(p, kslices, stream);
     }
     if constexpr (MT == 1 && (KIND == XFTHIP_W_UINT4 || KIND == XFTHIP_W_NF4)) {
         // 4-bit codes with the norm prologue: no activation registers are needed, so a batch can
@@ -592,7 +644,10 @@ static int dispatch_tail(const SkinnyParams &p, int kslices, hipStream_t stream)
     if constexpr (MT == 1) {
         if (p.norm_x) return launch<KIND, NT, MT, U, NEED_SUM, false, true>(p, kslices, stream);
     }
-    return launch<KIND, NT, MT, U, NEED_SUM, false, false>(p, kslices, stream);
+    // more than a few rows: activation rows loaded as contiguous runs (see STAGE)
+    if (MT == 2 || p.M > 4) return launch<KIND, NT, MT, U, NEED_SUM, false, false, false, true>(p, kslices, stream);
+    if constexpr (MT == 1) return launch<KIND, NT, MT, U, NEED_SUM, false, false>(p, kslices, stream);
+    return 0;
 }
 
 template <int KIND, int NT, int MT>

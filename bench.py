@@ -457,10 +457,11 @@ def moe_layer(xh, iters=5):
     us_queued = (time.time() - t0) * 1e6 / (4 * iters)
     wbytes, flops = 8 * (4096 * 28672 + 14336 * 4096), 512 * 3 * 2 * 4096 * 14336
     moe.free()
-    return dict(tokens=T, experts=E, us_per_layer=round(us, 1), us_per_layer_no_wait=round(us_queued, 1), weight_gbs=round(wbytes / us / 1e3, 1),
-                frac_of_hbm_peak=round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4), tflops=round(flops / us / 1e6, 1),
+    return dict(tokens=T, experts=E, us_per_layer=round(us, 1), us_per_layer_no_wait=round(us_queued, 1),
+                weight_gbs=round(wbytes / us_queued / 1e3, 1), frac_of_hbm_peak=round(wbytes / us_queued / 1e3 / HBM_PEAK_GBS, 4),
+                tflops=round(flops / us_queued / 1e6, 1),
                 note="us_per_layer: wall time of xfthip_moe_forward with the routing copied back to the host (one wait a call); "
-                     "us_per_layer_no_wait: calls that return no routing, queued back to back (nothing waits: the row "
+                     "us_per_layer_no_wait (the rates are quoted on it): calls that return no routing, queued back to back (nothing waits: the row "
                      "counts stay on the device)")
 
 

@@ -72,7 +72,9 @@ struct StepTraits<XFTHIP_W_BF16> {
     static constexpr int KTILE = 32, GROUPS = 2, SUB = 1, WREGS = 4;
 };
 
-template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL>
+// DEVROWS: the row count (and, for a group of weights, the weight) comes from device memory (SkinnyParams::rows_dev /
+// group); a form of its own, so that the plain kernels carry none of it
+template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL, bool DEVROWS = false>
 __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nblocks_n, int nblocks_m) {
     using T = StepTraits<KIND>;
     constexpr int KTILE = T::KTILE, GROUPS = T::GROUPS, SUB = T::SUB, WREGS = T::WREGS;
@@ -97,9 +99,11 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
         // that do work then come first in the launch order and spread over the CUs; the ones past the count
         // (which leave at once) follow them instead of sitting between them.
         int BAND = 8;
-        if (p.rows_dev && !p.group) {
-            const int want = (p.m_hint + ROWS - 1) / ROWS;
-            BAND = want < 1 ? 1 : want < 8 ? want : 8;
+        if constexpr (DEVROWS) {
+            if (!p.group) {
+                const int want = (p.m_hint + ROWS - 1) / ROWS;
+                BAND = want < 1 ? 1 : want < 8 ? want : 8;
+            }
         }
         const int parts = p.ksplit > 1 ? p.ksplit : 1;
         const int id = blockIdx.y * gridDim.x + blockIdx.x, xcd = id & 7, slot = id >> 3; // gridDim.x is a multiple of 8
@@ -114,6 +118,7 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
         if (nb >= nblocks_n) return;
     }
     int c_row = 0, part_row = 0; // first row of this GEMM in C and in a K part
+    if constexpr (DEVROWS) {
     if (p.group) {
         // several weights of one shape behind one launch: the row blocks of all of them are numbered in a
         // row, weight after weight, by their device-side row counts; blocks past the last one leave
@@ -138,6 +143,7 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
         c_row = p.rows_dev[2]; // the K parts hold local rows, the kernel that adds them shifts
     }
     p.C = (char *)p.C + (size_t)c_row * p.ldc * (p.c_dtype == XFTHIP_F32 ? 4 : 2);
+    }
     if (p.ksplit > 1) {
         // this workgroup owns a range of k tiles: shift the operands to it, the result goes to its part
         const int kt0 = part * p.split_ktiles;
@@ -152,7 +158,9 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     }
     const int n32_0 = (nb * 4 + wave) * WN; // first 32-column tile of this wave
     const int m0 = mb * ROWS;
-    if (m0 >= p.M) return; // fewer rows than the grid was sized for (the whole workgroup leaves)
+    if constexpr (DEVROWS) {
+        if (m0 >= p.M) return; // fewer rows than the grid was sized for (the whole workgroup leaves)
+    }
 
     uint2 *lut = nullptr;
     unsigned char *abuf_base = lds;
@@ -590,7 +598,7 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     }
 }
 
-template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL>
+template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL, bool DEVROWS = false>
 static int launch_big2(const SkinnyParams &p, hipStream_t stream) {
     using T = StepTraits<KIND>;
     constexpr int ROWS = 32 * WM, ROWB = T::KTILE * 2 + 16;
@@ -605,11 +613,11 @@ static int launch_big2(const SkinnyParams &p, hipStream_t stream) {
     const size_t smem = (pipe > patches ? pipe : patches) + (KIND == XFTHIP_W_NF4 ? 2048 : 0);
     if (smem > 64 * 1024) {
         // more dynamic LDS than the default limit: raise it once per instantiation
-        static const hipError_t attr = hipFuncSetAttribute((const void *)qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL>,
+        static const hipError_t attr = hipFuncSetAttribute((const void *)qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL, DEVROWS>,
                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         XFT_CHECK_HIP(attr);
     }
-    hipLaunchKernelGGL((qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL>), dim3(blocks, p.ksplit > 1 ? p.ksplit : 1), dim3(256), smem, stream,
+    hipLaunchKernelGGL((qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL, DEVROWS>), dim3(blocks, p.ksplit > 1 ? p.ksplit : 1), dim3(256), smem, stream,
             p, nblocks_n, nblocks_m);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
@@ -617,6 +625,16 @@ static int launch_big2(const SkinnyParams &p, hipStream_t stream) {
 
 template <int KIND, int WN, int WM, bool NEED_SUM>
 static int launch_big(const SkinnyParams &p, hipStream_t stream) {
+    if (p.rows_dev) {
+        // device-side row counts: built for the 32- and 64-row tiles only (dispatch_big_tile picks no other then)
+        if constexpr (WN == 1 && WM <= 2) {
+            if (p.K % StepTraits<KIND>::KTILE != 0) return launch_big2<KIND, WN, WM, NEED_SUM, true, true>(p, stream);
+            return launch_big2<KIND, WN, WM, NEED_SUM, false, true>(p, stream);
+        } else {
+            set_error("qgemm_mfma: no device-side row count for this tile");
+            return 2;
+        }
+    }
     if (p.K % StepTraits<KIND>::KTILE != 0) return launch_big2<KIND, WN, WM, NEED_SUM, true>(p, stream);
     return launch_big2<KIND, WN, WM, NEED_SUM, false>(p, stream);
 }
@@ -634,6 +652,14 @@ static int dispatch_big_tile(const SkinnyParams &p, hipStream_t stream) {
     const long t_large = (long)((n32 + 7) / 8) * ((rows + 127) / 128);
     const long t_mid = (long)((n32 + 3) / 4) * ((rows + 127) / 128);
     const long t_small = (long)((n32 + 3) / 4) * ((rows + 63) / 64);
+    if (p.rows_dev) {
+        // 32- or 64-row tiles.  A group's weights with more than 32 rows each keep 64-row tiles: the 32-row ones
+        // read every weight tile twice, and with all the weights' workgroups side by side there is no CU left to fill.
+        if constexpr (KIND != XFTHIP_W_BF16) {
+            if (t_small < 2 * cus && !(p.group && p.M > 32 * p.group_n)) return launch_big<KIND, 1, 1, NEED_SUM>(p, stream);
+        }
+        return launch_big<KIND, 1, 2, NEED_SUM>(p, stream);
+    }
     if constexpr (KIND == XFTHIP_W_BF16) {
         if (t_large >= cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
         if (t_mid >= cus) return launch_big<KIND, 1, 4, NEED_SUM>(p, stream);
@@ -652,9 +678,7 @@ static int dispatch_big_tile(const SkinnyParams &p, hipStream_t stream) {
         // Few rows against a deep K (512 tokens x 4096 columns): 64-row tiles would leave one
         // workgroup per CU, whose k loop is then a chain of load latencies; 32-row tiles put two
         // on a CU.
-        // (a group's weights with more than 32 rows each keep 64-row tiles: the 32-row ones read every weight
-        // tile twice, and with all the weights' workgroups side by side there is no CU left to fill)
-        if (t_small < 2 * cus && !(p.group && p.M > 32 * p.group_n)) return launch_big<KIND, 1, 1, NEED_SUM>(p, stream);
+        if (t_small < 2 * cus) return launch_big<KIND, 1, 1, NEED_SUM>(p, stream);
         return launch_big<KIND, 1, 2, NEED_SUM>(p, stream);
     }
 }

@@ -331,14 +331,16 @@ def test_persistent_decode_matches_per_kernel_decode(xh, orc, B, S):
             break
 
 
-@pytest.mark.parametrize("kind,B", [(0, 1), (0, 3), (1, 2), (2, 4)])
+@pytest.mark.parametrize("kind,B", [(0, 1), (0, 3), (1, 2), (2, 4), (0, 9), (1, 16), (0, 24), (1, 32), (2, 17)])
 def test_fused_decode_step_matches_unfused(xh, orc, kind, B):
     """The decode-step fusions (RMSNorm as the GEMV prologue, RoPE + cache append as the QKV
     GEMV's epilogue) keep every bf16 hand-over point of the unfused step; only the fp32 summation
     order inside the norm differs.  Logits of every step within 1e-2, ids equal unless the
     top-2 logits are that close."""
     S, steps, vocab = 21, 10, 1000
-    model, _ = build_small_model(xh, orc, kind, 13, layers=3, B=4)
+    # (above 4 sequences only the rotation + cache append stays fused, with one pair of column tiles a block up
+    # to 16 sequences and two up to 32)
+    model, _ = build_small_model(xh, orc, kind, 13, layers=3, B=max(4, B))
     ids = np.random.default_rng(38).integers(0, vocab, (B, S)).astype(np.int32)
     runs = []
     for fused in (False, True):

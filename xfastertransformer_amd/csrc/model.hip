@@ -403,7 +403,7 @@ static int attention_block(xfthip_model *m, int idx, const float *x_in, int in_s
     const PackedWeight &wq = L.qkv->pw;
     const bool small = m->fuse_decode && wq.kind != XFTHIP_W_W8A8;
     const bool fuse_norm = small && do_norm && skinny_can_fuse_norm(wq, T);
-    const bool fuse_rope = small && S == 1 && T <= 16 && c.kv_dtype == XFTHIP_FP16 && !L.qkv_bias && c.head_size == 128
+    const bool fuse_rope = small && S == 1 && T <= 32 && c.kv_dtype == XFTHIP_FP16 && !L.qkv_bias && c.head_size == 128
             && wq.KT * ktile_of(wq.kind) == wq.K;
     if (!fuse_norm) {
         if (do_norm) {

@@ -27,8 +27,10 @@ int qgemm_skinny(const PackedWeight &pw, const SkinnyParams &p0, hipStream_t str
         set_error("qgemm_skinny: RMSNorm prologue not available for M=%d K=%d kind=%d", p.M, pw.K, pw.kind);
         return 2;
     }
-    if (p.rope && (p.M > 16 || p.gateup || (p.qH + 2 * p.kvH) * 128 != pw.N || p.kv.int8 != 0 || p.kv.D != 128)) {
-        set_error("qgemm_skinny: RoPE / cache-append epilogue needs M <= 16, head size 128, an FP16 cache and a [K, (q+2kv)*128] weight");
+    if (p.rope && (p.M > 32 || p.M > p.kv.B || p.kvH != p.kv.H || p.gateup || (p.qH + 2 * p.kvH) * 128 != pw.N || p.kv.int8 != 0 || p.kv.D != 128
+                || (p.M > 16 && p.norm_x))) {
+        set_error("qgemm_skinny: RoPE / cache-append epilogue needs M <= 32 rows (one per cache row), head size 128, an FP16 cache and a "
+                  "[K, (q+2kv)*128] weight");
         return 2;
     }
     p.packed = pw.packed;

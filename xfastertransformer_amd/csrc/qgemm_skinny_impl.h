@@ -121,7 +121,7 @@ template <int KIND, int NT, int MT, int U, bool NEED_SUM, bool KTAIL, bool NORM,
 __global__ __launch_bounds__(512, (STAGE && MT == 1 && NT == 1) ? 4 : 1) void qgemm_skinny_kernel(SkinnyParams p) {
     // (the one-tile staged form is held to 128 registers, two workgroups a CU like its unstaged twin)
     static_assert(!NORM || (MT == 1 && !KTAIL), "the norm prologue covers M <= 4 without a K tail");
-    static_assert(!ROPE || (NT == 2 && MT == 1 && !KTAIL), "the RoPE epilogue works on tile pairs of up to 16 rows");
+    static_assert(!ROPE || (NT % 2 == 0 && !KTAIL), "the RoPE epilogue works on tile pairs");
     static_assert(!STAGE || (!NORM && !ROPE), "staged activation loads belong to the plain kernels");
     using T = KindTraits<KIND>;
     constexpr int MPT = T::MPT, KL = T::KL, KTILE = T::KTILE;
@@ -173,8 +173,13 @@ __global__ __launch_bounds__(512, (STAGE && MT == 1 && NT == 1) ? 4 : 1) void qg
     int xn_row = 0;
     // column tile t of column block `it`; the RoPE epilogue pairs dims (d, d + 64) of a head, then V tiles
     const int rope_pairs = ROPE ? (p.qH + p.kvH) * 4 : 0;
+    // (a block holds NT / 2 such pairs; the pair count of the rotated heads is even, so no block straddles the
+    // border between rotated and value tiles when NT = 4)
     auto tile_index = [&](int it, int t) {
-        if constexpr (ROPE) return it < rope_pairs ? (it >> 2) * 8 + (it & 3) + 4 * t : (p.qH + p.kvH) * 8 + 2 * (it - rope_pairs) + t;
+        if constexpr (ROPE) {
+            const int pi = it * (NT / 2) + (t >> 1), tt = t & 1;
+            return pi < rope_pairs ? (pi >> 2) * 8 + (pi & 3) + 4 * tt : (p.qH + p.kvH) * 8 + 2 * (pi - rope_pairs) + tt;
+        }
         return it * NT + t;
     };
     // Every weight load is unconditional: out-of-range column tiles are clamped to the last valid
@@ -450,16 +455,17 @@ __global__ __launch_bounds__(512, (STAGE && MT == 1 && NT == 1) ? 4 : 1) void qg
 
         if constexpr (ROPE) {
             // one new token per sequence: row m is sequence m at position pos
-            const int it = blk;
-            const int qcols = p.qH * 128;
+#pragma unroll
+            for (int sub = 0; sub < NT / 2; ++sub) {
+            const int it = blk * (NT / 2) + sub, cofs = 32 * sub; // pair index, its first column in the block
             if (it < rope_pairs) {
                 const int hh = it >> 2, jj = it & 3;
                 for (int v = threadIdx.x; v < p.M * 16; v += blockDim.x) {
                     const int m = v >> 4, c = v & 15;
                     const float sumA = need_sum ? total_sum(m) : 0.0f;
                     // the projection's output is bf16 in the reference (the rotation reads it back)
-                    const float lo = bf16_to_f32(f32_to_bf16_ref(column_value(m, c, sumA)));
-                    const float hi = bf16_to_f32(f32_to_bf16_ref(column_value(m, 16 + c, sumA)));
+                    const float lo = bf16_to_f32(f32_to_bf16_ref(column_value(m, cofs + c, sumA)));
+                    const float hi = bf16_to_f32(f32_to_bf16_ref(column_value(m, cofs + 16 + c, sumA)));
                     int pos = p.pos_dev ? p.pos_dev[m] : p.pos_host;
                     pos = pos < 0 ? 0 : (pos >= p.kv.S ? p.kv.S - 1 : pos); // held inside the cache whatever the device value is
                     const int i = jj * 16 + c;
@@ -482,7 +488,7 @@ __global__ __launch_bounds__(512, (STAGE && MT == 1 && NT == 1) ? 4 : 1) void qg
                     const int m = v >> 5, cc = v & 31;
                     const int vt = 2 * (it - rope_pairs) + (cc >> 4);
                     const float sumA = need_sum ? total_sum(m) : 0.0f;
-                    const float val = bf16_to_f32(f32_to_bf16_ref(column_value(m, cc, sumA)));
+                    const float val = bf16_to_f32(f32_to_bf16_ref(column_value(m, cofs + cc, sumA)));
                     int pos = p.pos_dev ? p.pos_dev[m] : p.pos_host;
                     pos = pos < 0 ? 0 : (pos >= p.kv.S ? p.kv.S - 1 : pos);
                     if (pos < p.kv.S) {
@@ -493,7 +499,7 @@ __global__ __launch_bounds__(512, (STAGE && MT == 1 && NT == 1) ? 4 : 1) void qg
                     }
                 }
             }
-            (void)qcols;
+            }
         } else if (!p.gateup) {
             // up to two tiles: all lanes along the block's rows at once; more: tile by tile (a static index into
             // the per-tile scales), 16 lanes along a row
@@ -583,7 +589,7 @@ static int launch(const SkinnyParams &p, int kslices, hipStream_t stream) {
     smem += (KIND == XFTHIP_W_NF4 ? 2048 : 0);
     if (NORM) smem += 64 + skinny_norm_lds_bytes(p.M, p.K);
     int blocks = (p.NTILES + NT - 1) / NT;
-    if (ROPE) blocks = (p.qH + 2 * p.kvH) * 4; // rotation pairs of the query and key heads, then value tile pairs
+    if (ROPE) blocks = (p.qH + 2 * p.kvH) * 4 / (NT / 2); // rotation pairs of the query and key heads, then value tile pairs
     SkinnyParams q = p;
     q.nblocks = blocks;
     if (NORM) {
@@ -637,8 +643,12 @@ static int dispatch_tail(const SkinnyParams &p, int kslices, hipStream_t stream)
             return launch<KIND, NT, MT, U, NEED_SUM, false, false, true>(p, kslices, stream);
         }
     }
+    if constexpr (MT == 2 && NT == 4) {
+        // 17 .. 32 rows: two pairs a block, one round over the CUs for a 7B QKV projection
+        if (p.rope && !p.norm_x) return launch<KIND, NT, MT, U, NEED_SUM, false, false, true>(p, kslices, stream);
+    }
     if (p.rope) {
-        set_error("qgemm_skinny: the RoPE epilogue needs M <= 16");
+        set_error("qgemm_skinny: no RoPE epilogue for this shape");
         return 2;
     }
     if constexpr (MT == 1) {
@@ -686,6 +696,7 @@ static int dispatch_shape(const SkinnyParams &p, hipStream_t stream) {
     // enough for one round over the CUs where the registers allow it: 3 tiles for the 768 of a 7B QKV projection
     // (384 two-tile blocks took two rounds: 23.2 us), 6 for the 1376 of its gate/up
     const int per_cu = (p.NTILES + cus - 1) / cus;
+    if (p.rope) return dispatch_sum<KIND, 4, 2>(p, kslices, stream);
     if (p.gateup) {
         if (per_cu > 4) return dispatch_sum<KIND, 6, 2>(p, kslices, stream);
         if (per_cu > 2) return dispatch_sum<KIND, 4, 2>(p, kslices, stream);

@@ -237,6 +237,40 @@ def test_decode_batch64(xh, orc, int8, ctx):
         assert _cos(got[b], ref[0]) >= 0.9999
 
 
+@pytest.mark.parametrize("B,S,qh,kvh", [(4, 2048, 32, 8), (2, 1056, 16, 16), (3, 700, 8, 2)])
+def test_prefill_int8_cache_large(xh, orc, B, S, qh, kvh):
+    """Prefill over an INT8 cache at sizes that take the prefill kernel (codes widened on their way into LDS, key
+    scale on the score, value scale on the probability): sampled query rows must match float64 attention over
+    the cache the oracle quantises from the same rows (the device's append is bit-exact with it, tested elsewhere)."""
+    print(f"case B={B} S={S} qh={qh} kvh={kvh}", flush=True)
+    rng = np.random.default_rng(B * 1000 + S)
+    stride = (qh + 2 * kvh) * D
+    qkv = orc.round_bf16(rng.standard_normal((B * S, stride), dtype=np.float32))
+    # token scales that differ by orders of magnitude inside a block (the value-scale normalisation has work to do)
+    qkv[:, qh * D:] *= np.exp2(rng.integers(-6, 3, (B * S, 1))).astype(np.float32)
+    Sc = (S + 31) // 32 * 32
+    dc = xh.KVCache(xh.INT8, B, kvh, Sc, D)
+    dev = xh.DeviceBuffer.from_numpy(orc.to_bf16(qkv))
+    xh.rope_kvstore(dc, dev.ptr, xh.BF16, stride, B, S, qh, None, 0)
+    od = xh.DeviceBuffer(B * S * qh * D * 4)
+    xh.attention(dc, dev.ptr, stride, od.ptr, qh * D, xh.F32, B, S, qh, SCALE, 0)
+    xh.synchronize()
+    got = od.to_numpy(np.float32, (B * S, qh * D))
+    assert np.isfinite(got).all()
+    worst = 0.0
+    for b in range(B):
+        kc, vc = orc.KVCache(1, 1, kvh, Sc, D), orc.KVCache(1, 1, kvh, Sc, D)
+        kc.store(0, 0, qkv[b * S:(b + 1) * S, qh * D:(qh + kvh) * D].copy())
+        vc.store(0, 0, qkv[b * S:(b + 1) * S, (qh + kvh) * D:].copy())
+        K4, V4 = kc.as_f32()[:, :, :S], vc.as_f32()[:, :, :S]
+        for s in sorted({0, 1, 31, 32, 33, S // 2, S - 2, S - 1} | set(rng.integers(0, S, 4).tolist())):
+            q = qkv[b * S + s:b * S + s + 1, :qh * D].copy()
+            ref = orc.attention_ref_f64(q, np.ascontiguousarray(K4), np.ascontiguousarray(V4), qh, kvh, D, [1], [s], SCALE)
+            worst = max(worst, float(np.abs(got[b * S + s] - ref[0]).max()) / max(1.0, float(np.abs(ref[0]).max())))
+    print("int8 prefill worst relative max-abs over sampled rows", worst, flush=True)
+    assert worst < 3e-3
+
+
 @pytest.mark.parametrize("int8", [0, 1])
 def test_chunk_256_over_3840_cached(xh, orc, int8):
     """The attention block of the sparse-MLP configuration: 256 new tokens attend to 3840 cached rows

@@ -33,20 +33,12 @@ __global__ __launch_bounds__(256, 4) void attn_kernel(AttnParams p) {
     attn_unit<INT8, 4>(p, blockIdx.x, blockIdx.y % p.kv.H, blockIdx.y / p.kv.H, blockIdx.z, lds, [] { __syncthreads(); });
 }
 
-// prefill form: 4 waves = 4 neighbouring groups of 16 CT columns of one (sequence, KV head)
-template <bool INT8, int CT>
-__global__ __launch_bounds__(256, 2) void attn_prefill_kernel(AttnParams p) {
-    // the column groups that see the longest history are dispatched first (the causal triangle's long rows
-    // would otherwise start last and finish alone)
-    attn_prefill_unit<INT8, CT>(p, blockIdx.y, (gridDim.x - 1 - blockIdx.x) * 4 + (threadIdx.x >> 6), blockIdx.z);
-}
-
 // FP16 cache, K / V blocks shared through LDS: a workgroup = 64 CT neighbouring columns of one (sequence, KV head)
-template <int CT>
+template <int CT, bool INT8 = false>
 // launch bounds: three workgroups a CU with one column tile a wave (140 registers), two with two (216)
 __global__ __launch_bounds__(256, (CT == 1 ? 3 : 2)) void attn_prefill_lds_kernel(AttnParams p) {
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kPfBufBytes];
-    attn_prefill_lds_unit<CT>(p, blockIdx.y, gridDim.x - 1 - blockIdx.x, blockIdx.z, lds); // longest history first
+    attn_prefill_lds_unit<CT, INT8>(p, blockIdx.y, gridDim.x - 1 - blockIdx.x, blockIdx.z, lds); // longest history first
 }
 
 // Split-KV merge workspace: `slots` partial-result slots of kSlotFloats floats and one ticket per
@@ -156,8 +148,9 @@ int xfthip::attention_launch(xfthip_kvcache_t c, const void *q, int qStride, voi
                 if (ctl == 2) hipLaunchKernelGGL(attn_prefill_lds_kernel<2>, grid, dim3(256), 0, stream, p);
                 else hipLaunchKernelGGL(attn_prefill_lds_kernel<1>, grid, dim3(256), 0, stream, p);
             } else {
+                // INT8 cache: the same kernel, codes widened once per workgroup on their way into LDS
                 dim3 grid((p.CG + 3) / 4, c->kv.H, B);
-                hipLaunchKernelGGL((attn_prefill_kernel<true, 1>), grid, dim3(256), 0, stream, p);
+                hipLaunchKernelGGL((attn_prefill_lds_kernel<1, true>), grid, dim3(256), 0, stream, p);
             }
             XFT_CHECK_HIP(hipGetLastError());
             return 0;

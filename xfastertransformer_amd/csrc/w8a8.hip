@@ -6,6 +6,8 @@
 // The packed INT8 tile (16 columns x 64 rows, 16 K-consecutive codes per lane) is exactly the
 // "A" operand of v_mfma_i32_16x16x64_i8, so the weight goes from HBM to the matrix core without
 // a single ALU instruction; the quantised activation rows are the "B" operand.
+#include <mutex>
+
 #include "qgemm.h"
 
 // The dequantisation formula is evaluated as written (multiply, multiply, add): no contraction
@@ -603,6 +605,7 @@ static int launch_w8a8_mfma(const W8A8Params &p, hipStream_t stream) {
 static int8_t *g_qa = nullptr;
 static float *g_qstat = nullptr;
 static size_t g_qa_cap = 0, g_qstat_cap = 0;
+static std::mutex g_qa_mu;
 
 } // namespace xfthip
 
@@ -695,21 +698,25 @@ int xfthip_gemm_w8a8(xfthip_weight_t w, int M, const int8_t *qa, int ldq, const 
 namespace xfthip {
 
 // xfthip_gemm on a W8A8 weight: quantise the bf16 activations into a library-owned scratch, then
-// run the int8 GEMM.  The scratch grows with hipMalloc: not for use under stream capture.
+// run the int8 GEMM.  The scratch grows with hipMalloc (after waiting for the whole device: launches on any
+// stream may still read the old one), so a first call of a given size is not for use under stream capture; calls
+// that overlap on different streams share the scratch and must be serialised by the caller.  The model driver
+// keeps a scratch of its own, sized when the weights are attached.
 int gemm_w8a8_from_bf16(xfthip_weight_t w, int M, const void *A, int lda, void *C, int ldc, int c_dtype, int epilogue,
         const float *bias, const void *res, int ldres, int res_dtype, float gamma, hipStream_t stream) {
     const int K = w->pw.K;
     const int ldq = (K + 15) / 16 * 16;
     const size_t need = (size_t)M * ldq;
+    std::lock_guard<std::mutex> lk(g_qa_mu);
     if (need > g_qa_cap) {
-        XFT_CHECK_HIP(hipStreamSynchronize(stream));
+        XFT_CHECK_HIP(hipDeviceSynchronize());
         if (g_qa) (void)hipFree(g_qa);
         g_qa = nullptr;
         XFT_CHECK_HIP(hipMalloc((void **)&g_qa, need));
         g_qa_cap = need;
     }
     if ((size_t)M * 3 > g_qstat_cap) {
-        XFT_CHECK_HIP(hipStreamSynchronize(stream));
+        XFT_CHECK_HIP(hipDeviceSynchronize());
         if (g_qstat) (void)hipFree(g_qstat);
         g_qstat = nullptr;
         XFT_CHECK_HIP(hipMalloc((void **)&g_qstat, (size_t)M * 3 * sizeof(float)));

@@ -411,22 +411,24 @@ def attention_sweep(xh, iters=10):
                                 gbs=round(byts / us / 1e3, 1), frac_of_hbm_peak=round(byts / us / 1e3 / HBM_PEAK_GBS, 4)))
             cache.free()
     B, S = 4, 2048
-    cache = xh.KVCache(xh.FP16, B, kvh, S, D)
     stride = (qh + 2 * kvh) * D
-    qkv = xh.DeviceBuffer(B * S * stride * 2)
-    qkv.zero()
+    # N(0, 1) rows (bf16): the running maxima move as they do on real activations (all-zero rows never rescale)
+    qkv = xh.DeviceBuffer.from_numpy(xh.f32_to_bf16_bits(np.random.default_rng(5).standard_normal((B * S, stride), dtype=np.float32)))
     o = xh.DeviceBuffer(B * S * qh * D * 2)
-    xh.rope_kvstore(cache, qkv.ptr, xh.BF16, stride, B, S, qh, None, 0)
-    xh.attention(cache, qkv.ptr, stride, o.ptr, qh * D, xh.BF16, B, S, qh, scale, 0)
-    xh.synchronize()
-    t = xh.Timer()
-    t.start()
-    for _ in range(3):
-        xh.attention(cache, qkv.ptr, stride, o.ptr, qh * D, xh.BF16, B, S, qh, scale, 0)
-    us = t.stop() * 1e3 / 3
     flops = 4.0 * B * qh * S * S * D / 2
-    out.append(dict(phase="prefill", kv="fp16", batch=B, seq=S, avg_launch_us=round(us, 1), tflops=round(flops / us / 1e6, 1),
-                    frac_of_bf16_mfma_peak=round(flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)))
+    for int8 in (0, 1):
+        cache = xh.KVCache(xh.INT8 if int8 else xh.FP16, B, kvh, S, D)
+        xh.rope_kvstore(cache, qkv.ptr, xh.BF16, stride, B, S, qh, None, 0)
+        xh.attention(cache, qkv.ptr, stride, o.ptr, qh * D, xh.BF16, B, S, qh, scale, 0)
+        xh.synchronize()
+        t = xh.Timer()
+        t.start()
+        for _ in range(3):
+            xh.attention(cache, qkv.ptr, stride, o.ptr, qh * D, xh.BF16, B, S, qh, scale, 0)
+        us = t.stop() * 1e3 / 3
+        out.append(dict(phase="prefill", kv="int8" if int8 else "fp16", batch=B, seq=S, avg_launch_us=round(us, 1),
+                        tflops=round(flops / us / 1e6, 1), frac_of_bf16_mfma_peak=round(flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4)))
+        cache.free()
     return out
 
 

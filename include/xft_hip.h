@@ -480,8 +480,10 @@ int xfthip_moe_top2(const float *logits, int M, int E, int *sel, float *weights,
  * starts as the input (residual).  Replaces MixtralMLP::forward (mlp_mixtral.h:85-187).  Expert
  * weights: gateup [hidden, 2*intermediate] created with XFTHIP_WF_GATEUP, down [intermediate, hidden].
  * logits_override: optional device fp32 [tokens, experts] used instead of the router GEMM.
- * sel_host_out / w_host_out: optional host copies of the routing decision.
- * The call synchronises the stream once (the per-expert row counts size the expert GEMMs).
+ * sel_host_out / w_host_out: optional host copies of the routing decision; asking for either makes the call
+ * wait for the stream once.  Without them the call only enqueues work (the per-expert row counts stay in device
+ * memory, where the expert GEMMs read them) and may be recorded into a graph.  The workspace of one xfthip_moe
+ * serves one call at a time: calls on the same object must be ordered on one stream.
  */
 int xfthip_moe_create(int hidden, int intermediate, int experts, int max_tokens, const float *router_host, const float *ln_host,
         xfthip_moe_t *out);

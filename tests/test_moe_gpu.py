@@ -112,6 +112,40 @@ def test_mixtral_mlp_four_bit_experts(xh, orc, kind, tokens):
     assert np.abs(got - exp).max() < 2e-2 and _cos(got, exp) >= 0.9999
 
 
+@pytest.mark.parametrize("tokens", [6, 40])
+def test_mixtral_mlp_bf16_experts(xh, orc, tokens):
+    """BF16 expert weights (no codes to widen), per-expert launches and the launch that serves all experts: against a
+    float64 restatement with the same bf16 hand-over points (normalised input, hidden activations)."""
+    hidden, inter, E = 512, 1024, 8
+    rng = np.random.default_rng(500 + tokens)
+    Wgu = [orc.round_bf16(rng.standard_normal((hidden, 2 * inter)) * 0.05) for _ in range(E)]
+    Wdn = [orc.round_bf16(rng.standard_normal((inter, hidden)) * 0.05) for _ in range(E)]
+    ln = rng.uniform(0.8, 1.2, hidden).astype(np.float32)
+    x = orc.round_bf16(rng.standard_normal((tokens, hidden)))
+    lo = rng.standard_normal((tokens, E)).astype(np.float32)
+    moe = xh.MoE(hidden, inter, E, tokens, np.zeros((hidden, E), np.float32), ln)
+    for e in range(E):
+        moe.set_expert(e, xh.Weight(xh.W_BF16, hidden, 2 * inter, orc.to_bf16(Wgu[e]), flags=xh.WF_GATEUP),
+                       xh.Weight(xh.W_BF16, inter, hidden, orc.to_bf16(Wdn[e])))
+    xd, lod = xh.DeviceBuffer.from_numpy(x), xh.DeviceBuffer.from_numpy(lo)
+    od = xh.DeviceBuffer(x.nbytes)
+    sel, w = moe.forward(xd.ptr, od.ptr, tokens, True, lod.ptr)
+    xh.synchronize()
+    got = od.to_numpy(np.float32, x.shape)
+    esel, ew = orc.moe_top2(lo)
+    assert np.array_equal(sel, esel) and np.abs(w - ew).max() < 1e-6
+    xn = orc.round_bf16(orc.rmsnorm(x, ln)).astype(np.float64)
+    exp = x.astype(np.float64).copy()
+    for t in range(tokens):
+        for s_ in range(2):
+            e = int(esel[t, s_])
+            gu = xn[t] @ Wgu[e].astype(np.float64)
+            g, u = gu[:inter], gu[inter:]
+            h = orc.round_bf16((g / (1.0 + np.exp(-g)) * u).astype(np.float32)[None])[0].astype(np.float64)
+            exp[t] += float(ew[t, s_]) * (h @ Wdn[e].astype(np.float64))
+    assert np.abs(got - exp).max() < 2e-2 and _cos(got, exp) >= 0.9999
+
+
 def test_mixtral_shape_full_size_spot_check(xh, orc):
     """Mixtral-8x7B shape (hidden 4096, FFN 14336, 8 INT8 experts, 256 tokens, overridden N(0,1)
     logits): routing must equal the oracle's, and a handful of tokens are recomputed by the oracle."""

@@ -20,12 +20,15 @@ __device__ inline float silu_split(float x) {
     return x / (1.0f + fast_exp(-x));
 }
 
-// One thread per output value: the K parts are added in order (the same result on every run), then the
-// epilogue of the call.  p.C / p.ldc / p.c_dtype / p.epi are the caller's.
+// One thread per VEC neighbouring output values of a row (4 where N allows 16-byte part loads, else 1): the K parts are
+// added in order (the same result on every run), then the epilogue of the call.  p.C / p.ldc / p.c_dtype / p.epi are
+// the caller's.
+template <int VEC>
 __global__ __launch_bounds__(256) void qgemm_split_finish_kernel(SkinnyParams p) {
+    const int nv = p.N / VEC;
     const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (size_t)p.M * p.N) return;
-    const int m = (int)(idx / p.N), n = (int)(idx - (size_t)m * p.N);
+    if (idx >= (size_t)p.M * nv) return;
+    const int m = (int)(idx / nv), n0 = (int)(idx - (size_t)m * nv) * VEC;
     int row_out = m;
     if (p.group) {
         // the parts hold the rows where C holds them; rows past the last weight's were never written
@@ -36,28 +39,59 @@ __global__ __launch_bounds__(256) void qgemm_split_finish_kernel(SkinnyParams p)
         if (m >= p.rows_dev[0]) return;
         row_out = m + p.rows_dev[2];
     }
-    float x = 0.0f;
-    for (int s = 0; s < p.ksplit; ++s) x += p.split_part[((size_t)s * p.M + m) * p.N + n];
-    switch (p.epi) {
-        case XFTHIP_EPI_BIAS: x += p.bias[n]; break;
-        case XFTHIP_EPI_SILU: x = silu_split(x); break;
-        case XFTHIP_EPI_GELU: {
-            const float e = fast_exp(1.702f * x);
-            x = e / (e + 1.0f) * x;
-            break;
+    float x[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) x[v] = 0.0f;
+    for (int s = 0; s < p.ksplit; ++s) {
+        const float *src = p.split_part + ((size_t)s * p.M + m) * p.N + n0;
+        if constexpr (VEC == 4) {
+            const float4 t = *(const float4 *)src;
+            x[0] += t.x, x[1] += t.y, x[2] += t.z, x[3] += t.w;
+        } else {
+            x[0] += src[0];
         }
-        case XFTHIP_EPI_RESMUL: x *= load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + n); break;
-        case XFTHIP_EPI_RESIDENTIAL:
-            if (p.bias) x += p.bias[n];
-            x += load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + n);
-            break;
-        case XFTHIP_EPI_RESEXT:
-            if (p.bias) x += p.bias[n];
-            x = fmaf(p.gamma, load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + n), x);
-            break;
-        default: break;
     }
-    store_from_f32(p.C, p.c_dtype, (size_t)row_out * p.ldc + n, x);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+        const int n = n0 + v;
+        float y = x[v];
+        switch (p.epi) {
+            case XFTHIP_EPI_BIAS: y += p.bias[n]; break;
+            case XFTHIP_EPI_SILU: y = silu_split(y); break;
+            case XFTHIP_EPI_GELU: {
+                const float e = fast_exp(1.702f * y);
+                y = e / (e + 1.0f) * y;
+                break;
+            }
+            case XFTHIP_EPI_RESMUL: y *= load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + n); break;
+            case XFTHIP_EPI_RESIDENTIAL:
+                if (p.bias) y += p.bias[n];
+                y += load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + n);
+                break;
+            case XFTHIP_EPI_RESEXT:
+                if (p.bias) y += p.bias[n];
+                y = fmaf(p.gamma, load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + n), y);
+                break;
+            default: break;
+        }
+        x[v] = y;
+    }
+    const size_t ci = (size_t)row_out * p.ldc + n0;
+    if constexpr (VEC == 4) {
+        // whole 16-byte (fp32) or 8-byte (16-bit) stores where the row start allows them
+        if (p.c_dtype == XFTHIP_F32 && ((((uintptr_t)p.C) | ((size_t)p.ldc * 4)) & 15) == 0) {
+            *(float4 *)((float *)p.C + ci) = make_float4(x[0], x[1], x[2], x[3]);
+            return;
+        }
+        if (p.c_dtype == XFTHIP_BF16 && ((((uintptr_t)p.C) | ((size_t)p.ldc * 2)) & 7) == 0) {
+            const uint32_t lo = f32_to_bf16_ref(x[0]) | ((uint32_t)f32_to_bf16_ref(x[1]) << 16);
+            const uint32_t hi = f32_to_bf16_ref(x[2]) | ((uint32_t)f32_to_bf16_ref(x[3]) << 16);
+            *(uint2 *)((uint16_t *)p.C + ci) = make_uint2(lo, hi);
+            return;
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) store_from_f32(p.C, p.c_dtype, ci + v, x[v]);
 }
 
 // Partial results of the K split: one buffer per process and device, allocated once at its upper bound (a
@@ -137,7 +171,10 @@ int qgemm_mfma(const PackedWeight &pw, const SkinnyParams &p0, hipStream_t strea
     }
     if (rc || p.ksplit <= 1) return rc;
     const size_t outs = (size_t)p.M * p.N;
-    hipLaunchKernelGGL(qgemm_split_finish_kernel, dim3((unsigned)((outs + 255) / 256)), dim3(256), 0, stream, p);
+    if (p.N % 4 == 0) // the parts are [M][N] fp32 in a 256-byte aligned buffer: 16-byte loads need only N % 4 == 0
+        hipLaunchKernelGGL(qgemm_split_finish_kernel<4>, dim3((unsigned)((outs / 4 + 255) / 256)), dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL(qgemm_split_finish_kernel<1>, dim3((unsigned)((outs + 255) / 256)), dim3(256), 0, stream, p);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }

@@ -599,7 +599,8 @@ static int launch(const SkinnyParams &p, int kslices, hipStream_t stream) {
         // projection as 384 workgroups 13.6 us against 14.9 as 256 workgroups looping; the 688 blocks
         // of gate/up as 512 workgroups 20.0 us against 21.3 as 256 and 24.7 as 688 (every workgroup
         // pays the prologue).
-        const int cus = device_cu_count() * 2;
+        // (workgroups of at most 4 waves, the 4-bit kinds at K = 4096: four a CU, UINT4 decode 550 -> 567 tok/s)
+        const int cus = device_cu_count() * (kslices <= 4 ? 4 : 2);
         blocks = blocks < cus ? blocks : cus;
     }
     if (smem > 64 * 1024) {

@@ -601,6 +601,8 @@ def main():
         for k2, b2 in ((0, 32), (1, 1), (1, 32)):
             if (k2, b2) != (kind, B):
                 extra["decode"].append(decode_run(xh, k2, b2, args.prompt, 64, 8))
+        # the INT8 KV cache at the batch where the cache is most of the step's bytes
+        extra["decode"].append(decode_run(xh, 0, 32, args.prompt, 64, 8, kv_int8=True))
         extra["prefill_gemm"] = prefill_gemm_sweep(xh, 2048)
         extra["attention"] = attention_sweep(xh)
         extra["moe"] = moe_layer(xh)

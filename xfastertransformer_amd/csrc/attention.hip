@@ -24,11 +24,14 @@
 
 namespace xfthip {
 
-// launch bounds: four workgroups a CU (128 registers, nothing spilled): over an FP16 cache 0.52 -> 0.71 of the HBM
-// peak at batch 64 over 16384 tokens; an INT8 block is kept as codes and widened at its MFMA to fit (16 x 4096 tokens
-// 57 -> 42 us; the longest INT8 cases stay bound by the widening and softmax arithmetic)
+// launch bounds: three workgroups a CU.  The next block's keys are requested as soon as this block's scores are
+// scaled and its values once this block's P.V products are issued, into the registers those have just left; at 128
+// registers (four workgroups a CU) the compiler spills to keep that order and everything is slower, at 168 it fits
+// (146 FP16, 168 INT8).  Against four workgroups a CU that request each block only when they need it: INT8 cache,
+// batch 64 x 16384 tokens 594 -> 388 us (5.7 TB/s), 16 x 4096 42 -> 30 us; FP16 725 -> 713 us (6.0 TB/s), 16 x 4096
+// 61 -> 44 us, 64 x 1024 58 -> 48 us.
 template <bool INT8>
-__global__ __launch_bounds__(256, 4) void attn_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, 3) void attn_kernel(AttnParams p) {
     __shared__ AttnLds<4> lds;
     attn_unit<INT8, 4>(p, blockIdx.x, blockIdx.y % p.kv.H, blockIdx.y / p.kv.H, blockIdx.z, lds, [] { __syncthreads(); });
 }
@@ -189,7 +192,7 @@ int xfthip::attention_launch(xfthip_kvcache_t c, const void *q, int qStride, voi
 
 int xfthip::attention_split_count(int len, int units) {
     const int nblk = (len + 31) / 32;
-    int nsplit = (4 * device_cu_count() + units - 1) / units;
+    int nsplit = (3 * device_cu_count() + units - 1) / units; // three workgroups a CU are resident
     const int cap = (nblk + 3) / 4;
     if (nsplit > cap) nsplit = cap;
     if (nsplit > 64) nsplit = 64;

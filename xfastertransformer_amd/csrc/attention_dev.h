@@ -103,8 +103,9 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
     wg_begin = wg_begin < wg_end ? wg_begin : wg_end;
     const int wn = wg_end - wg_begin;
     const int wbase = wn / NW, wrem = wn % NW;
-    const int blk_begin = wg_begin + wave * wbase + (wave < wrem ? wave : wrem);
-    const int blk_end = blk_begin + wbase + (wave < wrem ? 1 : 0);
+    // (the same for every lane of a wave: scalar values, so that the loop and its load branches are uniform)
+    const int blk_begin = __builtin_amdgcn_readfirstlane(wg_begin + wave * wbase + (wave < wrem ? wave : wrem));
+    const int blk_end = __builtin_amdgcn_readfirstlane(blk_begin + wbase + (wave < wrem ? 1 : 0));
 
     const size_t bh = (size_t)b * p.kv.H + kvh;
     const ATTN_GLOBAL char *kbase = (const ATTN_GLOBAL char *)p.kv.k + bh * p.kv.S * D * (INT8 ? 1 : 2);
@@ -119,7 +120,10 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
     u32x4 kraw[INT8 ? 2 : 1][INT8 ? 2 : 1];
     u32x2 vraw[INT8 ? 8 : 1];
     f32x4 ks[2], vs[2];
-    auto load_block = [&](const int blk) {
+    // The keys of block blk + 1 are requested as soon as the scores of block blk are scaled (the key registers and
+    // key scales are free then) and its values once the P.V products of block blk are issued: the next block
+    // travels while this one goes through the softmax and the value products, in the same registers.
+    auto load_keys = [&](const int blk) {
         const int t0 = blk << 5;
         if constexpr (INT8) {
 #pragma unroll
@@ -128,10 +132,7 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
 #pragma unroll
                 for (int j = 0; j < 2; ++j) kraw[a][j] = *(const ATTN_GLOBAL u32x4 *)(row + 64 * j);
                 ks[a] = *(const ATTN_GLOBAL f32x4 *)(ksc + t0 + 16 * a + 4 * g);
-                vs[a] = *(const ATTN_GLOBAL f32x4 *)(vsc + t0 + 16 * a + 4 * g);
             }
-#pragma unroll
-            for (int dt = 0; dt < 8; ++dt) vraw[dt] = *(const ATTN_GLOBAL u32x2 *)(vbase + ((size_t)blk * D + 16 * dt + cl) * 32 + 8 * g);
         } else {
 #pragma unroll
             for (int a = 0; a < 2; ++a) {
@@ -139,6 +140,16 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
 #pragma unroll
                 for (int s = 0; s < 4; ++s) kf[a][s].q = *(const ATTN_GLOBAL u32x4 *)(row + 64 * s);
             }
+        }
+    };
+    auto load_values = [&](const int blk) {
+        const int t0 = blk << 5;
+        if constexpr (INT8) {
+#pragma unroll
+            for (int a = 0; a < 2; ++a) vs[a] = *(const ATTN_GLOBAL f32x4 *)(vsc + t0 + 16 * a + 4 * g);
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt) vraw[dt] = *(const ATTN_GLOBAL u32x2 *)(vbase + ((size_t)blk * D + 16 * dt + cl) * 32 + 8 * g);
+        } else {
 #pragma unroll
             for (int dt = 0; dt < 8; ++dt) {
                 const ATTN_GLOBAL char *src = vbase + (((size_t)blk * D + 16 * dt + cl) * 32 + 8 * g) * 2;
@@ -163,7 +174,10 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
             }
         }
     }
-    if (blk_begin < blk_end) load_block(blk_begin);
+    if (blk_begin < blk_end) {
+        load_keys(blk_begin);
+        load_values(blk_begin);
+    }
 #pragma unroll
     for (int s = 0; s < 4; ++s)
 #pragma unroll
@@ -179,7 +193,6 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
 
     for (int blk = blk_begin; blk < blk_end; ++blk) {
         const int t0 = blk << 5;
-        if (blk != blk_begin) load_block(blk);
 
         // ---- scores S^T[token = t0 + 16a + 4g + r][col] ----
         f32x4 sc[2];
@@ -212,6 +225,9 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
                 sc[a][r] = x;
                 bmax = fmaxf(bmax, vis[a][r] ? x : kNegBig);
             }
+        __builtin_amdgcn_sched_barrier(0);
+        if (blk + 1 < blk_end) load_keys(blk + 1);
+        __builtin_amdgcn_sched_barrier(0);
         // column max across the 4 lane groups
         bmax = fmaxf(bmax, __shfl_xor(bmax, 16, 64));
         bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
@@ -260,6 +276,9 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
                 o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[dt].v, pf.v, o[dt], 0, 0, 0);
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
+        if (blk + 1 < blk_end) load_values(blk + 1);
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     // ---- merge the 4 waves in LDS ----

@@ -30,10 +30,12 @@ namespace xfthip {
 // (146 FP16, 168 INT8).  Against four workgroups a CU that request each block only when they need it: INT8 cache,
 // batch 64 x 16384 tokens 594 -> 388 us (5.7 TB/s), 16 x 4096 42 -> 30 us; FP16 725 -> 713 us (6.0 TB/s), 16 x 4096
 // 61 -> 44 us, 64 x 1024 58 -> 48 us.
-template <bool INT8>
+// With at most one block a wave (short contexts at small batches) nothing can be requested ahead: that form keeps
+// the plain order, the shorter program (few workgroups then: the same launch bounds do no harm).
+template <bool INT8, bool PIPE>
 __global__ __launch_bounds__(256, 3) void attn_kernel(AttnParams p) {
     __shared__ AttnLds<4> lds;
-    attn_unit<INT8, 4>(p, blockIdx.x, blockIdx.y % p.kv.H, blockIdx.y / p.kv.H, blockIdx.z, lds, [] { __syncthreads(); });
+    attn_unit<INT8, 4, PIPE>(p, blockIdx.x, blockIdx.y % p.kv.H, blockIdx.y / p.kv.H, blockIdx.z, lds, [] { __syncthreads(); });
 }
 
 // FP16 cache, K / V blocks shared through LDS: a workgroup = 64 CT neighbouring columns of one (sequence, KV head)
@@ -182,10 +184,15 @@ int xfthip::attention_launch(xfthip_kvcache_t c, const void *q, int qStride, voi
     p.ws = wsp ? wsp->ws : nullptr;
     p.tickets = wsp ? wsp->tickets : nullptr;
     dim3 grid(nsplit, c->kv.H * p.CG, B);
-    if (c->kv.int8)
-        hipLaunchKernelGGL(attn_kernel<true>, grid, dim3(256), 0, stream, p);
-    else
-        hipLaunchKernelGGL(attn_kernel<false>, grid, dim3(256), 0, stream, p);
+    // more than one 32-token block a wave somewhere: the form that requests blocks ahead
+    const bool pipe = (len + 31) / 32 > 4 * nsplit;
+    if (c->kv.int8) {
+        if (pipe) hipLaunchKernelGGL((attn_kernel<true, true>), grid, dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL((attn_kernel<true, false>), grid, dim3(256), 0, stream, p);
+    } else {
+        if (pipe) hipLaunchKernelGGL((attn_kernel<false, true>), grid, dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL((attn_kernel<false, false>), grid, dim3(256), 0, stream, p);
+    }
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }

@@ -68,7 +68,9 @@ struct AttnLds {
 // the XCD and costs several microseconds per launch.  It also lets the unit run inside a kernel
 // whose other workgroups produced q and will consume the output in the same launch (the cache
 // rows appended in that launch must then have been written with st_dev as well).
-template <bool INT8, int NW, typename Sync>
+// PIPE: request the next block behind the current block's arithmetic (pays once a wave walks several blocks; with
+// one block a wave the plain order is the shorter program)
+template <bool INT8, int NW, bool PIPE, typename Sync>
 __device__ inline void attn_unit(const AttnParams &p, const int split, const int kvh, const int cg, const int b, AttnLds<NW> &L,
         const Sync &wg_sync) {
     constexpr int D = 128;
@@ -193,6 +195,12 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
 
     for (int blk = blk_begin; blk < blk_end; ++blk) {
         const int t0 = blk << 5;
+        if constexpr (!PIPE) {
+            if (blk != blk_begin) {
+                load_keys(blk);
+                load_values(blk);
+            }
+        }
 
         // ---- scores S^T[token = t0 + 16a + 4g + r][col] ----
         f32x4 sc[2];
@@ -225,9 +233,11 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
                 sc[a][r] = x;
                 bmax = fmaxf(bmax, vis[a][r] ? x : kNegBig);
             }
-        __builtin_amdgcn_sched_barrier(0);
-        if (blk + 1 < blk_end) load_keys(blk + 1);
-        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (PIPE) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (blk + 1 < blk_end) load_keys(blk + 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         // column max across the 4 lane groups
         bmax = fmaxf(bmax, __shfl_xor(bmax, 16, 64));
         bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
@@ -276,9 +286,11 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
                 o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[dt].v, pf.v, o[dt], 0, 0, 0);
             }
         }
-        __builtin_amdgcn_sched_barrier(0);
-        if (blk + 1 < blk_end) load_values(blk + 1);
-        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (PIPE) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (blk + 1 < blk_end) load_values(blk + 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
 
     // ---- merge the 4 waves in LDS ----

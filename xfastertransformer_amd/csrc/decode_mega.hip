@@ -535,7 +535,7 @@ __device__ inline void attention_phase(const MegaParams &p, int layer, AttnLds<8
     const int units = p.M * p.kvH * p.nsplit;
     for (int it = blockIdx.x; it < units; it += gridDim.x) {
         const int split = it % p.nsplit, kvh = (it / p.nsplit) % p.kvH, b = it / (p.nsplit * p.kvH);
-        attn_unit<false, 8>(ap, split, kvh, 0, b, lds, [] { __syncthreads(); });
+        attn_unit<false, 8, false>(ap, split, kvh, 0, b, lds, [] { __syncthreads(); });
         __syncthreads();
     }
 }

@@ -232,3 +232,15 @@ def test_layer_without_routing_output_is_capturable(xh, orc):
         assert np.array_equal(od.to_numpy(np.float32, xs[i].shape), eager[i]), i
     graph.free()
     side.free()
+
+
+def test_graph_helpers_reject_the_null_stream(xh):
+    """Capture needs a stream of the caller's own: the null stream and null handles are refused with a message,
+    nothing is recorded."""
+    import ctypes as C
+    assert xh.lib.xfthip_graph_begin(None) != 0
+    assert b"null stream" in xh.lib.xfthip_last_error()
+    g = C.c_void_p()
+    assert xh.lib.xfthip_graph_end(None, C.byref(g)) != 0
+    assert xh.lib.xfthip_graph_launch(None, None) != 0
+    assert xh.lib.xfthip_graph_destroy(None) == 0

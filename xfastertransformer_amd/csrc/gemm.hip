@@ -38,11 +38,11 @@ int gemm_rows_dev(xfthip_weight_t w, int m_max, int m_hint, const int *rows_dev,
     return qgemm_mfma(pw, p, stream);
 }
 
-int gemm_grouped_rows_dev(const xfthip_weight_t *w, int n_group, const GroupWeight *table_dev, int rows_max, const int *rows_dev,
-        int rows_stride, const void *A, int lda, void *C, int ldc, int c_dtype, hipStream_t stream) {
+int gemm_grouped_rows_dev(const xfthip_weight_t *w, int n_group, const GroupWeight *table_dev, int rows_max, int rows_each_max,
+        const int *rows_dev, int rows_stride, const void *A, int lda, void *C, int ldc, int c_dtype, hipStream_t stream) {
     XFT_REQUIRE(w && n_group >= 1 && table_dev && rows_dev && rows_stride >= 3, "gemm_grouped_rows_dev: bad group arguments");
     if (int rc = check_common("gemm_grouped_rows_dev", w[0], rows_max, A, lda, C, ldc)) return rc;
-    XFT_REQUIRE(rows_max > 32, "gemm_grouped_rows_dev: needs more than 32 rows in all (the few-row kernel has no grouped form)");
+    XFT_REQUIRE(rows_each_max >= 1 && rows_each_max <= rows_max, "gemm_grouped_rows_dev: bad row bounds %d / %d", rows_each_max, rows_max);
     const PackedWeight &pw = w[0]->pw;
     XFT_REQUIRE(pw.kind != XFTHIP_W_W8A8, "gemm_grouped_rows_dev: needs a weight-only kind");
     for (int e = 1; e < n_group; ++e) {
@@ -67,6 +67,10 @@ int gemm_grouped_rows_dev(const xfthip_weight_t *w, int n_group, const GroupWeig
     p.group = table_dev;
     p.group_n = n_group;
     p.rows_stride = rows_stride;
+    if (rows_each_max <= 32) {
+        p.M = rows_each_max; // the few-row kernel: a grid row a weight, each with at most this many rows
+        return qgemm_skinny(pw, p, stream);
+    }
     return qgemm_mfma(pw, p, stream);
 }
 

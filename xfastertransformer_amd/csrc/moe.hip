@@ -270,20 +270,21 @@ int xfthip_moe_forward(xfthip_moe_t m, const float *x_in, int in_stride, float *
     }
     // The host never learns how many rows an expert got: the GEMMs read row counts and row offsets from the
     // records build_lists_kernel left in device memory, and nothing here synchronises, so the layer can be
-    // captured into a graph.  With more than 32 gathered rows and experts of one kind, one launch serves the gate/up
-    // projections of all experts and one their down projections (their workgroups run side by side instead of
-    // one expert after another); otherwise every expert's two GEMMs are launched for up to T rows, in the form
-    // for the 2 T / E rows an expert gets on average, and workgroups past the count leave at once.
-    bool uniform = 2 * T > 32;
+    // captured into a graph.  With experts of one kind, one launch serves the gate/up projections of all experts and
+    // one their down projections (up to 32 tokens: the few-row kernel, a grid row an expert, experts without rows
+    // leave at once; more: the tiled kernel, row blocks numbered across the experts); their workgroups run side by
+    // side instead of one expert after another.  Otherwise every expert's two GEMMs are launched for up to T rows, in
+    // the form for the 2 T / E rows an expert gets on average, and workgroups past the count leave at once.
+    bool uniform = true;
     for (int e = 1; e < m->E && uniform; ++e) {
         const PackedWeight &g0 = m->gateup[0]->pw, &g = m->gateup[e]->pw, &d0 = m->down[0]->pw, &d = m->down[e]->pw;
         uniform = g.kind == g0.kind && g.flags == g0.flags && (g.zero != nullptr) == (g0.zero != nullptr) && d.kind == d0.kind
                 && d.flags == d0.flags && (d.zero != nullptr) == (d0.zero != nullptr);
     }
     if (uniform && m->gateup[0]->pw.kind != XFTHIP_W_W8A8 && m->down[0]->pw.kind != XFTHIP_W_W8A8) {
-        if (int rc = gemm_grouped_rows_dev(m->gateup.data(), m->E, m->group, 2 * T, gemm_rows + 6, 9, m->xg, H, m->h, m->inter, XFTHIP_BF16, st))
+        if (int rc = gemm_grouped_rows_dev(m->gateup.data(), m->E, m->group, 2 * T, T, gemm_rows + 6, 9, m->xg, H, m->h, m->inter, XFTHIP_BF16, st))
             return rc;
-        if (int rc = gemm_grouped_rows_dev(m->down.data(), m->E, m->group + m->E, 2 * T, gemm_rows + 6, 9, m->h, m->inter, m->eo, H, XFTHIP_F32, st))
+        if (int rc = gemm_grouped_rows_dev(m->down.data(), m->E, m->group + m->E, 2 * T, T, gemm_rows + 6, 9, m->h, m->inter, m->eo, H, XFTHIP_F32, st))
             return rc;
     } else {
         const int hint = (2 * T + m->E - 1) / m->E;

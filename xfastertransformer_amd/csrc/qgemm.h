@@ -73,10 +73,11 @@ int gemm_rows_dev(xfthip_weight_t w, int m_max, int m_hint, const int *rows_dev,
         hipStream_t stream);
 
 // The same for n_group weights of one shape behind one launch: table_dev holds their device pointers, record e
-// of rows_dev (rows_stride ints apart) the rows of weight e; rows_max bounds the sum of the rows (and must be
-// above 32: the few-row kernel has no grouped form); the weights' rows of C tile [0, sum of rows).
-int gemm_grouped_rows_dev(const xfthip_weight_t *w, int n_group, const GroupWeight *table_dev, int rows_max, const int *rows_dev,
-        int rows_stride, const void *A, int lda, void *C, int ldc, int c_dtype, hipStream_t stream);
+// of rows_dev (rows_stride ints apart) the rows of weight e; rows_max bounds the sum of the rows, rows_each_max the
+// rows of one weight (up to 32 of those: the few-row kernel, one grid row a weight; more: the tiled kernel, row
+// blocks numbered across the weights); the weights' rows of C tile [0, sum of rows).
+int gemm_grouped_rows_dev(const xfthip_weight_t *w, int n_group, const GroupWeight *table_dev, int rows_max, int rows_each_max,
+        const int *rows_dev, int rows_stride, const void *A, int lda, void *C, int ldc, int c_dtype, hipStream_t stream);
 
 int gemm_w8a8_from_bf16(xfthip_weight_t w, int M, const void *A, int lda, void *C, int ldc, int c_dtype, int epilogue,
         const float *bias, const void *res, int ldres, int res_dtype, float gamma, hipStream_t stream);

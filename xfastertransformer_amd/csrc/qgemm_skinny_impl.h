@@ -133,10 +133,18 @@ __global__ __launch_bounds__(512, (STAGE && MT == 1 && NT == 1) ? 4 : 1) void qg
     const int g = lane >> 4, ml = lane & 15;
     constexpr bool need_sum = NEED_SUM;
     if (p.rows_dev) {
-        if (p.rows_dev[0] <= 0) return; // uniform: the whole workgroup leaves
-        p.M = p.rows_dev[0] < p.M ? p.rows_dev[0] : p.M;
-        p.A += (size_t)p.rows_dev[1] * p.lda;
-        p.C = (char *)p.C + (size_t)p.rows_dev[2] * p.ldc * (p.c_dtype == XFTHIP_F32 ? 4 : 2);
+        // row count (and, for a group of weights of one shape, the weight: blockIdx.y) from device memory
+        const int *rec = p.rows_dev;
+        if (p.group) {
+            rec += blockIdx.y * p.rows_stride;
+            p.packed = p.group[blockIdx.y].packed;
+            p.scale = p.group[blockIdx.y].scale;
+            p.zero = p.group[blockIdx.y].zero;
+        }
+        if (rec[0] <= 0) return; // uniform: the whole workgroup leaves
+        p.M = rec[0] < p.M ? rec[0] : p.M;
+        p.A += (size_t)rec[1] * p.lda;
+        p.C = (char *)p.C + (size_t)rec[2] * p.ldc * (p.c_dtype == XFTHIP_F32 ? 4 : 2);
     }
 
     uint2 *lut = nullptr;
@@ -609,8 +617,8 @@ static int launch(const SkinnyParams &p, int kslices, hipStream_t stream) {
                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         XFT_CHECK_HIP(attr);
     }
-    hipLaunchKernelGGL((qgemm_skinny_kernel<KIND, NT, MT, U, NEED_SUM, KTAIL, NORM, ROPE, STAGE>), dim3(blocks), dim3(64 * kslices), smem,
-            stream, q);
+    hipLaunchKernelGGL((qgemm_skinny_kernel<KIND, NT, MT, U, NEED_SUM, KTAIL, NORM, ROPE, STAGE>), dim3(blocks, p.group ? p.group_n : 1),
+            dim3(64 * kslices), smem, stream, q);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }

@@ -146,6 +146,31 @@ def test_mixtral_mlp_bf16_experts(xh, orc, tokens):
     assert np.abs(got - exp).max() < 2e-2 and _cos(got, exp) >= 0.9999
 
 
+@pytest.mark.parametrize("tokens", [12, 70])
+def test_mixtral_mlp_experts_of_different_layouts(xh, orc, tokens):
+    """Experts that cannot share a launch (some INT8 weights carry a zero-point vector, some do not) go through the
+    per-expert launches with device-side row counts."""
+    hidden, inter, E = 1024, 3584, 8
+    rng = np.random.default_rng(700 + tokens)
+    experts = _experts(orc, rng, 0, hidden, inter, E)
+    router = np.zeros((hidden, E), np.float32)
+    ln = rng.uniform(0.8, 1.2, hidden).astype(np.float32)
+    x = orc.round_bf16(rng.standard_normal((tokens, hidden)))
+    lo = rng.standard_normal((tokens, E)).astype(np.float32)
+    moe = xh.MoE(hidden, inter, E, tokens, router, ln)
+    for e, (gu, dn) in enumerate(experts):
+        zg, zd = (gu.zero, dn.zero) if e % 3 else (None, None)  # all zeros either way: same values, other kernel form
+        moe.set_expert(e, xh.Weight(0, gu.K, gu.N, gu.q, gu.scale, zg, flags=xh.WF_GATEUP), xh.Weight(0, dn.K, dn.N, dn.q, dn.scale, zd))
+    xd, lod = xh.DeviceBuffer.from_numpy(x), xh.DeviceBuffer.from_numpy(lo)
+    od = xh.DeviceBuffer(x.nbytes)
+    sel, w = moe.forward(xd.ptr, od.ptr, tokens, True, lod.ptr)
+    xh.synchronize()
+    got = od.to_numpy(np.float32, x.shape)
+    exp, esel, ew = orc.mixtral_mlp(x, ln, router, experts, lo, rounding="bf16")
+    assert np.array_equal(sel, esel) and np.abs(w - ew).max() < 1e-6
+    assert np.abs(got - exp).max() < 2e-2 and _cos(got, exp) >= 0.9999
+
+
 def test_mixtral_shape_full_size_spot_check(xh, orc):
     """Mixtral-8x7B shape (hidden 4096, FFN 14336, 8 INT8 experts, 256 tokens, overridden N(0,1)
     logits): routing must equal the oracle's, and a handful of tokens are recomputed by the oracle."""

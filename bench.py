@@ -457,11 +457,20 @@ def moe_layer(xh, iters=5):
         moe.forward(x.ptr, y.ptr, T, True, lg.ptr, want_routing=False)
     xh.synchronize()
     us_queued = (time.time() - t0) * 1e6 / (4 * iters)
+    # one token (a decode step): two of the eight experts work, 352 MB of their weights
+    moe.forward(x.ptr, y.ptr, 1, True, lg.ptr, want_routing=False)
+    xh.synchronize()
+    t0 = time.time()
+    for _ in range(20 * iters):
+        moe.forward(x.ptr, y.ptr, 1, True, lg.ptr, want_routing=False)
+    xh.synchronize()
+    us_one = (time.time() - t0) * 1e6 / (20 * iters)
     wbytes, flops = 8 * (4096 * 28672 + 14336 * 4096), 512 * 3 * 2 * 4096 * 14336
     moe.free()
     return dict(tokens=T, experts=E, us_per_layer=round(us, 1), us_per_layer_no_wait=round(us_queued, 1),
                 weight_gbs=round(wbytes / us_queued / 1e3, 1), frac_of_hbm_peak=round(wbytes / us_queued / 1e3 / HBM_PEAK_GBS, 4),
-                tflops=round(flops / us_queued / 1e6, 1),
+                tflops=round(flops / us_queued / 1e6, 1), us_per_layer_one_token=round(us_one, 1),
+                one_token_weight_gbs=round(wbytes / 4 / us_one / 1e3, 1),
                 note="us_per_layer: wall time of xfthip_moe_forward with the routing copied back to the host (one wait a call); "
                      "us_per_layer_no_wait (the rates are quoted on it): calls that return no routing, queued back to back (nothing waits: the row "
                      "counts stay on the device)")

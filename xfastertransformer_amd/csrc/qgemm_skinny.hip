@@ -23,8 +23,9 @@ bool skinny_can_fuse_norm(const PackedWeight &pw, int M) {
 
 int qgemm_skinny(const PackedWeight &pw, const SkinnyParams &p0, hipStream_t stream) {
     SkinnyParams p = p0;
-    if (p.group && (p.norm_x || p.rope || !p.rows_dev)) {
-        set_error("qgemm_skinny: a group of weights needs device row records and takes no norm prologue or RoPE epilogue");
+    if (p.group && (p.norm_x || p.rope || !p.rows_dev || pw.KT * ktile_of(pw.kind) != pw.K)) {
+        set_error("qgemm_skinny: a group of weights needs device row records and K a whole number of weight tiles, and takes no norm "
+                  "prologue or RoPE epilogue");
         return 2;
     }
     if (p.norm_x && !skinny_can_fuse_norm(pw, p.M)) {

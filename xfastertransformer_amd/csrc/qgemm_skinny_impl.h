@@ -117,12 +117,15 @@ __constant__ float c_nf4_gemm[16] = XFTHIP_NF4_CODE_VALUES;
 // MFMA fragments through a wave-private LDS patch.  Loaded straight in fragment order a wave-load is 16 rows x
 // four 16-byte pieces, which the memory pipeline serves at a third of the rate of contiguous runs (37 against
 // 125 GB/s a CU from L2, measured): with more than a few rows those loads, not the weights, set the time.
-template <int KIND, int NT, int MT, int U, bool NEED_SUM, bool KTAIL, bool NORM, bool ROPE, bool STAGE = false>
+// GROUP: several weights of one shape behind one launch (SkinnyParams::group, one grid row a weight); a form of its
+// own: with the weight pointers possibly read from memory the plain kernels lost 6 % of the decode step.
+template <int KIND, int NT, int MT, int U, bool NEED_SUM, bool KTAIL, bool NORM, bool ROPE, bool STAGE = false, bool GROUP = false>
 __global__ __launch_bounds__(512, (STAGE && MT == 1 && NT == 1) ? 4 : 1) void qgemm_skinny_kernel(SkinnyParams p) {
     // (the one-tile staged form is held to 128 registers, two workgroups a CU like its unstaged twin)
     static_assert(!NORM || (MT == 1 && !KTAIL), "the norm prologue covers M <= 4 without a K tail");
     static_assert(!ROPE || (NT % 2 == 0 && !KTAIL), "the RoPE epilogue works on tile pairs");
     static_assert(!STAGE || (!NORM && !ROPE), "staged activation loads belong to the plain kernels");
+    static_assert(!GROUP || (!NORM && !ROPE && !KTAIL), "grouped launches: plain kernels, whole k tiles");
     using T = KindTraits<KIND>;
     constexpr int MPT = T::MPT, KL = T::KL, KTILE = T::KTILE;
     extern __shared__ float smem[];
@@ -135,7 +138,7 @@ __global__ __launch_bounds__(512, (STAGE && MT == 1 && NT == 1) ? 4 : 1) void qg
     if (p.rows_dev) {
         // row count (and, for a group of weights of one shape, the weight: blockIdx.y) from device memory
         const int *rec = p.rows_dev;
-        if (p.group) {
+        if constexpr (GROUP) {
             rec += blockIdx.y * p.rows_stride;
             p.packed = p.group[blockIdx.y].packed;
             p.scale = p.group[blockIdx.y].scale;
@@ -586,7 +589,7 @@ constexpr int batch_tiles() {
     return MT == 1 ? 2 : 1;
 }
 
-template <int KIND, int NT, int MT, int U, bool NEED_SUM, bool KTAIL, bool NORM, bool ROPE = false, bool STAGE = false>
+template <int KIND, int NT, int MT, int U, bool NEED_SUM, bool KTAIL, bool NORM, bool ROPE = false, bool STAGE = false, bool GROUP = false>
 static int launch(const SkinnyParams &p, int kslices, hipStream_t stream) {
     constexpr int ROWS = 16 * MT, COLS = 16 * NT;
     size_t smem = (size_t)kslices * (ROWS * (COLS + 1) + ROWS) * sizeof(float);
@@ -613,11 +616,11 @@ static int launch(const SkinnyParams &p, int kslices, hipStream_t stream) {
     }
     if (smem > 64 * 1024) {
         // more dynamic LDS than the default limit (wide column blocks at 17 .. 32 rows): raise it once per instantiation
-        static const hipError_t attr = hipFuncSetAttribute((const void *)qgemm_skinny_kernel<KIND, NT, MT, U, NEED_SUM, KTAIL, NORM, ROPE, STAGE>,
+        static const hipError_t attr = hipFuncSetAttribute((const void *)qgemm_skinny_kernel<KIND, NT, MT, U, NEED_SUM, KTAIL, NORM, ROPE, STAGE, GROUP>,
                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         XFT_CHECK_HIP(attr);
     }
-    hipLaunchKernelGGL((qgemm_skinny_kernel<KIND, NT, MT, U, NEED_SUM, KTAIL, NORM, ROPE, STAGE>), dim3(blocks, p.group ? p.group_n : 1),
+    hipLaunchKernelGGL((qgemm_skinny_kernel<KIND, NT, MT, U, NEED_SUM, KTAIL, NORM, ROPE, STAGE, GROUP>), dim3(blocks, GROUP ? p.group_n : 1),
             dim3(64 * kslices), smem, stream, q);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
@@ -664,6 +667,10 @@ static int dispatch_tail(const SkinnyParams &p, int kslices, hipStream_t stream)
         if (p.norm_x) return launch<KIND, NT, MT, U, NEED_SUM, false, true>(p, kslices, stream);
     }
     // more than a few rows: activation rows loaded as contiguous runs (see STAGE)
+    if (p.group) {
+        if (MT == 2 || p.M > 4) return launch<KIND, NT, MT, U, NEED_SUM, false, false, false, true, true>(p, kslices, stream);
+        if constexpr (MT == 1) return launch<KIND, NT, MT, U, NEED_SUM, false, false, false, false, true>(p, kslices, stream);
+    }
     if (MT == 2 || p.M > 4) return launch<KIND, NT, MT, U, NEED_SUM, false, false, false, true>(p, kslices, stream);
     if constexpr (MT == 1) return launch<KIND, NT, MT, U, NEED_SUM, false, false>(p, kslices, stream);
     return 0;

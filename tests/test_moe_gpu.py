@@ -68,6 +68,11 @@ def test_mixtral_mlp_vs_oracle(xh, orc, tokens, override):
     sel, w = moe.forward(xd.ptr, od.ptr, tokens, True, None if lod is None else lod.ptr)
     xh.synchronize()
     got = od.to_numpy(np.float32, x.shape)
+    # output over the input (the residual is read where it is written): the same bits
+    sel2, w2 = moe.forward(xd.ptr, xd.ptr, tokens, True, None if lod is None else lod.ptr)
+    xh.synchronize()
+    assert np.array_equal(sel, sel2) and np.array_equal(w, w2)
+    assert np.array_equal(xd.to_numpy(np.float32, x.shape), got)
     exp, esel, ew = orc.mixtral_mlp(x, ln, router, experts, lo, rounding="bf16")
     if override:
         assert np.array_equal(sel, esel)

@@ -120,8 +120,10 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t *__rest
 // out[t] += eo[row of choice] * weight, the lower expert index first: the order in which the reference's
 // loop over the experts adds a token's two contributions (xft::addto: one fused multiply-add per element).
 // grid = tokens
-__global__ __launch_bounds__(256) void combine_kernel(float *__restrict__ out, int ld, const float *__restrict__ eo, const int *__restrict__ sel,
-        const int *__restrict__ slot_row, const float *__restrict__ w, int hidden, int wide) {
+// The residual comes straight from the layer's input (`in`, which may be `out` itself: a thread reads an element
+// before it writes it), so no copy of the input into the output runs first.
+__global__ __launch_bounds__(256) void combine_kernel(float *out, int ld, const float *in, int in_ld, const float *__restrict__ eo,
+        const int *__restrict__ sel, const int *__restrict__ slot_row, const float *__restrict__ w, int hidden, int wide) {
     const int t = blockIdx.x;
     const int first = sel[2 * t] < sel[2 * t + 1] ? 0 : 1;
     const int ga = slot_row[2 * t + first], gb = slot_row[2 * t + 1 - first];
@@ -129,8 +131,9 @@ __global__ __launch_bounds__(256) void combine_kernel(float *__restrict__ out, i
     if (wide) { // rows of out start on 16-byte boundaries
         const float4 *ea = (const float4 *)(eo + (size_t)ga * hidden), *eb = (const float4 *)(eo + (size_t)gb * hidden);
         float4 *dst = (float4 *)(out + (size_t)t * ld);
+        const float4 *src = (const float4 *)(in + (size_t)t * in_ld);
         for (int c = threadIdx.x; c < hidden / 4; c += blockDim.x) {
-            float4 o = dst[c];
+            float4 o = src[c];
             const float4 a = ea[c], b = eb[c];
             o.x = fmaf(b.x, wb, fmaf(a.x, wa, o.x));
             o.y = fmaf(b.y, wb, fmaf(a.y, wa, o.y));
@@ -141,13 +144,9 @@ __global__ __launch_bounds__(256) void combine_kernel(float *__restrict__ out, i
     } else {
         const float *ea = eo + (size_t)ga * hidden, *eb = eo + (size_t)gb * hidden;
         float *dst = out + (size_t)t * ld;
-        for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = fmaf(eb[c], wb, fmaf(ea[c], wa, dst[c]));
+        const float *src = in + (size_t)t * in_ld;
+        for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = fmaf(eb[c], wb, fmaf(ea[c], wa, src[c]));
     }
-}
-
-__global__ void copy_rows_kernel(const float *__restrict__ in, int in_ld, float *__restrict__ out, int out_ld, int hidden) {
-    const int r = blockIdx.x;
-    for (int c = threadIdx.x; c < hidden; c += blockDim.x) out[(size_t)r * out_ld + c] = in[(size_t)r * in_ld + c];
 }
 
 __global__ void narrow_rows_kernel2(const float *__restrict__ in, int in_stride, uint16_t *__restrict__ out, int cols) {
@@ -244,9 +243,7 @@ int xfthip_moe_forward(xfthip_moe_t m, const float *x_in, int in_stride, float *
     for (int e = 0; e < m->E; ++e) XFT_REQUIRE(m->gateup[e] && m->down[e], "xfthip_moe_forward: expert %d has no weights", e);
     hipStream_t st = (hipStream_t)stream;
     const int T = tokens, H = m->hidden;
-    // residual: the output starts as a copy of the input (mlp_mixtral.h:116-121)
-    if ((const void *)x_in != (const void *)x_out)
-        hipLaunchKernelGGL(copy_rows_kernel, dim3(T), dim3(256), 0, st, x_in, in_stride, x_out, out_stride, H);
+    // residual (mlp_mixtral.h:116-121: the output starts as a copy of the input): combine_kernel reads it from x_in
     if (do_norm) {
         if (int rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, x_in, XFTHIP_F32, m->ln, T, H, in_stride, H, 1e-6f, st)) return rc;
     } else {
@@ -293,8 +290,8 @@ int xfthip_moe_forward(xfthip_moe_t m, const float *x_in, int in_stride, float *
             if (int rc = gemm_rows_dev(m->down[e], T, hint, gemm_rows + 9 * e + 3, m->h, m->inter, m->eo, H, XFTHIP_F32, st)) return rc;
         }
     }
-    const int wide = (((size_t)x_out | ((size_t)out_stride * 4)) & 15) == 0;
-    hipLaunchKernelGGL(combine_kernel, dim3(T), dim3(256), 0, st, x_out, out_stride, m->eo, m->sel, m->slot_row, m->w, H, wide);
+    const int wide = (((size_t)x_out | ((size_t)out_stride * 4) | (size_t)x_in | ((size_t)in_stride * 4)) & 15) == 0 && H % 4 == 0;
+    hipLaunchKernelGGL(combine_kernel, dim3(T), dim3(256), 0, st, x_out, out_stride, x_in, in_stride, m->eo, m->sel, m->slot_row, m->w, H, wide);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }

@@ -367,14 +367,23 @@ __global__ __launch_bounds__(512, (STAGE && MT == 1 && NT == 1) ? 4 : 1) void qg
             // kinds, whose short weight stream leaves the prologue in the open: UINT4 decode 561 -> 574 tok/s; the
             // INT8 kernels, at their 128 registers, lose 0.7 % to the extra one)
             constexpr bool TOUCH = KIND == XFTHIP_W_UINT4 || KIND == XFTHIP_W_NF4;
+            constexpr int NB = TOUCH ? 4 : 2;
             float w_touch = 0.0f;
             if (TOUCH && (int)threadIdx.x * 32 < p.K) w_touch = p.norm_w[threadIdx.x * 32];
             for (int m = 0; m < p.M; ++m) {
                 const float *row = p.norm_x + (size_t)m * p.ldx;
                 float sq = 0.0f;
-                for (int c = threadIdx.x * 4; c < p.K; c += blockDim.x * 4) {
-                    const float4 v = *(const float4 *)(row + c);
-                    sq = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, sq))));
+                // NB loads in flight a thread (the 4-wave workgroups of the 4-bit kinds walk a 4096-wide row in four
+                // steps: one round trip instead of four); the sums keep the order of the plain loop
+                for (int c = threadIdx.x * 4; c < p.K; c += blockDim.x * 4 * NB) {
+                    float4 v[NB];
+#pragma unroll
+                    for (int i = 0; i < NB; ++i) {
+                        const int ci = c + i * (int)blockDim.x * 4;
+                        v[i] = ci < p.K ? *(const float4 *)(row + ci) : make_float4(0.f, 0.f, 0.f, 0.f);
+                    }
+#pragma unroll
+                    for (int i = 0; i < NB; ++i) sq = fmaf(v[i].x, v[i].x, fmaf(v[i].y, v[i].y, fmaf(v[i].z, v[i].z, fmaf(v[i].w, v[i].w, sq))));
                 }
 #pragma unroll
                 for (int off = 32; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
@@ -384,12 +393,23 @@ __global__ __launch_bounds__(512, (STAGE && MT == 1 && NT == 1) ? 4 : 1) void qg
                 float tot = 0.0f;
                 for (int w = 0; w < nwaves; ++w) tot += part[(m & 1) * 8 + w];
                 const float var = 1.0f / sqrtf(tot / (float)p.K + p.norm_eps);
-                for (int c = threadIdx.x * 4; c < p.K; c += blockDim.x * 4) {
-                    const float4 v = *(const float4 *)(row + c);
-                    const float4 w = *(const float4 *)(p.norm_w + c);
-                    const uint32_t lo = f32_to_bf16_ref((v.x * var) * w.x) | ((uint32_t)f32_to_bf16_ref((v.y * var) * w.y) << 16);
-                    const uint32_t hi = f32_to_bf16_ref((v.z * var) * w.z) | ((uint32_t)f32_to_bf16_ref((v.w * var) * w.w) << 16);
-                    *(uint2 *)(xn + (size_t)m * pitch + c) = make_uint2(lo, hi);
+                for (int c = threadIdx.x * 4; c < p.K; c += blockDim.x * 4 * NB) {
+                    float4 vv[NB], ww[NB];
+#pragma unroll
+                    for (int i = 0; i < NB; ++i) {
+                        const int ci = c + i * (int)blockDim.x * 4;
+                        const int cl = ci < p.K ? ci : c; // past the row: a second read of this step's first chunk, not stored
+                        vv[i] = *(const float4 *)(row + cl);
+                        ww[i] = *(const float4 *)(p.norm_w + cl);
+                    }
+#pragma unroll
+                    for (int i = 0; i < NB; ++i) {
+                        const int ci = c + i * (int)blockDim.x * 4;
+                        const float4 v = vv[i], w = ww[i];
+                        const uint32_t lo = f32_to_bf16_ref((v.x * var) * w.x) | ((uint32_t)f32_to_bf16_ref((v.y * var) * w.y) << 16);
+                        const uint32_t hi = f32_to_bf16_ref((v.z * var) * w.z) | ((uint32_t)f32_to_bf16_ref((v.w * var) * w.w) << 16);
+                        if (ci < p.K) *(uint2 *)(xn + (size_t)m * pitch + ci) = make_uint2(lo, hi);
+                    }
                 }
             }
             __syncthreads();

@@ -338,6 +338,12 @@ __global__ __launch_bounds__(512, (STAGE && MT == 1 && NT == 1) ? 4 : 1) void qg
         // sched_barrier keeps the compiler from sinking the next batch's loads below the MFMAs of
         // the current one: all loads of a batch are issued back to back, then the math runs.
 #define XFT_FENCE() __builtin_amdgcn_sched_barrier(0)
+        // ROPE: the position of the first row (the only one of a single sequence) is requested ahead of the weights,
+        // into a scalar register, so that the epilogue's chain position -> cos / sin -> store is one round trip
+        // shorter (the cos / sin values themselves stay in the epilogue: requested here, the wait for their address
+        // would hold up the weight stream)
+        int pos_pre = 0;
+        if constexpr (ROPE) pos_pre = __builtin_amdgcn_readfirstlane(p.pos_dev ? p.pos_dev[0] : p.pos_host);
         if (nb > 0 && !pre_issued) {
             issue(0, b_begin);
             XFT_FENCE();
@@ -501,14 +507,15 @@ __global__ __launch_bounds__(512, (STAGE && MT == 1 && NT == 1) ? 4 : 1) void qg
                 const int hh = it >> 2, jj = it & 3;
                 for (int v = threadIdx.x; v < p.M * 16; v += blockDim.x) {
                     const int m = v >> 4, c = v & 15;
+                    int pos = m == 0 ? pos_pre : (p.pos_dev ? p.pos_dev[m] : p.pos_host);
+                    pos = pos < 0 ? 0 : (pos >= p.kv.S ? p.kv.S - 1 : pos); // held inside the cache whatever the device value is
+                    const int i = jj * 16 + c;
+                    // (requested before the sums over the waves' partial results are read, not behind them)
+                    const float cs = p.cosT[(size_t)pos * 64 + i], sn = p.sinT[(size_t)pos * 64 + i];
                     const float sumA = need_sum ? total_sum(m) : 0.0f;
                     // the projection's output is bf16 in the reference (the rotation reads it back)
                     const float lo = bf16_to_f32(f32_to_bf16_ref(column_value(m, cofs + c, sumA)));
                     const float hi = bf16_to_f32(f32_to_bf16_ref(column_value(m, cofs + 16 + c, sumA)));
-                    int pos = p.pos_dev ? p.pos_dev[m] : p.pos_host;
-                    pos = pos < 0 ? 0 : (pos >= p.kv.S ? p.kv.S - 1 : pos); // held inside the cache whatever the device value is
-                    const int i = jj * 16 + c;
-                    const float cs = p.cosT[(size_t)pos * 64 + i], sn = p.sinT[(size_t)pos * 64 + i];
                     // reference: fmsub(q, cos, qHalf*sin) ; fmadd(qHalf, cos, q*sin)
                     const float nlo = fmaf(lo, cs, -(hi * sn)), nhi = fmaf(hi, cs, lo * sn);
                     if (hh < p.qH) {

@@ -535,7 +535,7 @@ __global__ __launch_bounds__(512, (STAGE && MT == 1 && NT == 1) ? 4 : 1) void qg
                     const int vt = 2 * (it - rope_pairs) + (cc >> 4);
                     const float sumA = need_sum ? total_sum(m) : 0.0f;
                     const float val = bf16_to_f32(f32_to_bf16_ref(column_value(m, cofs + cc, sumA)));
-                    int pos = p.pos_dev ? p.pos_dev[m] : p.pos_host;
+                    int pos = m == 0 ? pos_pre : (p.pos_dev ? p.pos_dev[m] : p.pos_host);
                     pos = pos < 0 ? 0 : (pos >= p.kv.S ? p.kv.S - 1 : pos);
                     if (pos < p.kv.S) {
                         const size_t bh = (size_t)m * p.kv.H + (vt >> 3);
@@ -554,6 +554,10 @@ __global__ __launch_bounds__(512, (STAGE && MT == 1 && NT == 1) ? 4 : 1) void qg
                 const int m = v / PCOLS, c = t * 16 + v % PCOLS;
                 const int np = nt0 * 16 + c;
                 if (m >= p.M || np >= p.N) return;
+                // the residual value is requested before the sums over the waves' partial results are read
+                float resv = 0.0f;
+                if (p.epi == XFTHIP_EPI_RESMUL || p.epi == XFTHIP_EPI_RESIDENTIAL || p.epi == XFTHIP_EPI_RESEXT)
+                    resv = load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + np);
                 const float sumA = need_sum ? total_sum(m) : 0.0f;
                 float x = column_value(m, c, sumA);
                 switch (p.epi) {
@@ -564,14 +568,14 @@ __global__ __launch_bounds__(512, (STAGE && MT == 1 && NT == 1) ? 4 : 1) void qg
                         x = e / (e + 1.0f) * x;
                         break;
                     }
-                    case XFTHIP_EPI_RESMUL: x *= load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + np); break;
+                    case XFTHIP_EPI_RESMUL: x *= resv; break;
                     case XFTHIP_EPI_RESIDENTIAL:
                         if (p.bias) x += p.bias[np];
-                        x += load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + np);
+                        x += resv;
                         break;
                     case XFTHIP_EPI_RESEXT:
                         if (p.bias) x += p.bias[np];
-                        x = fmaf(p.gamma, load_as_f32(p.res, p.res_dtype, (size_t)m * p.ldres + np), x);
+                        x = fmaf(p.gamma, resv, x);
                         break;
                     default: break;
                 }

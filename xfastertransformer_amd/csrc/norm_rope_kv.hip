@@ -50,16 +50,18 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(void *__restrict__ out
     __shared__ float part[4];
     const int row = blockIdx.x;
     const size_t ibase = (size_t)row * iStride, obase = (size_t)row * oStride;
-    float x[CHUNKS][8];
+    // the norm weights are requested with the row, not behind the reduction's barrier (a second, cold round trip)
+    float x[CHUNKS][8], w[CHUNKS][8];
     float sq = 0.0f;
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
         const int col = (c * 256 + threadIdx.x) * 8;
         if (col < cols) {
             load8<IN_BF16>(in, ibase + col, x[c]);
+            load8<false>(weight, col, w[c]);
         } else {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) x[c][i] = 0.0f;
+            for (int i = 0; i < 8; ++i) x[c][i] = 0.0f, w[c][i] = 0.0f;
         }
     }
 #pragma unroll
@@ -75,21 +77,19 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(void *__restrict__ out
     for (int c = 0; c < CHUNKS; ++c) {
         const int col = (c * 256 + threadIdx.x) * 8;
         if (col < cols) {
-            float w[8];
-            load8<false>(weight, col, w);
             if constexpr (OUT_BF16) {
                 uint32_t pk[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const uint32_t lo = f32_to_bf16_ref((x[c][2 * i] * var) * w[2 * i]);
-                    const uint32_t hi = f32_to_bf16_ref((x[c][2 * i + 1] * var) * w[2 * i + 1]);
+                    const uint32_t lo = f32_to_bf16_ref((x[c][2 * i] * var) * w[c][2 * i]);
+                    const uint32_t hi = f32_to_bf16_ref((x[c][2 * i + 1] * var) * w[c][2 * i + 1]);
                     pk[i] = lo | (hi << 16);
                 }
                 *(uint4 *)((uint16_t *)out + obase + col) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
             } else {
                 float *o = (float *)out + obase + col;
-                *(float4 *)o = make_float4((x[c][0] * var) * w[0], (x[c][1] * var) * w[1], (x[c][2] * var) * w[2], (x[c][3] * var) * w[3]);
-                *(float4 *)(o + 4) = make_float4((x[c][4] * var) * w[4], (x[c][5] * var) * w[5], (x[c][6] * var) * w[6], (x[c][7] * var) * w[7]);
+                *(float4 *)o = make_float4((x[c][0] * var) * w[c][0], (x[c][1] * var) * w[c][1], (x[c][2] * var) * w[c][2], (x[c][3] * var) * w[c][3]);
+                *(float4 *)(o + 4) = make_float4((x[c][4] * var) * w[c][4], (x[c][5] * var) * w[c][5], (x[c][6] * var) * w[c][6], (x[c][7] * var) * w[c][7]);
             }
         }
     }

@@ -483,7 +483,9 @@ int xfthip_moe_top2(const float *logits, int M, int E, int *sel, float *weights,
  * sel_host_out / w_host_out: optional host copies of the routing decision; asking for either makes the call
  * wait for the stream once.  Without them the call only enqueues work (the per-expert row counts stay in device
  * memory, where the expert GEMMs read them) and may be recorded into a graph.  The workspace of one xfthip_moe
- * serves one call at a time: calls on the same object must be ordered on one stream.
+ * serves one call at a time: calls on the same object must be ordered on one stream.  x_out may be x_in itself
+ * (same pointer and stride: the result is then written over the input); buffers that overlap in any other way are
+ * not supported.
  */
 int xfthip_moe_create(int hidden, int intermediate, int experts, int max_tokens, const float *router_host, const float *ln_host,
         xfthip_moe_t *out);

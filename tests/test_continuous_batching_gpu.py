@@ -158,3 +158,61 @@ def test_cache_rows_copied_and_reordered_for_beams(xh, orc, kv):
         err = float(np.abs(got - want[r]).max())
         assert err < 2e-2, (r, err)
     print(f"six rows agree with their solo runs after three re-mappings ({kv=})", flush=True)
+
+
+def test_lockstep_and_per_sequence_decode_alternate_at_one_batch(xh, orc):
+    """The captured decode step differs between the two modes (the per-sequence one carries the mask of
+    the rows that sit out), so a change of mode at an unchanged batch, stream and split count must not
+    replay the other mode's step: a subset decode that leaves a zero in the mask, then a lockstep
+    prompt + decode at the same batch, and the reverse order, each compared with a fresh model."""
+    from test_layer_model_gpu import make_layer_weights, to_device_weights
+    layers, hidden, inter, qh, kvh, D, vocab, rows, max_seq = 2, 512, 1408, 4, 2, 128, 1000, 2, 96
+
+    def build():
+        rng = np.random.default_rng(77)
+        model = xh.Model(layers, hidden, inter, qh, kvh, D, vocab=vocab, max_batch=rows, max_seq=max_seq, max_tokens=rows * max_seq)
+        for l in range(layers):
+            ws = make_layer_weights(orc, rng, 0, hidden, inter, qh, kvh, D)
+            model.set_layer(l, *to_device_weights(xh, ws, 0), rng.uniform(0.8, 1.2, hidden).astype(np.float32),
+                            rng.uniform(0.8, 1.2, hidden).astype(np.float32))
+        lm = orc.round_bf16(rng.standard_normal((hidden, vocab)) * 0.05)
+        model.set_head(orc.to_fp16(rng.standard_normal((vocab, hidden)) * 0.5), rng.uniform(0.8, 1.2, hidden).astype(np.float32),
+                       xh.Weight(xh.W_BF16, hidden, vocab, orc.to_bf16(lm)))
+        return model
+
+    rng = np.random.default_rng(5)
+    pa, pb = rng.integers(0, vocab, 11).tolist(), rng.integers(0, vocab, 11).tolist()
+    both = np.asarray([pa, pb], np.int32)
+    steps = 6
+
+    def lockstep(model):
+        first, _ = model.prefill(both)
+        out = model.decode(steps, 2)
+        return [int(first[0]), int(first[1])], out.tolist()
+
+    def per_sequence(model):
+        model.seq_prefill(0, pa)
+        model.seq_prefill(1, pb)
+        ids = [[int(t) for t in model.last_ids(2)]]
+        for _ in range(2):
+            ids.append([int(t) for t in model.seq_decode([0, 1])])
+        only_b = [int(model.seq_decode([1])[0]) for _ in range(3)]  # row 0 sits out: the mask ends as [0, 1]
+        return ids, only_b
+
+    want_lock = lockstep(build())
+    want_seq = per_sequence(build())
+    # (in the per-sequence run row 0 must stay where it was while it sat out)
+    m = build()
+    assert per_sequence(m) == want_seq
+    assert lockstep(m) == want_lock, "a lockstep decode replayed the masked step of the per-sequence mode"
+    assert per_sequence(m) == want_seq, "a per-sequence decode replayed the unmasked lockstep step"
+    m2 = build()
+    assert lockstep(m2) == want_lock
+    got_ids, got_b = per_sequence(m2)
+    assert (got_ids, got_b) == want_seq
+    # row 0 sat out three steps: stepping it now continues from its own position
+    a_next = int(m2.seq_decode([0])[0])
+    fresh = build()
+    fresh.seq_prefill(0, pa)
+    solo = [int(fresh.seq_decode([0])[0]) for _ in range(3)]
+    assert a_next == solo[2], (a_next, solo)

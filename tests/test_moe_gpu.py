@@ -274,3 +274,73 @@ def test_graph_helpers_reject_the_null_stream(xh):
     assert xh.lib.xfthip_graph_end(None, C.byref(g)) != 0
     assert xh.lib.xfthip_graph_launch(None, None) != 0
     assert xh.lib.xfthip_graph_destroy(None) == 0
+
+
+@pytest.mark.parametrize("kind,hidden,inter", [(0, 1056, 1104), (1, 1088, 1168)])
+@pytest.mark.parametrize("tokens", [3, 8])
+def test_mixtral_mlp_few_tokens_k_not_a_whole_tile(xh, orc, kind, hidden, inter, tokens):
+    """Up to 32 tokens with a hidden / intermediate size that is not a whole number of weight tiles along K (64 rows
+    for INT8, 128 for the 4-bit kinds): the one-launch form of the few-row GEMM has no K-tail variant, so these
+    shapes go expert by expert; every expert's rows must still be multiplied."""
+    E = 8
+    rng = np.random.default_rng(hidden + tokens)
+    experts = _experts(orc, rng, kind, hidden, inter, E)
+    ln = rng.uniform(0.8, 1.2, hidden).astype(np.float32)
+    x = orc.round_bf16(rng.standard_normal((tokens, hidden)))
+    lo = rng.standard_normal((tokens, E)).astype(np.float32)
+    moe = xh.MoE(hidden, inter, E, tokens, np.zeros((hidden, E), np.float32), ln)
+    for e, (gu, dn) in enumerate(experts):
+        moe.set_expert(e, xh.Weight(kind, gu.K, gu.N, gu.q, gu.scale, gu.zero, flags=xh.WF_GATEUP),
+                       xh.Weight(kind, dn.K, dn.N, dn.q, dn.scale, dn.zero))
+    xd, lod = xh.DeviceBuffer.from_numpy(x), xh.DeviceBuffer.from_numpy(lo)
+    od = xh.DeviceBuffer(x.nbytes)
+    sel, w = moe.forward(xd.ptr, od.ptr, tokens, True, lod.ptr)
+    xh.synchronize()
+    got = od.to_numpy(np.float32, x.shape)
+    exp, esel, ew = orc.mixtral_mlp(x, ln, np.zeros((hidden, E), np.float32), experts, lo, rounding="bf16")
+    assert np.array_equal(sel, esel)
+    assert len(set(sel.ravel().tolist())) >= 3  # several experts take part
+    assert np.abs(got - exp).max() < 2e-2 and _cos(got, exp) >= 0.9999
+
+
+@pytest.mark.parametrize("tokens", [5, 70])
+def test_mixtral_mlp_token_without_two_choices(xh, orc, tokens):
+    """Router logits that are NaN (no comparison is true: no expert) or all -inf but one (a single expert): such a
+    choice takes no row, as in the reference, whose loop over the experts never matches index -1
+    (mlp_mixtral.h:165-186, 262-283); the token keeps its residual plus what its valid choice adds, and the
+    other tokens are not disturbed."""
+    hidden, inter, E = 512, 1024, 8
+    rng = np.random.default_rng(900 + tokens)
+    experts = _experts(orc, rng, 0, hidden, inter, E)
+    ln = rng.uniform(0.8, 1.2, hidden).astype(np.float32)
+    x = orc.round_bf16(rng.standard_normal((tokens, hidden)))
+    lo = rng.standard_normal((tokens, E)).astype(np.float32)
+    lo[1] = np.nan
+    lo[3] = -np.inf
+    lo[3, 5] = 0.25
+    moe = xh.MoE(hidden, inter, E, tokens, np.zeros((hidden, E), np.float32), ln)
+    for e, (gu, dn) in enumerate(experts):
+        moe.set_expert(e, xh.Weight(0, gu.K, gu.N, gu.q, gu.scale, gu.zero, flags=xh.WF_GATEUP),
+                       xh.Weight(0, dn.K, dn.N, dn.q, dn.scale, dn.zero))
+    xd, lod = xh.DeviceBuffer.from_numpy(x), xh.DeviceBuffer.from_numpy(lo)
+    od = xh.DeviceBuffer(x.nbytes)
+    sel, w = moe.forward(xd.ptr, od.ptr, tokens, True, lod.ptr)
+    xh.synchronize()
+    got = od.to_numpy(np.float32, x.shape)
+    assert list(sel[1]) == [-1, -1] and list(sel[3]) == [5, -1]
+    assert np.array_equal(got[1], x[1]), "a token without an expert keeps its input"
+    # the well-formed tokens: as the oracle computes them from finite logits
+    keep = np.ones(tokens, bool)
+    keep[[1, 3]] = False
+    lo_ok = lo.copy()
+    lo_ok[1] = 0.0
+    lo_ok[3] = 0.0
+    exp, esel, _ = orc.mixtral_mlp(x, ln, np.zeros((hidden, E), np.float32), experts, lo_ok, rounding="bf16")
+    assert np.array_equal(sel[keep], esel[keep])
+    assert np.abs(got[keep] - exp[keep]).max() < 2e-2
+    # token 3: residual + weight 1 (exp(-inf) = 0 for the missing one) times expert 5 alone
+    lo_one = lo_ok.copy()
+    lo_one[3] = -40.0
+    lo_one[3, 5] = 40.0  # the second choice's weight underflows to 0
+    exp1, _, _ = orc.mixtral_mlp(x, ln, np.zeros((hidden, E), np.float32), experts, lo_one, rounding="bf16")
+    assert np.isfinite(got[3]).all() and np.abs(got[3] - exp1[3]).max() < 2e-2

@@ -92,3 +92,35 @@ def test_static_scratch_attention_prefill_and_rejection(xh, orc):
         xh.attention_static(big, qd.ptr, 32 * D, od.ptr, 32 * D, xh.F32, 80, 1, 32, SCALE, 400)
     xh.attention(big, qd.ptr, 32 * D, od.ptr, 32 * D, xh.F32, 80, 1, 32, SCALE, 400)  # the allocating entry point takes it
     xh.synchronize()
+
+
+def test_static_scratch_attention_records_into_a_graph(xh, orc):
+    """The property the entry point exists for: nothing in the call allocates.  A device allocation (or any
+    other synchronising call) while a stream is being captured makes the capture fail, so a split shape is
+    recorded into a graph and the graph replayed three times, with eager work between the replays, against
+    the eager result."""
+    rng = np.random.default_rng(79)
+    qh, kvh, B, ctx = 32, 8, 2, 900
+    kc, vc, dc = _filled(xh, orc, rng, 0, B, kvh, 1024, ctx)
+    q = orc.round_bf16(rng.standard_normal((B, qh * D)))
+    qd = xh.DeviceBuffer.from_numpy(orc.to_bf16(q))
+    eager = xh.DeviceBuffer(q.size * 4)
+    xh.attention_static(dc, qd.ptr, qh * D, eager.ptr, qh * D, xh.F32, B, 1, qh, SCALE, ctx - 1)
+    xh.synchronize()
+    want = eager.to_numpy(np.float32, q.shape)
+    ref = orc.attention_ref_f64(q, kc.as_f32(), vc.as_f32(), qh, kvh, D, [1] * B, [ctx - 1] * B, SCALE)
+    assert np.abs(want - ref).max() < 3e-3
+    st = xh.Stream()
+    od = xh.DeviceBuffer(q.size * 4)
+    with xh.Graph(st) as g:
+        xh.attention_static(dc, qd.ptr, qh * D, od.ptr, qh * D, xh.F32, B, 1, qh, SCALE, ctx - 1, stream=st.h)
+    for replay in range(3):
+        od.zero()
+        xh.synchronize()
+        g.launch()
+        st.synchronize()
+        assert np.array_equal(od.to_numpy(np.float32, q.shape), want), replay
+        # eager work of the same kind between the replays (shares the scratch array, one call at a time)
+        xh.attention_static(dc, qd.ptr, qh * D, eager.ptr, qh * D, xh.F32, B, 1, qh, SCALE, ctx - 1)
+        xh.synchronize()
+    g.free()

@@ -17,6 +17,7 @@
 // INT8 caches are widened to fp16 in registers (exact); the per-token key scale multiplies
 // the score column, the value scale multiplies the probability (gemm_kernel_ext.cpp:471-500,
 // gemm_kernel_ext2.cpp:75-91).
+#include <atomic>
 #include <mutex>
 
 
@@ -82,7 +83,7 @@ constexpr size_t kStaticTicketOffset = (size_t)kStaticSlots * kSlotFloats * size
 static __device__ __align__(256) unsigned char scratch[kStaticTicketOffset + (size_t)kStaticSlots * sizeof(unsigned int)];
 
 constexpr int kMaxDevices = 64;
-static void *g_scratch_ptr[kMaxDevices] = {};
+static std::atomic<void *> g_scratch_ptr[kMaxDevices] = {}; // written once under g_scratch_mu, read without it
 static std::mutex g_scratch_mu;
 
 // Resolves (once per device, with that device current) the device address of `scratch` and clears
@@ -92,13 +93,13 @@ int attention_static_scratch_init() {
     XFT_CHECK_HIP(hipGetDevice(&dev));
     XFT_REQUIRE(dev >= 0 && dev < kMaxDevices, "attention_static_scratch_init: device index %d out of range", dev);
     std::lock_guard<std::mutex> lk(g_scratch_mu);
-    if (g_scratch_ptr[dev] != nullptr) return 0;
+    if (g_scratch_ptr[dev].load(std::memory_order_acquire) != nullptr) return 0;
     void *ptr = nullptr;
     XFT_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
     XFT_REQUIRE(ptr != nullptr, "attention_static_scratch_init: no device address for the static scratch");
     XFT_CHECK_HIP(hipMemset((unsigned char *)ptr + kStaticTicketOffset, 0, (size_t)kStaticSlots * sizeof(unsigned int)));
     XFT_CHECK_HIP(hipDeviceSynchronize());
-    g_scratch_ptr[dev] = ptr;
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
     return 0;
 }
 
@@ -224,11 +225,12 @@ extern "C" int xfthip_attention_static(xfthip_kvcache_t c, const void *q, int qS
     int dev = -1;
     XFT_CHECK_HIP(hipGetDevice(&dev));
     XFT_REQUIRE(dev >= 0 && dev < kMaxDevices, "xfthip_attention_static: device index %d out of range", dev);
-    if (g_scratch_ptr[dev] == nullptr)
+    if (g_scratch_ptr[dev].load(std::memory_order_acquire) == nullptr)
         if (int rc = attention_static_scratch_init()) return rc;
+    unsigned char *base = (unsigned char *)g_scratch_ptr[dev].load(std::memory_order_acquire);
     AttnWorkspace w;
-    w.ws = (float *)g_scratch_ptr[dev];
-    w.tickets = (unsigned int *)((unsigned char *)g_scratch_ptr[dev] + kStaticTicketOffset);
+    w.ws = (float *)base;
+    w.tickets = (unsigned int *)(base + kStaticTicketOffset);
     w.slots = kStaticSlots;
     return attention_launch(c, q, qStride, out, oStride, out_dtype, B, S, qHeads, scale, past, past_dev, 0, (hipStream_t)stream, &w,
             true);

@@ -68,6 +68,8 @@ int gemm_grouped_rows_dev(const xfthip_weight_t *w, int n_group, const GroupWeig
     p.group_n = n_group;
     p.rows_stride = rows_stride;
     if (rows_each_max <= 32) {
+        XFT_REQUIRE(pw.KT * ktile_of(pw.kind) == pw.K, "gemm_grouped_rows_dev: the few-row form needs K = %d to be a whole number of %d-row weight tiles",
+                pw.K, ktile_of(pw.kind));
         p.M = rows_each_max; // the few-row kernel: a grid row a weight, each with at most this many rows
         return qgemm_skinny(pw, p, stream);
     }

@@ -195,6 +195,7 @@ struct xfthip_model {
     hipGraphExec_t graph = nullptr;
     int graph_B = 0;
     int graph_nsplit = 0; // attention split count the captured step was built with
+    bool graph_ragged = false; // the captured step's last node holds the `active` mask only in this mode
     int len_hint = 0; // upper bound of the sequence length during the current decode call (0 = unknown)
     hipStream_t graph_stream = nullptr;
     bool use_graph = true;
@@ -814,7 +815,8 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
     } else if (!m->use_graph) {
         for (int i = 0; i < steps; ++i)
             if (int rc = decode_step(m, B, st)) return rc;
-    } else if (m->graph == nullptr || m->graph_B != B || m->graph_stream != st || m->graph_nsplit != nsplit) {
+    } else if (m->graph == nullptr || m->graph_B != B || m->graph_stream != st || m->graph_nsplit != nsplit
+            || m->graph_ragged != m->ragged) {
         if (m->graph) {
             (void)hipGraphExecDestroy(m->graph);
             m->graph = nullptr;
@@ -844,6 +846,7 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
         XFT_CHECK_HIP(e);
         m->graph_B = B;
         m->graph_nsplit = nsplit;
+        m->graph_ragged = m->ragged;
         m->graph_stream = st;
     }
     if (!persistent && m->use_graph)

@@ -100,8 +100,21 @@ __global__ __launch_bounds__(512) void build_lists_kernel(const int *__restrict_
         }
     }
     __syncthreads();
+    // A token whose logits are NaN (or all -inf) has fewer than two choices: top2_kernel leaves -1 there, no wave
+    // ranked that choice, and it takes no row, as in the reference, whose loop over the experts never matches it
+    // (mlp_mixtral.h:165-186).  The gathered rows past the last expert's stay defined (token 0, weight 0): the
+    // gather runs over all 2 M rows.
+    const int total = s_off[E - 1] + s_count[E - 1];
     for (int i = threadIdx.x; i < 2 * M; i += blockDim.x) {
-        const int t = i >> 1, g = s_off[sel[i]] + rank[i];
+        const int e_sel = sel[i];
+        if (i >= total) row_token[i] = 0, row_weight[i] = 0.0f;
+        if (e_sel < 0 || e_sel >= E) slot_row[i] = -1;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 2 * M; i += blockDim.x) {
+        const int e_sel = sel[i];
+        if (e_sel < 0 || e_sel >= E) continue;
+        const int t = i >> 1, g = s_off[e_sel] + rank[i];
         slot_row[i] = g;
         row_token[g] = t;
         row_weight[g] = w[i];
@@ -128,6 +141,17 @@ __global__ __launch_bounds__(256) void combine_kernel(float *out, int ld, const 
     const int first = sel[2 * t] < sel[2 * t + 1] ? 0 : 1;
     const int ga = slot_row[2 * t + first], gb = slot_row[2 * t + 1 - first];
     const float wa = w[2 * t + first], wb = w[2 * t + 1 - first];
+    if (ga < 0 || gb < 0) {
+        // a choice without an expert (NaN logits) contributes nothing; not the common case, kept simple
+        const float *ea = eo + (size_t)(ga < 0 ? 0 : ga) * hidden, *eb = eo + (size_t)(gb < 0 ? 0 : gb) * hidden;
+        for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+            float o = in[(size_t)t * in_ld + c];
+            if (ga >= 0) o = fmaf(ea[c], wa, o);
+            if (gb >= 0) o = fmaf(eb[c], wb, o);
+            out[(size_t)t * ld + c] = o;
+        }
+        return;
+    }
     if (wide) { // rows of out start on 16-byte boundaries
         const float4 *ea = (const float4 *)(eo + (size_t)ga * hidden), *eb = (const float4 *)(eo + (size_t)gb * hidden);
         float4 *dst = (float4 *)(out + (size_t)t * ld);
@@ -277,6 +301,12 @@ int xfthip_moe_forward(xfthip_moe_t m, const float *x_in, int in_stride, float *
         const PackedWeight &g0 = m->gateup[0]->pw, &g = m->gateup[e]->pw, &d0 = m->down[0]->pw, &d = m->down[e]->pw;
         uniform = g.kind == g0.kind && g.flags == g0.flags && (g.zero != nullptr) == (g0.zero != nullptr) && d.kind == d0.kind
                 && d.flags == d0.flags && (d.zero != nullptr) == (d0.zero != nullptr);
+    }
+    // (the few-row form of the grouped launch has no K-tail variant: a K that is not a whole number of weight
+    // tiles goes expert by expert)
+    if (T <= 32) {
+        const PackedWeight &g0 = m->gateup[0]->pw, &d0 = m->down[0]->pw;
+        uniform = uniform && g0.KT * ktile_of(g0.kind) == g0.K && d0.KT * ktile_of(d0.kind) == d0.K;
     }
     if (uniform && m->gateup[0]->pw.kind != XFTHIP_W_W8A8 && m->down[0]->pw.kind != XFTHIP_W_W8A8) {
         if (int rc = gemm_grouped_rows_dev(m->gateup.data(), m->E, m->group, 2 * T, T, gemm_rows + 6, 9, m->xg, H, m->h, m->inter, XFTHIP_BF16, st))

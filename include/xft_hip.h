@@ -187,6 +187,15 @@ int xfthip_gemm_w8a8(xfthip_weight_t w, int M, const int8_t *qa, int ldq, const 
 int xfthip_rmsnorm(void *out, int out_dtype, const void *in, int in_dtype, const float *weight, int rows, int cols,
         int iStride, int oStride, float eps, xfthip_stream_t stream);
 
+/* ---- LayerNorm ---------------------------------------------------------------------- */
+/*
+ * y = (x - mean) * gamma / sqrt(E[x^2] - mean^2 + eps) + beta, fp32 arithmetic.  Replaces
+ * xft::invokeLayerNorm / LayerNorm::forward (src/kernels/layernorm_kernels.cpp:27-160).  in/out:
+ * XFTHIP_F32 or XFTHIP_BF16; gamma, beta: fp32 [cols]; strides in elements (-1 = cols).
+ */
+int xfthip_layernorm(void *out, int out_dtype, const void *in, int in_dtype, const float *gamma, const float *beta, int rows,
+        int cols, int iStride, int oStride, float eps, xfthip_stream_t stream);
+
 /* ---- rotary embedding --------------------------------------------------------------- */
 /*
  * cos/sin tables [maxPos, dim/2] fp32 in device memory, built as LlamaRotaryEmbedding does
@@ -348,6 +357,12 @@ int xfthip_model_set_layer(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthi
 int xfthip_model_set_attention(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthip_weight_t o, const float *ln1_host,
         const float *qkv_bias_host, const float *o_bias_host);
 int xfthip_model_set_mlp(xfthip_model_t m, int idx, xfthip_weight_t gateup, xfthip_weight_t down, const float *ln2_host);
+/* NormType::LN of the layer API (src/layers/decoder_layer.cpp:179-181, 195-197: the layer built over
+ * LayerNorm instead of RmsNorm): with shifts set, layer idx runs its two norms as LayerNorms with the
+ * weights given to xfthip_model_set_layer as gamma and these fp32 [hidden] host arrays as beta (as
+ * kernels of their own: the norm prologue of the decode GEMVs is RMSNorm only).  Null pointers turn the
+ * layer back into an RMSNorm layer. */
+int xfthip_model_set_layer_norm_shifts(xfthip_model_t m, int idx, const float *ln1_beta_host, const float *ln2_beta_host);
 /* A second weight set for layer idx that only the prompt pass (xfthip_model_prefill / _seq_prefill) uses; the
  * decode steps keep the layer's own set.  The reference's HybridModel (src/models/hybrid_model.h:25-84: one
  * model per weight type sharing context and KV cache, behind the "bf16_int8"-style type names).  Shapes as in
@@ -421,6 +436,11 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
  *   _seq_release: frees the row.
  * xfthip_model_prefill resets this state (all rows in lockstep again).
  */
+/* Logits of every prompt position (Model::forward(logitsAll = true), src/models/models.cpp:760-830,
+ * CommonDecoder::forward's logitsAll branch): final norm + lm_head over rows [first_row, first_row + rows)
+ * of the last prompt pass (xfthip_model_prefill: B * S rows, sequence after sequence; xfthip_model_seq_prefill:
+ * S rows), fp32 [rows, vocab] to host memory.  Valid until the next forward call of the model. */
+int xfthip_model_prompt_logits(xfthip_model_t m, int first_row, int rows, float *logits_host, xfthip_stream_t stream);
 int xfthip_model_seq_prefill(xfthip_model_t m, int row, const int *ids_host, int S, float *logits_host, xfthip_stream_t stream);
 int xfthip_model_seq_decode(xfthip_model_t m, const int *rows_host, int n, int *ids_out_host, xfthip_stream_t stream);
 int xfthip_model_seq_set_next_id(xfthip_model_t m, int row, int id);

@@ -259,6 +259,14 @@ def rmsnorm(x, weight, eps=1e-6):
     return out
 
 
+def layernorm(x, gamma, beta, eps=1e-5):
+    x = f32(x)
+    out = np.empty_like(x)
+    rows, cols = x.shape
+    lib.orc_layernorm(p(out), p(x), p(f32(gamma)), p(f32(beta)), rows, cols, -1, -1, C.c_float(eps))
+    return out
+
+
 def rope_tables(dim, max_pos, base=10000, scaling=1.0):
     half = (dim + 1) // 2
     cos = np.empty((max_pos, half), np.float32)
@@ -398,8 +406,11 @@ class LlamaLayerOracle:
 
     def __init__(self, hidden, inter, q_heads, kv_heads, head, wqkv, wo, wgateup, wdown, ln1, ln2, kv_int8=0,
                  batch=1, max_seq=256, eps=1e-6, rope_base=10000, max_pos=2048, rounding="fp32", gemm="oracle",
-                 prefill_attention="flash"):
+                 prefill_attention="flash", ln1_beta=None, ln2_beta=None):
         self.hidden, self.inter, self.qh, self.kvh, self.D = hidden, inter, q_heads, kv_heads, head
+        # shifts given: the layer built over LayerNorm instead of RmsNorm (NormType::LN, decoder_layer.cpp:179-181)
+        self.ln1_beta = None if ln1_beta is None else f32(ln1_beta)
+        self.ln2_beta = None if ln2_beta is None else f32(ln2_beta)
         self.wqkv, self.wo, self.wgateup, self.wdown = wqkv, wo, wgateup, wdown
         self.ln1, self.ln2, self.eps = f32(ln1), f32(ln2), eps
         self.kc = KVCache(kv_int8, batch, kv_heads, max_seq, head)
@@ -430,7 +441,7 @@ class LlamaLayerOracle:
         x = f32(x)
         T = B * S
         qcols, kvcols = self.qh * self.D, self.kvh * self.D
-        xn = self._r(rmsnorm(x, self.ln1, self.eps))
+        xn = self._r(rmsnorm(x, self.ln1, self.eps) if self.ln1_beta is None else layernorm(x, self.ln1, self.ln1_beta, self.eps))
         qkv = self._r(self._mm(self.wqkv, xn))
         stride = qkv.shape[1]
         flat = qkv.reshape(-1)
@@ -451,7 +462,7 @@ class LlamaLayerOracle:
             att = cross_attn_by_head(q, k, v, self.qh, self.kvh, self.D, [S] * B, [past] * B, scale, self.kc, self.vc)
         att = self._r(att)
         x1 = self._mm(self.wo, att, epi=EPI_RESIDENTIAL, res=x)
-        xn2 = self._r(rmsnorm(x1, self.ln2, 1e-6))
+        xn2 = self._r(rmsnorm(x1, self.ln2, 1e-6) if self.ln2_beta is None else layernorm(x1, self.ln2, self.ln2_beta, 1e-6))
         h = self._r(silu_sum(self._mm(self.wgateup, xn2)))
         return self._mm(self.wdown, h, epi=EPI_RESIDENTIAL, res=x1)
 

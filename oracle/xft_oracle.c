@@ -531,6 +531,35 @@ ORC_API void orc_rmsnorm(float *out, const float *in, const float *weight, int r
     }
 }
 
+/* LayerNorm (src/kernels/layernorm_kernels.cpp:27-81): sum and sum of squares in one pass over 16 lanes,
+ * mean = sum / n, var = 1 / sqrt(sq / n - mean^2 + eps), y = (x - mean) * gamma * var + beta (that order).
+ * Pinned by the two-pass float64 definition the reference's own test uses (tests/ut/layers_norm_test.cpp:24-52). */
+ORC_API void orc_layernorm(float *out, const float *in, const float *gamma, const float *beta, int rows, int cols, int iStride,
+        int oStride, float eps) {
+    if (iStride == -1) iStride = cols;
+    if (oStride == -1) oStride = cols;
+#pragma omp parallel for
+    for (int r = 0; r < rows; ++r) {
+        const float *px = in + (int64_t)r * iStride;
+        float *py = out + (int64_t)r * oStride;
+        float ls[16], lq[16];
+        for (int l = 0; l < 16; ++l) ls[l] = 0.0f, lq[l] = 0.0f;
+        for (int c = 0; c < cols; ++c) {
+            ls[c & 15] = ls[c & 15] + px[c];
+            float t = px[c] * px[c];
+            lq[c & 15] = lq[c & 15] + t;
+        }
+        float sum = reduce_add16(ls), sq = reduce_add16(lq);
+        float mean = sum / cols;
+        float var = (float)(1 / sqrt((double)(sq / cols - mean * mean + eps)));
+        for (int c = 0; c < cols; ++c) {
+            float t = (px[c] - mean) * gamma[c];
+            t = t * var;
+            py[c] = t + beta[c];
+        }
+    }
+}
+
 /* ------------------------------------------------------------------------- */
 /* RoPE  (src/layers/rotary_embedding.cpp:21-66, kernels :21-199)             */
 /* ------------------------------------------------------------------------- */

@@ -42,7 +42,7 @@ def test_c_abi_exports_every_declared_symbol():
 def test_host_layer_exports_reference_entry_points(tmp_path):
     out = subprocess.check_output(["nm", "-DC", "--defined-only", LIB_LAYERS], text=True)
     for fn in ("xft::invokeLayerLLaMA(", "xft::invokeAttentionLLaMA(", "xft::invokeAttention(", "xft::invokeMLPLLaMA(", "xft::invokeGemm(",
-               "xft::invokeRmsNorm(", "xft::invokeRotaryEmbedding("):
+               "xft::invokeRmsNorm(", "xft::invokeLayerNorm(", "xft::invokeRotaryEmbedding("):
         assert fn in out, fn
     # the signatures are the reference's: a translation unit written against its headers links
     src = r'''
@@ -65,6 +65,7 @@ def test_host_layer_exports_reference_entry_points(tmp_path):
                     nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, false, nullptr);
             xft::invokeGemm(xft::DataType::bf16, false, false, 1, 1, 8, 1.0f, nullptr, 8, nullptr, 0.0f, nullptr, 1);
             xft::invokeRmsNorm(xft::DataType::fp32, nullptr, nullptr, nullptr, 1, 8);
+            xft::invokeLayerNorm(xft::DataType::fp32, nullptr, nullptr, nullptr, nullptr, 1, 8);
             xft::invokeRotaryEmbedding(xft::DataType::bf16, nullptr, nullptr, nullptr, nullptr, nullptr, 128, 128, 128, 1, 1,
                     128, 1);
         }
@@ -124,3 +125,36 @@ def test_package_refuses_to_import_without_the_library(tmp_path):
     code = "import sys; sys.path.insert(0, %r); import xfastertransformer_amd.capi" % str(tmp_path)
     r = subprocess.run(["python3", "-c", code], capture_output=True, text=True)
     assert r.returncode != 0 and "no CPU fallback" in r.stderr
+
+
+@pytest.mark.skipif(not os.path.exists(LIB_LAYERS), reason="host library not built")
+def test_model_header_declares_what_the_reference_declares():
+    """Every public member function the reference's include/models.h declares for xft::Model (its
+    lines 24-141) is declared here with the same parameter list, apart from the documented exclusions;
+    all nine set_input overloads are exported."""
+    ours = open(os.path.join(ROOT, "include", "models.h")).read()
+    ours = re.sub(r"//[^\n]*", "", ours)
+    flat = re.sub(r"\s+", " ", ours)
+    # the reference's declarations, parameter lists normalised to single spaces
+    want = [
+        "void input(std::vector<int32_t> &inputIds_, int batchSize_);",
+        "void config(SearcherConfig &config_, const std::vector<std::vector<int>> &stopWordsList_ = {});",
+        "std::vector<int> set_input(std::vector<int32_t> &inputIds_, int batchSize_, int maxLen_ = -1, int numBeams_ = 1,",
+        "std::vector<int> set_input(std::vector<int32_t> &inputIds_, int batchSize_, SearcherConfig &config_,",
+        "std::vector<int> set_input(std::vector<std::vector<int32_t>> &inputIds_, SearcherConfig &config_,",
+        "std::vector<int> set_input(std::vector<std::vector<int32_t>> &inputIds_, int maxLen_ = -1, int numBeams_ = 1,",
+        "std::vector<int> set_input(std::vector<std::vector<int32_t>> &inputIds_, std::vector<int> seqIDs, SearcherConfig &config_,",
+        "std::vector<int> set_input( std::vector<std::vector<int32_t>> &inputIds_, std::vector<int> seqIDs = {}, int maxLen = -1);",
+        "std::vector<int> set_input( std::vector<int32_t> &inputIds_, int batchSize_, std::vector<int> seqIDs = {}, int maxLen = -1);",
+        "std::vector<int> set_input( std::vector<int32_t> &inputIds_, int batchSize_, std::vector<int> seqIDs, const std::vector<int> &maxLen);",
+        "std::vector<int> set_input(std::vector<int32_t> &inputIds_, std::vector<int32_t> &seqLens_, std::vector<int> seqIDs, std::vector<int> &maxLen);",
+        "bool isDone();", "std::tuple<float *, int, int> forward(bool logitsAll = true);", "std::vector<int32_t> generate();",
+        "void createSearcher(SearcherConfig &config_);", "void initMaxSeqLen();", "std::vector<int32_t> finalize();",
+        "void setPrefix(std::vector<int32_t> &prefixIDs);", "void unsetPrefix();",
+        "bool setStopWords(std::vector<std::vector<int>> stopWordsList);", "bool freeSeqs(std::vector<int> &seqIDs);",
+    ]
+    for decl in want:
+        assert decl in flat, decl
+    out = subprocess.check_output(["nm", "-D", "--defined-only", LIB_LAYERS], text=True)
+    assert len([l for l in out.splitlines() if "_ZN3xft5Model9set_inputE" in l]) == 9
+    assert "_ZN3xft15invokeLayerNormENS_8DataTypeEPvPKvS3_S3_iiiif" in out

@@ -374,3 +374,39 @@ def test_first_token_and_next_token_weight_types(xh, orc, am, tmp_path, dtype):
             for t in (first, nxt)]
     print(f"{dtype}: equal to pure {first}: {np.array_equal(out, pure[0])}, to pure {nxt}: {np.array_equal(out, pure[1])}", flush=True)
     model.free()
+
+
+def test_every_set_input_overload_through_the_cpp_api(am, tmp_path):
+    """tests/set_input_driver.cpp (built with the libraries) calls all nine Model::set_input overloads of
+    include/models.h, generate(), forward(false / true) and freeSeqs the way a program written against the
+    reference's header does (include/models.h:40-73, src/models/models.cpp:238-683) and checks that every
+    sequence continues as it does alone.  Here: it must pass, and its lockstep ids must be the ones the
+    Python face gets for the same prompts."""
+    import subprocess
+    import make_llama_fixture as fx
+    driver = os.path.join(ROOT, "xfastertransformer_amd", "csrc", "build", "set_input_driver")
+    assert os.path.exists(driver), "tests/set_input_driver.cpp is not built; run `python -m xfastertransformer_amd.build`"
+    held = fx.write_model_dir(str(tmp_path / "model"), None, 31)
+    V = held["cfg"]["vocab"]
+    run = subprocess.run([driver, str(tmp_path / "model"), "int8", str(V)], capture_output=True, text=True, timeout=300)
+    print(run.stdout[-3000:], run.stderr[-2000:], flush=True)
+    assert run.returncode == 0 and "PASSED" in run.stdout and "FAIL" not in run.stdout.replace("FAILED", "")
+    alone = [[int(t) for t in line.split()[1:]] for line in run.stdout.splitlines() if line.startswith("ALONE")]
+    assert len(alone) == 3 and all(len(a) == 6 for a in alone)
+
+    def prompt_of(n, salt):  # the driver's generator (xorshift64)
+        s = (88172645463325252 + salt * 7919) & (2 ** 64 - 1)
+        out = []
+        for _ in range(n):
+            s ^= (s << 13) & (2 ** 64 - 1)
+            s ^= s >> 7
+            s ^= (s << 17) & (2 ** 64 - 1)
+            out.append(s % V)
+        return np.asarray(out, np.int32)
+
+    model = am.AutoModel.from_pretrained(str(tmp_path / "model"), dtype="int8")
+    for k, (n, salt) in enumerate(((7, 1), (7, 2), (12, 3))):
+        p = prompt_of(n, salt)
+        out = model.generate(p[None, :], max_length=n + 6, eos_token_id=V + 5)
+        assert out[0, n:].tolist() == alone[k], (k, out[0, n:].tolist(), alone[k])
+    model.free()

@@ -10,8 +10,13 @@ activations to bf16 where the GPU pipeline does, runs its prefill attention at t
 FP16 cache (the reference's route for a prefill over a past; its flash-style route for a first
 prefill narrows K, V and the probabilities to bf16, and through 32 randomly initialised layers that
 one point alone moves the logits by ~0.2, which the INT8 batch-1 case prints), and is teacher-forced
-with the GPU's tokens, so every step is checked: the GPU's id must be the oracle's best logit or
-within the logit tolerance."""
+with the GPU's tokens, so every step is checked against the GPU's own logits of that step:
+  * prompt logits: cosine >= 0.9997, max-abs <= 0.15 (|logit| reaches 6);
+  * every decode step's logits: the same two bars;
+  * a GPU token that is not the oracle's best must lie within 1.5 x that step's measured max-abs
+    logit difference of the oracle's best (in the oracle's logits): the two pipelines then
+    disagree only about a pair they cannot tell apart;
+  * at least 85 % of the choices are the oracle's best."""
 import time
 
 import numpy as np
@@ -21,9 +26,7 @@ pytestmark = pytest.mark.gpu
 
 HIDDEN, INTER, QH, KVH, D, LAYERS, VOCAB = 4096, 11008, 32, 32, 128, 32, 32000
 PROMPT, STEPS = 512, 32
-# a GPU token may differ from the oracle's best only where the oracle's own logits put the two
-# closer than the noise two faithful pipelines of this random 32-layer model show (see the prefill check)
-LOGIT_TOL = 0.2
+COS_BAR, ABS_BAR, GAP_FACTOR, EXACT_SHARE = 0.9997, 0.15, 1.5, 0.85
 
 
 @pytest.fixture(scope="module")
@@ -79,7 +82,7 @@ def _build(xh, orc, head, kind, B_gpu, B_orc, also_flash=False):
     return model, orc.LlamaModelOracle(olayers, emb, fn, lm), flash, (dws, lmw)
 
 
-@pytest.mark.parametrize("kind,B", [(0, 1), (1, 1), (0, 32)])
+@pytest.mark.parametrize("kind,B", [(0, 1), (1, 1), (0, 32), (1, 32)])
 def test_full_model_greedy_32_steps(xh, orc, head, kind, B):
     print(f"case kind={kind} B={B}", flush=True)
     t0 = time.time()
@@ -87,7 +90,10 @@ def test_full_model_greedy_32_steps(xh, orc, head, kind, B):
     model, ref, flash, keep = _build(xh, orc, head, kind, B, len(follow), also_flash=(kind == 0 and B == 1))
     ids = np.random.default_rng(3).integers(0, VOCAB, (B, PROMPT)).astype(np.int32)
     first, logits = model.prefill(ids, want_logits=True)
-    got = model.decode(STEPS, B)
+    got, glogits = [], []
+    for t in range(STEPS):  # one graph replay a step, so that every step's logits can be read
+        got.append(model.decode(1, B)[0])
+        glogits.append(model.logits(B)[follow].copy())
     assert model.decode_mode() == 1  # replays of the captured decode graph
     t1 = time.time()
     Bo = len(follow)
@@ -98,7 +104,7 @@ def test_full_model_greedy_32_steps(xh, orc, head, kind, B):
     # Through 32 randomly initialised layers every bf16 hand-over re-rounds the difference it
     # receives (an intermediate that differs by 5e-5 lands on the neighbouring bf16 value in a few
     # per cent of the elements), so one layer's 5e-3 rms grows to ~2e-2 rms on the logits.
-    assert cos >= 0.9995 and err < 0.2
+    assert cos >= COS_BAR and err <= ABS_BAR
     if flash is not None:
         flogits, _ = flash.step(ids[follow], Bo, PROMPT, 0)
         print(f"oracle with the flash-style prefill (bf16 K/V/probabilities): differs from the cache-precision oracle by "
@@ -106,24 +112,33 @@ def test_full_model_greedy_32_steps(xh, orc, head, kind, B):
               f"(cosine {_cos(logits[follow], flogits):.6f})", flush=True)
         assert _cos(logits[follow], flogits) >= 0.999
 
-    def check(g, lg):
+    worst = dict(err=err, cos=cos, gap_ratio=0.0)
+
+    def check(g, gpu_lg, lg, what):
+        """g: the GPU's tokens; gpu_lg / lg: the GPU's and the oracle's logits of the same step."""
         same = 0
+        step_err = float(np.abs(gpu_lg - lg).max())
+        step_cos = _cos(gpu_lg, lg)
+        worst["err"], worst["cos"] = max(worst["err"], step_err), min(worst["cos"], step_cos)
+        assert step_cos >= COS_BAR and step_err <= ABS_BAR, (what, step_cos, step_err)
         for j in range(Bo):
+            assert int(g[j]) == int(gpu_lg[j].argmax()), (what, j)  # the device arg-max picked the GPU's own best logit
             best = int(lg[j].argmax())
             gap = float(lg[j, best] - lg[j, g[j]])
-            assert gap <= LOGIT_TOL, (j, int(g[j]), best, gap)
+            worst["gap_ratio"] = max(worst["gap_ratio"], gap / step_err)
+            assert gap <= GAP_FACTOR * step_err, (what, j, int(g[j]), best, gap, step_err)
             same += int(g[j] == best)
         return same
 
-    exact = check(first[follow], elogits)
+    exact = check(first[follow], logits[follow], elogits, "prompt")
     cur = first[follow]
     for t in range(STEPS):
         elogits, _ = ref.step(cur.reshape(Bo, 1), Bo, 1, PROMPT + t)
-        exact += check(got[t][follow], elogits)
+        exact += check(got[t][follow], glogits[t], elogits, f"step {t}")
         cur = got[t][follow]
     total = (STEPS + 1) * Bo
-    print(f"greedy ids equal to the oracle's best in {exact} of {total} choices; gpu {t1 - t0:.1f} s, "
-          f"oracle {time.time() - t1:.1f} s", flush=True)
-    assert exact >= total * 3 // 4
+    print(f"greedy ids equal to the oracle's best in {exact} of {total} choices; worst step: max-abs {worst['err']:.3e}, cosine "
+          f"{worst['cos']:.6f}, gap / max-abs {worst['gap_ratio']:.2f}; gpu {t1 - t0:.1f} s, oracle {time.time() - t1:.1f} s", flush=True)
+    assert exact >= EXACT_SHARE * total
     orc.clear_blas_cache()
     model.free()

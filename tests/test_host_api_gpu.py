@@ -278,3 +278,78 @@ def test_invoke_rotary_embedding_reads_the_second_half_of_the_tables(host, orc):
             buf[t, :, h:] = b * cos[pos[t], h:] + a * sin[pos[t], h:]
     host["rope"](FP32, ptr(pos), ptr(q), ptr(k), ptr(cos), ptr(sin), D, heads * D, heads * D, T, heads, D, heads)
     assert np.abs(q - eq.reshape(T, -1)).max() < 1e-6 and np.abs(k - ek.reshape(T, -1)).max() < 1e-6
+
+
+@pytest.fixture(scope="module")
+def host_ln():
+    C.CDLL(os.path.join(ROOT, "xfastertransformer_amd", "libxft_hip.so"), mode=C.RTLD_GLOBAL)
+    lib = C.CDLL(os.path.join(ROOT, "xfastertransformer_amd", "libxft_layers.so"))
+    fn = getattr(lib, "_ZN3xft15invokeLayerNormENS_8DataTypeEPvPKvS3_S3_iiiif")
+    fn.argtypes = [I, P, P, P, P, I, I, I, I, F]
+    fn.restype = None
+    return fn
+
+
+@pytest.mark.parametrize("rows,cols", [(128, 128), (33, 5120), (7, 5120 * 3), (5, 137)])
+def test_invoke_layer_norm_reference_test_shapes(host_ln, orc, rows, cols):
+    """xft::invokeLayerNorm against the two-pass definition and at the tolerance of the reference's own test
+    (tests/ut/layers_norm_test.cpp:24-96: inputs uniform on [0, 1), |d| < 0.01), fp32 and bf16 buffers, with
+    gamma and beta that are not the identity, and with row strides."""
+    rng = np.random.default_rng(rows + cols)
+    x = rng.random((rows, cols)).astype(np.float32)
+    g = rng.uniform(0.5, 1.5, cols).astype(np.float32)
+    b = rng.uniform(-1, 1, cols).astype(np.float32)
+    x64 = x.astype(np.float64)
+    mean = x64.mean(1, keepdims=True)
+    exp = g * (x64 - mean) / np.sqrt(((x64 - mean) ** 2).mean(1, keepdims=True) + 1e-5) + b
+    out = np.zeros_like(x)
+    host_ln(FP32, ptr(out), ptr(x), ptr(g), ptr(b), rows, cols, -1, -1, 1e-5)
+    assert np.abs(out - exp).max() < 1e-4
+    assert np.abs(out - orc.layernorm(x, g, b, 1e-5)).max() < 1e-4
+    # strided rows: the gaps of the output stay as they were
+    xs = np.full((rows, cols + 8), 7.0, np.float32)
+    xs[:, :cols] = x
+    outs = np.full((rows, cols + 16), -3.0, np.float32)
+    host_ln(FP32, ptr(outs), ptr(xs), ptr(g), ptr(b), rows, cols, cols + 8, cols + 16, 1e-5)
+    assert np.array_equal(outs[:, :cols], out) and (outs[:, cols:] == -3.0).all()
+    # bf16 buffers (input, gamma, beta and output all bf16)
+    xb, gb, bb = orc.to_bf16(x), orc.to_bf16(g), orc.to_bf16(b)
+    outb = np.zeros((rows, cols), np.uint16)
+    host_ln(BF16, ptr(outb), ptr(xb), ptr(gb), ptr(bb), rows, cols, -1, -1, 1e-5)
+    xr, gr, br = orc.round_bf16(x).astype(np.float64), orc.round_bf16(g).astype(np.float64), orc.round_bf16(b).astype(np.float64)
+    m = xr.mean(1, keepdims=True)
+    expb = gr * (xr - m) / np.sqrt(((xr - m) ** 2).mean(1, keepdims=True) + 1e-5) + br
+    gotb = orc.from_bf16(outb) if hasattr(orc, "from_bf16") else (outb.astype(np.uint32) << 16).view(np.float32)
+    assert np.abs(gotb - expb).max() < 0.01 * max(1.0, float(np.abs(expb).max()))
+
+
+def test_invoke_layer_llama_with_layer_norm(host, orc):
+    """NormType::LN (decoder_layer.cpp:179-181, 195-197): the layer over LayerNorm with gamma and beta, prefill
+    of 18 tokens and two decode steps as in layers_decoder_test.cpp:25-60, against the oracle's layer with the
+    same norm; and the result differs from the RMSNorm layer's (the shifts are used)."""
+    LN = 1
+    hidden, inter, qh, kvh, D = 1024, 2816, 8, 8, 128
+    rng = np.random.default_rng(44)
+    qkv, wo, gate, up, down = _layer_weights(rng, hidden, inter, qh, kvh, D)
+    ln1 = rng.uniform(0.8, 1.2, hidden).astype(np.float32)
+    ln2 = rng.uniform(0.8, 1.2, hidden).astype(np.float32)
+    b1 = rng.uniform(-0.3, 0.3, hidden).astype(np.float32)
+    b2 = rng.uniform(-0.3, 0.3, hidden).astype(np.float32)
+    ow = [_oracle_weight(orc, BF16, w) for w in (qkv, wo, np.concatenate([gate, up], 1), down)]
+    ref = orc.LlamaLayerOracle(hidden, inter, qh, kvh, D, *ow, ln1, ln2, max_seq=32, ln1_beta=b1, ln2_beta=b2)
+    rms = orc.LlamaLayerOracle(hidden, inter, qh, kvh, D, *ow, ln1, ln2, max_seq=32)
+    qcols, kvcols = qh * D, kvh * D
+    past = 0
+    for step, S in enumerate((18, 1, 1)):
+        x = (rng.standard_normal((S, hidden)) + 0.5).astype(np.float32)  # a mean that RMSNorm would keep
+        out = np.zeros_like(x)
+        host["layer"](BF16, SILU, LN, 1, S, D, qh, kvh, 32, 32, past, past + S, step, hidden, inter, ptr(out), hidden, ptr(x), hidden,
+                      ptr(ln1), ptr(b1), ptr(qkv), C.c_void_p(qkv.ctypes.data + qcols * 4),
+                      C.c_void_p(qkv.ctypes.data + (qcols + kvcols) * 4), ptr(wo), ptr(ln2), ptr(b2), ptr(gate), ptr(up), ptr(down),
+                      None, None, None, None)
+        exp = ref.forward(x, 1, S, past)
+        other = rms.forward(x, 1, S, past)
+        err = np.abs(out - exp)
+        assert _cos(out, exp) >= 0.9999 and err.max() < 5e-2 and np.sqrt((err ** 2).mean()) < 1e-2, (step, err.max())
+        assert np.abs(out - other).max() > 10 * err.max()
+        past += S

@@ -320,6 +320,26 @@ def test_rmsnorm_closed_form():
         assert np.abs(orc.rmsnorm(x, w) - exp).max() < 2e-6 * np.abs(exp).max() + 1e-6
 
 
+def test_layernorm_two_pass_definition():
+    """orc_layernorm (one pass, E[x^2] - mean^2) against the two-pass float64 definition that the reference's
+    own test compares with (tests/ut/layers_norm_test.cpp:24-52, tolerance 0.01 there), at its shapes and with
+    an offset that would expose a dropped mean or a wrong sign of the shift."""
+    rng = np.random.default_rng(93)
+    for rows, cols in ((4, 128), (3, 5120), (2, 137)):
+        x = (rng.random((rows, cols)) + 3.0).astype(np.float32)
+        g = rng.uniform(0.5, 1.5, cols).astype(np.float32)
+        b = rng.uniform(-1, 1, cols).astype(np.float32)
+        x64 = x.astype(np.float64)
+        mean = x64.mean(1, keepdims=True)
+        var = ((x64 - mean) ** 2).mean(1, keepdims=True)
+        exp = g * (x64 - mean) / np.sqrt(var + 1e-5) + b
+        got = orc.layernorm(x, g, b, 1e-5)
+        assert np.abs(got - exp).max() < 2e-4  # the one-pass variance of values near 3.5 loses ~5 digits in fp32
+        # unit gamma, zero beta: rows have mean 0 and variance 1 - eps / (var + eps)
+        y = orc.layernorm(x, np.ones(cols, np.float32), np.zeros(cols, np.float32), 1e-5).astype(np.float64)
+        assert np.abs(y.mean(1)).max() < 1e-4 and np.abs(y.var(1) - var.ravel() / (var.ravel() + 1e-5)).max() < 2e-3
+
+
 def test_softmax_closed_form():
     x = _rand(1000, 92, 3.0)
     s = orc.softmax_scaled(x, 0.25)

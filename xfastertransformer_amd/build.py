@@ -14,6 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 ROOT = os.path.dirname(HERE)
 LIB_HIP = os.path.join(HERE, "libxft_hip.so")
 LIB_LAYERS = os.path.join(HERE, "libxft_layers.so")
+LIB_TORCH = os.path.join(HERE, "libxft_pt.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # gfx950 only; packed-FP32 VALU ops stay off (the compiler must not form v_pk_*_f32)
@@ -85,9 +86,42 @@ def build_host(force=True):
     return LIB_LAYERS
 
 
+def build_torch(force=True):
+    """torch.classes.xfastertransformer.AutoModel over libxft_layers.so: g++ against the Torch headers of this
+    interpreter's torch (no HIP code, no torch device memory: token ids and logits are host tensors)."""
+    src = os.path.join(CSRC, "torch", "xft_torch.cpp")
+    deps = [src, os.path.join(ROOT, "include", "models.h"), LIB_LAYERS]
+    if not (force or _stale(LIB_TORCH, deps)):
+        return LIB_TORCH
+    import torch
+    from torch.utils import cpp_extension
+    inc = []
+    for d in cpp_extension.include_paths():
+        inc += ["-isystem", d]
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    abi = "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    _run([os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-variable", abi, src, "-o", LIB_TORCH]
+         + inc + ["-L" + HERE, "-lxft_layers", "-lxft_hip", "-L" + tlib, "-ltorch", "-ltorch_cpu", "-lc10", "-Wl,-rpath,$ORIGIN",
+                  "-Wl,-rpath," + tlib])
+    return LIB_TORCH
+
+
+def build_test_drivers(force=True):
+    """C++ programs of the test suite that call the host API the way a program written against the reference's
+    headers would (built here, not inside a GPU test)."""
+    out = os.path.join(CSRC, "build", "set_input_driver")
+    src = os.path.join(ROOT, "tests", "set_input_driver.cpp")
+    if force or _stale(out, [src, LIB_LAYERS, os.path.join(ROOT, "include", "models.h")]):
+        _run([os.environ.get("CXX", "g++"), "-O1", "-std=c++17", "-Wall", "-I" + os.path.join(ROOT, "include"), src, "-o", out, "-L" + HERE,
+              "-lxft_layers", "-lxft_hip", "-Wl,-rpath," + HERE])
+    return out
+
+
 def build_all(force=True):
     build_hip(force)
-    return build_host(force)
+    build_host(force)
+    build_test_drivers(force)
+    return build_torch(force)
 
 
 if __name__ == "__main__":

@@ -88,6 +88,7 @@ struct Entry {
     xfthip_model_t model = nullptr;
     xfthip_weight_t qkv = nullptr, o = nullptr, gateup = nullptr, down = nullptr;
     std::vector<float> ln1, ln2, qkvBias, oBias;
+    std::vector<float> ln1Beta, ln2Beta; // NormType::LN layers only
     xfthip_model_config cfg {};
     bool hasAttn = false, hasMlp = false;
 };
@@ -100,6 +101,7 @@ void build_model(Entry &e) {
         CK(xfthip_model_set_attention(e.model, 0, e.qkv, e.o, e.ln1.empty() ? nullptr : e.ln1.data(),
                 e.qkvBias.empty() ? nullptr : e.qkvBias.data(), e.oBias.empty() ? nullptr : e.oBias.data()));
     if (e.hasMlp) CK(xfthip_model_set_mlp(e.model, 0, e.gateup, e.down, e.ln2.empty() ? nullptr : e.ln2.data()));
+    if (!e.ln1Beta.empty()) CK(xfthip_model_set_layer_norm_shifts(e.model, 0, e.ln1Beta.data(), e.ln2Beta.data()));
 }
 
 // grow the model when a call needs more batch / tokens / positions than it was built for
@@ -141,13 +143,17 @@ void invokeLayerLLaMA(DataType dt, ActivationType at, NormType nt, int batchSize
         const float *keyBias, const float *valueBias, const float *attnOutBias) {
     static std::mutex mutex;
     std::lock_guard<std::mutex> lock(mutex);
-    (void)ln1Beta; (void)ln2Beta; (void)currentSeqLen; (void)step;
+    (void)currentSeqLen; (void)step;
 
     const int kind = kind_of(dt);
     if (kind < 0) return; // message printed, output untouched, as the reference (decoder_layer.cpp:172-206)
-    if (nt != NormType::RMS) {
-        printf(">> unsupported norm type (this build implements RMSNorm layers)\n");
+    if (nt != NormType::RMS && nt != NormType::LN) {
+        printf(">> unsupported norm type\n");
         return;
+    }
+    if (nt == NormType::LN && (!ln1Beta || !ln2Beta)) {
+        printf(">> NormType::LN needs ln1Beta and ln2Beta\n");
+        exit(-1);
     }
     if (at != ActivationType::SILU && at != ActivationType::SWIGLU) {
         printf(">> unsupported activation type\n");
@@ -170,6 +176,11 @@ void invokeLayerLLaMA(DataType dt, ActivationType at, NormType nt, int batchSize
         e.down = make_weight(kind, intermediateSize, hiddenSize, (const float *)downWeight, XFTHIP_WF_NONE);
         e.ln1.assign(ln1Gamma, ln1Gamma + hiddenSize);
         e.ln2.assign(ln2Gamma, ln2Gamma + hiddenSize);
+        if (nt == NormType::LN) {
+            // the layer over LayerNorm instead of RmsNorm (decoder_layer.cpp:179-181, 195-197)
+            e.ln1Beta.assign(ln1Beta, ln1Beta + hiddenSize);
+            e.ln2Beta.assign(ln2Beta, ln2Beta + hiddenSize);
+        }
         e.qkvBias = concat_bias(queryBias, keyBias, valueBias, qCols, kvCols);
         if (attnOutBias) e.oBias.assign(attnOutBias, attnOutBias + hiddenSize);
         e.hasAttn = e.hasMlp = true;
@@ -353,6 +364,36 @@ void invokeRmsNorm(DataType dt, void *output, const void *input, const void *wei
     CK(xfthip_memcpy_h2d(dop, output, ((size_t)(rows - 1) * oStride + cols) * esz, nullptr)); // keep the gaps between rows
     CK(xfthip_memcpy_h2d(dw, w.data(), (size_t)cols * 4, nullptr));
     CK(xfthip_rmsnorm(dop, et, di, et, (const float *)dw, rows, cols, iStride, oStride, epsilon, nullptr));
+    CK(xfthip_memcpy_d2h(output, dop, ((size_t)(rows - 1) * oStride + cols) * esz, nullptr));
+    xfthip_free(di);
+    xfthip_free(dop);
+    xfthip_free(dw);
+}
+
+void invokeLayerNorm(DataType dt, void *output, const void *input, const void *gamma, const void *beta, int rows, int cols,
+        int iStride, int oStride, float epsilon) {
+    // fp32 and bf16 buffers; fp16 activations are not offered by this build (the reference's dispatch has no
+    // else-branch either: an unknown dt is a silent no-op, layernorm_kernels.cpp:148-160)
+    if (dt != DataType::fp32 && dt != DataType::bf16) return;
+    ensure_init();
+    if (iStride == -1) iStride = cols;
+    if (oStride == -1) oStride = cols;
+    const int et = dt == DataType::fp32 ? XFTHIP_F32 : XFTHIP_BF16;
+    const size_t esz = dt == DataType::fp32 ? 4 : 2;
+    // gamma and beta have the element type of dt; the kernel wants fp32
+    std::vector<float> gb((size_t)2 * cols);
+    for (int i = 0; i < cols; ++i) {
+        gb[i] = dt == DataType::fp32 ? ((const float *)gamma)[i] : from_bf16(((const uint16_t *)gamma)[i]);
+        gb[cols + i] = dt == DataType::fp32 ? ((const float *)beta)[i] : from_bf16(((const uint16_t *)beta)[i]);
+    }
+    void *di = nullptr, *dop = nullptr, *dw = nullptr;
+    CK(xfthip_malloc(&di, (size_t)rows * iStride * esz));
+    CK(xfthip_malloc(&dop, (size_t)rows * oStride * esz));
+    CK(xfthip_malloc(&dw, gb.size() * 4));
+    CK(xfthip_memcpy_h2d(di, input, ((size_t)(rows - 1) * iStride + cols) * esz, nullptr));
+    CK(xfthip_memcpy_h2d(dop, output, ((size_t)(rows - 1) * oStride + cols) * esz, nullptr)); // keep the gaps between rows
+    CK(xfthip_memcpy_h2d(dw, gb.data(), gb.size() * 4, nullptr));
+    CK(xfthip_layernorm(dop, et, di, et, (const float *)dw, (const float *)dw + cols, rows, cols, iStride, oStride, epsilon, nullptr));
     CK(xfthip_memcpy_d2h(output, dop, ((size_t)(rows - 1) * oStride + cols) * esz, nullptr));
     xfthip_free(di);
     xfthip_free(dop);

@@ -469,6 +469,7 @@ struct ModelImpl {
     struct Seq {
         int id = 0, row = 0, step = 0;
         bool done = false;
+        bool forwardOnly = false; // made by the set_input forms that carry no searcher config: Model::forward() runs it
         std::vector<int32_t> prompt, generated;
         SearcherConfig cfg;
         std::vector<int> cachedRepetVec;
@@ -901,14 +902,53 @@ bool Model::isDone() {
     return true;
 }
 
+// models.cpp:760-830.  After input(): the prompt pass of the whole batch, (logits, 0, vocab) with the logits of
+// the last position of every sequence, or of every position when logitsAll.  After set_input(): one pass of
+// the working sequences, all prompts or all decodes, (logits, rows, vocab) with one row a sequence, or one a
+// prompt token when logitsAll and the sequences are prompts.
 std::tuple<float *, int, int> Model::forward(bool logitsAll) {
     ModelImpl &s = *impl;
-    if (logitsAll) unsupported("Model::forward(logitsAll = true)");
+    if (s.cbMode) {
+        if (s.working.empty()) {
+            printf("Please input prompt first.\n");
+            exit(-1);
+        }
+        const int n = (int)s.working.size();
+        std::vector<ModelImpl::Seq *> seqs;
+        for (int id : s.working) seqs.push_back(&s.pool.at(id));
+        const bool prompts = seqs[0]->step == 0;
+        for (auto *q : seqs)
+            if ((q->step == 0) != prompts) {
+                printf("[ERROR] The sequences of one step must be all prompts or all decodes.\n");
+                exit(-1);
+            }
+        if (prompts) {
+            size_t total = 0;
+            for (auto *q : seqs) total += logitsAll ? q->prompt.size() : 1;
+            s.logitsHost.resize(total * s.vocab);
+            float *out = s.logitsHost.data();
+            for (auto *q : seqs) {
+                const int S = (int)q->prompt.size();
+                CK(xfthip_model_seq_prefill(s.model, q->row, q->prompt.data(), S, logitsAll ? nullptr : out, nullptr));
+                if (logitsAll) CK(xfthip_model_prompt_logits(s.model, 0, S, out, nullptr));
+                out += (size_t)(logitsAll ? S : 1) * s.vocab;
+            }
+            return std::make_tuple(s.logitsHost.data(), (int)total, s.vocab);
+        }
+        std::vector<int> rows(n);
+        for (int i = 0; i < n; ++i) rows[i] = seqs[i]->row;
+        CK(xfthip_model_seq_decode(s.model, rows.data(), n, nullptr, nullptr));
+        s.logitsHost.resize((size_t)n * s.vocab);
+        for (int i = 0; i < n; ++i) CK(xfthip_model_seq_logits(s.model, rows[i], s.logitsHost.data() + (size_t)i * s.vocab));
+        return std::make_tuple(s.logitsHost.data(), n, s.vocab);
+    }
     if (inputIds.empty() || !isNewInput) unsupported("Model::forward without a new input");
     s.batch = batchSize;
     s.fit(batchSize, seqLen, std::max(seqLen + 1, s.maxLen));
-    s.logitsHost.resize((size_t)batchSize * s.vocab);
-    CK(xfthip_model_prefill(s.model, inputIds.data(), batchSize, seqLen, s.logitsHost.data(), nullptr));
+    const size_t rows = logitsAll ? (size_t)batchSize * seqLen : (size_t)batchSize;
+    s.logitsHost.resize(rows * s.vocab);
+    CK(xfthip_model_prefill(s.model, inputIds.data(), batchSize, seqLen, logitsAll ? nullptr : s.logitsHost.data(), nullptr));
+    if (logitsAll) CK(xfthip_model_prompt_logits(s.model, 0, (int)rows, s.logitsHost.data(), nullptr));
     return std::make_tuple(s.logitsHost.data(), 0, s.vocab);
 }
 
@@ -1221,6 +1261,186 @@ std::vector<int> Model::set_input(std::vector<std::vector<int32_t>> &inputIds_, 
         }
     }
     return seqIDs;
+}
+
+static SearcherConfig flat_config(int maxLen_, int numBeams_, int numBeamHypsToKeep_, float lenPenalty_, bool doEarlyStopping_,
+        int eosTokenId_, int padTokenId_, bool doSample_, float temperature_, int topK_, float topP_, float repetitionPenalty_) {
+    SearcherConfig c;
+    c.maxLen = maxLen_;
+    c.numBeams = numBeams_;
+    c.numBeamHypsToKeep = numBeamHypsToKeep_;
+    c.lenPenalty = lenPenalty_;
+    c.doEarlyStopping = doEarlyStopping_;
+    c.eosTokenId = eosTokenId_;
+    c.padTokenId = padTokenId_;
+    c.doSample = doSample_;
+    c.temperature = temperature_;
+    c.topK = topK_;
+    c.topP = topP_;
+    c.repetitionPenalty = repetitionPenalty_;
+    return c;
+}
+
+// models.cpp:238-273: the flat-argument forms fill a SearcherConfig and forward
+std::vector<int> Model::set_input(std::vector<int32_t> &inputIds_, int batchSize_, int maxLen_, int numBeams_, int numBeamHypsToKeep_,
+        float lenPenalty_, bool doEarlyStopping_, int eosTokenId_, int padTokenId_, bool doSample_, float temperature_, int topK_,
+        float topP_, float repetitionPenalty_, const std::vector<std::vector<int>> &stopWordsList_) {
+    configuration = flat_config(maxLen_, numBeams_, numBeamHypsToKeep_, lenPenalty_, doEarlyStopping_, eosTokenId_, padTokenId_, doSample_,
+            temperature_, topK_, topP_, repetitionPenalty_);
+    return set_input(inputIds_, batchSize_, configuration, stopWordsList_);
+}
+
+std::vector<int> Model::set_input(std::vector<std::vector<int32_t>> &inputIds_, int maxLen_, int numBeams_, int numBeamHypsToKeep_,
+        float lenPenalty_, bool doEarlyStopping_, int eosTokenId_, int padTokenId_, bool doSample_, float temperature_, int topK_,
+        float topP_, float repetitionPenalty_, const std::vector<std::vector<int>> &stopWordsList_) {
+    configuration = flat_config(maxLen_, numBeams_, numBeamHypsToKeep_, lenPenalty_, doEarlyStopping_, eosTokenId_, padTokenId_, doSample_,
+            temperature_, topK_, topP_, repetitionPenalty_);
+    return set_input(inputIds_, configuration, stopWordsList_);
+}
+
+// ---- the forms "only used for model.forward()" (models.cpp:412-683): sequences without a searcher.  With no
+// ids the prompts become new sequences, each with room for its own maximum length; with ids, every listed
+// sequence steps forward with the token the caller chose for it (SequenceMeta::stepForward,
+// src/common/sequence.h:104-113) and forms the batch of the next forward() call.
+static std::vector<int> forward_input(ModelImpl &s, int modelMaxLen, const std::vector<std::vector<int32_t>> &prompts,
+        const std::vector<int32_t> &tokens, std::vector<int> seqIDs, const std::vector<int> &maxLens) {
+    s.cbMode = true;
+    s.working.clear();
+    if (seqIDs.empty()) {
+        const int n = (int)prompts.size();
+        int needLen = 0, longest = 0;
+        std::vector<int> lens(n);
+        for (int i = 0; i < n; ++i) {
+            if (prompts[i].empty()) {
+                printf("[ERROR] Empty prompt.\n");
+                exit(-1);
+            }
+            const int want = maxLens.empty() ? -1 : maxLens[maxLens.size() == 1 ? 0 : i];
+            lens[i] = want < 0 ? modelMaxLen : std::min(want, modelMaxLen);
+            lens[i] = std::max(lens[i], (int)prompts[i].size());
+            needLen = std::max(needLen, lens[i]);
+            longest = std::max(longest, (int)prompts[i].size());
+        }
+        s.fit_rows(n, needLen, longest);
+        for (int i = 0; i < n; ++i) {
+            ModelImpl::Seq q;
+            q.id = s.nextSeqId++;
+            q.prompt = prompts[i];
+            q.forwardOnly = true;
+            q.cfg.maxLen = lens[i];
+            q.row = s.free_row();
+            if (q.row < 0) {
+                printf("[ERROR] No free KV cache row.\n");
+                exit(-1);
+            }
+            s.pool[q.id] = q;
+            s.working.push_back(q.id);
+            seqIDs.push_back(q.id);
+        }
+        return seqIDs;
+    }
+    if (tokens.size() != seqIDs.size()) {
+        printf("[ERROR] Input size and seqIDs size mismatch.\n");
+        exit(-1);
+    }
+    for (size_t i = 0; i < seqIDs.size(); ++i) {
+        auto it = s.pool.find(seqIDs[i]);
+        if (it == s.pool.end()) {
+            printf("[ERROR] Sequence ID %d not found.\n", seqIDs[i]);
+            exit(-1);
+        }
+        ModelImpl::Seq &q = it->second;
+        if (tokens[i] < 0 || tokens[i] >= s.vocab) {
+            printf("[ERROR] Token %d of sequence %d is outside the vocabulary.\n", tokens[i], seqIDs[i]);
+            exit(-1);
+        }
+        if ((int)(q.prompt.size() + q.generated.size()) + 1 > s.cfg.max_seq) {
+            printf("[ERROR] Sequence ID %d is at the end of its KV cache (%d positions).\n", seqIDs[i], s.cfg.max_seq);
+            exit(-1);
+        }
+        q.generated.push_back(tokens[i]);
+        q.step++;
+        CK(xfthip_model_seq_set_next_id(s.model, q.row, tokens[i]));
+        s.working.push_back(q.id);
+    }
+    return seqIDs;
+}
+
+std::vector<int> Model::set_input(std::vector<std::vector<int32_t>> &inputIds_, std::vector<int> seqIDs, int maxLen) {
+    batchSize = (int)inputIds_.size();
+    std::vector<int32_t> tokens;
+    if (!seqIDs.empty()) {
+        if (inputIds_.size() != seqIDs.size()) {
+            printf("[ERROR] Input size and seqIDs size mismatch.\n");
+            exit(-1);
+        }
+        for (auto &ids : inputIds_) {
+            if (ids.empty()) {
+                printf("[ERROR] Empty input for a sequence.\n");
+                exit(-1);
+            }
+            tokens.push_back(ids[0]);
+        }
+    }
+    return forward_input(*impl, maxSeqLen, inputIds_, tokens, seqIDs, {maxLen});
+}
+
+std::vector<int> Model::set_input(std::vector<int32_t> &inputIds_, int batchSize_, std::vector<int> seqIDs, int maxLen) {
+    return set_input(inputIds_, batchSize_, seqIDs, std::vector<int> {maxLen});
+}
+
+std::vector<int> Model::set_input(std::vector<int32_t> &inputIds_, int batchSize_, std::vector<int> seqIDs, const std::vector<int> &maxLen) {
+    if (batchSize_ <= 0 || inputIds_.size() % (size_t)batchSize_ != 0) {
+        printf("Model::set_input: %zu ids do not form %d sequences of equal length.\n", inputIds_.size(), batchSize_);
+        exit(-1);
+    }
+    batchSize = batchSize_;
+    seqLen = (int)(inputIds_.size() / (size_t)batchSize_);
+    if (!(maxLen.size() == (size_t)batchSize || maxLen.size() == 1 || maxLen.empty())) {
+        printf("[ERROR] maxLen size and batch size mismatch.\n");
+        exit(-1);
+    }
+    std::vector<std::vector<int32_t>> prompts;
+    if (seqIDs.empty()) {
+        for (int b = 0; b < batchSize_; ++b) prompts.emplace_back(inputIds_.begin() + (size_t)b * seqLen, inputIds_.begin() + (size_t)(b + 1) * seqLen);
+    } else if (inputIds_.size() != (size_t)batchSize_) {
+        printf("[ERROR] Input size and batch size mismatch.\n");
+        exit(-1);
+    }
+    return forward_input(*impl, maxSeqLen, prompts, inputIds_, seqIDs, maxLen);
+}
+
+std::vector<int> Model::set_input(std::vector<int32_t> &inputIds_, std::vector<int32_t> &seqLens_, std::vector<int> seqIDs,
+        std::vector<int> &maxLen) {
+    std::vector<std::vector<int32_t>> prompts;
+    if (seqIDs.empty()) {
+        batchSize = (int)seqLens_.size();
+        if (!(maxLen.size() == (size_t)batchSize || maxLen.size() == 1 || maxLen.empty())) {
+            printf("[ERROR] maxLen size and batch size mismatch.\n");
+            exit(-1);
+        }
+        size_t at = 0;
+        for (int len : seqLens_) {
+            if (len < 0 || at + (size_t)len > inputIds_.size()) {
+                printf("[ERROR] seqLens do not fit the %zu input ids.\n", inputIds_.size());
+                exit(-1);
+            }
+            prompts.emplace_back(inputIds_.begin() + at, inputIds_.begin() + at + len);
+            at += (size_t)len;
+        }
+    } else {
+        batchSize = (int)seqIDs.size();
+    }
+    return forward_input(*impl, maxSeqLen, prompts, inputIds_, seqIDs, maxLen);
+}
+
+// models.cpp:905-935: the searcher half of config(), without the stop words
+void Model::createSearcher(SearcherConfig &config_) {
+    this->config(config_, {});
+}
+
+void Model::initMaxSeqLen() {
+    maxSeqLen = impl->maxSeqLength > 0 ? impl->maxSeqLength : impl->maxPositions;
 }
 
 AutoModel::AutoModel(std::string modelPath, xft::DataType dataType, xft::DataType KVCacheDataType) : Model() {

@@ -31,6 +31,8 @@ struct LayerW {
     // first token, another for the following ones, src/models/hybrid_model.h:25-84)
     xfthip_weight_t first_qkv = nullptr, first_o = nullptr, first_gateup = nullptr, first_down = nullptr;
     float *ln1 = nullptr, *ln2 = nullptr, *qkv_bias = nullptr, *o_bias = nullptr;
+    // set: the layer's two norms are LayerNorms with these shifts (NormType::LN of the layer API) instead of RMSNorms
+    float *ln1_beta = nullptr, *ln2_beta = nullptr;
 };
 
 __global__ void embed_kernel(const uint16_t *__restrict__ table, const int *__restrict__ ids, float *__restrict__ x,
@@ -183,6 +185,7 @@ struct xfthip_model {
     xfthip_weight_t lm_head = nullptr;
     // decode state
     int cur_B = 0, cur_pos = 0;
+    int prompt_rows = 0; // rows of `x` that hold the last layer's output of the most recent prompt pass (0 after a decode step)
     // continuous batching: sequences live in cache rows of their own, each at its own position
     int row0 = 0; // cache row of the first sequence of the forward call in flight
     bool ragged = false; // rows may differ in position or sit out a step (set by the xfthip_model_seq_* calls)
@@ -243,7 +246,7 @@ static int mega_prepare(xfthip_model *m) {
     std::vector<MegaLayer> tab(c.layers);
     for (int l = 0; l < c.layers; ++l) {
         const LayerW &L = m->layers[l];
-        if (!L.qkv || !L.o || !L.gateup || !L.down || !L.ln1 || !L.ln2 || L.qkv_bias || L.o_bias) return 0;
+        if (!L.qkv || !L.o || !L.gateup || !L.down || !L.ln1 || !L.ln2 || L.qkv_bias || L.o_bias || L.ln1_beta || L.ln2_beta) return 0;
         const PackedWeight *w[4] = {&L.qkv->pw, &L.o->pw, &L.gateup->pw, &L.down->pw};
         for (const PackedWeight *pw : w)
             if (pw->kind != XFTHIP_W_INT8 || pw->zero != nullptr || pw->KT % 4 != 0) return 0;
@@ -403,11 +406,14 @@ static int attention_block(xfthip_model *m, int idx, const float *x_in, int in_s
     // (and their gaps) out of every layer.
     const PackedWeight &wq = L.qkv->pw;
     const bool small = m->fuse_decode && wq.kind != XFTHIP_W_W8A8;
-    const bool fuse_norm = small && do_norm && skinny_can_fuse_norm(wq, T);
+    const bool fuse_norm = small && do_norm && !L.ln1_beta && skinny_can_fuse_norm(wq, T);
     const bool fuse_rope = small && S == 1 && T <= 32 && c.kv_dtype == XFTHIP_FP16 && !L.qkv_bias && c.head_size == 128
             && wq.KT * ktile_of(wq.kind) == wq.K;
     if (!fuse_norm) {
-        if (do_norm) {
+        if (do_norm && L.ln1_beta) {
+            if ((rc = xfthip_layernorm(m->xn, XFTHIP_BF16, x_in, XFTHIP_F32, L.ln1, L.ln1_beta, T, c.hidden, in_stride, c.hidden, c.rms_eps, st)))
+                return rc;
+        } else if (do_norm) {
             if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, x_in, XFTHIP_F32, L.ln1, T, c.hidden, in_stride, c.hidden, c.rms_eps, st))) return rc;
         } else {
             hipLaunchKernelGGL(narrow_rows_kernel, dim3(T), dim3(256), 0, st, x_in, in_stride, m->xn, c.hidden);
@@ -466,7 +472,7 @@ static int mlp_block(xfthip_model *m, int idx, const float *x_in, int in_stride,
     int rc;
     const PackedWeight &wg = L.gateup->pw;
     // epsilon 1e-6 is hard-coded on the MLP side of the reference (src/layers/mlp_llama.h:212)
-    if (m->fuse_decode && do_norm && wg.kind != XFTHIP_W_W8A8 && skinny_can_fuse_norm(wg, T)) {
+    if (m->fuse_decode && do_norm && !L.ln2_beta && wg.kind != XFTHIP_W_W8A8 && skinny_can_fuse_norm(wg, T)) {
         SkinnyParams sp = {};
         sp.M = T;
         sp.A = m->xn;
@@ -478,7 +484,10 @@ static int mlp_block(xfthip_model *m, int idx, const float *x_in, int in_stride,
         sp.norm_x = x_in, sp.ldx = in_stride, sp.norm_w = L.ln2, sp.norm_eps = 1e-6f;
         if ((rc = qgemm_skinny(wg, sp, st))) return rc;
     } else {
-        if (do_norm) {
+        if (do_norm && L.ln2_beta) {
+            if ((rc = xfthip_layernorm(m->xn, XFTHIP_BF16, x_in, XFTHIP_F32, L.ln2, L.ln2_beta, T, c.hidden, in_stride, c.hidden, 1e-6f, st)))
+                return rc;
+        } else if (do_norm) {
             if ((rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, x_in, XFTHIP_F32, L.ln2, T, c.hidden, in_stride, c.hidden, 1e-6f, st))) return rc;
         } else {
             hipLaunchKernelGGL(narrow_rows_kernel, dim3(T), dim3(256), 0, st, x_in, in_stride, m->xn, c.hidden);
@@ -607,6 +616,8 @@ int xfthip_model_destroy(xfthip_model_t m) {
     for (auto &L : m->layers) {
         if (L.ln1) (void)hipFree(L.ln1);
         if (L.ln2) (void)hipFree(L.ln2);
+        if (L.ln1_beta) (void)hipFree(L.ln1_beta);
+        if (L.ln2_beta) (void)hipFree(L.ln2_beta);
         if (L.qkv_bias) (void)hipFree(L.qkv_bias);
         if (L.o_bias) (void)hipFree(L.o_bias);
     }
@@ -677,6 +688,21 @@ int xfthip_model_set_layer(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthi
     XFT_REQUIRE(ln1_host && ln2_host, "xfthip_model_set_layer: norm weights are required");
     if (int rc = xfthip_model_set_attention(m, idx, qkv, o, ln1_host, qkv_bias_host, o_bias_host)) return rc;
     return xfthip_model_set_mlp(m, idx, gateup, down, ln2_host);
+}
+
+int xfthip_model_set_layer_norm_shifts(xfthip_model_t m, int idx, const float *ln1_beta_host, const float *ln2_beta_host) {
+    XFT_REQUIRE(m && idx >= 0 && idx < m->cfg.layers, "xfthip_model_set_layer_norm_shifts: bad model or layer");
+    LayerW &L = m->layers[idx];
+    // a captured decode step holds the kernels of the other norm
+    if (m->graph) {
+        XFT_CHECK_HIP(hipDeviceSynchronize());
+        (void)hipGraphExecDestroy(m->graph);
+        m->graph = nullptr;
+    }
+    mega_invalidate(m);
+    XFT_CHECK_HIP(hipDeviceSynchronize());
+    if (int rc = upload_f32(&L.ln1_beta, ln1_beta_host, m->cfg.hidden)) return rc; // (a null pointer drops the shift)
+    return upload_f32(&L.ln2_beta, ln2_beta_host, m->cfg.hidden);
 }
 
 int xfthip_model_set_first_token_weights(xfthip_model_t m, int idx, xfthip_weight_t qkv, xfthip_weight_t o, xfthip_weight_t gateup,
@@ -784,6 +810,7 @@ int xfthip_model_prefill(xfthip_model_t m, const int *ids_host, int B, int S, fl
     if (logits_host) XFT_CHECK_HIP(hipMemcpy(logits_host, m->logits, (size_t)B * c.vocab * 4, hipMemcpyDeviceToHost));
     m->cur_B = B;
     m->cur_pos = S;
+    m->prompt_rows = B * S;
     return 0;
 }
 
@@ -796,6 +823,7 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
     XFT_REQUIRE(steps <= m->idlog_cap, "xfthip_model_decode: too many steps for the id log");
     hipStream_t st = (hipStream_t)stream;
     const int B = m->cur_B;
+    m->prompt_rows = 0; // the step overwrites the residual rows of the prompt pass
     hipLaunchKernelGGL(fill_int_kernel, dim3(1), dim3(64), 0, st, m->step, 1, 0);
     // the positions are read from device memory, but the attention split count is fixed at launch
     // (capture) time: it follows an upper bound of the length, rounded up so that the graph is
@@ -918,6 +946,7 @@ int xfthip_model_seq_prefill(xfthip_model_t m, int row, const int *ids_host, int
     if (logits_host) XFT_CHECK_HIP(hipMemcpy(logits_host, m->logits + (size_t)row * c.vocab, (size_t)c.vocab * 4, hipMemcpyDeviceToHost));
     m->row_pos[row] = S;
     if (row + 1 > m->cur_B) m->cur_B = row + 1;
+    m->prompt_rows = S;
     return 0;
 }
 
@@ -1154,6 +1183,38 @@ int xfthip_model_set_next_ids(xfthip_model_t m, const int *ids_host, xfthip_stre
     XFT_CHECK_HIP(hipMemcpyAsync(m->ids, ids_host, (size_t)m->cur_B * 4, hipMemcpyHostToDevice, (hipStream_t)stream));
     XFT_CHECK_HIP(hipStreamSynchronize((hipStream_t)stream));
     return 0;
+}
+
+int xfthip_model_prompt_logits(xfthip_model_t m, int first_row, int rows, float *logits_host, xfthip_stream_t stream) {
+    XFT_REQUIRE(m && logits_host && m->lm_head && m->final_norm, "xfthip_model_prompt_logits: bad argument or no head");
+    XFT_REQUIRE(first_row >= 0 && rows > 0 && first_row + rows <= m->prompt_rows,
+            "xfthip_model_prompt_logits: rows [%d, %d) outside the %d rows of the last prompt pass (a decode step discards them)", first_row,
+            first_row + rows, m->prompt_rows);
+    const xfthip_model_config &c = m->cfg;
+    hipStream_t st = (hipStream_t)stream;
+    // final norm + lm_head over the prompt's residual rows, a chunk at a time through a buffer that lives for the
+    // call (not a hot path: the reference's logitsAll = true serves scoring, not generation)
+    const int chunk = rows < 256 ? rows : 256;
+    float *tmp = nullptr;
+    XFT_CHECK_HIP(hipMalloc((void **)&tmp, (size_t)chunk * c.vocab * 4));
+    int rc = 0;
+    for (int r = 0; r < rows && rc == 0; r += chunk) {
+        const int n = rows - r < chunk ? rows - r : chunk;
+        const float *x = m->x + (size_t)(first_row + r) * c.hidden;
+        rc = xfthip_rmsnorm(m->xn, XFTHIP_BF16, x, XFTHIP_F32, m->final_norm, n, c.hidden, c.hidden, c.hidden, c.rms_eps, st);
+        if (rc == 0)
+            rc = xfthip_gemm(m->lm_head, n, m->xn, c.hidden, tmp, c.vocab, XFTHIP_F32, XFTHIP_EPI_NONE, nullptr, nullptr, 0, XFTHIP_F32, 1.0f, st);
+        if (rc == 0 && hipMemcpyAsync(logits_host + (size_t)r * c.vocab, tmp, (size_t)n * c.vocab * 4, hipMemcpyDeviceToHost, st) != hipSuccess) {
+            set_error("xfthip_model_prompt_logits: copy to the host failed");
+            rc = 1;
+        }
+        if (rc == 0 && hipStreamSynchronize(st) != hipSuccess) {
+            set_error("xfthip_model_prompt_logits: the stream failed");
+            rc = 1;
+        }
+    }
+    (void)hipFree(tmp);
+    return rc;
 }
 
 int xfthip_model_logits(xfthip_model_t m, const float **logits_dev) {

@@ -118,6 +118,33 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(void *__restrict__ out, in
     }
 }
 
+// ---- LayerNorm: one 256-thread block per row -----------------------------------------------
+// y = (x - mean) * gamma * (1 / sqrt(E[x^2] - mean^2 + eps)) + beta with the sum and the sum of squares taken in
+// one pass and fp32 arithmetic in the reference's order (src/kernels/layernorm_kernels.cpp:27-81).  Not on the
+// Llama path's hot loop (its layers use RMSNorm): the generic form only.
+__global__ __launch_bounds__(256) void layernorm_kernel(void *__restrict__ out, int out_dtype, const void *__restrict__ in, int in_dtype,
+        const float *__restrict__ gamma, const float *__restrict__ beta, int cols, int iStride, int oStride, float eps) {
+    __shared__ float part[8];
+    const int row = blockIdx.x;
+    const size_t ibase = (size_t)row * iStride, obase = (size_t)row * oStride;
+    float sum = 0.0f, sq = 0.0f;
+    for (int c = threadIdx.x; c < cols; c += 256) {
+        const float x = load_as_f32(in, in_dtype, ibase + c);
+        sum += x;
+        sq = fmaf(x, x, sq);
+    }
+    sum = wave_sum(sum);
+    sq = wave_sum(sq);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = sum, part[4 + (threadIdx.x >> 6)] = sq;
+    __syncthreads();
+    const float mean = ((part[0] + part[1]) + (part[2] + part[3])) / (float)cols;
+    const float var = 1.0f / sqrtf(((part[4] + part[5]) + (part[6] + part[7])) / (float)cols - mean * mean + eps);
+    for (int c = threadIdx.x; c < cols; c += 256) {
+        const float x = load_as_f32(in, in_dtype, ibase + c);
+        store_from_f32(out, out_dtype, obase + c, (x - mean) * gamma[c] * var + beta[c]);
+    }
+}
+
 // ---- RoPE + KV append ---------------------------------------------------------------------
 // One wavefront per (token, head); lane l owns elements l, l+64, ... of the two halves.
 // D <= 256, D % 2 == 0.  heads [0, qHeads) are query heads (rotated in place), heads
@@ -347,6 +374,21 @@ int xfthip_rmsnorm(void *out, int out_dtype, const void *in, int in_dtype, const
         hipLaunchKernelGGL(rmsnorm_kernel, dim3(rows), dim3(256), 0, st, out, out_dtype, in, in_dtype, weight, cols, iStride,
                 oStride, eps);
     }
+    XFT_CHECK_HIP(hipGetLastError());
+    return 0;
+}
+
+int xfthip_layernorm(void *out, int out_dtype, const void *in, int in_dtype, const float *gamma, const float *beta, int rows, int cols,
+        int iStride, int oStride, float eps, xfthip_stream_t stream) {
+    XFT_REQUIRE(out && in && gamma && beta, "xfthip_layernorm: null argument");
+    XFT_REQUIRE(rows > 0 && cols > 0, "xfthip_layernorm: bad shape %d x %d", rows, cols);
+    XFT_REQUIRE((out_dtype == XFTHIP_F32 || out_dtype == XFTHIP_BF16) && (in_dtype == XFTHIP_F32 || in_dtype == XFTHIP_BF16),
+            "xfthip_layernorm: dtypes must be f32 or bf16");
+    if (iStride == -1) iStride = cols;
+    if (oStride == -1) oStride = cols;
+    XFT_REQUIRE(iStride >= cols && oStride >= cols, "xfthip_layernorm: stride smaller than cols");
+    hipLaunchKernelGGL(layernorm_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, out, out_dtype, in, in_dtype, gamma, beta, cols,
+            iStride, oStride, eps);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }

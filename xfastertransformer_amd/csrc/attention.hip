@@ -22,6 +22,7 @@
 
 
 #include "attention_dev.h"
+#include "attention_prefill.h"
 
 namespace xfthip {
 
@@ -47,10 +48,29 @@ __global__ __launch_bounds__(256, (CT == 1 ? 3 : 2)) void attn_prefill_lds_kerne
     attn_prefill_lds_unit<CT, INT8>(p, blockIdx.y, gridDim.x - 1 - blockIdx.x, blockIdx.z, lds); // longest history first
 }
 
+// 32 x 32 MFMA tiles, 32 columns a wave, K / V blocks shared through LDS (attention_prefill.h); two workgroups a CU
+// Workgroups are handed to the 8 XCDs in turn by their linear index, and each XCD has an L2 of its own: the
+// (sequence, KV head) pairs are dealt to the XCDs (pair = 8 k + XCD), and an XCD walks the column groups of one
+// pair, longest history first, before it starts the next, so that the workgroups resident on an XCD share one or
+// two pairs' keys and values in its L2 instead of all of them.
+template <bool INT8>
+__global__ __launch_bounds__(256, 2) void attn_prefill32_kernel(AttnParams p, int ncg, int npairs) {
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kP32BufBytes];
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int pair = (slot / ncg) * 8 + xcd;
+    if (pair >= npairs) return;
+    attn_prefill32_unit<4, INT8>(p, pair % p.kv.H, ncg - 1 - slot % ncg, pair / p.kv.H, lds);
+}
+
 // Split-KV merge workspace: `slots` partial-result slots of kSlotFloats floats and one ticket per
 // column group.  The library keeps one for plain xfthip_attention calls (allocated on first use);
 // a model owns its own, so that two models on two streams never share partials or tickets.
 static AttnWorkspace g_shared_ws;
+// 0: the 32-column form above; 1: the 16-column form it replaced (XFT_PREFILL_FORM=16, kept for comparison runs)
+static const int g_prefill_form = [] {
+    const char *e = getenv("XFT_PREFILL_FORM");
+    return (e && atoi(e) == 16) ? 1 : 0;
+}();
 
 int attention_workspace_create(AttnWorkspace *w, int slots) {
     w->ws = nullptr, w->tickets = nullptr, w->slots = 0;
@@ -148,6 +168,14 @@ int xfthip::attention_launch(xfthip_kvcache_t c, const void *q, int qStride, voi
         const long waves1 = (long)B * c->kv.H * p.CG; // waves with one column tile each
         if (S > 1 && waves1 >= 4L * device_cu_count()) {
             p.nsplit = 1;
+            if (g_prefill_form == 0) {
+                const int ncg = (S * p.G + 127) / 128, npairs = B * c->kv.H;
+                dim3 grid(8 * ((npairs + 7) / 8) * ncg);
+                if (c->kv.int8) hipLaunchKernelGGL(attn_prefill32_kernel<true>, grid, dim3(256), 0, stream, p, ncg, npairs);
+                else hipLaunchKernelGGL(attn_prefill32_kernel<false>, grid, dim3(256), 0, stream, p, ncg, npairs);
+                XFT_CHECK_HIP(hipGetLastError());
+                return 0;
+            }
             if (!c->kv.int8) {
                 const int ctl = (p.G == 1 && waves1 >= 16L * device_cu_count()) ? 2 : 1;
                 dim3 grid((p.CG + 4 * ctl - 1) / (4 * ctl), c->kv.H, B);

@@ -1,0 +1,289 @@
+// Prefill attention on 32 x 32 MFMA tiles: many (query token, query head) columns per (sequence, KV head).
+//
+// Replaces the reference's flash-style prefill (xft::selfScaledDpAttention, src/kernels/attention_kernels.h:1283-1408;
+// DecoderUtil::incrementalTileAttention / softmaxTile / updateOutTile, src/utils/decoder_util.h:606-889) and its
+// chunked prefill over a cache (xft::crossAttnByHead, attention_kernels.h:988-1123) when a launch has enough
+// columns to fill the device.
+//
+// Why this shape.  A workgroup shares each 32-token block of keys and values through LDS, and every MFMA of a wave
+// takes one operand from there.  The LDS port delivers 128 bytes a clock to the whole CU; a 16 x 16 x 32 MFMA
+// (16 cycles) needs a 1 KiB operand, four SIMDs issuing them back to back would need 256 bytes a clock - the
+// 16-column form is bound by the LDS port at half the MFMA rate before any softmax arithmetic.  A
+// 32 x 32 x 16 MFMA (32 cycles) does twice the work on the same 1 KiB operand: the port and the MFMA pipes are
+// in balance, and a wave owns 32 columns instead of 16, so a K / V byte is read from LDS half as often per flop.
+//
+//   S^T = K . Q^T   tile: 32 tokens (rows) x 32 columns; A = keys from LDS, B = the wave's queries, held in
+//                   registers for the whole walk (8 k-steps of 16 dims)
+//   O^T += V^T . P^T  4 tiles of 32 dims x 32 columns; A = values from LDS (token index innermost, as the cache
+//                   stores them), B = probabilities straight from the score registers
+// In the 32 x 32 accumulator a lane owns one column and 16 of the 32 rows (rows 8 q + 4 h + s; h = lane / 32,
+// q = 0..3, s = 0..3), the other 16 sit in the lane 32 away.  The cache stores a value block with its tokens
+// permuted (kvcache.h: 16-byte chunk c of a dim row = tokens 4 c .. 4 c + 3 and 16 + 4 c .. 16 + 4 c + 3); with the
+// score rows in natural token order, chunk c = 2 t + h is exactly what lane half h holds in registers q = t and
+// q = t + 2, so the probabilities of k-step t need no exchange between lanes.
+//
+// Online softmax per column in the log2 domain, fp32; the reference point moves only when a block's maximum
+// exceeds it by more than 2^8 (probabilities up to 256 are exact enough in fp16 and in the fp32 sums), so the
+// 64 accumulator registers of a lane are rescaled in few blocks only.  INT8 cache: codes are widened to fp16
+// (exact) on their way into LDS, the key scale multiplies the score row, the value scale the probability; the
+// value scales are taken relative to a running reference that is part of the same lazy rescaling (it moves when
+// a block's largest scale leaves [ref / 1024, 4 ref]), so fp16 probabilities stay in range whatever the scales.
+#pragma once
+#include "attention_dev.h"
+
+namespace xfthip {
+
+constexpr int kP32ScaleBytes = 256; // 32 key scales + 32 value scales of a block (INT8 cache)
+constexpr int kP32BufBytes = kPfBufBytes + kP32ScaleBytes;
+
+union HFrag32 {
+    f16x8 v;
+    uint32_t u[4];
+    u32x4 q;
+};
+
+// NW waves a workgroup, 32 columns a wave
+template <int NW, bool INT8>
+__device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, const int cgroup, const int b, unsigned char *lds) {
+    constexpr int D = 128, NT = NW * 64;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int h = lane >> 5, cl = lane & 31;
+    int past = p.past;
+    if (p.past_dev) {
+        past = p.past_dev[b];
+        past = past < 0 ? 0 : (past > p.kv.S - p.S ? p.kv.S - p.S : past);
+    }
+    const int ncols = p.S * p.G;
+    const int c0 = (cgroup * NW + wave) * 32; // first column of this wave
+    const int c = c0 + cl;
+    const bool cvalid = c < ncols;
+    const int cs = cvalid ? c / p.G : 0, cj = cvalid ? c % p.G : 0;
+    const int limit = cvalid ? past + cs + 1 : 0; // tokens [0, limit) are visible to this column
+    const int lim_min = c0 + 31 < ncols ? past + c0 / p.G + 1 : 0; // every column of the wave sees at least this many
+    int wave_last = c0 + 31;
+    wave_last = wave_last < ncols ? wave_last : ncols - 1;
+    const int wave_nblk = c0 < ncols ? (past + wave_last / p.G + 1 + 31) >> 5 : 0;
+    int wg_last = (cgroup + 1) * NW * 32 - 1;
+    wg_last = wg_last < ncols ? wg_last : ncols - 1;
+    const int nblk = (past + wg_last / p.G + 1 + 31) >> 5;
+
+    const size_t bh = (size_t)b * p.kv.H + kvh;
+    constexpr int ESZ = INT8 ? 1 : 2;
+    const ATTN_GLOBAL char *kbase = (const ATTN_GLOBAL char *)p.kv.k + bh * p.kv.S * D * ESZ;
+    const ATTN_GLOBAL char *vbase = (const ATTN_GLOBAL char *)p.kv.v + bh * p.kv.S * D * ESZ;
+    const ATTN_GLOBAL float *ksc = INT8 ? (const ATTN_GLOBAL float *)p.kv.kscale + bh * p.kv.S : nullptr;
+    const ATTN_GLOBAL float *vsc = INT8 ? (const ATTN_GLOBAL float *)p.kv.vscale + bh * p.kv.S : nullptr;
+
+    // ---- the block copy global -> registers -> LDS: 512 + 512 chunks of 16 bytes (FP16) or 256 + 256 (INT8) ----
+    constexpr int CHUNKS = INT8 ? 256 : 512, PER = (CHUNKS + NT - 1) / NT;
+    u32x4 kstage[PER], vstage[PER];
+    f32x4 sstage; // INT8: threads 0..7 carry 4 key scales each, threads 8..15 4 value scales
+    auto fetch = [&](const int blk) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int ch = threadIdx.x + NT * i;
+            if (CHUNKS % NT == 0 || ch < CHUNKS) {
+                kstage[i] = *(const ATTN_GLOBAL u32x4 *)(kbase + (size_t)blk * (32 * D * ESZ) + (size_t)ch * 16);
+                vstage[i] = *(const ATTN_GLOBAL u32x4 *)(vbase + (size_t)blk * (32 * D * ESZ) + (size_t)ch * 16);
+            }
+        }
+        if constexpr (INT8) {
+            if (threadIdx.x < 16) sstage = *(const ATTN_GLOBAL f32x4 *)((threadIdx.x < 8 ? ksc : vsc) + (blk << 5) + 4 * (threadIdx.x & 7));
+        }
+    };
+    auto widen16 = [&](const u32x4 raw, u32x4 &lo, u32x4 &hi) {
+        HFrag x, y;
+        widen_i8x4(raw[0], x.h[0], x.h[1]);
+        widen_i8x4(raw[1], x.h[2], x.h[3]);
+        widen_i8x4(raw[2], y.h[0], y.h[1]);
+        widen_i8x4(raw[3], y.h[2], y.h[3]);
+        lo = x.q, hi = y.q;
+    };
+    auto stash = [&](const int buf) {
+        unsigned char *kb = lds + buf * kP32BufBytes, *vb = kb + 32 * kPfKPitch;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int ch = threadIdx.x + NT * i;
+            if (CHUNKS % NT == 0 || ch < CHUNKS) {
+                if constexpr (INT8) {
+                    u32x4 lo, hi;
+                    widen16(kstage[i], lo, hi); // token ch / 8, dims 16 (ch % 8) ..
+                    *(u32x4 *)(kb + (ch >> 3) * kPfKPitch + (ch & 7) * 32) = lo;
+                    *(u32x4 *)(kb + (ch >> 3) * kPfKPitch + (ch & 7) * 32 + 16) = hi;
+                    widen16(vstage[i], lo, hi); // dim ch / 2, token slots 16 (ch % 2) ..
+                    *(u32x4 *)(vb + (ch >> 1) * kPfVPitch + (ch & 1) * 32) = lo;
+                    *(u32x4 *)(vb + (ch >> 1) * kPfVPitch + (ch & 1) * 32 + 16) = hi;
+                } else {
+                    *(u32x4 *)(kb + (ch >> 4) * kPfKPitch + (ch & 15) * 16) = kstage[i]; // token ch / 16, dims 8 (ch % 16) ..
+                    *(u32x4 *)(vb + (ch >> 2) * kPfVPitch + (ch & 3) * 16) = vstage[i]; // dim ch / 4, tokens 8 (ch % 4) ..
+                }
+            }
+        }
+        if constexpr (INT8) {
+            if (threadIdx.x < 16) *(f32x4 *)(kb + kPfBufBytes + 16 * threadIdx.x) = sstage;
+        }
+    };
+
+    // ---- this wave's queries: B operand of the score MFMA, k-step s covers dims 16 s + 8 h .. + 8 ----
+    HFrag32 qf[8];
+    {
+        const uint16_t *qrow = p.q + ((size_t)b * p.S + cs) * p.qStride + (size_t)(kvh * p.G + cj) * D;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            uint32_t raw[4] = {0u, 0u, 0u, 0u};
+            if (cvalid) ld_dev16(qrow + 16 * s + 8 * h, raw);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) qf[s].u[i] = pack_f16(u2f(raw[i] << 16), u2f(raw[i] & 0xFFFF0000u));
+        }
+    }
+    float m_run = kNegBig, l_run = 0.0f;
+    float vref = 0.0f; // INT8: the value scales are taken relative to this (0 = not set yet)
+    f32x16 o[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[dt][r] = 0.0f;
+    const float c1 = p.scale * 1.4426950408889634f; // scores live in the log2 domain
+
+    auto compute = [&](const int buf, const int blk) {
+        const int t0 = blk << 5;
+        const unsigned char *kb = lds + buf * kP32BufBytes, *vb = kb + 32 * kPfKPitch;
+        // scores: 8 k-steps on one accumulator; the key operands are read two steps ahead of their use
+        f32x16 sc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[r] = 0.0f;
+        const unsigned char *krow = kb + cl * kPfKPitch + 16 * h;
+        HFrag32 kf[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) kf[s].q = *(const u32x4 *)(krow + 32 * s);
+#pragma unroll
+        for (int s = 0; s < 8; ++s) sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s].v, qf[s].v, sc, 0, 0, 0);
+        // the value operands are read only now: they reuse the key operands' registers and their LDS latency
+        // passes behind the softmax arithmetic
+        __builtin_amdgcn_sched_barrier(0);
+        HFrag32 vf[2][4];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt) vf[t][dt].q = *(const u32x4 *)(vb + (32 * dt + cl) * kPfVPitch + 16 * (2 * t + h));
+        // INT8: scales of this lane's 16 tokens (8 q + 4 h ..)
+        f32x4 ks[4], vs[4];
+        float vmax = 0.0f;
+        if constexpr (INT8) {
+            const float *sl = (const float *)(kb + kPfBufBytes);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                ks[q] = *(const f32x4 *)(sl + 8 * q + 4 * h) * c1; // key scale and softmax scale in one factor
+                vs[q] = *(const f32x4 *)(sl + 32 + 8 * q + 4 * h);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) vmax = fmaxf(vmax, vs[q][r]);
+            }
+            vmax = fmaxf(vmax, swap32(vmax)); // the block's largest value scale, the same in every lane
+        }
+        const bool masked = t0 + 32 > lim_min; // wave-uniform
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[r] *= INT8 ? ks[r >> 2][r & 3] : c1;
+        if (masked) {
+            // only the blocks on the causal diagonal pay for the mask (a real branch)
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sc[r] = (t0 + 8 * (r >> 2) + 4 * h + (r & 3)) < limit ? sc[r] : kNegBig;
+        }
+        float bmax = kNegBig;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) bmax = fmaxf(bmax, sc[r]);
+        bmax = fmaxf(bmax, swap32(bmax));
+        const float m_new = bmax > m_run + 8.0f ? bmax : m_run;
+        float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        m_run = m_new;
+        float pr[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) pr[r] = __builtin_amdgcn_exp2f(sc[r] - m_new);
+        if (masked) {
+            // a masked score is kNegBig: 2^(kNegBig - m) is already 0 unless the column has seen nothing yet
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int r = 0; r < 16; ++r) pr[r] = sc[r] > 0.5f * kNegBig ? pr[r] : 0.0f;
+        }
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) psum += pr[r];
+        l_run = l_run * alpha + psum; // (this lane's 16 rows; the two halves are added at the end)
+        float oscale = alpha; // what the running output is multiplied by before this block is added
+        if constexpr (INT8) {
+            // value scales relative to vref; vref follows the blocks' largest scale lazily, like the maximum
+            float nref = vref;
+            if (vmax > 4.0f * vref || (vmax > 0.0f && vmax * 1024.0f < vref)) nref = vmax; // wave-uniform
+            if (nref != vref) {
+                oscale = vref > 0.0f ? alpha * (vref / nref) : alpha;
+                vref = nref;
+            }
+            const float vinv = vref > 0.0f ? 1.0f / vref : 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) pr[r] *= vs[r >> 2][r & 3] * vinv;
+        }
+        HFrag32 pf[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            pf[t].u[0] = pack_f16(pr[4 * t], pr[4 * t + 1]);
+            pf[t].u[1] = pack_f16(pr[4 * t + 2], pr[4 * t + 3]);
+            pf[t].u[2] = pack_f16(pr[4 * t + 8], pr[4 * t + 9]);
+            pf[t].u[3] = pack_f16(pr[4 * t + 10], pr[4 * t + 11]);
+        }
+        if (__builtin_amdgcn_ballot_w64(oscale != 1.0f) != 0) {
+            // the running output is rescaled only when some column's reference point moved (a real branch)
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o[dt][r] *= oscale;
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[t][dt].v, pf[t].v, o[dt], 0, 0, 0);
+    };
+
+    if (nblk > 0) {
+        fetch(0);
+        stash(0);
+    }
+    __syncthreads();
+    for (int blk = 0; blk < nblk; ++blk) {
+        const bool more = blk + 1 < nblk; // uniform over the workgroup
+        if (more) fetch(blk + 1);
+        if (blk < wave_nblk) compute(blk & 1, blk);
+        if (more) stash((blk + 1) & 1);
+        __syncthreads();
+    }
+
+    float l = l_run;
+    l += swap32(l);
+    if (!cvalid) return;
+    const float vr = INT8 ? vref : 1.0f;
+    const size_t base = ((size_t)b * p.S + cs) * p.oStride + (size_t)(kvh * p.G + cj) * D;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const size_t idx = base + 32 * dt + 8 * q + 4 * h;
+            float v0 = o[dt][4 * q], v1 = o[dt][4 * q + 1], v2 = o[dt][4 * q + 2], v3 = o[dt][4 * q + 3];
+            if constexpr (INT8) v0 *= vr, v1 *= vr, v2 *= vr, v3 *= vr;
+            v0 /= l, v1 /= l, v2 /= l, v3 /= l;
+            if (p.out_dtype == XFTHIP_BF16) {
+                const uint32_t lo = f32_to_bf16_ref(v0) | ((uint32_t)f32_to_bf16_ref(v1) << 16);
+                const uint32_t hi = f32_to_bf16_ref(v2) | ((uint32_t)f32_to_bf16_ref(v3) << 16);
+                uint16_t *dst = (uint16_t *)p.out + idx;
+                if ((((uintptr_t)dst) & 7) == 0) {
+                    *(uint2 *)dst = make_uint2(lo, hi);
+                } else {
+                    dst[0] = (uint16_t)lo, dst[1] = (uint16_t)(lo >> 16), dst[2] = (uint16_t)hi, dst[3] = (uint16_t)(hi >> 16);
+                }
+            } else {
+                float *dst = (float *)p.out + idx;
+                dst[0] = v0, dst[1] = v1, dst[2] = v2, dst[3] = v3;
+            }
+        }
+}
+
+} // namespace xfthip

@@ -46,13 +46,14 @@ union HFrag32 {
 template <int NW, bool INT8>
 __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, const int cgroup, const int b, unsigned char *lds) {
     constexpr int D = 128, NT = NW * 64;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int h = lane >> 5, cl = lane & 31;
     int past = p.past;
     if (p.past_dev) {
         past = p.past_dev[b];
         past = past < 0 ? 0 : (past > p.kv.S - p.S ? p.kv.S - p.S : past);
     }
+    past = __builtin_amdgcn_readfirstlane(past);
     const int ncols = p.S * p.G;
     const int c0 = (cgroup * NW + wave) * 32; // first column of this wave
     const int c = c0 + cl;
@@ -125,6 +126,10 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
     };
 
     // ---- this wave's queries: B operand of the score MFMA, k-step s covers dims 16 s + 8 h .. + 8 ----
+    // FP16 cache: the queries carry the softmax scale and log2 e (rounded to fp16 once: 2^-12 relative, the size of
+    // the rounding of the fp16 probabilities), so that a score leaves the MFMA in the log2 domain.
+    const float c1 = p.scale * 1.4426950408889634f;
+    const float qmul = INT8 ? 1.0f : c1;
     HFrag32 qf[8];
     {
         const uint16_t *qrow = p.q + ((size_t)b * p.S + cs) * p.qStride + (size_t)(kvh * p.G + cj) * D;
@@ -133,29 +138,40 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
             uint32_t raw[4] = {0u, 0u, 0u, 0u};
             if (cvalid) ld_dev16(qrow + 16 * s + 8 * h, raw);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) qf[s].u[i] = pack_f16(u2f(raw[i] << 16), u2f(raw[i] & 0xFFFF0000u));
+            for (int i = 0; i < 4; ++i) qf[s].u[i] = pack_f16(u2f(raw[i] << 16) * qmul, u2f(raw[i] & 0xFFFF0000u) * qmul);
         }
     }
-    float m_run = kNegBig, l_run = 0.0f;
+    float m_run = kNegBig, l_run = 0.0f; // m_run == kNegBig: the column has seen no token yet
     float vref = 0.0f; // INT8: the value scales are taken relative to this (0 = not set yet)
     f32x16 o[4];
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) o[dt][r] = 0.0f;
-    const float c1 = p.scale * 1.4426950408889634f; // scores live in the log2 domain
+    // FP16 cache: the score MFMAs start from -m_run instead of 0, so a score arrives relative to the column's
+    // reference point with no vector instruction spent on it, and the row sums of the probabilities come out of
+    // two more MFMAs against a tile of ones (the matrix pipes have the slack, the vector ALUs do not).
+    f32x16 negm, lacc;
+    HFrag32 ones;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) negm[r] = 0.0f, lacc[r] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ones.u[i] = 0x3C003C00u;
 
     auto compute = [&](const int buf, const int blk) {
         const int t0 = blk << 5;
         const unsigned char *kb = lds + buf * kP32BufBytes, *vb = kb + 32 * kPfKPitch;
-        // scores: 8 k-steps on one accumulator; the key operands are read two steps ahead of their use
-        f32x16 sc;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sc[r] = 0.0f;
         const unsigned char *krow = kb + cl * kPfKPitch + 16 * h;
         HFrag32 kf[8];
 #pragma unroll
         for (int s = 0; s < 8; ++s) kf[s].q = *(const u32x4 *)(krow + 32 * s);
+        f32x16 sc;
+        if constexpr (INT8) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sc[r] = 0.0f;
+        } else {
+            sc = negm;
+        }
 #pragma unroll
         for (int s = 0; s < 8; ++s) sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s].v, qf[s].v, sc, 0, 0, 0);
         // the value operands are read only now: they reuse the key operands' registers and their LDS latency
@@ -166,10 +182,12 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt) vf[t][dt].q = *(const u32x4 *)(vb + (32 * dt + cl) * kPfVPitch + 16 * (2 * t + h));
-        // INT8: scales of this lane's 16 tokens (8 q + 4 h ..)
-        f32x4 ks[4], vs[4];
-        float vmax = 0.0f;
+        const bool masked = t0 + 32 > lim_min; // wave-uniform
+        float pr[16];
         if constexpr (INT8) {
+            // scales of this lane's 16 tokens (8 q + 4 h ..)
+            f32x4 ks[4], vs[4];
+            float vmax = 0.0f;
             const float *sl = (const float *)(kb + kPfBufBytes);
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
@@ -179,38 +197,35 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
                 for (int r = 0; r < 4; ++r) vmax = fmaxf(vmax, vs[q][r]);
             }
             vmax = fmaxf(vmax, swap32(vmax)); // the block's largest value scale, the same in every lane
-        }
-        const bool masked = t0 + 32 > lim_min; // wave-uniform
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sc[r] *= INT8 ? ks[r >> 2][r & 3] : c1;
-        if (masked) {
-            // only the blocks on the causal diagonal pay for the mask (a real branch)
-            asm volatile("" ::: "memory");
+            for (int r = 0; r < 16; ++r) sc[r] *= ks[r >> 2][r & 3];
+            if (masked) {
+                // only the blocks on the causal diagonal pay for the mask (a real branch)
+                asm volatile("" ::: "memory");
 #pragma unroll
-            for (int r = 0; r < 16; ++r) sc[r] = (t0 + 8 * (r >> 2) + 4 * h + (r & 3)) < limit ? sc[r] : kNegBig;
-        }
-        float bmax = kNegBig;
+                for (int r = 0; r < 16; ++r) sc[r] = (t0 + 8 * (r >> 2) + 4 * h + (r & 3)) < limit ? sc[r] : kNegBig;
+            }
+            float bmax = fmaxf(fmaxf(sc[0], sc[1]), sc[2]);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) bmax = fmaxf(bmax, sc[r]);
-        bmax = fmaxf(bmax, swap32(bmax));
-        const float m_new = bmax > m_run + 8.0f ? bmax : m_run;
-        float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        m_run = m_new;
-        float pr[16];
+            for (int r = 3; r < 15; r += 2) bmax = fmaxf(fmaxf(bmax, sc[r]), sc[r + 1]);
+            bmax = fmaxf(bmax, sc[15]);
+            bmax = fmaxf(bmax, swap32(bmax));
+            const float m_new = bmax > m_run + 8.0f ? bmax : m_run;
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            m_run = m_new;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) pr[r] = __builtin_amdgcn_exp2f(sc[r] - m_new);
-        if (masked) {
-            // a masked score is kNegBig: 2^(kNegBig - m) is already 0 unless the column has seen nothing yet
-            asm volatile("" ::: "memory");
+            for (int r = 0; r < 16; ++r) pr[r] = __builtin_amdgcn_exp2f(sc[r] - m_new);
+            if (masked) {
+                // a masked score is kNegBig: 2^(kNegBig - m) is already 0 unless the column has seen nothing yet
+                asm volatile("" ::: "memory");
 #pragma unroll
-            for (int r = 0; r < 16; ++r) pr[r] = sc[r] > 0.5f * kNegBig ? pr[r] : 0.0f;
-        }
-        float psum = 0.0f;
+                for (int r = 0; r < 16; ++r) pr[r] = sc[r] > 0.5f * kNegBig ? pr[r] : 0.0f;
+            }
+            float psum = (pr[0] + pr[1]) + (pr[2] + pr[3]);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) psum += pr[r];
-        l_run = l_run * alpha + psum; // (this lane's 16 rows; the two halves are added at the end)
-        float oscale = alpha; // what the running output is multiplied by before this block is added
-        if constexpr (INT8) {
+            for (int r = 4; r < 16; r += 4) psum += (pr[r] + pr[r + 1]) + (pr[r + 2] + pr[r + 3]);
+            l_run = l_run * alpha + psum; // (this lane's 16 rows; the two halves are added at the end)
+            float oscale = alpha; // what the running output is multiplied by before this block is added
             // value scales relative to vref; vref follows the blocks' largest scale lazily, like the maximum
             float nref = vref;
             if (vmax > 4.0f * vref || (vmax > 0.0f && vmax * 1024.0f < vref)) nref = vmax; // wave-uniform
@@ -221,6 +236,45 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
             const float vinv = vref > 0.0f ? 1.0f / vref : 0.0f;
 #pragma unroll
             for (int r = 0; r < 16; ++r) pr[r] *= vs[r >> 2][r & 3] * vinv;
+            if (__builtin_amdgcn_ballot_w64(oscale != 1.0f) != 0) {
+                // the running output is rescaled only when some column's reference point moved (a real branch)
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) o[dt][r] *= oscale;
+            }
+        } else {
+            if (masked) {
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sc[r] = (t0 + 8 * (r >> 2) + 4 * h + (r & 3)) < limit ? sc[r] : kNegBig;
+            }
+            // sc = log2-domain score minus the column's reference point (0 while the column has seen nothing)
+            float bmax = fmaxf(fmaxf(sc[0], sc[1]), sc[2]);
+#pragma unroll
+            for (int r = 3; r < 15; r += 2) bmax = fmaxf(fmaxf(bmax, sc[r]), sc[r + 1]);
+            bmax = fmaxf(bmax, sc[15]);
+            bmax = fmaxf(bmax, swap32(bmax));
+            // the reference point moves when the block's maximum exceeds it by more than 2^8, and is set by the first
+            // block a column sees anything of
+            const bool first = m_run == kNegBig;
+            const bool move = bmax > 8.0f || (first && bmax > 0.5f * kNegBig);
+            if (__builtin_amdgcn_ballot_w64(move) != 0) {
+                // a real branch: in most blocks no column of the wave moves
+                asm volatile("" ::: "memory");
+                const float delta = move ? bmax : 0.0f;
+                const float alpha = __builtin_amdgcn_exp2f(-delta); // (columns that see their first tokens hold zeros)
+                if (move) m_run = (first ? 0.0f : m_run) + delta;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sc[r] -= delta, negm[r] = move ? -m_run : negm[r], lacc[r] *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) pr[r] = __builtin_amdgcn_exp2f(sc[r]); // (a masked score is kNegBig: 0)
         }
         HFrag32 pf[2];
 #pragma unroll
@@ -230,18 +284,12 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
             pf[t].u[2] = pack_f16(pr[4 * t + 8], pr[4 * t + 9]);
             pf[t].u[3] = pack_f16(pr[4 * t + 10], pr[4 * t + 11]);
         }
-        if (__builtin_amdgcn_ballot_w64(oscale != 1.0f) != 0) {
-            // the running output is rescaled only when some column's reference point moved (a real branch)
-            asm volatile("" ::: "memory");
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) o[dt][r] *= oscale;
-        }
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < 2; ++t) {
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[t][dt].v, pf[t].v, o[dt], 0, 0, 0);
+            if constexpr (!INT8) lacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ones.v, pf[t].v, lacc, 0, 0, 0);
+        }
     };
 
     if (nblk > 0) {
@@ -259,17 +307,16 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
 
     float l = l_run;
     l += swap32(l);
+    if constexpr (!INT8) l = lacc[0]; // every row of the ones tile holds the column's sum over all 32 tokens of every block
     if (!cvalid) return;
-    const float vr = INT8 ? vref : 1.0f;
+    const float inv = (INT8 ? vref : 1.0f) / l;
     const size_t base = ((size_t)b * p.S + cs) * p.oStride + (size_t)(kvh * p.G + cj) * D;
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const size_t idx = base + 32 * dt + 8 * q + 4 * h;
-            float v0 = o[dt][4 * q], v1 = o[dt][4 * q + 1], v2 = o[dt][4 * q + 2], v3 = o[dt][4 * q + 3];
-            if constexpr (INT8) v0 *= vr, v1 *= vr, v2 *= vr, v3 *= vr;
-            v0 /= l, v1 /= l, v2 /= l, v3 /= l;
+            const float v0 = o[dt][4 * q] * inv, v1 = o[dt][4 * q + 1] * inv, v2 = o[dt][4 * q + 2] * inv, v3 = o[dt][4 * q + 3] * inv;
             if (p.out_dtype == XFTHIP_BF16) {
                 const uint32_t lo = f32_to_bf16_ref(v0) | ((uint32_t)f32_to_bf16_ref(v1) << 16);
                 const uint32_t hi = f32_to_bf16_ref(v2) | ((uint32_t)f32_to_bf16_ref(v3) << 16);

@@ -53,13 +53,13 @@ __global__ __launch_bounds__(256, (CT == 1 ? 3 : 2)) void attn_prefill_lds_kerne
 // (sequence, KV head) pairs are dealt to the XCDs (pair = 8 k + XCD), and an XCD walks the column groups of one
 // pair, longest history first, before it starts the next, so that the workgroups resident on an XCD share one or
 // two pairs' keys and values in its L2 instead of all of them.
-template <bool INT8>
-__global__ __launch_bounds__(256, 2) void attn_prefill32_kernel(AttnParams p, int ncg, int npairs) {
+template <bool INT8, int CT>
+__global__ __launch_bounds__(256, (CT == 1 ? 2 : 1)) void attn_prefill32_kernel(AttnParams p, int ncg, int npairs) {
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kP32BufBytes];
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int pair = (slot / ncg) * 8 + xcd;
     if (pair >= npairs) return;
-    attn_prefill32_unit<4, INT8>(p, pair % p.kv.H, ncg - 1 - slot % ncg, pair / p.kv.H, lds);
+    attn_prefill32_unit<4, CT, INT8>(p, pair % p.kv.H, ncg - 1 - slot % ncg, pair / p.kv.H, lds);
 }
 
 // Split-KV merge workspace: `slots` partial-result slots of kSlotFloats floats and one ticket per
@@ -171,8 +171,8 @@ int xfthip::attention_launch(xfthip_kvcache_t c, const void *q, int qStride, voi
             if (g_prefill_form == 0) {
                 const int ncg = (S * p.G + 127) / 128, npairs = B * c->kv.H;
                 dim3 grid(8 * ((npairs + 7) / 8) * ncg);
-                if (c->kv.int8) hipLaunchKernelGGL(attn_prefill32_kernel<true>, grid, dim3(256), 0, stream, p, ncg, npairs);
-                else hipLaunchKernelGGL(attn_prefill32_kernel<false>, grid, dim3(256), 0, stream, p, ncg, npairs);
+                if (c->kv.int8) hipLaunchKernelGGL((attn_prefill32_kernel<true, 1>), grid, dim3(256), 0, stream, p, ncg, npairs);
+                else hipLaunchKernelGGL((attn_prefill32_kernel<false, 1>), grid, dim3(256), 0, stream, p, ncg, npairs);
                 XFT_CHECK_HIP(hipGetLastError());
                 return 0;
             }

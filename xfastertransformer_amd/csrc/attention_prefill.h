@@ -43,9 +43,24 @@ union HFrag32 {
 };
 
 // NW waves a workgroup, 32 columns a wave
-template <int NW, bool INT8>
+// NW waves a workgroup, CT column tiles (32 CT columns) a wave; the library launches CT = 1, two workgroups a CU.
+// Measured in that form (4 x 2048 tokens, 32 query / 8 KV heads, 213 us): the LDS pipe busy 90 % of the time (16
+// operand reads and 4 staging writes a block and wave at about 22 cycles each), matrix pipes 29 %, vector ALUs 29 %;
+// taking the MFMAs out of the kernel left 143 us, the softmax as well 119 us: the operand reads bound it.
+// CT = 2 (every fragment read feeds two MFMAs; a wave then needs the registers of a whole SIMD, one workgroup a CU)
+// halves the LDS bytes per flop but ran 353 us: a single wave a SIMD executes score MFMAs, softmax and value MFMAs
+// strictly one after the other.  A three-stage software pipeline inside the wave (value MFMAs of block k - 1 and
+// score MFMAs of block k + 1 issued between the softmax instructions of block k, the order fixed with scheduling
+// fences) was built for both CT: correct, but 41 (CT = 1) and 182 (CT = 2) registers short, and the spill traffic
+// shares the counter of the block prefetch, so every reload waited for it: 542 and 1560 us.  Requesting blocks two
+// steps ahead, 8-wave workgroups and touching the pair's cache lines on arrival (L2 warm-up) each changed nothing:
+// global latency and barriers are not what the waves wait for.
+template <int NW, int CT, bool INT8>
 __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, const int cgroup, const int b, unsigned char *lds) {
-    constexpr int D = 128, NT = NW * 64;
+    constexpr int D = 128, NT = NW * 64, WC = 32 * CT;
+    // FP16 cache, one tile a wave: reference point and row sums through the MFMAs (below); with two tiles a wave the
+    // 64 registers this takes are not there, and the vector ALUs have the time
+    constexpr bool VIA_MFMA = !INT8 && CT == 1;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int h = lane >> 5, cl = lane & 31;
     int past = p.past;
@@ -55,16 +70,21 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
     }
     past = __builtin_amdgcn_readfirstlane(past);
     const int ncols = p.S * p.G;
-    const int c0 = (cgroup * NW + wave) * 32; // first column of this wave
-    const int c = c0 + cl;
-    const bool cvalid = c < ncols;
-    const int cs = cvalid ? c / p.G : 0, cj = cvalid ? c % p.G : 0;
-    const int limit = cvalid ? past + cs + 1 : 0; // tokens [0, limit) are visible to this column
-    const int lim_min = c0 + 31 < ncols ? past + c0 / p.G + 1 : 0; // every column of the wave sees at least this many
-    int wave_last = c0 + 31;
+    const int c0 = (cgroup * NW + wave) * WC; // first column of this wave
+    bool cvalid[CT];
+    int cs[CT], cj[CT], limit[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const int c = c0 + 32 * ct + cl;
+        cvalid[ct] = c < ncols;
+        cs[ct] = cvalid[ct] ? c / p.G : 0, cj[ct] = cvalid[ct] ? c % p.G : 0;
+        limit[ct] = cvalid[ct] ? past + cs[ct] + 1 : 0; // tokens [0, limit) are visible to this column
+    }
+    const int lim_min = c0 + WC - 1 < ncols ? past + c0 / p.G + 1 : 0; // every column of the wave sees at least this many
+    int wave_last = c0 + WC - 1;
     wave_last = wave_last < ncols ? wave_last : ncols - 1;
     const int wave_nblk = c0 < ncols ? (past + wave_last / p.G + 1 + 31) >> 5 : 0;
-    int wg_last = (cgroup + 1) * NW * 32 - 1;
+    int wg_last = (cgroup + 1) * NW * WC - 1;
     wg_last = wg_last < ncols ? wg_last : ncols - 1;
     const int nblk = (past + wg_last / p.G + 1 + 31) >> 5;
 
@@ -130,31 +150,34 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
     // the rounding of the fp16 probabilities), so that a score leaves the MFMA in the log2 domain.
     const float c1 = p.scale * 1.4426950408889634f;
     const float qmul = INT8 ? 1.0f : c1;
-    HFrag32 qf[8];
-    {
-        const uint16_t *qrow = p.q + ((size_t)b * p.S + cs) * p.qStride + (size_t)(kvh * p.G + cj) * D;
+    HFrag32 qf[CT][8];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const uint16_t *qrow = p.q + ((size_t)b * p.S + cs[ct]) * p.qStride + (size_t)(kvh * p.G + cj[ct]) * D;
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
             uint32_t raw[4] = {0u, 0u, 0u, 0u};
-            if (cvalid) ld_dev16(qrow + 16 * s + 8 * h, raw);
+            if (cvalid[ct]) ld_dev16(qrow + 16 * s + 8 * h, raw);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) qf[s].u[i] = pack_f16(u2f(raw[i] << 16) * qmul, u2f(raw[i] & 0xFFFF0000u) * qmul);
+            for (int i = 0; i < 4; ++i) qf[ct][s].u[i] = pack_f16(u2f(raw[i] << 16) * qmul, u2f(raw[i] & 0xFFFF0000u) * qmul);
         }
     }
-    float m_run = kNegBig, l_run = 0.0f; // m_run == kNegBig: the column has seen no token yet
+    float m_run[CT], l_run[CT]; // m_run == kNegBig: the column has seen no token yet
     float vref = 0.0f; // INT8: the value scales are taken relative to this (0 = not set yet)
-    f32x16 o[4];
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) o[dt][r] = 0.0f;
+    f32x16 o[CT][4];
     // FP16 cache: the score MFMAs start from -m_run instead of 0, so a score arrives relative to the column's
     // reference point with no vector instruction spent on it, and the row sums of the probabilities come out of
     // two more MFMAs against a tile of ones (the matrix pipes have the slack, the vector ALUs do not).
-    f32x16 negm, lacc;
+    f32x16 negm[VIA_MFMA ? CT : 1], lacc[VIA_MFMA ? CT : 1];
     HFrag32 ones;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) negm[r] = 0.0f, lacc[r] = 0.0f;
+    for (int r = 0; r < 16; ++r) negm[0][r] = 0.0f, lacc[0][r] = 0.0f;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        m_run[ct] = kNegBig, l_run[ct] = 0.0f;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) o[ct][dt] = negm[0];
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) ones.u[i] = 0x3C003C00u;
 
@@ -165,15 +188,20 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
         HFrag32 kf[8];
 #pragma unroll
         for (int s = 0; s < 8; ++s) kf[s].q = *(const u32x4 *)(krow + 32 * s);
-        f32x16 sc;
-        if constexpr (INT8) {
+        f32x16 sc[CT];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) sc[r] = 0.0f;
-        } else {
-            sc = negm;
+        for (int ct = 0; ct < CT; ++ct) {
+            if constexpr (!VIA_MFMA) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sc[ct][r] = 0.0f;
+            } else {
+                sc[ct] = negm[ct];
+            }
         }
 #pragma unroll
-        for (int s = 0; s < 8; ++s) sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s].v, qf[s].v, sc, 0, 0, 0);
+        for (int s = 0; s < 8; ++s)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) sc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s].v, qf[ct][s].v, sc[ct], 0, 0, 0);
         // the value operands are read only now: they reuse the key operands' registers and their LDS latency
         // passes behind the softmax arithmetic
         __builtin_amdgcn_sched_barrier(0);
@@ -183,11 +211,10 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt) vf[t][dt].q = *(const u32x4 *)(vb + (32 * dt + cl) * kPfVPitch + 16 * (2 * t + h));
         const bool masked = t0 + 32 > lim_min; // wave-uniform
-        float pr[16];
+        // INT8: scales of this lane's 16 tokens (8 q + 4 h ..)
+        f32x4 ks[4], vs[4];
+        float vmax = 0.0f, vinv = 1.0f, vmove = 1.0f;
         if constexpr (INT8) {
-            // scales of this lane's 16 tokens (8 q + 4 h ..)
-            f32x4 ks[4], vs[4];
-            float vmax = 0.0f;
             const float *sl = (const float *)(kb + kPfBufBytes);
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
@@ -197,98 +224,107 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
                 for (int r = 0; r < 4; ++r) vmax = fmaxf(vmax, vs[q][r]);
             }
             vmax = fmaxf(vmax, swap32(vmax)); // the block's largest value scale, the same in every lane
-#pragma unroll
-            for (int r = 0; r < 16; ++r) sc[r] *= ks[r >> 2][r & 3];
-            if (masked) {
-                // only the blocks on the causal diagonal pay for the mask (a real branch)
-                asm volatile("" ::: "memory");
-#pragma unroll
-                for (int r = 0; r < 16; ++r) sc[r] = (t0 + 8 * (r >> 2) + 4 * h + (r & 3)) < limit ? sc[r] : kNegBig;
-            }
-            float bmax = fmaxf(fmaxf(sc[0], sc[1]), sc[2]);
-#pragma unroll
-            for (int r = 3; r < 15; r += 2) bmax = fmaxf(fmaxf(bmax, sc[r]), sc[r + 1]);
-            bmax = fmaxf(bmax, sc[15]);
-            bmax = fmaxf(bmax, swap32(bmax));
-            const float m_new = bmax > m_run + 8.0f ? bmax : m_run;
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-            m_run = m_new;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) pr[r] = __builtin_amdgcn_exp2f(sc[r] - m_new);
-            if (masked) {
-                // a masked score is kNegBig: 2^(kNegBig - m) is already 0 unless the column has seen nothing yet
-                asm volatile("" ::: "memory");
-#pragma unroll
-                for (int r = 0; r < 16; ++r) pr[r] = sc[r] > 0.5f * kNegBig ? pr[r] : 0.0f;
-            }
-            float psum = (pr[0] + pr[1]) + (pr[2] + pr[3]);
-#pragma unroll
-            for (int r = 4; r < 16; r += 4) psum += (pr[r] + pr[r + 1]) + (pr[r + 2] + pr[r + 3]);
-            l_run = l_run * alpha + psum; // (this lane's 16 rows; the two halves are added at the end)
-            float oscale = alpha; // what the running output is multiplied by before this block is added
             // value scales relative to vref; vref follows the blocks' largest scale lazily, like the maximum
-            float nref = vref;
-            if (vmax > 4.0f * vref || (vmax > 0.0f && vmax * 1024.0f < vref)) nref = vmax; // wave-uniform
-            if (nref != vref) {
-                oscale = vref > 0.0f ? alpha * (vref / nref) : alpha;
-                vref = nref;
+            if (vmax > 4.0f * vref || (vmax > 0.0f && vmax * 1024.0f < vref)) { // wave-uniform
+                vmove = vref > 0.0f ? vref / vmax : 1.0f;
+                vref = vmax;
             }
-            const float vinv = vref > 0.0f ? 1.0f / vref : 0.0f;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) pr[r] *= vs[r >> 2][r & 3] * vinv;
-            if (__builtin_amdgcn_ballot_w64(oscale != 1.0f) != 0) {
-                // the running output is rescaled only when some column's reference point moved (a real branch)
-                asm volatile("" ::: "memory");
-#pragma unroll
-                for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) o[dt][r] *= oscale;
-            }
-        } else {
-            if (masked) {
-                asm volatile("" ::: "memory");
-#pragma unroll
-                for (int r = 0; r < 16; ++r) sc[r] = (t0 + 8 * (r >> 2) + 4 * h + (r & 3)) < limit ? sc[r] : kNegBig;
-            }
-            // sc = log2-domain score minus the column's reference point (0 while the column has seen nothing)
-            float bmax = fmaxf(fmaxf(sc[0], sc[1]), sc[2]);
-#pragma unroll
-            for (int r = 3; r < 15; r += 2) bmax = fmaxf(fmaxf(bmax, sc[r]), sc[r + 1]);
-            bmax = fmaxf(bmax, sc[15]);
-            bmax = fmaxf(bmax, swap32(bmax));
-            // the reference point moves when the block's maximum exceeds it by more than 2^8, and is set by the first
-            // block a column sees anything of
-            const bool first = m_run == kNegBig;
-            const bool move = bmax > 8.0f || (first && bmax > 0.5f * kNegBig);
-            if (__builtin_amdgcn_ballot_w64(move) != 0) {
-                // a real branch: in most blocks no column of the wave moves
-                asm volatile("" ::: "memory");
-                const float delta = move ? bmax : 0.0f;
-                const float alpha = __builtin_amdgcn_exp2f(-delta); // (columns that see their first tokens hold zeros)
-                if (move) m_run = (first ? 0.0f : m_run) + delta;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) sc[r] -= delta, negm[r] = move ? -m_run : negm[r], lacc[r] *= alpha;
-#pragma unroll
-                for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
-            }
-#pragma unroll
-            for (int r = 0; r < 16; ++r) pr[r] = __builtin_amdgcn_exp2f(sc[r]); // (a masked score is kNegBig: 0)
-        }
-        HFrag32 pf[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            pf[t].u[0] = pack_f16(pr[4 * t], pr[4 * t + 1]);
-            pf[t].u[1] = pack_f16(pr[4 * t + 2], pr[4 * t + 3]);
-            pf[t].u[2] = pack_f16(pr[4 * t + 8], pr[4 * t + 9]);
-            pf[t].u[3] = pack_f16(pr[4 * t + 10], pr[4 * t + 11]);
+            vinv = vref > 0.0f ? 1.0f / vref : 0.0f;
         }
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        for (int ct = 0; ct < CT; ++ct) {
+            f32x16 &x = sc[ct];
+            float pr[16];
+            if constexpr (!VIA_MFMA) {
+                if constexpr (INT8) {
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[t][dt].v, pf[t].v, o[dt], 0, 0, 0);
-            if constexpr (!INT8) lacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ones.v, pf[t].v, lacc, 0, 0, 0);
+                    for (int r = 0; r < 16; ++r) x[r] *= ks[r >> 2][r & 3];
+                }
+                if (masked) {
+                    // only the blocks on the causal diagonal pay for the mask (a real branch)
+                    asm volatile("" ::: "memory");
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) x[r] = (t0 + 8 * (r >> 2) + 4 * h + (r & 3)) < limit[ct] ? x[r] : kNegBig;
+                }
+                float bmax = fmaxf(fmaxf(x[0], x[1]), x[2]);
+#pragma unroll
+                for (int r = 3; r < 15; r += 2) bmax = fmaxf(fmaxf(bmax, x[r]), x[r + 1]);
+                bmax = fmaxf(bmax, x[15]);
+                bmax = fmaxf(bmax, swap32(bmax));
+                const float m_new = bmax > m_run[ct] + 8.0f ? bmax : m_run[ct];
+                const float alpha = __builtin_amdgcn_exp2f(m_run[ct] - m_new);
+                m_run[ct] = m_new;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) pr[r] = __builtin_amdgcn_exp2f(x[r] - m_new);
+                if (masked) {
+                    // a masked score is kNegBig: 2^(kNegBig - m) is already 0 unless the column has seen nothing yet
+                    asm volatile("" ::: "memory");
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) pr[r] = x[r] > 0.5f * kNegBig ? pr[r] : 0.0f;
+                }
+                float psum = (pr[0] + pr[1]) + (pr[2] + pr[3]);
+#pragma unroll
+                for (int r = 4; r < 16; r += 4) psum += (pr[r] + pr[r + 1]) + (pr[r + 2] + pr[r + 3]);
+                l_run[ct] = l_run[ct] * alpha + psum; // (this lane's 16 rows; the two halves are added at the end)
+                const float oscale = alpha * vmove; // what the running output is multiplied by before this block is added
+                if constexpr (INT8) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) pr[r] *= vs[r >> 2][r & 3] * vinv;
+                }
+                if (__builtin_amdgcn_ballot_w64(oscale != 1.0f) != 0) {
+                    // the running output is rescaled only when some column's reference point moved (a real branch)
+                    asm volatile("" ::: "memory");
+#pragma unroll
+                    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) o[ct][dt][r] *= oscale;
+                }
+            } else {
+                if (masked) {
+                    asm volatile("" ::: "memory");
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) x[r] = (t0 + 8 * (r >> 2) + 4 * h + (r & 3)) < limit[ct] ? x[r] : kNegBig;
+                }
+                // x = log2-domain score minus the column's reference point (0 while the column has seen nothing)
+                float bmax = fmaxf(fmaxf(x[0], x[1]), x[2]);
+#pragma unroll
+                for (int r = 3; r < 15; r += 2) bmax = fmaxf(fmaxf(bmax, x[r]), x[r + 1]);
+                bmax = fmaxf(bmax, x[15]);
+                bmax = fmaxf(bmax, swap32(bmax));
+                // the reference point moves when the block's maximum exceeds it by more than 2^8, and is set by the
+                // first block a column sees anything of
+                const bool first = m_run[ct] == kNegBig;
+                const bool move = bmax > 8.0f || (first && bmax > 0.5f * kNegBig);
+                if (__builtin_amdgcn_ballot_w64(move) != 0) {
+                    // a real branch: in most blocks no column of the wave moves
+                    asm volatile("" ::: "memory");
+                    const float delta = move ? bmax : 0.0f;
+                    const float alpha = __builtin_amdgcn_exp2f(-delta); // (columns that see their first tokens hold zeros)
+                    if (move) m_run[ct] = (first ? 0.0f : m_run[ct]) + delta;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) x[r] -= delta, negm[ct][r] = move ? -m_run[ct] : negm[ct][r], lacc[ct][r] *= alpha;
+#pragma unroll
+                    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) o[ct][dt][r] *= alpha;
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) pr[r] = __builtin_amdgcn_exp2f(x[r]); // (a masked score is kNegBig: 0)
+            }
+            HFrag32 pf[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                pf[t].u[0] = pack_f16(pr[4 * t], pr[4 * t + 1]);
+                pf[t].u[1] = pack_f16(pr[4 * t + 2], pr[4 * t + 3]);
+                pf[t].u[2] = pack_f16(pr[4 * t + 8], pr[4 * t + 9]);
+                pf[t].u[3] = pack_f16(pr[4 * t + 10], pr[4 * t + 11]);
+            }
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                for (int dt = 0; dt < 4; ++dt) o[ct][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[t][dt].v, pf[t].v, o[ct][dt], 0, 0, 0);
+                if constexpr (VIA_MFMA) lacc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ones.v, pf[t].v, lacc[ct], 0, 0, 0);
+            }
         }
     };
 
@@ -305,32 +341,36 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
         __syncthreads();
     }
 
-    float l = l_run;
-    l += swap32(l);
-    if constexpr (!INT8) l = lacc[0]; // every row of the ones tile holds the column's sum over all 32 tokens of every block
-    if (!cvalid) return;
-    const float inv = (INT8 ? vref : 1.0f) / l;
-    const size_t base = ((size_t)b * p.S + cs) * p.oStride + (size_t)(kvh * p.G + cj) * D;
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
+    for (int ct = 0; ct < CT; ++ct) {
+        float l = l_run[ct];
+        l += swap32(l);
+        if constexpr (VIA_MFMA) l = lacc[ct][0]; // every row of the ones tile holds the column's sum over all tokens
+        if (!cvalid[ct]) continue;
+        const float inv = (INT8 ? vref : 1.0f) / l;
+        const size_t base = ((size_t)b * p.S + cs[ct]) * p.oStride + (size_t)(kvh * p.G + cj[ct]) * D;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const size_t idx = base + 32 * dt + 8 * q + 4 * h;
-            const float v0 = o[dt][4 * q] * inv, v1 = o[dt][4 * q + 1] * inv, v2 = o[dt][4 * q + 2] * inv, v3 = o[dt][4 * q + 3] * inv;
-            if (p.out_dtype == XFTHIP_BF16) {
-                const uint32_t lo = f32_to_bf16_ref(v0) | ((uint32_t)f32_to_bf16_ref(v1) << 16);
-                const uint32_t hi = f32_to_bf16_ref(v2) | ((uint32_t)f32_to_bf16_ref(v3) << 16);
-                uint16_t *dst = (uint16_t *)p.out + idx;
-                if ((((uintptr_t)dst) & 7) == 0) {
-                    *(uint2 *)dst = make_uint2(lo, hi);
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const size_t idx = base + 32 * dt + 8 * q + 4 * h;
+                const float v0 = o[ct][dt][4 * q] * inv, v1 = o[ct][dt][4 * q + 1] * inv, v2 = o[ct][dt][4 * q + 2] * inv,
+                            v3 = o[ct][dt][4 * q + 3] * inv;
+                if (p.out_dtype == XFTHIP_BF16) {
+                    const uint32_t lo = f32_to_bf16_ref(v0) | ((uint32_t)f32_to_bf16_ref(v1) << 16);
+                    const uint32_t hi = f32_to_bf16_ref(v2) | ((uint32_t)f32_to_bf16_ref(v3) << 16);
+                    uint16_t *dst = (uint16_t *)p.out + idx;
+                    if ((((uintptr_t)dst) & 7) == 0) {
+                        *(uint2 *)dst = make_uint2(lo, hi);
+                    } else {
+                        dst[0] = (uint16_t)lo, dst[1] = (uint16_t)(lo >> 16), dst[2] = (uint16_t)hi, dst[3] = (uint16_t)(hi >> 16);
+                    }
                 } else {
-                    dst[0] = (uint16_t)lo, dst[1] = (uint16_t)(lo >> 16), dst[2] = (uint16_t)hi, dst[3] = (uint16_t)(hi >> 16);
+                    float *dst = (float *)p.out + idx;
+                    dst[0] = v0, dst[1] = v1, dst[2] = v2, dst[3] = v3;
                 }
-            } else {
-                float *dst = (float *)p.out + idx;
-                dst[0] = v0, dst[1] = v1, dst[2] = v2, dst[3] = v3;
             }
-        }
+    }
 }
 
 } // namespace xfthip

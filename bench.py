@@ -2,9 +2,9 @@
 """Decode-throughput benchmark of the MI355X decoder-layer hot path.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--weights int8|uint4] [--kv fp16|int8]
-                    [--eager | --no-fusion | --persistent]        (variants of the decode step)
+                    [--eager | --no-fusion]                       (variants of the decode step)
                     [--no-extras] [--no-cpu-baseline]
-                    [--prefill-gemm | --attention | --moe]        (one of the extra measurements alone, one JSON line)
+                    [--prefill-gemm | --attention | --moe | --stream-floor]   (one of the extra measurements alone, one JSON line)
                     [--pmc-workload | --pmc-summary FETCH_CSV WRITE_CSV]   (hardware-counter traffic)
 
 Workload (configs[3] of the benchmark definition): a 32-layer Llama-2-7B-shape model with random weights
@@ -137,6 +137,34 @@ def time_gemm_kernel(xh, layer_weights, which, M, iters):
     byts = sum(layer_weights[0][i].bytes() + in_bytes(i, layer_weights[0][i]) + out_bytes(i, layer_weights[0][i])
                for i in which) / len(which)
     return ms * 1e3 / n, byts
+
+
+def stream_floor(xh, sizes_mb=(16.8, 45.1, 50.4, 90.2), buffers=32, iters=4):
+    """The library's read-only kernel over `buffers` distinct device buffers of each size (the byte counts of
+    one decode layer's four packed INT8 weights), launched back to back and timed with HIP events: what
+    streaming that many bytes costs on this machine with nothing behind the loads, launch ramp and tail
+    included.  The weight-streaming GEMVs are held against these, not against bytes / 8 TB/s."""
+    out = []
+    for mb in sizes_mb:
+        nbytes = int(mb * 1e6) // 4096 * 4096
+        bufs = [xh.DeviceBuffer(nbytes) for _ in range(buffers)]
+        for b in bufs:
+            b.zero()
+        for b in bufs:
+            xh.read_kernel(b.ptr, nbytes)
+        xh.synchronize()
+        t = xh.Timer()
+        t.start()
+        for _ in range(iters):
+            for b in bufs:
+                xh.read_kernel(b.ptr, nbytes)
+        ms = t.stop()
+        us = ms * 1e3 / (iters * buffers)
+        out.append({"bytes": nbytes, "avg_launch_us": round(us, 2), "gbs": round(nbytes / us / 1e3, 1),
+                    "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
+        for b in bufs:
+            b.free()
+    return out
 
 
 PMC_COPY_BYTES = 256 << 20
@@ -487,7 +515,6 @@ def main():
     ap.add_argument("--kv", choices=["fp16", "int8"], default="fp16", help="KV cache format")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fusion", action="store_true", help="run RMSNorm / RoPE + cache append as their own kernels instead of inside the decode GEMVs")
-    ap.add_argument("--persistent", action="store_true", help="run each decode step as the single persistent kernel (experimental)")
     ap.add_argument("--pmc-workload", action="store_true", help="counter workload for rocprofv3 --pmc: a plain copy kernel of known size, then every distinct decode GEMV of the model once; prints no result line")
     ap.add_argument("--pmc-summary", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"), help="summarise the two counter CSVs of the --pmc-workload runs (CPU only)")
     ap.add_argument("--eager", action="store_true", help="launch decode kernels one by one instead of replaying the captured graph (for per-kernel profiling)")
@@ -495,6 +522,7 @@ def main():
     ap.add_argument("--prefill-gemm", action="store_true", help="only the weight-only GEMM sweep at M = 1, 8, 32, 256, 2048 (one JSON line)")
     ap.add_argument("--attention", action="store_true", help="only the GQA attention sweep (one JSON line)")
     ap.add_argument("--moe", action="store_true", help="only the sparse-MLP layer (one JSON line)")
+    ap.add_argument("--stream-floor", action="store_true", help="only the read-only streaming floor at the decode GEMVs' byte counts (one JSON line)")
     args = ap.parse_args()
     if args.pmc_summary:
         pmc_summary(*args.pmc_summary)
@@ -514,6 +542,9 @@ def main():
     if args.moe:
         print(json.dumps({"moe": moe_layer(xh)}))
         return
+    if args.stream_floor:
+        print(json.dumps({"stream_floor": stream_floor(xh), "hbm_peak_gbs": HBM_PEAK_GBS}))
+        return
     kind = 0 if args.weights == "int8" else 1
     B = args.batch
     max_seq = args.prompt + args.warmup + args.steps + 1
@@ -526,8 +557,6 @@ def main():
         model.use_graph(False)
     if args.no_fusion:
         model.use_fusion(False)
-    if args.persistent:
-        model.use_persistent(True)
     rng = np.random.default_rng(3)
     ids = rng.integers(0, CFG["vocab"], (B, args.prompt)).astype(np.int32)
     t0 = time.time()
@@ -615,6 +644,8 @@ def main():
         extra["prefill_gemm"] = prefill_gemm_sweep(xh, 2048)
         extra["attention"] = attention_sweep(xh)
         extra["moe"] = moe_layer(xh)
+        # what the bytes of a decode layer's four GEMVs cost as a pure read (out-proj, down, QKV, gate/up)
+        extra["stream_floor"] = stream_floor(xh)
         result["extra"] = extra
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(kind, host, shapes, B, args.prompt)

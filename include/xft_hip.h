@@ -70,6 +70,11 @@ int xfthip_memcpy_d2d(void *dst, const void *src, size_t bytes, xfthip_stream_t 
  * 16-byte aligned): reads `bytes` and writes `bytes`, which makes it the reference point when
  * hardware counters of HBM traffic are scaled.  No counterpart in the reference. */
 int xfthip_copy_kernel(void *dst, const void *src, size_t bytes, xfthip_stream_t stream);
+/* Reads `bytes` (a multiple of 16, 16-byte aligned) with `blocks` workgroups (0 = two per compute unit) and
+ * discards them: the time of a launch is what streaming that many bytes costs on this machine with nothing
+ * behind the loads, launch ramp and tail included - the floor bench.py prints beside the weight-streaming
+ * kernels.  A measurement aid with no counterpart in the reference. */
+int xfthip_read_kernel(const void *src, size_t bytes, int blocks, xfthip_stream_t stream);
 int xfthip_memset(void *dst, int value, size_t bytes, xfthip_stream_t stream);
 int xfthip_stream_create(xfthip_stream_t *stream);
 int xfthip_stream_destroy(xfthip_stream_t stream);
@@ -458,19 +463,7 @@ int xfthip_model_use_graph(xfthip_model_t m, int enable);
  * points except for the fp32 summation order inside the norm.  The reference keeps these as
  * separate calls (src/layers/attention.h:322-460, src/layers/mlp_llama.h:200-260). */
 int xfthip_model_use_fusion(xfthip_model_t m, int enable);
-/* Decode of up to 4 sequences with INT8 symmetric layer weights, FP16 cache and a BF16 lm_head runs
- * as ONE persistent kernel per step (device-wide barriers instead of launches).  enable = 0 falls
- * back to the per-kernel step (captured in a HIP graph when xfthip_model_use_graph allows).
- * The reference has no counterpart: its decode step is a host loop over layers
- * (src/models/common_decoder.h:290-420). */
-int xfthip_model_use_persistent(xfthip_model_t m, int enable);
-/* Per-phase timing of the persistent kernel, which a kernel-level profiler cannot see into.
- * Call once with ticks_host = NULL to arm it; after a decode call, a second call copies out
- * 5 * layers + 3 timestamps of the last step (100 MHz ticks): [0] kernel start, [i] the moment
- * workgroup 0 left device-wide barrier i (embedding; per layer qkv, attention, out-proj,
- * gate/up, down; lm_head).  No counterpart in the reference. */
-int xfthip_model_persistent_trace(xfthip_model_t m, unsigned long long *ticks_host, int capacity);
-/* How the last xfthip_model_decode ran: 2 = persistent kernel, 1 = graph replay, 0 = eager launches. */
+/* How the last xfthip_model_decode ran: 1 = graph replay, 0 = eager launches. */
 int xfthip_model_decode_mode(xfthip_model_t m);
 /* ids chosen by the last prefill / decode call (host int32 [B]) and the current position */
 int xfthip_model_last_ids(xfthip_model_t m, int *ids_host, int *position);

@@ -15,10 +15,14 @@ with the GPU's tokens, so every step is checked against the GPU's own logits of 
   * every decode step's logits: max-abs <= 0.2, cosine >= 0.9995 (a step attends over 512 + t cached rows
     that already carry the prompt pass's differences, and the maximum is taken over 32 steps x 32000 (x 2)
     logits instead of one set; measured at worst 0.182 and 0.99966, UINT4 at batch 32 / batch 1);
-  * a GPU token that is not the oracle's best must lie within 1.5 x that step's measured max-abs
-    logit difference of the oracle's best (in the oracle's logits): the two pipelines then
-    disagree only about a pair they cannot tell apart;
-  * at least 85 % of the choices are the oracle's best."""
+  * a GPU token that is not the oracle's best must lie within 0.75 x that step's measured max-abs
+    logit difference of the oracle's best (in the oracle's logits; measured at worst 0.37): the two
+    pipelines then disagree only about a pair they cannot tell apart;
+  * at least 70 % of the choices are the oracle's best.  With 32000 logits of unit spread the best two
+    of a step lie ~0.2 apart on average and closer than 0.04 in one step of six, and the logits differ
+    by ~0.02 rms, so a few of the 33 choices fall on such a pair by chance (measured: 26 to 33 of 33
+    between builds that differ only in the rounding order of the prompt pass); the gap rule above is
+    what bounds each of them."""
 import time
 
 import numpy as np
@@ -28,7 +32,7 @@ pytestmark = pytest.mark.gpu
 
 HIDDEN, INTER, QH, KVH, D, LAYERS, VOCAB = 4096, 11008, 32, 32, 128, 32, 32000
 PROMPT, STEPS = 512, 32
-COS_BAR, STEP_COS_BAR, ABS_BAR, STEP_ABS_BAR, GAP_FACTOR, EXACT_SHARE = 0.9997, 0.9995, 0.15, 0.2, 1.5, 0.85
+COS_BAR, STEP_COS_BAR, ABS_BAR, STEP_ABS_BAR, GAP_FACTOR, EXACT_SHARE = 0.9997, 0.9995, 0.15, 0.2, 0.75, 0.70
 
 
 @pytest.fixture(scope="module")
@@ -115,6 +119,7 @@ def test_full_model_greedy_32_steps(xh, orc, head, kind, B):
         assert _cos(logits[follow], flogits) >= 0.999
 
     worst = dict(err=err, cos=cos, gap_ratio=0.0)
+    misses = []
 
     def check(g, gpu_lg, lg, what, cos_bar=STEP_COS_BAR, abs_bar=STEP_ABS_BAR):
         """g: the GPU's tokens; gpu_lg / lg: the GPU's and the oracle's logits of the same step."""
@@ -130,6 +135,8 @@ def test_full_model_greedy_32_steps(xh, orc, head, kind, B):
             worst["gap_ratio"] = max(worst["gap_ratio"], gap / step_err)
             assert gap <= GAP_FACTOR * step_err, (what, j, int(g[j]), best, gap, step_err)
             same += int(g[j] == best)
+            if g[j] != best:
+                misses.append((what, j, round(gap, 4), round(step_err, 4)))
         return same
 
     exact = check(first[follow], logits[follow], elogits, "prompt", COS_BAR, ABS_BAR)
@@ -141,6 +148,7 @@ def test_full_model_greedy_32_steps(xh, orc, head, kind, B):
     total = (STEPS + 1) * Bo
     print(f"greedy ids equal to the oracle's best in {exact} of {total} choices; worst step: max-abs {worst['err']:.3e}, cosine "
           f"{worst['cos']:.6f}, gap / max-abs {worst['gap_ratio']:.2f}; gpu {t1 - t0:.1f} s, oracle {time.time() - t1:.1f} s", flush=True)
+    print("choices that are not the oracle's best (step, sequence, oracle's gap, step max-abs):", misses, flush=True)
     assert exact >= EXACT_SHARE * total
     orc.clear_blas_cache()
     model.free()

@@ -54,6 +54,11 @@ def copy_kernel(dst_ptr, src_ptr, nbytes, stream=None):
     check(lib.xfthip_copy_kernel(dst_ptr, src_ptr, C.c_size_t(nbytes), stream))
 
 
+def read_kernel(src_ptr, nbytes, blocks=0, stream=None):
+    """Read-only stream over nbytes (results discarded): the floor of a weight-streaming launch."""
+    check(lib.xfthip_read_kernel(src_ptr, C.c_size_t(nbytes), int(blocks), stream))
+
+
 def synchronize():
     check(lib.xfthip_device_synchronize())
 
@@ -440,19 +445,6 @@ class Model:
 
     def use_fusion(self, enable):
         check(lib.xfthip_model_use_fusion(self.h, int(bool(enable))))
-
-    def use_persistent(self, enable):
-        check(lib.xfthip_model_use_persistent(self.h, int(bool(enable))))
-
-    def persistent_trace(self, arm=False):
-        """arm=True: start recording; otherwise the barrier timestamps (seconds) of the last step."""
-        if arm:
-            check(lib.xfthip_model_persistent_trace(self.h, None, 0))
-            return None
-        n = 5 * self.cfg.layers + 3
-        out = np.zeros(n, np.uint64)
-        check(lib.xfthip_model_persistent_trace(self.h, _hp(out), len(out)))
-        return out.astype(np.float64) * 1e-8
 
     def decode_mode(self):
         return int(lib.xfthip_model_decode_mode(self.h))

@@ -40,14 +40,6 @@ __global__ __launch_bounds__(256, 3) void attn_kernel(AttnParams p) {
     attn_unit<INT8, 4, PIPE>(p, blockIdx.x, blockIdx.y % p.kv.H, blockIdx.y / p.kv.H, blockIdx.z, lds, [] { __syncthreads(); });
 }
 
-// FP16 cache, K / V blocks shared through LDS: a workgroup = 64 CT neighbouring columns of one (sequence, KV head)
-template <int CT, bool INT8 = false>
-// launch bounds: three workgroups a CU with one column tile a wave (140 registers), two with two (216)
-__global__ __launch_bounds__(256, (CT == 1 ? 3 : 2)) void attn_prefill_lds_kernel(AttnParams p) {
-    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kPfBufBytes];
-    attn_prefill_lds_unit<CT, INT8>(p, blockIdx.y, gridDim.x - 1 - blockIdx.x, blockIdx.z, lds); // longest history first
-}
-
 // 32 x 32 MFMA tiles, 32 columns a wave, K / V blocks shared through LDS (attention_prefill.h); two workgroups a CU
 // Workgroups are handed to the 8 XCDs in turn by their linear index, and each XCD has an L2 of its own: the
 // (sequence, KV head) pairs are dealt to the XCDs (pair = 8 k + XCD), and an XCD walks the column groups of one
@@ -66,12 +58,6 @@ __global__ __launch_bounds__(256, (CT == 1 ? 2 : 1)) void attn_prefill32_kernel(
 // column group.  The library keeps one for plain xfthip_attention calls (allocated on first use);
 // a model owns its own, so that two models on two streams never share partials or tickets.
 static AttnWorkspace g_shared_ws;
-// 0: the 32-column form above; 1: the 16-column form it replaced (XFT_PREFILL_FORM=16, kept for comparison runs)
-static const int g_prefill_form = [] {
-    const char *e = getenv("XFT_PREFILL_FORM");
-    return (e && atoi(e) == 16) ? 1 : 0;
-}();
-
 int attention_workspace_create(AttnWorkspace *w, int slots) {
     w->ws = nullptr, w->tickets = nullptr, w->slots = 0;
     XFT_CHECK_HIP(hipMalloc((void **)&w->ws, (size_t)slots * kSlotFloats * sizeof(float)));
@@ -159,33 +145,16 @@ int xfthip::attention_launch(xfthip_kvcache_t c, const void *q, int qStride, voi
     p.past = past;
     p.past_dev = past_dev;
     p.CG = (S * p.G + 15) / 16;
-    // Many columns per KV head (prefill, long chunks): the forms in which a wave walks the whole visible
-    // sequence for its 16 (or 32) columns, taken once they fill the device by themselves.  Occupancy decides
-    // here: with one column tile a wave the FP16 form runs three workgroups a CU, with two tiles two; measured
-    // (4 x 2048 and 8 x 1024 GQA, 1 x 512 / 1 x 2048 / 32 x 512 MHA) one tile wins or ties except for long
-    // sequences of a model without grouped heads, where a workgroup's 64 columns are 64 tokens.
+    // Many columns per KV head (prefill, long chunks): the form in which a wave walks the whole visible sequence
+    // for its 32 columns through LDS blocks shared by its workgroup, taken once such waves fill the device.
     {
         const long waves1 = (long)B * c->kv.H * p.CG; // waves with one column tile each
         if (S > 1 && waves1 >= 4L * device_cu_count()) {
             p.nsplit = 1;
-            if (g_prefill_form == 0) {
-                const int ncg = (S * p.G + 127) / 128, npairs = B * c->kv.H;
-                dim3 grid(8 * ((npairs + 7) / 8) * ncg);
-                if (c->kv.int8) hipLaunchKernelGGL((attn_prefill32_kernel<true, 1>), grid, dim3(256), 0, stream, p, ncg, npairs);
-                else hipLaunchKernelGGL((attn_prefill32_kernel<false, 1>), grid, dim3(256), 0, stream, p, ncg, npairs);
-                XFT_CHECK_HIP(hipGetLastError());
-                return 0;
-            }
-            if (!c->kv.int8) {
-                const int ctl = (p.G == 1 && waves1 >= 16L * device_cu_count()) ? 2 : 1;
-                dim3 grid((p.CG + 4 * ctl - 1) / (4 * ctl), c->kv.H, B);
-                if (ctl == 2) hipLaunchKernelGGL(attn_prefill_lds_kernel<2>, grid, dim3(256), 0, stream, p);
-                else hipLaunchKernelGGL(attn_prefill_lds_kernel<1>, grid, dim3(256), 0, stream, p);
-            } else {
-                // INT8 cache: the same kernel, codes widened once per workgroup on their way into LDS
-                dim3 grid((p.CG + 3) / 4, c->kv.H, B);
-                hipLaunchKernelGGL((attn_prefill_lds_kernel<1, true>), grid, dim3(256), 0, stream, p);
-            }
+            const int ncg = (S * p.G + 127) / 128, npairs = B * c->kv.H;
+            dim3 grid(8 * ((npairs + 7) / 8) * ncg);
+            if (c->kv.int8) hipLaunchKernelGGL((attn_prefill32_kernel<true, 1>), grid, dim3(256), 0, stream, p, ncg, npairs);
+            else hipLaunchKernelGGL((attn_prefill32_kernel<false, 1>), grid, dim3(256), 0, stream, p, ncg, npairs);
             XFT_CHECK_HIP(hipGetLastError());
             return 0;
         }

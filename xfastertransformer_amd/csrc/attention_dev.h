@@ -1,5 +1,4 @@
-// Device-side body of the attention kernel, shared by the stand-alone kernel and the persistent
-// decode kernel.  See attention.hip for the algorithm.
+// Device-side body of the attention kernels.  See attention.hip for the algorithm.
 #pragma once
 #include "kvcache.h"
 
@@ -435,301 +434,11 @@ __device__ inline float swap32(float x) { // value of lane ^ 32
 }
 
 
-// ---- prefill: many columns per (sequence, KV head), K / V blocks shared through LDS ----------------
-// With hundreds of (query token, query head) columns per KV head the unit above re-reads the keys and values
-// of a head once per 16 columns from L2, which is what bounds it.  Here a wave owns CT column tiles (16 CT
-// columns) and walks ALL token blocks its columns can see (no partials: every wave finishes its columns by
-// itself; same arithmetic per column as attn_unit: fp32 scores, online softmax, fp16 probabilities into the
-// P.V MFMA), and the 4 waves of a workgroup take 4 neighbouring column groups.  A form in which every wave kept
-// its own copy of a block in registers still pulled each block once per wave through L2 (the waves do not stay
-// close enough for the 32 KB L1 to serve them).  Here the workgroup copies each 32-token block
-// (8 KB of keys, 8 KB of values) into LDS once and its 4 waves, CT column tiles each, read their MFMA
-// operands from there: 64 CT columns per workgroup share one trip of the block through L2.  Rows are padded
-// (keys 272 B per token, values 80 B per dim) so that the 8 lanes one 128-bit LDS read serves together
-// touch different banks.  Two LDS buffers; the next block travels global -> registers while the current
-// one is multiplied, then registers -> LDS, one barrier per block.
+// ---- prefill: many columns per (sequence, KV head), K / V blocks shared through LDS (attention_prefill.h) -----
+// Layout of a 32-token block in LDS: keys 32 rows of 256 B at a pitch of 272 B, values 128 dim rows of 64 B (token
+// slots as in the cache) at a pitch of 80 B, so that the lanes one 128-bit LDS read serves together touch
+// different banks.
 constexpr int kPfKPitch = 272, kPfVPitch = 80;
 constexpr int kPfBufBytes = 32 * kPfKPitch + 128 * kPfVPitch; // 18,944 B per buffer
-
-// INT8: the cache holds codes and one scale a token.  The codes are widened to fp16 (exact) on their way into LDS,
-// once per workgroup, so the blocks in LDS look as they do for the FP16 cache; the key scale multiplies the score,
-// the value scale the probability (normalised by the block's largest scale, which multiplies the block's product:
-// probabilities stay in fp16's range whatever the scales).  The scales of the next block travel with its codes.
-template <int CT, bool INT8 = false>
-__device__ inline void attn_prefill_lds_unit(const AttnParams &p, const int kvh, const int cgroup, const int b, unsigned char *lds) {
-    constexpr int D = 128;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int g = lane >> 4, cl = lane & 15;
-    const int cgw = cgroup * 4 + wave; // this wave's group of 16 CT columns
-    int past = p.past;
-    if (p.past_dev) {
-        past = p.past_dev[b];
-        past = past < 0 ? 0 : (past > p.kv.S - p.S ? p.kv.S - p.S : past);
-    }
-    const int ncols = p.S * p.G;
-    bool cvalid[CT];
-    int cs[CT], cj[CT], limit[CT], lim_min[CT];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        const int c = (cgw * CT + ct) * 16 + cl;
-        cvalid[ct] = c < ncols;
-        cs[ct] = cvalid[ct] ? c / p.G : 0;
-        cj[ct] = cvalid[ct] ? c % p.G : 0;
-        limit[ct] = cvalid[ct] ? past + cs[ct] + 1 : 0;
-        lim_min[ct] = (cgw * CT + ct) * 16 + 15 < ncols ? past + ((cgw * CT + ct) * 16) / p.G + 1 : 0;
-    }
-    // blocks this wave needs / the workgroup walks (its last wave sees the most)
-    int wave_last = (cgw * CT + CT) * 16 - 1;
-    wave_last = wave_last < ncols ? wave_last : ncols - 1;
-    const int wave_nblk = (cgw * CT) * 16 < ncols ? (past + wave_last / p.G + 1 + 31) >> 5 : 0;
-    int wg_last = (cgroup * 4 + 4) * CT * 16 - 1;
-    wg_last = wg_last < ncols ? wg_last : ncols - 1;
-    const int nblk = (past + wg_last / p.G + 1 + 31) >> 5;
-
-    const size_t bh = (size_t)b * p.kv.H + kvh;
-    constexpr int ESZ = INT8 ? 1 : 2;
-    const ATTN_GLOBAL char *kbase = (const ATTN_GLOBAL char *)p.kv.k + bh * p.kv.S * D * ESZ;
-    const ATTN_GLOBAL char *vbase = (const ATTN_GLOBAL char *)p.kv.v + bh * p.kv.S * D * ESZ;
-    const ATTN_GLOBAL float *ksc = INT8 ? (const ATTN_GLOBAL float *)p.kv.kscale + bh * p.kv.S : nullptr;
-    const ATTN_GLOBAL float *vsc = INT8 ? (const ATTN_GLOBAL float *)p.kv.vscale + bh * p.kv.S : nullptr;
-
-    // the block copy: 512 + 512 chunks of 16 bytes, two of each per thread (INT8: 256 + 256, one of each)
-    u32x4 kstage[2], vstage[2];
-    f32x4 ks_next[2], vs_next[2], ks_cur[2], vs_cur[2]; // INT8: scales of tokens t0 + 16 a + 4 g + r
-    auto fetch = [&](const int blk) {
-        if constexpr (INT8) {
-            kstage[0] = *(const ATTN_GLOBAL u32x4 *)(kbase + (size_t)blk * (32 * D) + (size_t)threadIdx.x * 16);
-            vstage[0] = *(const ATTN_GLOBAL u32x4 *)(vbase + (size_t)blk * (32 * D) + (size_t)threadIdx.x * 16);
-#pragma unroll
-            for (int a = 0; a < 2; ++a) {
-                ks_next[a] = *(const ATTN_GLOBAL f32x4 *)(ksc + (blk << 5) + 16 * a + 4 * g);
-                vs_next[a] = *(const ATTN_GLOBAL f32x4 *)(vsc + (blk << 5) + 16 * a + 4 * g);
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const int ch = threadIdx.x + 256 * i;
-                kstage[i] = *(const ATTN_GLOBAL u32x4 *)(kbase + (size_t)blk * (32 * D * 2) + (size_t)ch * 16);
-                vstage[i] = *(const ATTN_GLOBAL u32x4 *)(vbase + (size_t)blk * (32 * D * 2) + (size_t)ch * 16);
-            }
-        }
-    };
-    // 16 codes -> 16 fp16 values (two 16-byte pieces)
-    auto widen16 = [&](const u32x4 raw, u32x4 &lo, u32x4 &hi) {
-        HFrag x, y;
-        widen_i8x4(raw[0], x.h[0], x.h[1]);
-        widen_i8x4(raw[1], x.h[2], x.h[3]);
-        widen_i8x4(raw[2], y.h[0], y.h[1]);
-        widen_i8x4(raw[3], y.h[2], y.h[3]);
-        lo = x.q, hi = y.q;
-    };
-    auto stash = [&](const int buf) {
-        unsigned char *kb = lds + buf * kPfBufBytes, *vb = kb + 32 * kPfKPitch;
-        if constexpr (INT8) {
-            const int ch = threadIdx.x;
-            u32x4 lo, hi;
-            widen16(kstage[0], lo, hi); // token ch / 8, dims 16 (ch % 8) ..
-            *(u32x4 *)(kb + (ch >> 3) * kPfKPitch + (ch & 7) * 32) = lo;
-            *(u32x4 *)(kb + (ch >> 3) * kPfKPitch + (ch & 7) * 32 + 16) = hi;
-            widen16(vstage[0], lo, hi); // dim ch / 2, token slots 16 (ch % 2) ..
-            *(u32x4 *)(vb + (ch >> 1) * kPfVPitch + (ch & 1) * 32) = lo;
-            *(u32x4 *)(vb + (ch >> 1) * kPfVPitch + (ch & 1) * 32 + 16) = hi;
-#pragma unroll
-            for (int a = 0; a < 2; ++a) ks_cur[a] = ks_next[a], vs_cur[a] = vs_next[a];
-        } else {
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const int ch = threadIdx.x + 256 * i;
-                *(u32x4 *)(kb + (ch >> 4) * kPfKPitch + (ch & 15) * 16) = kstage[i]; // token ch / 16, dims 8 (ch % 16) ..
-                *(u32x4 *)(vb + (ch >> 2) * kPfVPitch + (ch & 3) * 16) = vstage[i]; // dim ch / 4, tokens 8 (ch % 4) ..
-            }
-        }
-    };
-
-    HFrag qf[CT][4];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        const uint16_t *qrow = p.q + ((size_t)b * p.S + cs[ct]) * p.qStride + (size_t)(kvh * p.G + cj[ct]) * D;
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            uint32_t raw[4] = {0u, 0u, 0u, 0u};
-            if (cvalid[ct]) ld_dev16(qrow + 32 * s + 8 * g, raw);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) qf[ct][s].u[i] = pack_f16(u2f(raw[i] << 16), u2f(raw[i] & 0xFFFF0000u));
-        }
-    }
-    float m_run[CT], l_run[CT];
-    f32x4 o[CT][8];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        m_run[ct] = kNegBig, l_run[ct] = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) o[ct][i] = f32x4 {0.f, 0.f, 0.f, 0.f};
-    }
-    const float c1 = p.scale * 1.4426950408889634f; // scores live in the log2 domain
-
-    auto compute = [&](const int buf, const int blk) {
-        const int t0 = blk << 5;
-        const unsigned char *kb = lds + buf * kPfBufBytes, *vb = kb + 32 * kPfKPitch;
-        HFrag kf[2][4], vf[8];
-        // INT8: this block's scales (stash() moved them here when it put the block into LDS)
-        f32x4 ks[2], vs[2];
-        float vmax = 0.0f;
-        if constexpr (INT8) {
-#pragma unroll
-            for (int a = 0; a < 2; ++a) {
-                ks[a] = ks_cur[a] * c1; // key scale and softmax scale in one factor
-                vs[a] = vs_cur[a];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) vmax = fmaxf(vmax, vs[a][r]);
-            }
-            vmax = fmaxf(vmax, swap16(vmax));
-            vmax = fmaxf(vmax, swap32(vmax));
-        }
-        const float vinv = (INT8 && vmax > 0.0f) ? 1.0f / vmax : 1.0f;
-#pragma unroll
-        for (int a = 0; a < 2; ++a)
-#pragma unroll
-            for (int s = 0; s < 4; ++s) kf[a][s].q = *(const u32x4 *)(kb + (16 * a + cl) * kPfKPitch + (8 * g + 32 * s) * 2);
-        // all score tiles first, k step by k step over the 2 CT independent accumulators: no MFMA waits for the
-        // one before it, and the scores of the later column tiles are ready while the earlier ones go through
-        // the softmax arithmetic (their P.V products then run behind that arithmetic instead of in front of it)
-        f32x4 sc_all[CT][2];
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-            for (int a = 0; a < 2; ++a) sc_all[ct][a] = f32x4 {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < 4; ++s)
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-                for (int a = 0; a < 2; ++a)
-                    sc_all[ct][a] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[a][s].v, qf[ct][s].v, sc_all[ct][a], 0, 0, 0);
-        // the value operands are read only now (the fence keeps the compiler from hoisting the reads): they reuse
-        // the registers of the key operands, and their LDS latency passes behind the softmax arithmetic
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int dt = 0; dt < 8; ++dt) vf[dt].q = *(const u32x4 *)(vb + (16 * dt + cl) * kPfVPitch + 8 * g * 2);
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            f32x4 sc[2] = {sc_all[ct][0], sc_all[ct][1]};
-            float bmax = kNegBig;
-            const bool masked = t0 + 32 > lim_min[ct]; // wave-uniform
-#pragma unroll
-            for (int a = 0; a < 2; ++a)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) sc[a][r] *= INT8 ? ks[a][r] : c1;
-            if (masked) {
-                // only the blocks on the causal diagonal pay for the mask (a real branch: the empty asm keeps
-                // the compiler from turning it into selects executed by every block)
-                asm volatile("" ::: "memory");
-#pragma unroll
-                for (int a = 0; a < 2; ++a)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) sc[a][r] = (t0 + 16 * a + 4 * g + r) < limit[ct] ? sc[a][r] : kNegBig;
-            }
-#pragma unroll
-            for (int a = 0; a < 2; ++a)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) bmax = fmaxf(bmax, sc[a][r]);
-            bmax = fmaxf(bmax, swap16(bmax));
-            bmax = fmaxf(bmax, swap32(bmax));
-            // The reference point of the exponentials only moves when the block's maximum exceeds it by more than
-            // 2^8: softmax does not depend on the reference point, probabilities up to 256 are exact enough in
-            // fp16 and in the fp32 sums, and the running output (in AGPRs) is rescaled in few blocks only.
-            const float m_new = bmax > m_run[ct] + 8.0f ? bmax : m_run[ct];
-            const float alpha = __builtin_amdgcn_exp2f(m_run[ct] - m_new);
-            m_run[ct] = m_new;
-            float psum = 0.0f;
-            float pr[2][4];
-#pragma unroll
-            for (int a = 0; a < 2; ++a)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) pr[a][r] = __builtin_amdgcn_exp2f(sc[a][r] - m_new);
-            if (masked) {
-                // a masked score is kNegBig: 2^(kNegBig - m) is already 0 unless the column has seen nothing yet
-                asm volatile("" ::: "memory");
-#pragma unroll
-                for (int a = 0; a < 2; ++a)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) pr[a][r] = sc[a][r] > 0.5f * kNegBig ? pr[a][r] : 0.0f;
-            }
-#pragma unroll
-            for (int a = 0; a < 2; ++a)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) psum += pr[a][r];
-            l_run[ct] = l_run[ct] * alpha + psum;
-            const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0;
-            if constexpr (INT8) {
-#pragma unroll
-                for (int a = 0; a < 2; ++a)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) pr[a][r] *= vs[a][r] * vinv;
-            }
-            HFrag pf;
-            pf.u[0] = pack_f16(pr[0][0], pr[0][1]);
-            pf.u[1] = pack_f16(pr[0][2], pr[0][3]);
-            pf.u[2] = pack_f16(pr[1][0], pr[1][1]);
-            pf.u[3] = pack_f16(pr[1][2], pr[1][3]);
-            if (rescale) {
-                // the running output is rescaled only when some column's maximum moved (a real branch: the
-                // accumulators live in AGPRs and a rescale costs a read, a multiply and a write each)
-                asm volatile("" ::: "memory");
-#pragma unroll
-                for (int dt = 0; dt < 8; ++dt) o[ct][dt] = o[ct][dt] * alpha;
-            }
-#pragma unroll
-            for (int dt = 0; dt < 8; ++dt) {
-                if constexpr (INT8) {
-                    f32x4 tmp = {0.f, 0.f, 0.f, 0.f};
-                    tmp = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[dt].v, pf.v, tmp, 0, 0, 0);
-                    o[ct][dt] = o[ct][dt] + tmp * vmax;
-                } else {
-                    o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[dt].v, pf.v, o[ct][dt], 0, 0, 0);
-                }
-            }
-        }
-    };
-
-    if (nblk > 0) {
-        fetch(0);
-        stash(0);
-    }
-    __syncthreads();
-    for (int blk = 0; blk < nblk; ++blk) {
-        const bool more = blk + 1 < nblk; // uniform over the workgroup
-        if (more) fetch(blk + 1);
-        if (blk < wave_nblk) compute(blk & 1, blk);
-        if (more) stash((blk + 1) & 1);
-        __syncthreads();
-    }
-
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        float l = l_run[ct];
-        l += swap16(l);
-        l += swap32(l);
-        if (!cvalid[ct]) continue;
-        const size_t base = ((size_t)b * p.S + cs[ct]) * p.oStride + (size_t)(kvh * p.G + cj[ct]) * D;
-#pragma unroll
-        for (int dt = 0; dt < 8; ++dt) {
-            const size_t idx = base + 16 * dt + 4 * g;
-            if (p.out_dtype == XFTHIP_BF16) {
-                const uint32_t lo = f32_to_bf16_ref(o[ct][dt][0] / l) | ((uint32_t)f32_to_bf16_ref(o[ct][dt][1] / l) << 16);
-                const uint32_t hi = f32_to_bf16_ref(o[ct][dt][2] / l) | ((uint32_t)f32_to_bf16_ref(o[ct][dt][3] / l) << 16);
-                uint16_t *dst = (uint16_t *)p.out + idx;
-                if ((((uintptr_t)dst) & 7) == 0) {
-                    *(uint2 *)dst = make_uint2(lo, hi);
-                } else {
-                    dst[0] = (uint16_t)lo, dst[1] = (uint16_t)(lo >> 16), dst[2] = (uint16_t)hi, dst[3] = (uint16_t)(hi >> 16);
-                }
-            } else {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) store_from_f32(p.out, p.out_dtype, idx + r, o[ct][dt][r] / l);
-            }
-        }
-    }
-}
 
 } // namespace xfthip

@@ -19,7 +19,6 @@
 #include <vector>
 
 #include "attention_dev.h"
-#include "decode_mega.h"
 #include "kvcache.h"
 #include "qgemm.h"
 
@@ -203,17 +202,6 @@ struct xfthip_model {
     hipStream_t graph_stream = nullptr;
     bool use_graph = true;
     bool fuse_decode = true; // RMSNorm prologue / RoPE + cache-append epilogue inside the decode GEMVs
-    // persistent whole-step decode kernel: 0 = not examined yet, 1 = usable, -1 = configuration not covered
-    bool use_persistent = false;
-    int mega_state = 0, mega_grid = 0;
-    MegaLayer *mega_layers = nullptr;
-    float *mega_ws = nullptr;
-    unsigned int *mega_sync = nullptr; // [0, 640) barrier counters, [16] abort flag, [1024, ...) attention tickets
-    int mega_lds_B = 0; // batch the kernel's LDS size was last set up for
-    size_t mega_lds = 0;
-    int mega_pitch = 0;
-    unsigned long long *mega_trace = nullptr;
-    int mega_trace_cap = 0;
 };
 
 // While one of these lives, the layers that hold first-token weights run with them.
@@ -231,94 +219,6 @@ struct FirstTokenWeights {
         }
     }
 };
-
-static void mega_invalidate(xfthip_model *m) {
-    m->mega_state = 0;
-}
-
-// Decides whether the persistent kernel covers this model and builds its per-layer table.
-static int mega_prepare(xfthip_model *m) {
-    const xfthip_model_config &c = m->cfg;
-    m->mega_state = -1;
-    if (c.kv_dtype != XFTHIP_FP16 || c.head_size != 128) return 0;
-    if (c.hidden > 8192 || c.hidden % 64 != 0 || c.intermediate % 16 != 0 || c.vocab <= 0) return 0;
-    if (!m->lm_head || m->lm_head->pw.kind != XFTHIP_W_BF16 || !m->embedding) return 0;
-    std::vector<MegaLayer> tab(c.layers);
-    for (int l = 0; l < c.layers; ++l) {
-        const LayerW &L = m->layers[l];
-        if (!L.qkv || !L.o || !L.gateup || !L.down || !L.ln1 || !L.ln2 || L.qkv_bias || L.o_bias || L.ln1_beta || L.ln2_beta) return 0;
-        const PackedWeight *w[4] = {&L.qkv->pw, &L.o->pw, &L.gateup->pw, &L.down->pw};
-        for (const PackedWeight *pw : w)
-            if (pw->kind != XFTHIP_W_INT8 || pw->zero != nullptr || pw->KT % 4 != 0) return 0;
-        MegaLayer &t = tab[l];
-        t.wqkv = w[0]->packed, t.wo = w[1]->packed, t.wgu = w[2]->packed, t.wdown = w[3]->packed;
-        t.sqkv = w[0]->scale, t.so = w[1]->scale, t.sgu = w[2]->scale, t.sdown = w[3]->scale;
-        t.kt_qkv = w[0]->KT, t.kt_o = w[1]->KT, t.kt_gu = w[2]->KT, t.kt_down = w[3]->KT;
-        t.ln1 = L.ln1, t.ln2 = L.ln2;
-        t.kv = m->caches[l]->kv;
-    }
-    if (m->lm_head->pw.KT % 4 != 0) return 0;
-    m->mega_grid = device_cu_count();
-    if (m->mega_grid < 8) return 0;
-    int kmax = c.hidden > c.intermediate ? c.hidden : c.intermediate;
-    if (c.q_heads * c.head_size > kmax) kmax = c.q_heads * c.head_size;
-    m->mega_pitch = kmax + 8;
-    m->mega_lds_B = 0;
-    if (!m->mega_layers) XFT_CHECK_HIP(hipMalloc((void **)&m->mega_layers, tab.size() * sizeof(MegaLayer)));
-    XFT_CHECK_HIP(hipMemcpy(m->mega_layers, tab.data(), tab.size() * sizeof(MegaLayer), hipMemcpyHostToDevice));
-    if (!m->mega_ws) XFT_CHECK_HIP(hipMalloc((void **)&m->mega_ws, (size_t)kWsSlots * kSlotFloats * sizeof(float)));
-    if (!m->mega_sync) {
-        XFT_CHECK_HIP(hipMalloc((void **)&m->mega_sync, (size_t)(1024 + kWsSlots) * sizeof(unsigned int)));
-        XFT_CHECK_HIP(hipMemset(m->mega_sync, 0, (size_t)(1024 + kWsSlots) * sizeof(unsigned int)));
-    }
-    m->mega_state = 1;
-    return 0;
-}
-
-// LDS of the kernel depends on the batch; returns 0 with *ok = false when it does not fit
-static int mega_fit(xfthip_model *m, int B, bool *ok) {
-    *ok = false;
-    if (m->mega_lds_B != B) {
-        const size_t lds = mega_lds_bytes(B, m->mega_pitch);
-        if (lds > (size_t)160 * 1024) return 0;
-        int per_cu = 0;
-        if (int rc = mega_decode_max_blocks(&per_cu, lds)) return rc;
-        if (per_cu < 1) return 0;
-        m->mega_lds = lds;
-        m->mega_lds_B = B;
-    }
-    *ok = true;
-    return 0;
-}
-
-static int mega_step(xfthip_model *m, int B, int position, hipStream_t st) {
-    const xfthip_model_config &c = m->cfg;
-    MegaParams p = {};
-    p.layers = m->mega_layers;
-    p.nlayers = c.layers, p.M = B, p.hidden = c.hidden, p.inter = c.intermediate, p.qH = c.q_heads, p.kvH = c.kv_heads;
-    p.x = m->x, p.q = m->qkv, p.att = m->att, p.h = m->h, p.pos = m->pos;
-    p.cosT = m->cosT, p.sinT = m->sinT;
-    p.rms_eps = c.rms_eps, p.scale = 1.0f / sqrtf((float)c.head_size);
-    p.ws = m->mega_ws, p.tickets = m->mega_sync + 1024;
-    // a unit is 8 waves: one token block of 32 per wave keeps its load chain at a single round
-    // trip, so the context is split as far as there are workgroups
-    const int nblk = (position + 1 + 31) / 32;
-    int nsplit = (nblk + 7) / 8;
-    const int room = m->mega_grid / (B * c.kv_heads);
-    nsplit = nsplit > room ? room : nsplit;
-    nsplit = nsplit < 1 ? 1 : (nsplit > 64 ? 64 : nsplit);
-    while (nsplit > 1 && (size_t)B * c.kv_heads * nsplit > (size_t)kWsSlots) --nsplit;
-    p.nsplit = nsplit;
-    p.act_pitch = m->mega_pitch;
-    p.red_off = (int)((((size_t)B * m->mega_pitch * 2) + 15) & ~(size_t)15);
-    p.embedding = m->embedding, p.ids = m->ids, p.final_norm = m->final_norm;
-    p.lm_head = m->lm_head->pw.packed, p.kt_lm = m->lm_head->pw.KT, p.vocab = c.vocab;
-    p.logits = m->logits, p.idlog = m->idlog, p.step = m->step;
-    p.counter = m->mega_sync, p.abort_flag = (int *)(m->mega_sync + 16);
-    p.spin_limit = 400000u;
-    p.trace = m->mega_trace, p.trace_cap = m->mega_trace_cap;
-    return mega_decode_launch(p, m->mega_grid, m->mega_lds, st);
-}
 
 static int upload_f32(float **dst, const float *src, size_t n) {
     if (*dst) {
@@ -621,7 +521,7 @@ int xfthip_model_destroy(xfthip_model_t m) {
         if (L.qkv_bias) (void)hipFree(L.qkv_bias);
         if (L.o_bias) (void)hipFree(L.o_bias);
     }
-    void *bufs[] = {m->w8a8_qa, m->w8a8_stat, m->gu, m->mega_trace, m->mega_layers, m->mega_ws, m->mega_sync, m->cosT, m->sinT, m->xn, m->qkv, m->att, m->h, m->x, m->xlast, m->logits, m->ids, m->pos, m->step, m->idlog,
+    void *bufs[] = {m->w8a8_qa, m->w8a8_stat, m->gu, m->cosT, m->sinT, m->xn, m->qkv, m->att, m->h, m->x, m->xlast, m->logits, m->ids, m->pos, m->step, m->idlog,
             m->embedding, m->final_norm, m->active, m->prompt_ids, m->kv_stage, m->reorder_rows};
     for (void *b : bufs)
         if (b) (void)hipFree(b);
@@ -652,7 +552,6 @@ int xfthip_model_set_attention(xfthip_model_t m, int idx, xfthip_weight_t qkv, x
         (void)hipGraphExecDestroy(m->graph);
         m->graph = nullptr;
     }
-    mega_invalidate(m);
     return 0;
 }
 
@@ -678,7 +577,6 @@ int xfthip_model_set_mlp(xfthip_model_t m, int idx, xfthip_weight_t gateup, xfth
         (void)hipGraphExecDestroy(m->graph);
         m->graph = nullptr;
     }
-    mega_invalidate(m);
     return 0;
 }
 
@@ -699,7 +597,6 @@ int xfthip_model_set_layer_norm_shifts(xfthip_model_t m, int idx, const float *l
         (void)hipGraphExecDestroy(m->graph);
         m->graph = nullptr;
     }
-    mega_invalidate(m);
     XFT_CHECK_HIP(hipDeviceSynchronize());
     if (int rc = upload_f32(&L.ln1_beta, ln1_beta_host, m->cfg.hidden)) return rc; // (a null pointer drops the shift)
     return upload_f32(&L.ln2_beta, ln2_beta_host, m->cfg.hidden);
@@ -750,7 +647,6 @@ int xfthip_model_set_head(xfthip_model_t m, const uint16_t *embedding_fp16_host,
     XFT_CHECK_HIP(hipMemcpy(m->embedding, embedding_fp16_host, eb, hipMemcpyHostToDevice));
     if (int rc = upload_f32(&m->final_norm, final_norm_host, c.hidden)) return rc;
     m->lm_head = lm_head;
-    mega_invalidate(m);
     return 0;
 }
 
@@ -830,17 +726,10 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
     // re-captured only every 128 tokens
     m->len_hint = ((m->cur_pos + steps + 127) / 128) * 128;
     const int nsplit = attention_split_count(m->len_hint < c.max_seq ? m->len_hint : c.max_seq, B * c.kv_heads);
-    bool persistent = false;
-    if (m->use_persistent && !m->ragged && B <= 4 && (size_t)B * c.kv_heads <= (size_t)kWsSlots) {
-        if (m->mega_state == 0)
-            if (int rc = mega_prepare(m)) return rc;
-        if (m->mega_state == 1)
-            if (int rc = mega_fit(m, B, &persistent)) return rc;
-    }
-    if (persistent) {
+    if (!m->use_graph) {
         for (int i = 0; i < steps; ++i)
-            if (int rc = mega_step(m, B, m->cur_pos + i, st)) return rc;
-    } else if (!m->use_graph) {
+            if (int rc = decode_step(m, B, st)) return rc;
+    } else if (!m->use_graph) {    } else if (!m->use_graph) {
         for (int i = 0; i < steps; ++i)
             if (int rc = decode_step(m, B, st)) return rc;
     } else if (m->graph == nullptr || m->graph_B != B || m->graph_stream != st || m->graph_nsplit != nsplit
@@ -877,20 +766,9 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
         m->graph_ragged = m->ragged;
         m->graph_stream = st;
     }
-    if (!persistent && m->use_graph)
+    if (m->use_graph)
         for (int i = 0; i < steps; ++i) XFT_CHECK_HIP(hipGraphLaunch(m->graph, st));
     XFT_CHECK_HIP(hipStreamSynchronize(st));
-    if (persistent) {
-        int aborted = 0;
-        XFT_CHECK_HIP(hipMemcpy(&aborted, m->mega_sync + 16, 4, hipMemcpyDeviceToHost));
-        if (aborted) {
-            // the kernel gave up at a barrier: the caches and the residual stream are unusable
-            XFT_CHECK_HIP(hipMemset(m->mega_sync, 0, (size_t)(1024 + kWsSlots) * sizeof(unsigned int)));
-            m->cur_B = 0;
-            set_error("xfthip_model_decode: the persistent decode kernel timed out at a device-wide barrier");
-            return 3;
-        }
-    }
     if (ids_out_host) {
         // the log holds the input id of every step; the outputs are rows 1..steps-1 plus the final ids
         std::vector<int> log((size_t)steps * B);
@@ -1122,33 +1000,9 @@ int xfthip_model_seq_logits(xfthip_model_t m, int row, float *logits_host) {
     return 0;
 }
 
-int xfthip_model_use_persistent(xfthip_model_t m, int enable) {
-    XFT_REQUIRE(m != nullptr, "xfthip_model_use_persistent: null model");
-    m->use_persistent = enable != 0;
-    return 0;
-}
-
-int xfthip_model_persistent_trace(xfthip_model_t m, unsigned long long *ticks_host, int capacity) {
-    XFT_REQUIRE(m && capacity >= 0, "xfthip_model_persistent_trace: bad argument");
-    const int need = 5 * m->cfg.layers + 3;
-    if (ticks_host == nullptr) {
-        // arm: later persistent steps record their barrier times
-        if (!m->mega_trace) {
-            XFT_CHECK_HIP(hipMalloc((void **)&m->mega_trace, (size_t)need * 8));
-            XFT_CHECK_HIP(hipMemset(m->mega_trace, 0, (size_t)need * 8));
-            m->mega_trace_cap = need;
-        }
-        return 0;
-    }
-    XFT_REQUIRE(m->mega_trace != nullptr, "xfthip_model_persistent_trace: tracing was not armed");
-    XFT_REQUIRE(capacity >= need, "xfthip_model_persistent_trace: capacity %d < %d entries", capacity, need);
-    XFT_CHECK_HIP(hipMemcpy(ticks_host, m->mega_trace, (size_t)need * 8, hipMemcpyDeviceToHost));
-    return 0;
-}
-
 int xfthip_model_decode_mode(xfthip_model_t m) {
     if (!m) return -1;
-    return m->mega_state == 1 && m->use_persistent ? 2 : (m->use_graph ? 1 : 0);
+    return m->use_graph ? 1 : 0;
 }
 
 int xfthip_model_use_fusion(xfthip_model_t m, int enable) {

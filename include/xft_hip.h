@@ -287,7 +287,8 @@ int xfthip_attention(xfthip_kvcache_t c, const void *q, int qStride, void *out, 
  * process ends) instead of the workspace xfthip_attention allocates on first use.  The call
  * allocates and frees nothing.  A shape whose split needs more than 1024 slots (column groups
  * B * kvHeads * ceil(S * qHeads / kvHeads / 16) times sequence splits) is rejected with an error
- * that says so.  All calls on one GPU share the array: calls that overlap on one GPU (two streams)
+ * that says so; the split rule makes at most two slots a compute unit, so that on a device of up to
+ * 512 compute units no shape is.  All calls on one GPU share the array: calls that overlap on one GPU (two streams)
  * race; calls on one stream do not.  No counterpart in the reference.
  */
 int xfthip_attention_static(xfthip_kvcache_t c, const void *q, int qStride, void *out, int oStride, int out_dtype, int B,

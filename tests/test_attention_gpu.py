@@ -157,24 +157,26 @@ def test_chunked_prefill_over_cache(xh, orc, int8):
     assert _cos(got, exp) >= 0.9999
 
 
-def test_split_count_independence(xh, orc):
-    """The same query against the same rows gives the same answer whether the cache is short
-    (one workgroup per head) or long (sequence split over many workgroups)."""
+@pytest.mark.parametrize("n,S", [(900, 1024), (4000, 4096)])
+def test_split_count_independence(xh, orc, n, S):
+    """The same query against the same rows gives the same answer whether the sequence is left whole (a large batch:
+    one workgroup per sequence and KV head) or split: 8 parts merged by the last workgroup to finish at 900 tokens,
+    32 parts merged by a launch of their own at 4000."""
     rng = np.random.default_rng(41)
-    qh, kvh, n = 32, 8, 900
+    qh, kvh = 32, 8
     rows_k = rng.standard_normal((n, kvh * D)).astype(np.float32)
     rows_v = rng.standard_normal((n, kvh * D)).astype(np.float32)
     q = orc.round_bf16(rng.standard_normal((1, qh * D)))
     outs = []
-    for B in (1, 40):  # a large batch removes the need to split
-        kc, vc = orc.KVCache(0, B, kvh, 1024, D), orc.KVCache(0, B, kvh, 1024, D)
-        for b in range(B):
-            kc.store(b, 0, rows_k)
-            vc.store(b, 0, rows_v)
-        dc = xh.KVCache(xh.FP16, B, kvh, 1024, D)
-        dc.load(0, kc.data)
-        dc.load(1, vc.data)
+    for B in (1, 40):  # 320 (sequence, KV head) pairs: more than the device has CUs, nothing is split
+        kc, vc = orc.KVCache(0, 1, kvh, S, D), orc.KVCache(0, 1, kvh, S, D)
+        kc.store(0, 0, rows_k)
+        vc.store(0, 0, rows_v)
+        dc = xh.KVCache(xh.FP16, B, kvh, S, D)
+        dc.load(0, np.repeat(kc.data, B, 0))
+        dc.load(1, np.repeat(vc.data, B, 0))
         outs.append(_attend(xh, orc, dc, np.repeat(q, B, 0), B, 1, qh, n - 1)[0])
+        dc.free()
     # probabilities are narrowed to fp16 relative to a different running max per split
     assert np.abs(outs[0] - outs[1]).max() < 1e-4
 

@@ -68,7 +68,7 @@ def test_static_scratch_attention_two_calls_in_a_row(xh, orc, int8):
     assert np.array_equal(static3, static) and np.array_equal(plain3, plain)
 
 
-def test_static_scratch_attention_prefill_and_rejection(xh, orc):
+def test_static_scratch_attention_prefill_and_widest_split(xh, orc):
     rng = np.random.default_rng(73)
     qh, kvh, B, S = 8, 2, 2, 100
     stride = (qh + 2 * kvh) * D
@@ -83,15 +83,19 @@ def test_static_scratch_attention_prefill_and_rejection(xh, orc):
         xh.synchronize()
         outs.append(od.to_numpy(np.float32, (B * S, qh * D)))
     assert np.array_equal(outs[0], outs[1])
-    # 80 sequences x 8 KV heads = 640 column groups, split in two at this length: 1280 slots > 1024
-    big = xh.KVCache(xh.FP16, 80, 8, 512, D)
-    qd = xh.DeviceBuffer(80 * 32 * D * 2)
-    qd.zero()
-    od = xh.DeviceBuffer(80 * 32 * D * 4)
-    with pytest.raises(xh.XftHipError, match="static"):
-        xh.attention_static(big, qd.ptr, 32 * D, od.ptr, 32 * D, xh.F32, 80, 1, 32, SCALE, 400)
-    xh.attention(big, qd.ptr, 32 * D, od.ptr, 32 * D, xh.F32, 80, 1, 32, SCALE, 400)  # the allocating entry point takes it
-    xh.synchronize()
+    # the widest split the library makes: 16 sequences x 8 KV heads = 128 column groups in 4 parts at 2048 tokens or
+    # more = 512 of the array's 1024 slots (with as many column groups as CUs or more, nothing is split at all)
+    big = xh.KVCache(xh.FP16, 16, 8, 2304, D)
+    for which in (0, 1):
+        big.load(which, orc.to_fp16(rng.standard_normal((16, 8, 2304, D), dtype=np.float32)))
+    qd = xh.DeviceBuffer.from_numpy(orc.to_bf16(orc.round_bf16(rng.standard_normal((16, 32 * D)))))
+    wide = []
+    for fn in (xh.attention, xh.attention_static):
+        od = xh.DeviceBuffer(16 * 32 * D * 4)
+        fn(big, qd.ptr, 32 * D, od.ptr, 32 * D, xh.F32, 16, 1, 32, SCALE, 2200)
+        xh.synchronize()
+        wide.append(od.to_numpy(np.float32, (16, 32 * D)))
+    assert np.array_equal(wide[0], wide[1])
 
 
 def test_static_scratch_attention_records_into_a_graph(xh, orc):

@@ -40,6 +40,13 @@ __global__ __launch_bounds__(256, 3) void attn_kernel(AttnParams p) {
     attn_unit<INT8, 4, PIPE>(p, blockIdx.x, blockIdx.y % p.kv.H, blockIdx.y / p.kv.H, blockIdx.z, lds, [] { __syncthreads(); });
 }
 
+constexpr int kTicketParts = 8, kMaxParts = 32;
+// merges the parts of a launch of attn_kernel that took no tickets: grid (columns of a group, groups), at most 128 parts
+__global__ __launch_bounds__(128) void attn_merge_kernel(AttnParams p) {
+    __shared__ float s_pm[128], s_f[128];
+    attn_merge_unit(p, blockIdx.y, blockIdx.x, s_pm, s_f);
+}
+
 // 32 x 32 MFMA tiles, 32 columns a wave, K / V blocks shared through LDS (attention_prefill.h); two workgroups a CU
 // Workgroups are handed to the 8 XCDs in turn by their linear index, and each XCD has an L2 of its own: the
 // (sequence, KV head) pairs are dealt to the XCDs (pair = 8 k + XCD), and an XCD walks the column groups of one
@@ -159,9 +166,8 @@ int xfthip::attention_launch(xfthip_kvcache_t c, const void *q, int qStride, voi
             return 0;
         }
     }
-    // split the KV sequence so that the launch has ~4 workgroups per CU, each wave keeping at
-    // least one 32-token block; the longest visible sequence is bounded by the cache length
-    // when the real one lives in device memory
+    // split the KV sequence so that the launch has about one workgroup a CU (attention_split_count); the longest
+    // visible sequence is bounded by the cache length when the real one lives in device memory
     const int len = past_dev ? ((len_hint > 0 && len_hint < c->maxSeq) ? len_hint : c->maxSeq) : past + S;
     const int wgs = B * c->kv.H * p.CG;
     int nsplit = attention_split_count(len, wgs);
@@ -180,7 +186,10 @@ int xfthip::attention_launch(xfthip_kvcache_t c, const void *q, int qStride, voi
     }
     p.nsplit = nsplit;
     p.ws = wsp ? wsp->ws : nullptr;
-    p.tickets = wsp ? wsp->tickets : nullptr;
+    // up to kTicketParts parts the last workgroup of a column group merges them; beyond, a second launch does (8 KV
+    // heads, 2048 tokens, 16 parts: 11.7 us merged by the last workgroup, 10.2 by the launch; 4096 tokens 13.7 / 12.7)
+    const bool merge_launch = nsplit > kTicketParts;
+    p.tickets = (wsp && !merge_launch) ? wsp->tickets : nullptr;
     dim3 grid(nsplit, c->kv.H * p.CG, B);
     // more than one 32-token block a wave somewhere: the form that requests blocks ahead
     const bool pipe = (len + 31) / 32 > 4 * nsplit;
@@ -191,21 +200,30 @@ int xfthip::attention_launch(xfthip_kvcache_t c, const void *q, int qStride, voi
         if (pipe) hipLaunchKernelGGL((attn_kernel<false, true>), grid, dim3(256), 0, stream, p);
         else hipLaunchKernelGGL((attn_kernel<false, false>), grid, dim3(256), 0, stream, p);
     }
+    if (merge_launch) {
+        const int cols = S * p.G < 16 ? S * p.G : 16;
+        hipLaunchKernelGGL(attn_merge_kernel, dim3(cols, wgs), dim3(128), 0, stream, p);
+    }
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }
 
 int xfthip::attention_split_count(int len, int units) {
-    // Three workgroups a CU are resident.  Every wave keeps at least one 32-token block, two once the sequence is
-    // longer than 1024 tokens (the next block then travels behind the current one), and at most 16 parts are made: the
-    // last workgroup of a column group merges all its parts alone, which at 64 parts cost more than the split gained
-    // (batch 1, 8 KV heads, 16384 tokens: 30.2 us with 64 parts, 22.1 with 16; 4096 tokens 15.8 -> 13.1; 32 KV heads,
-    // 2048 tokens 13.2 -> 11.0).
+    // Measured over batch 1 .. 64, 8 and 32 KV heads, 512 .. 16384 tokens, both cache kinds: a launch is fastest with
+    // about one workgroup a CU.  With at least that many (batch, KV head, column group) units nothing is split, and the
+    // partials, tickets and merge fall away with it (64 sequences x 8 KV heads x 512 tokens: 35 -> 27 us FP16, 26 ->
+    // 17 us INT8, against two parts); below, the sequence is cut into CUs / units parts, twice that where this gives
+    // at most 4 parts and the sequence has 2048 tokens or more (16 x 8 KV heads x 4096 tokens INT8: 37.5 us with 2
+    // parts, 32.8 with 4), every wave keeping at least one 32-token block, 32 parts at most (batch 1, 8 KV heads,
+    // 16384 tokens: 23.0 us with 16 parts, 20.2 with 32, 23.0 with 64; INT8 21.6 / 16.2 / 16.9).
     const int nblk = (len + 31) / 32;
-    int nsplit = (3 * device_cu_count() + units - 1) / units;
-    const int cap = nblk <= 32 ? (nblk + 3) / 4 : (nblk + 7) / 8;
+    const int cus = device_cu_count();
+    if (units >= cus) return 1;
+    int nsplit = cus / units;
+    if (nsplit <= 4 && nblk >= 64) nsplit *= 2;
+    const int cap = (nblk + 3) / 4;
     if (nsplit > cap) nsplit = cap;
-    if (nsplit > 16) nsplit = 16;
+    if (nsplit > kMaxParts) nsplit = kMaxParts;
     if (nsplit < 1) nsplit = 1;
     while (nsplit > 1 && (size_t)units * nsplit > (size_t)kWsSlots) --nsplit;
     return nsplit;

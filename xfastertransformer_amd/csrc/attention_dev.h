@@ -34,7 +34,7 @@ struct AttnParams {
     const int *past_dev;
     int nsplit, CG;
     float *ws;
-    unsigned int *tickets; // one per (batch, kv head, column group), zero between launches
+    unsigned int *tickets; // one per (batch, kv head, column group), zero between launches; null: the parts are merged by a launch of their own
 };
 
 // 4 int8 -> 2 x (2 fp16), exact: (q ^ 0x80) | 0x6400 is 1152 + q, then subtract 1152
@@ -336,7 +336,7 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
             }
         }
     }
-    if (p.nsplit == 1) return;
+    if (p.nsplit == 1 || p.tickets == nullptr) return; // no tickets: a launch of attn_merge_unit follows
 
     // ---- the workgroup that finishes last merges the splits of its column group ----
     // (no waiting: every workgroup publishes its partial, takes a ticket and leaves; the one
@@ -357,9 +357,19 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
     float *s_pm = s_linv + 16, *s_pl = s_pm + 64 * 16; // [nsplit][16] partial maxima and sums
     // one load per thread (independent round trips), then the per-column arithmetic from LDS
     // (up to 8 a thread at 64 splits: all sent before the first is used)
+    // (at up to 8 parts this thread's first output is requested in the same round trip: with one query
+    // row a KV head, the decode step of a single sequence, that is the whole merge)
+    constexpr int EARLY = 8;
+    const bool early = p.nsplit <= EARLY && (int)threadIdx.x < 16 * D && cg * 16 + (int)threadIdx.x / D < ncols;
+    float t_early[EARLY];
     {
         constexpr int PER = 64 * 32 / (64 * NW) > 0 ? 64 * 32 / (64 * NW) : 1;
         float x[PER];
+        if (early) {
+#pragma unroll
+            for (int u = 0; u < EARLY; ++u)
+                t_early[u] = u < p.nsplit ? ws_ld(&base[(size_t)u * kSlotFloats + 32 + threadIdx.x]) : 0.0f;
+        }
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
             const int v = threadIdx.x + i * 64 * NW;
@@ -396,6 +406,11 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
         const int cc = cg * 16 + col;
         if (cc >= ncols) continue;
         float acc = 0.0f;
+        if (early && v == (int)threadIdx.x) {
+#pragma unroll
+            for (int u = 0; u < EARLY; ++u)
+                if (u < p.nsplit) acc = fmaf(t_early[u], s_f[u * 16 + col], acc);
+        } else
         // 32 partials in flight a thread (4 made the merge of 64 splits a chain of 16 round trips per output)
         for (int s0 = 0; s0 < p.nsplit; s0 += 32) {
             float t[32];
@@ -415,6 +430,51 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
 }
 
 
+
+// Merge of the parts of one column as a launch of its own (more than 16 parts: the last workgroup of a column
+// group merging them alone would take longer than the finer split saves).  One 128-thread workgroup a column,
+// one thread a dim; same arithmetic and order over the parts as the in-kernel merge above.
+__device__ inline void attn_merge_unit(const AttnParams &p, const int group, const int col, float *s_pm, float *s_f) {
+    constexpr int D = 128;
+    const int cg = group % p.CG, kvh = (group / p.CG) % p.kv.H, b = group / (p.CG * p.kv.H);
+    const int cc = cg * 16 + col, d = threadIdx.x;
+    if (cc >= p.S * p.G) return; // uniform over the workgroup
+    const float *base = p.ws + (size_t)group * p.nsplit * kSlotFloats;
+    float pm = kNegBig, pl = 0.0f;
+    if (d < p.nsplit) {
+        pm = ld_dev(&base[(size_t)d * kSlotFloats + col]);
+        pl = ld_dev(&base[(size_t)d * kSlotFloats + 16 + col]);
+    }
+    float acc = 0.0f;
+    for (int s0 = 0; s0 < p.nsplit; s0 += 32) {
+        float t[32];
+#pragma unroll
+        for (int u = 0; u < 32; ++u) t[u] = s0 + u < p.nsplit ? ld_dev(&base[(size_t)(s0 + u) * kSlotFloats + 32 + col * D + d]) : 0.0f;
+        if (s0 == 0) {
+            // factors of all parts (the loads above are in flight meanwhile)
+            s_pm[d] = pm;
+            __syncthreads();
+            float m = kNegBig;
+            for (int s = 0; s < p.nsplit; ++s) m = fmaxf(m, s_pm[s]);
+            __syncthreads();
+            s_f[d] = fast_exp(pm - m);
+            s_pm[d] = pl;
+            __syncthreads();
+        }
+#pragma unroll
+        for (int u = 0; u < 32; ++u)
+            if (s0 + u < p.nsplit) acc = fmaf(t[u], s_f[s0 + u], acc);
+    }
+    float l = 0.0f;
+    for (int s = 0; s < p.nsplit; ++s) l += s_pm[s] * s_f[s];
+    const float r = acc * (1.0f / l);
+    const int s_tok = cc / p.G, j = cc % p.G;
+    const size_t idx = ((size_t)b * p.S + s_tok) * p.oStride + (size_t)(kvh * p.G + j) * D + d;
+    if (p.out_dtype == XFTHIP_BF16)
+        st_dev((uint16_t *)p.out + idx, f32_to_bf16_ref(r));
+    else
+        store_from_f32(p.out, p.out_dtype, idx, r);
+}
 
 // Exchange with the lanes 16 / 32 away (the other lane groups holding the same column) through the gfx950
 // lane-swap instructions: unlike __shfl_xor (ds_bpermute) they do not go through the LDS pipeline, whose

@@ -54,7 +54,13 @@ union HFrag32 {
 // fences) was built for both CT: correct, but 41 (CT = 1) and 182 (CT = 2) registers short, and the spill traffic
 // shares the counter of the block prefetch, so every reload waited for it: 542 and 1560 us.  Requesting blocks two
 // steps ahead, 8-wave workgroups and touching the pair's cache lines on arrival (L2 warm-up) each changed nothing:
-// global latency and barriers are not what the waves wait for.
+// global latency and barriers are not what the waves wait for.  The LDS port itself, measured with a kernel of
+// nothing but conflict-free 128-bit reads: 7.2 ns a wave-read a CU (about 140 bytes/ns; 64- and 32-bit reads move
+// 75 - 80), so the 16 KB a wave reads per block put a floor of about 150 us under this shape.  Taking the value
+// operands straight from the cache instead (they are laid out as the MFMA wants them; one block ahead, into the
+// registers the products have just read: 209 registers) to share the bytes between the LDS port and the vector
+// memory pipeline ran 262 us: a lane's 16 bytes lie 64 bytes from its neighbour's, and the memory pipeline serves
+// such a load line by line.
 template <int NW, int CT, bool INT8>
 __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, const int cgroup, const int b, unsigned char *lds) {
     constexpr int D = 128, NT = NW * 64, WC = 32 * CT;

@@ -107,6 +107,17 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
     // (the same for every lane of a wave: scalar values, so that the loop and its load branches are uniform)
     const int blk_begin = __builtin_amdgcn_readfirstlane(wg_begin + wave * wbase + (wave < wrem ? wave : wrem));
     const int blk_end = __builtin_amdgcn_readfirstlane(blk_begin + wbase + (wave < wrem ? 1 : 0));
+    // A wave walks its blocks from a starting point of its own and wraps around (the online softmax does not care
+    // about the order).  With a cache whose rows per head are a power of two long, the waves of all heads and parts
+    // would otherwise be at the same offset modulo the memory channels' stripe at every step, on a fraction of the
+    // channels (16 sequences x 8 KV heads x 4096 tokens in a cache of 16384: 67.5 us in step, 54 us staggered; INT8
+    // 41.6 / 35.7).  The pipelined INT8 form sits at its register limit and spills with the two scalars more that
+    // this takes (33 -> 37 us on the same shape in a cache of 4096): it keeps the plain order.
+    constexpr bool STAGGER = !(INT8 && PIPE);
+    const int wblk = blk_end - blk_begin;
+    const int rot = STAGGER
+            ? __builtin_amdgcn_readfirstlane(wblk > 1 ? (int)((unsigned)((b * p.kv.H + kvh) * 5 + split * 3 + wave) % (unsigned)wblk) : 0)
+            : 0;
 
     const size_t bh = (size_t)b * p.kv.H + kvh;
     const ATTN_GLOBAL char *kbase = (const ATTN_GLOBAL char *)p.kv.k + bh * p.kv.S * D * (INT8 ? 1 : 2);
@@ -176,8 +187,8 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
         }
     }
     if (blk_begin < blk_end) {
-        load_keys(blk_begin);
-        load_values(blk_begin);
+        load_keys(blk_begin + rot);
+        load_values(blk_begin + rot);
     }
 #pragma unroll
     for (int s = 0; s < 4; ++s)
@@ -192,10 +203,13 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
 #pragma unroll
     for (int i = 0; i < 8; ++i) o[i] = f32x4 {0.f, 0.f, 0.f, 0.f};
 
-    for (int blk = blk_begin; blk < blk_end; ++blk) {
+    // (one loop for both orders; in the plain order `bi` is dead and the conditions are those of a loop over blk)
+    for (int bi = 0, blk = blk_begin + rot; STAGGER ? bi < wblk : blk < blk_end; ++bi) {
+        const auto more = [&] { return STAGGER ? bi + 1 < wblk : blk + 1 < blk_end; };
+        const auto next = [&] { return (STAGGER && blk + 1 == blk_end) ? blk_begin : blk + 1; };
         const int t0 = blk << 5;
         if constexpr (!PIPE) {
-            if (blk != blk_begin) {
+            if (STAGGER ? bi != 0 : blk != blk_begin) {
                 load_keys(blk);
                 load_values(blk);
             }
@@ -234,7 +248,7 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
             }
         if constexpr (PIPE) {
             __builtin_amdgcn_sched_barrier(0);
-            if (blk + 1 < blk_end) load_keys(blk + 1);
+            if (more()) load_keys(next());
             __builtin_amdgcn_sched_barrier(0);
         }
         // column max across the 4 lane groups
@@ -287,9 +301,10 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
         }
         if constexpr (PIPE) {
             __builtin_amdgcn_sched_barrier(0);
-            if (blk + 1 < blk_end) load_values(blk + 1);
+            if (more()) load_values(next());
             __builtin_amdgcn_sched_barrier(0);
         }
+        blk = next();
     }
 
     // ---- merge the 4 waves in LDS ----

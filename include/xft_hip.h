@@ -503,10 +503,22 @@ int xfthip_moe_top2(const float *logits, int M, int E, int *sel, float *weights,
  */
 int xfthip_moe_create(int hidden, int intermediate, int experts, int max_tokens, const float *router_host, const float *ln_host,
         xfthip_moe_t *out);
+/* A further sparse MLP of the same shape that works in the per-call buffers of `first` (the layers of one model run
+ * one after the other on one stream): only the router, the norm weight and the experts' table are its own.  `first`
+ * must outlive it. */
+int xfthip_moe_create_beside(xfthip_moe_t first, const float *router_host, const float *ln_host, xfthip_moe_t *out);
+int xfthip_moe_shape(xfthip_moe_t m, int *hidden, int *intermediate, int *experts, int *max_tokens);
 int xfthip_moe_destroy(xfthip_moe_t m);
 int xfthip_moe_set_expert(xfthip_moe_t m, int e, xfthip_weight_t gateup, xfthip_weight_t down);
 int xfthip_moe_forward(xfthip_moe_t m, const float *x_in, int in_stride, float *x_out, int out_stride, int tokens, int do_norm,
         const float *logits_override, int *sel_host_out, float *w_host_out, xfthip_stream_t stream);
+/*
+ * Layer idx of a model takes this sparse MLP in place of its gate/up/down weights (set its attention half with
+ * xfthip_model_set_attention): the layer of MixtralLLM (src/models/mixtral.h:25-54: CommonDecoder over Attention +
+ * MixtralMLP).  The object must have been created for at least the model's max_tokens and outlive the model; prompt
+ * pass, decode steps (graph replay included) and the per-sequence entry points run it like any other layer.
+ */
+int xfthip_model_set_moe(xfthip_model_t m, int idx, xfthip_moe_t moe);
 
 #ifdef __cplusplus
 }

@@ -406,8 +406,11 @@ class LlamaLayerOracle:
 
     def __init__(self, hidden, inter, q_heads, kv_heads, head, wqkv, wo, wgateup, wdown, ln1, ln2, kv_int8=0,
                  batch=1, max_seq=256, eps=1e-6, rope_base=10000, max_pos=2048, rounding="fp32", gemm="oracle",
-                 prefill_attention="flash", ln1_beta=None, ln2_beta=None):
+                 prefill_attention="flash", ln1_beta=None, ln2_beta=None, moe=None):
         self.hidden, self.inter, self.qh, self.kvh, self.D = hidden, inter, q_heads, kv_heads, head
+        # moe = (router fp32 [hidden, experts], [(gateup, down) per expert]): the layer of MixtralLLM
+        # (src/models/mixtral.h:25-54), whose MLP half is MixtralMLP; wgateup / wdown are then unused
+        self.moe = moe
         # shifts given: the layer built over LayerNorm instead of RmsNorm (NormType::LN, decoder_layer.cpp:179-181)
         self.ln1_beta = None if ln1_beta is None else f32(ln1_beta)
         self.ln2_beta = None if ln2_beta is None else f32(ln2_beta)
@@ -462,6 +465,8 @@ class LlamaLayerOracle:
             att = cross_attn_by_head(q, k, v, self.qh, self.kvh, self.D, [S] * B, [past] * B, scale, self.kc, self.vc)
         att = self._r(att)
         x1 = self._mm(self.wo, att, epi=EPI_RESIDENTIAL, res=x)
+        if self.moe is not None:
+            return mixtral_mlp(x1, self.ln2, self.moe[0], self.moe[1], rounding=self.rounding)[0]
         xn2 = self._r(rmsnorm(x1, self.ln2, 1e-6) if self.ln2_beta is None else layernorm(x1, self.ln2, self.ln2_beta, 1e-6))
         h = self._r(silu_sum(self._mm(self.wgateup, xn2)))
         return self._mm(self.wdown, h, epi=EPI_RESIDENTIAL, res=x1)
@@ -504,8 +509,9 @@ def mixtral_mlp(x, ln, router, experts, logits_override=None, do_norm=True, roun
         order = np.argsort(rows, kind="stable")
         rows, slot = rows[order], slot[order]
         xe = np.ascontiguousarray(xn[rows])
-        h = r(silu_sum(qgemm(gu, xe)))
-        eo = qgemm(dn, h)
+        mm = lambda w, a: qgemm(w, a) if isinstance(w, QWeight) else gemm_f32(a, w)  # (plain fp32 / bf16-valued experts)
+        h = r(silu_sum(mm(gu, xe)))
+        eo = mm(dn, h)
         idx = i32(rows)
         wt = f32(w[rows, slot])
         lib.orc_scatter_add(p(out), out.shape[1], p(f32(eo)), out.shape[1], p(idx), p(wt), rows.size)

@@ -11,6 +11,12 @@ shapes: src/layers/decoder_block.h:205-343, common_decoder.h:857-874, llama.cpp:
     model.layers.N.{input,post_attention}_layernorm.weight.bin  [hidden]
     model.final_layernorm.weight.bin            [hidden]
     model.lm_head.weight.bin                    [vocab, hidden]
+  a Mixtral directory (`experts=8`; section [mixtral], src/xfastertransformer/tools/mixtral_convert.py:120-160,
+  src/layers/decoder_block.h:640-676) holds instead of the three mlp matrices
+    model.layers.N.moe.gate.weight.bin                      [hidden, experts]   (the router)
+    model.layers.N.moe.sparse_experts.E.w1.0.bin            [hidden, inter]     (gate)
+    model.layers.N.moe.sparse_experts.E.w2.0.bin            [hidden, inter]     (up)
+    model.layers.N.moe.sparse_experts.E.w3.0.bin            [inter, hidden]     (down)
   pre-quantised directories hold .qweight.0.bin (int8, or two 4-bit codes per byte with the even
   column in the low nibble) + .scales.0.bin + .zeros.0.bin (fp32 per output column) instead of
   .weight.0.bin.
@@ -66,12 +72,13 @@ def _quantize(w, quant):
     return q, scale, zero
 
 
-def write_model_dir(out, cfg=None, seed=0, weight_type="fp32", quant=None):
+def write_model_dir(out, cfg=None, seed=0, weight_type="fp32", quant=None, experts=0):
     cfg = dict(TINY if cfg is None else cfg)
+    assert not (experts and quant), "pre-quantised Mixtral directories are not written here"
     os.makedirs(out, exist_ok=True)
     L, H, I, qh, kvh, D, V = (cfg[k] for k in ("layers", "hidden", "inter", "heads", "kv_heads", "head", "vocab"))
     with open(os.path.join(out, "config.ini"), "w") as f:
-        f.write("[llama]\n")
+        f.write("[mixtral]\n" if experts else "[llama]\n")
         f.write("model_name = fixture\n")
         f.write(f"head_num = {qh}\nkv_head_num = {kvh}\nsize_per_head = {D}\ninter_size = {I}\n")
         f.write(f"max_pos_seq_len = {cfg['max_pos']}\nnum_layer = {L}\nlayernorm_eps = {cfg['eps']}\n")
@@ -79,6 +86,10 @@ def write_model_dir(out, cfg=None, seed=0, weight_type="fp32", quant=None):
         f.write(f"rope_theta = {cfg['rope_theta']}\nhas_post_decoder_layernorm = 1\nvocab_size = {V}\n")
         f.write("start_id = 1\nend_id = 2\n")
         f.write(f"weight_data_type = {weight_type}\n")
+        if experts:
+            f.write("attn_params_type = GQAttnParams\nffn_params_type = MixtralFFNParams\n")
+            if experts != 8:
+                f.write(f"sparse_experts = {experts}\n")
         if quant:
             f.write(f"quant_qweight_data_type = {quant}\nquant_scales_data_type = fp32\nquant_zeros_data_type = fp32\n")
             f.write("quant_groupsize = -1\n")
@@ -103,9 +114,19 @@ def write_model_dir(out, cfg=None, seed=0, weight_type="fp32", quant=None):
         lay = {}
         lay["qkv"] = matrix(l, "attention.query_key_value", H, (qh + 2 * kvh) * D, 0.05)
         lay["o"] = matrix(l, "attention.dense", qh * D, H, 0.05)
-        lay["gate"] = matrix(l, "mlp.gate_proj", H, I, 0.05)
-        lay["up"] = matrix(l, "mlp.up_proj", H, I, 0.05)
-        lay["down"] = matrix(l, "mlp.down_proj", I, H, 0.05)
+        if experts:
+            lay["router"] = _store(os.path.join(out, f"model.layers.{l}.moe.gate.weight.bin"),
+                                   rng.standard_normal((H, experts)) * 0.2, weight_type)
+            lay["experts"] = []
+            for e in range(experts):
+                base = os.path.join(out, f"model.layers.{l}.moe.sparse_experts.{e}.")
+                lay["experts"].append({"gate": _store(base + "w1.0.bin", rng.standard_normal((H, I)) * 0.05, weight_type),
+                                       "up": _store(base + "w2.0.bin", rng.standard_normal((H, I)) * 0.05, weight_type),
+                                       "down": _store(base + "w3.0.bin", rng.standard_normal((I, H)) * 0.05, weight_type)})
+        else:
+            lay["gate"] = matrix(l, "mlp.gate_proj", H, I, 0.05)
+            lay["up"] = matrix(l, "mlp.up_proj", H, I, 0.05)
+            lay["down"] = matrix(l, "mlp.down_proj", I, H, 0.05)
         lay["ln1"] = _store(os.path.join(out, f"model.layers.{l}.input_layernorm.weight.bin"),
                             1.0 + 0.1 * rng.standard_normal(H), weight_type)
         lay["ln2"] = _store(os.path.join(out, f"model.layers.{l}.post_attention_layernorm.weight.bin"),
@@ -124,6 +145,7 @@ if __name__ == "__main__":
     ap.add_argument("--weight-type", default="fp32", choices=["fp32", "fp16", "bf16"])
     ap.add_argument("--quant", default=None, choices=["int8", "uint4"])
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--experts", type=int, default=0, help="8: a Mixtral directory")
     a = ap.parse_args()
-    write_model_dir(a.out, None, a.seed, a.weight_type, a.quant)
+    write_model_dir(a.out, None, a.seed, a.weight_type, a.quant, a.experts)
     print("wrote", a.out)

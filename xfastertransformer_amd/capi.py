@@ -409,6 +409,14 @@ class Model:
         check(lib.xfthip_model_set_layer(self.h, idx, qkv.h, o.h, gateup.h, down.h, _hp(ln1), _hp(ln2), _hp(qkv_bias),
                                          _hp(o_bias)))
 
+    def set_sparse_layer(self, idx, qkv, o, moe, ln1, qkv_bias=None, o_bias=None):
+        """Layer idx = attention half + a sparse MLP (capi.MoE created with its own norm weight)."""
+        self._keep += [qkv, o, moe]
+        f = lambda a: None if a is None else np.ascontiguousarray(a, np.float32)
+        ln1, qkv_bias, o_bias = f(ln1), f(qkv_bias), f(o_bias)
+        check(lib.xfthip_model_set_attention(self.h, idx, qkv.h, o.h, _hp(ln1), _hp(qkv_bias), _hp(o_bias)))
+        check(lib.xfthip_model_set_moe(self.h, idx, moe.h))
+
     def set_first_token_weights(self, idx, qkv, o, gateup, down):
         """A second weight set of layer idx for the prompt pass only (None x 4 drops it)."""
         ws = [qkv, o, gateup, down]
@@ -550,14 +558,18 @@ def gemm_w8a8(w, M, qa, ldq, s, z, sm, C_dev, ldc, c_dtype=F32, epi=EPI_NONE, bi
 
 # ---------------------------------------------------------------------------- Mixtral MoE
 class MoE:
-    def __init__(self, hidden, inter, experts, max_tokens, router, ln=None):
+    def __init__(self, hidden, inter, experts, max_tokens, router, ln=None, beside=None):
+        """beside: another MoE of the same shape whose per-call buffers this one works in (layers of one model)."""
         self.hidden, self.inter, self.E = hidden, inter, experts
         router = np.ascontiguousarray(router, np.float32)
         ln = None if ln is None else np.ascontiguousarray(ln, np.float32)
         h = C.c_void_p()
-        check(lib.xfthip_moe_create(hidden, inter, experts, max_tokens, _hp(router), _hp(ln), C.byref(h)))
+        if beside is None:
+            check(lib.xfthip_moe_create(hidden, inter, experts, max_tokens, _hp(router), _hp(ln), C.byref(h)))
+        else:
+            check(lib.xfthip_moe_create_beside(beside.h, _hp(router), _hp(ln), C.byref(h)))
         self.h = h
-        self._keep = []
+        self._keep = [beside]
 
     def set_expert(self, e, gateup, down):
         self._keep += [gateup, down]

@@ -437,7 +437,13 @@ struct ModelImpl {
         xfthip_weight_t qkv = nullptr, o = nullptr, gateup = nullptr, down = nullptr;
         xfthip_weight_t firstQkv = nullptr, firstO = nullptr, firstGateup = nullptr, firstDown = nullptr;
         std::vector<float> ln1, ln2, qkvBias, oBias;
+        // [mixtral] directories: the router [hidden, experts] and every expert's gate/up and down weights
+        // (MixtralFFNParams, decoder_block.h:640-676); gateup / down above stay empty
+        std::vector<float> router;
+        std::vector<xfthip_weight_t> expertGateup, expertDown;
     };
+    int experts = 0; // sparse_experts of a [mixtral] section, 0 for a dense model
+    std::vector<xfthip_moe_t> moe; // one per layer, rebuilt with the device model (their buffers are sized by its token capacity)
     std::vector<Layer> L;
     std::vector<uint16_t> embedding;
     std::vector<float> finalNorm;
@@ -518,10 +524,23 @@ struct ModelImpl {
 
     ~ModelImpl() {
         if (model) xfthip_model_destroy(model);
-        for (auto &l : L)
+        drop_moe();
+        for (auto &l : L) {
             for (xfthip_weight_t w : {l.qkv, l.o, l.gateup, l.down, l.firstQkv, l.firstO, l.firstGateup, l.firstDown})
                 if (w) xfthip_weight_destroy(w);
+            for (xfthip_weight_t w : l.expertGateup)
+                if (w) xfthip_weight_destroy(w);
+            for (xfthip_weight_t w : l.expertDown)
+                if (w) xfthip_weight_destroy(w);
+        }
         if (lmHead) xfthip_weight_destroy(lmHead);
+    }
+
+    // the sparse MLPs work in the first one's buffers: the others go first
+    void drop_moe() {
+        for (size_t i = moe.size(); i-- > 0;)
+            if (moe[i]) xfthip_moe_destroy(moe[i]);
+        moe.clear();
     }
 
     std::string layer_file(int l, const std::string &name) const { return path + "/model.layers." + std::to_string(l) + "." + name; }
@@ -585,17 +604,31 @@ struct ModelImpl {
                 printf("The model directory holds a two-matrix MLP (dense_h_to_4h); only gate/up/down MLPs are served.\n");
                 exit(-1);
             }
-            {
+            if (experts > 0) {
+                // loadMixtralFFNWeights (decoder_block.h:640-676): w1 = gate, w2 = up, w3 = down, all [in, out]
+                y.router = read_floats(layer_file(l, "moe.gate.weight.bin"), (size_t)hidden * experts, fileType);
+                for (int e = 0; e < experts; ++e) {
+                    const std::string stem = "moe.sparse_experts." + std::to_string(e) + ".";
+                    HostMatrix gate, up, down;
+                    gate.K = up.K = hidden, gate.N = up.N = inter, down.K = inter, down.N = hidden;
+                    gate.w = read_floats(layer_file(l, stem + "w1.0.bin"), (size_t)hidden * inter, fileType);
+                    up.w = read_floats(layer_file(l, stem + "w2.0.bin"), (size_t)hidden * inter, fileType);
+                    down.w = read_floats(layer_file(l, stem + "w3.0.bin"), (size_t)inter * hidden, fileType);
+                    HostMatrix gu = hcat({&gate, &up});
+                    y.expertGateup.push_back(to_device(gu, XFTHIP_WF_GATEUP));
+                    y.expertDown.push_back(to_device(down, XFTHIP_WF_NONE));
+                }
+            } else {
                 HostMatrix gate = load_matrix(l, "mlp.gate_proj", hidden, inter);
                 HostMatrix up = load_matrix(l, "mlp.up_proj", hidden, inter);
                 HostMatrix gu = hcat({&gate, &up});
                 // the W8A8 path runs gate/up as one plain GEMM followed by silu(gate) * up
                 y.gateup = to_device(gu, wkind == XFTHIP_W_W8A8 ? XFTHIP_WF_NONE : XFTHIP_WF_GATEUP);
                 if (mixed) y.firstGateup = to_device(gu, firstKind == XFTHIP_W_W8A8 ? XFTHIP_WF_NONE : XFTHIP_WF_GATEUP, firstKind);
+                HostMatrix down = load_matrix(l, "mlp.down_proj", inter, hidden);
+                y.down = to_device(down, XFTHIP_WF_NONE);
+                if (mixed) y.firstDown = to_device(down, XFTHIP_WF_NONE, firstKind);
             }
-            HostMatrix down = load_matrix(l, "mlp.down_proj", inter, hidden);
-            y.down = to_device(down, XFTHIP_WF_NONE);
-            if (mixed) y.firstDown = to_device(down, XFTHIP_WF_NONE, firstKind);
             y.ln1 = read_floats(layer_file(l, "input_layernorm.weight.bin"), hidden, fileType);
             y.ln2 = read_floats(layer_file(l, "post_attention_layernorm.weight.bin"), hidden, fileType);
             y.qkvBias = read_floats(layer_file(l, "attention.query_key_value.bias.0.bin"), qkvCols, fileType, false);
@@ -630,6 +663,7 @@ struct ModelImpl {
         if (!grow) return;
         if (model) CK(xfthip_model_destroy(model));
         model = nullptr;
+        drop_moe();
         cfg.layers = layers, cfg.hidden = hidden, cfg.intermediate = inter;
         cfg.q_heads = heads, cfg.kv_heads = kvHeads, cfg.head_size = headSize;
         cfg.vocab = vocab;
@@ -643,6 +677,20 @@ struct ModelImpl {
         CK(xfthip_model_create(&cfg, &model));
         for (int l = 0; l < layers; ++l) {
             Layer &y = L[l];
+            if (experts > 0) {
+                // MixtralLLM's layer: the attention half and a sparse MLP that carries the post-attention norm weight
+                CK(xfthip_model_set_attention(model, l, y.qkv, y.o, y.ln1.data(), y.qkvBias.empty() ? nullptr : y.qkvBias.data(),
+                        y.oBias.empty() ? nullptr : y.oBias.data()));
+                xfthip_moe_t sparse = nullptr;
+                if (moe.empty())
+                    CK(xfthip_moe_create(hidden, inter, experts, cfg.max_tokens, y.router.data(), y.ln2.data(), &sparse));
+                else
+                    CK(xfthip_moe_create_beside(moe[0], y.router.data(), y.ln2.data(), &sparse));
+                moe.push_back(sparse);
+                for (int e = 0; e < experts; ++e) CK(xfthip_moe_set_expert(sparse, e, y.expertGateup[e], y.expertDown[e]));
+                CK(xfthip_model_set_moe(model, l, sparse));
+                continue;
+            }
             CK(xfthip_model_set_layer(model, l, y.qkv, y.o, y.gateup, y.down, y.ln1.data(), y.ln2.data(),
                     y.qkvBias.empty() ? nullptr : y.qkvBias.data(), y.oBias.empty() ? nullptr : y.oBias.data()));
             if (y.firstQkv) CK(xfthip_model_set_first_token_weights(model, l, y.firstQkv, y.firstO, y.firstGateup, y.firstDown));
@@ -1475,8 +1523,14 @@ AutoModel::AutoModel(std::string modelPath, xft::DataType dataType, xft::DataTyp
         default: break; // fp8_e4m3 and unknown
     }
     const bool kvOk = KVCacheDataType == xft::DataType::fp16 || KVCacheDataType == xft::DataType::int8;
-    if (Ini::lower(sec) != "llama" || wkind < 0 || !kvOk) {
+    const bool mixtral = Ini::lower(sec) == "mixtral";
+    if ((Ini::lower(sec) != "llama" && !mixtral) || wkind < 0 || !kvOk) {
         printf("Unsupported data type or KV cache data type: %s\n", modelKey.c_str());
+        exit(-1);
+    }
+    if (mixtral && (firstKind >= 0 || wkind == XFTHIP_W_W8A8)) {
+        // (the experts run the weight-only GEMMs with the fused SwiGLU; one weight set)
+        printf("Unsupported data type for a sparse-MLP model: %s\n", modelKey.c_str());
         exit(-1);
     }
 
@@ -1501,6 +1555,7 @@ AutoModel::AutoModel(std::string modelPath, xft::DataType dataType, xft::DataTyp
     s.hidden = (int)ini.get_int(sec, "hidden_size", (long)s.heads * s.headSize);
     s.eps = (float)ini.get_float(sec, "layernorm_eps", 1e-6);
     s.ropeTheta = (float)ini.get_float(sec, "rope_theta", 10000.0);
+    s.experts = mixtral ? (int)ini.get_int(sec, "sparse_experts", 8) : 0; // common_decoder.h:249
     s.startId = (int)ini.get_int(sec, "start_id", 0);
     s.endId = (int)ini.get_int(sec, "end_id", s.startId);
     if (s.heads <= 0 || s.headSize <= 0 || s.inter <= 0 || s.layers <= 0 || s.vocab <= 0 || s.hidden <= 0) {
@@ -1540,6 +1595,10 @@ AutoModel::AutoModel(std::string modelPath, xft::DataType dataType, xft::DataTyp
         }
         if (ini.get_int(sec, "quant_groupsize", -1) != -1) {
             printf("Quantization with groupsize is not supported.\n");
+            exit(-1);
+        }
+        if (mixtral) {
+            printf("Pre-quantised sparse-MLP model directories are not supported by this build.\n");
             exit(-1);
         }
     }

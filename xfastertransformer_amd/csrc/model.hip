@@ -32,6 +32,8 @@ struct LayerW {
     float *ln1 = nullptr, *ln2 = nullptr, *qkv_bias = nullptr, *o_bias = nullptr;
     // set: the layer's two norms are LayerNorms with these shifts (NormType::LN of the layer API) instead of RMSNorms
     float *ln1_beta = nullptr, *ln2_beta = nullptr;
+    // set: the layer's MLP is this sparse one (MixtralMLP; it carries its own norm weight and router), not gateup / down
+    xfthip_moe_t moe = nullptr;
 };
 
 __global__ void embed_kernel(const uint16_t *__restrict__ table, const int *__restrict__ ids, float *__restrict__ x,
@@ -367,6 +369,8 @@ static int mlp_block(xfthip_model *m, int idx, const float *x_in, int in_stride,
         bool do_norm, hipStream_t st) {
     const xfthip_model_config &c = m->cfg;
     const LayerW &L = m->layers[idx];
+    if (L.moe) // router, top-2, expert GEMMs and the weighted sum over the residual: only enqueues work
+        return xfthip_moe_forward(L.moe, x_in, in_stride, x_out, out_stride, T, do_norm ? 1 : 0, nullptr, nullptr, nullptr, st);
     XFT_REQUIRE(L.gateup && L.down, "layer %d has no MLP weights attached", idx);
     XFT_REQUIRE(!do_norm || L.ln2, "layer %d has no MLP norm weight", idx);
     int rc;
@@ -570,9 +574,30 @@ int xfthip_model_set_mlp(xfthip_model_t m, int idx, xfthip_weight_t gateup, xfth
     LayerW &L = m->layers[idx];
     L.gateup = gateup;
     L.down = down;
+    L.moe = nullptr;
     if (int rc = upload_f32(&L.ln2, ln2_host, c.hidden)) return rc;
     if (int rc = w8a8_reserve(m, gateup->pw, true)) return rc;
     if (int rc = w8a8_reserve(m, down->pw, false)) return rc;
+    if (m->graph) {
+        (void)hipGraphExecDestroy(m->graph);
+        m->graph = nullptr;
+    }
+    return 0;
+}
+
+int xfthip_model_set_moe(xfthip_model_t m, int idx, xfthip_moe_t moe) {
+    XFT_REQUIRE(m && moe, "xfthip_model_set_moe: null argument");
+    XFT_REQUIRE(idx >= 0 && idx < m->cfg.layers, "xfthip_model_set_moe: layer %d out of range", idx);
+    const xfthip_model_config &c = m->cfg;
+    int hidden = 0, inter = 0, experts = 0, max_tokens = 0;
+    if (int rc = xfthip_moe_shape(moe, &hidden, &inter, &experts, &max_tokens)) return rc;
+    XFT_REQUIRE(hidden == c.hidden && inter == c.intermediate, "xfthip_model_set_moe: the sparse MLP is %d x %d, the model %d x %d", hidden, inter,
+            c.hidden, c.intermediate);
+    XFT_REQUIRE(max_tokens >= c.max_tokens, "xfthip_model_set_moe: the sparse MLP takes %d tokens a call, the model up to %d", max_tokens,
+            c.max_tokens);
+    LayerW &L = m->layers[idx];
+    L.moe = moe;
+    L.gateup = L.down = nullptr;
     if (m->graph) {
         (void)hipGraphExecDestroy(m->graph);
         m->graph = nullptr;

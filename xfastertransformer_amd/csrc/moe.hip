@@ -191,6 +191,7 @@ struct xfthip_moe {
     float *eo = nullptr, *logits = nullptr, *w = nullptr, *row_weight = nullptr;
     GroupWeight *group = nullptr; // device pointers of the experts' weights: [E] gate/up, [E] down
     int *sel = nullptr, *counts = nullptr, *row_token = nullptr, *slot_row = nullptr, *rank = nullptr; // counts: [E] counts, [E] offsets, [9 E] GEMM row records
+    bool owns_workspace = true; // false: the per-call buffers belong to the object this one was created beside
 };
 
 extern "C" {
@@ -236,12 +237,47 @@ int xfthip_moe_create(int hidden, int intermediate, int experts, int max_tokens,
     return 0;
 }
 
+int xfthip_moe_create_beside(xfthip_moe_t first, const float *router_host, const float *ln_host, xfthip_moe_t *out) {
+    XFT_REQUIRE(first && out && router_host, "xfthip_moe_create_beside: null argument");
+    XFT_REQUIRE(first->owns_workspace, "xfthip_moe_create_beside: the first object must own its workspace");
+    xfthip_moe *m = new xfthip_moe(*first);
+    m->owns_workspace = false;
+    m->router = nullptr, m->ln = nullptr, m->group = nullptr;
+    m->gateup.assign(m->E, nullptr);
+    m->down.assign(m->E, nullptr);
+    bool ok = hipMalloc((void **)&m->router, (size_t)m->hidden * m->E * 4) == hipSuccess
+            && hipMalloc((void **)&m->group, 2 * 64 * sizeof(GroupWeight)) == hipSuccess
+            && hipMemcpy(m->router, router_host, (size_t)m->hidden * m->E * 4, hipMemcpyHostToDevice) == hipSuccess;
+    if (ok && ln_host) ok = hipMalloc((void **)&m->ln, (size_t)m->hidden * 4) == hipSuccess
+            && hipMemcpy(m->ln, ln_host, (size_t)m->hidden * 4, hipMemcpyHostToDevice) == hipSuccess;
+    if (!ok) {
+        set_error("xfthip_moe_create_beside: allocation failed");
+        xfthip_moe_destroy(m);
+        return 3;
+    }
+    *out = m;
+    return 0;
+}
+
 int xfthip_moe_destroy(xfthip_moe_t m) {
     if (!m) return 0;
-    void *bufs[] = {m->router, m->ln, m->xn, m->xg, m->h, m->eo, m->logits, m->w, m->row_weight, m->sel, m->counts, m->row_token, m->slot_row, m->rank, m->group};
-    for (void *b : bufs)
+    void *own[] = {m->router, m->ln, m->group};
+    void *workspace[] = {m->xn, m->xg, m->h, m->eo, m->logits, m->w, m->row_weight, m->sel, m->counts, m->row_token, m->slot_row, m->rank};
+    for (void *b : own)
         if (b) (void)hipFree(b);
+    if (m->owns_workspace)
+        for (void *b : workspace)
+            if (b) (void)hipFree(b);
     delete m;
+    return 0;
+}
+
+int xfthip_moe_shape(xfthip_moe_t m, int *hidden, int *intermediate, int *experts, int *max_tokens) {
+    XFT_REQUIRE(m, "xfthip_moe_shape: null argument");
+    if (hidden) *hidden = m->hidden;
+    if (intermediate) *intermediate = m->inter;
+    if (experts) *experts = m->E;
+    if (max_tokens) *max_tokens = m->max_tokens;
     return 0;
 }
 

@@ -175,7 +175,8 @@ int xfthip_gemm_qkv_rmsnorm_rope(xfthip_weight_t w, xfthip_kvcache_t cache, int 
  * q = rne(fma(x, 1/scale, -zero/scale)), sum = (sum q)*scale + K*zero.  gemm_w8a8: int8 x int8 ->
  * int32 GEMM against an XFTHIP_W_W8A8 weight, then C = s32*sA*sB + sumB*sB*zA + sumA*zB and the
  * epilogue.  qa: int8 [M, ldq], 16-byte aligned, ldq % 16 == 0.  xfthip_gemm on a W8A8 weight runs
- * both, quantising its bf16 A into a library-owned scratch (not for use under stream capture).
+ * both, quantising its bf16 A into the scratch of the call's stream (grown on demand: a first call of a size is not
+ * for use under stream capture).
  */
 int xfthip_w8a8_quantize_rows(const void *A, int a_dtype, int M, int K, int lda, int8_t *qa, int ldq, float *scale,
         float *zero, float *sum, xfthip_stream_t stream);

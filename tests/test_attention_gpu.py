@@ -181,6 +181,30 @@ def test_split_count_independence(xh, orc, n, S):
     assert np.abs(outs[0] - outs[1]).max() < 1e-4
 
 
+def test_two_streams_each_merge_their_splits_in_their_own_workspace(xh, orc):
+    """Split launches on two streams, queued alternately without a wait in between, over different caches and
+    queries: each stream's results equal what the same call gives alone (the partial results and tickets of plain
+    calls belong to the stream they are made on)."""
+    rng = np.random.default_rng(77)
+    qh, kvh, n = 32, 8, 3000  # batch 1: 24 parts, merged by a launch of their own
+    cases = []
+    for i in range(2):
+        kc, vc, dc = _filled(xh, orc, rng, 0, 1, kvh, 3072, n)
+        q = orc.round_bf16(rng.standard_normal((1, qh * D)))
+        alone = _attend(xh, orc, dc, q, 1, 1, qh, n - 1)
+        cases.append((dc, xh.DeviceBuffer.from_numpy(orc.to_bf16(q)), xh.DeviceBuffer(q.size * 4), alone, q.shape))
+    streams = [xh.Stream(), xh.Stream()]
+    for rep in range(20):
+        for (dc, qd, od, _, shape), st in zip(cases, streams):
+            xh.attention(dc, qd.ptr, shape[1], od.ptr, shape[1], xh.F32, 1, 1, qh, SCALE, n - 1, None, st.h)
+    for st in streams:
+        st.synchronize()
+    for dc, qd, od, alone, shape in cases:
+        assert np.array_equal(od.to_numpy(np.float32, shape), alone)
+    for st in streams:
+        st.free()
+
+
 def test_past_from_device_memory(xh, orc):
     rng = np.random.default_rng(51)
     B, qh, kvh = 3, 32, 8

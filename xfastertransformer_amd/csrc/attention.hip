@@ -62,9 +62,8 @@ __global__ __launch_bounds__(256, (CT == 1 ? 2 : 1)) void attn_prefill32_kernel(
 }
 
 // Split-KV merge workspace: `slots` partial-result slots of kSlotFloats floats and one ticket per
-// column group.  The library keeps one for plain xfthip_attention calls (allocated on first use);
-// a model owns its own, so that two models on two streams never share partials or tickets.
-static AttnWorkspace g_shared_ws;
+// column group.  Plain xfthip_attention calls take one per stream from the library's per-stream scratch
+// (allocated on a stream's first call); a model owns its own.
 int attention_workspace_create(AttnWorkspace *w, int slots) {
     w->ws = nullptr, w->tickets = nullptr, w->slots = 0;
     XFT_CHECK_HIP(hipMalloc((void **)&w->ws, (size_t)slots * kSlotFloats * sizeof(float)));
@@ -81,8 +80,12 @@ void attention_workspace_destroy(AttnWorkspace *w) {
     w->ws = nullptr, w->tickets = nullptr, w->slots = 0;
 }
 
-int attention_workspace_init() {
-    if (g_shared_ws.slots == 0) return attention_workspace_create(&g_shared_ws, kWsSlots);
+// the workspace of plain calls on `stream`
+static int attention_stream_workspace(hipStream_t stream, AttnWorkspace *w) {
+    void *parts = nullptr, *tickets = nullptr;
+    if (int rc = stream_scratch(kScratchAttnParts, stream, (size_t)kWsSlots * kSlotFloats * sizeof(float), false, &parts)) return rc;
+    if (int rc = stream_scratch(kScratchAttnTickets, stream, (size_t)kWsSlots * sizeof(unsigned int), true, &tickets)) return rc;
+    w->ws = (float *)parts, w->tickets = (unsigned int *)tickets, w->slots = kWsSlots;
     return 0;
 }
 
@@ -171,10 +174,11 @@ int xfthip::attention_launch(xfthip_kvcache_t c, const void *q, int qStride, voi
     const int len = past_dev ? ((len_hint > 0 && len_hint < c->maxSeq) ? len_hint : c->maxSeq) : past + S;
     const int wgs = B * c->kv.H * p.CG;
     int nsplit = attention_split_count(len, wgs);
+    AttnWorkspace of_stream;
     if (nsplit > 1) {
         if (wsp == nullptr) {
-            if (int rc = attention_workspace_init()) return rc;
-            wsp = &g_shared_ws;
+            if (int rc = attention_stream_workspace(stream, &of_stream)) return rc;
+            wsp = &of_stream;
         }
         if ((size_t)wgs * nsplit > (size_t)wsp->slots) {
             XFT_REQUIRE(!strict,

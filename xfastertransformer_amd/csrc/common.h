@@ -146,6 +146,30 @@ __device__ inline void dev_drain() {
 __device__ inline float fast_exp(float x) { return __expf(x); }
 
 int device_cu_count();
+// Scratch memory of the stand-alone entry points: one buffer per (purpose, device, stream), so that calls on different
+// streams never share one (calls on one stream are ordered).  Returns a buffer of at least `bytes`; a buffer that has
+// to grow is replaced (which waits for the device).  Allocates on first use for a stream: not during a stream capture
+// (xfthip_graph_begin reserves what the recordable entry points need; a caller that captures by itself makes one
+// eager call on that stream first).  zero_new: a new buffer starts cleared.
+enum ScratchPurpose {
+    kScratchGemmSplit, // fp32 parts of a K-split weight-only GEMM
+    kScratchAttnParts, // split-KV partial results of xfthip_attention
+    kScratchAttnTickets,
+    kScratchW8a8Codes, // quantised activation rows of xfthip_gemm_w8a8_from_bf16
+    kScratchW8a8Stats,
+    kScratchPagedParts, // context splits of xfthip_paged_attention_decode
+    kScratchPagedQkv, // fused q|k|v rows of xfthip_paged_attention_prefill
+    kScratchPurposes
+};
+int stream_scratch(ScratchPurpose purpose, hipStream_t stream, size_t bytes, bool zero_new, void **out);
+// While one of these lives, the calling thread's stream_scratch calls take the buffers of `key` whatever stream they
+// name: for work recorded on a capture stream of the library's own that will be launched on `key`.
+struct ScratchKeyScope {
+    explicit ScratchKeyScope(hipStream_t key);
+    ~ScratchKeyScope();
+    ScratchKeyScope(const ScratchKeyScope &) = delete;
+    ScratchKeyScope &operator=(const ScratchKeyScope &) = delete;
+};
 // Split-KV merge workspace of the attention kernel: partial (max, sum, output) slots and one
 // ticket per column group (tickets are zero between launches).
 struct AttnWorkspace {
@@ -155,8 +179,6 @@ struct AttnWorkspace {
 };
 int attention_workspace_create(AttnWorkspace *w, int slots); // allocates; not for use during stream capture
 void attention_workspace_destroy(AttnWorkspace *w);
-// allocates the library's shared workspace (idempotent; must not run during stream capture)
-int attention_workspace_init();
 // resolves the device address of the statically allocated workspace behind xfthip_attention_static
 // for the current device (idempotent, allocates nothing)
 int attention_static_scratch_init();

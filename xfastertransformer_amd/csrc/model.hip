@@ -454,7 +454,6 @@ int xfthip_argmax(const float *logits, int rows, int cols, int *ids_dev, xfthip_
 }
 
 int xfthip_model_create(const xfthip_model_config *cfg, xfthip_model_t *out) {
-    if (int rc = qgemm_split_reserve()) return rc; // decode steps at more than 32 rows are captured into graphs: no allocation there
     XFT_REQUIRE(cfg && out, "xfthip_model_create: null argument");
     const xfthip_model_config &c = *cfg;
     XFT_REQUIRE(c.layers > 0 && c.hidden > 0 && c.intermediate > 0, "xfthip_model_create: bad sizes");
@@ -754,9 +753,6 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
     if (!m->use_graph) {
         for (int i = 0; i < steps; ++i)
             if (int rc = decode_step(m, B, st)) return rc;
-    } else if (!m->use_graph) {    } else if (!m->use_graph) {
-        for (int i = 0; i < steps; ++i)
-            if (int rc = decode_step(m, B, st)) return rc;
     } else if (m->graph == nullptr || m->graph_B != B || m->graph_stream != st || m->graph_nsplit != nsplit
             || m->graph_ragged != m->ragged) {
         if (m->graph) {
@@ -773,6 +769,11 @@ int xfthip_model_decode(xfthip_model_t m, int steps, int *ids_out_host, xfthip_s
             XFT_CHECK_HIP(hipDeviceSynchronize());
         }
         hipGraph_t g = nullptr;
+        // A step at more than 32 rows, or with sparse MLPs, may split K: the parts go to the scratch of the stream the
+        // graph will be launched on (not of the capture stream, which may be a temporary one), which has to exist
+        // before the capture starts.
+        ScratchKeyScope scratch_of_launch_stream(st);
+        if (int rc0 = qgemm_split_reserve(st)) return rc0;
         XFT_CHECK_HIP(hipStreamBeginCapture(cap, hipStreamCaptureModeThreadLocal));
         int rc = decode_step(m, B, cap);
         hipError_t e = hipStreamEndCapture(cap, &g);

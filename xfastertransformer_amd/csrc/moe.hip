@@ -208,7 +208,6 @@ int xfthip_moe_create(int hidden, int intermediate, int experts, int max_tokens,
     XFT_REQUIRE(out && router_host, "xfthip_moe_create: null argument");
     XFT_REQUIRE(experts == 8, "xfthip_moe_create: %d experts unsupported (the router kernel is built for 8)", experts);
     XFT_REQUIRE(hidden > 0 && hidden % 8 == 0 && intermediate % 16 == 0 && max_tokens > 0, "xfthip_moe_create: bad sizes");
-    if (int rc = qgemm_split_reserve()) return rc; // the down projections split K: have the workspace before any capture
     xfthip_moe *m = new xfthip_moe();
     m->hidden = hidden;
     m->inter = intermediate;

@@ -21,6 +21,7 @@
 // selfAttention call), through this library's FP16-cache attention kernel on a scratch cache, and
 // every token's key / value row stored to its slot (slot_mapping holds one entry per token; the
 // reference's closures, marked "TODO: debug and fix", pass only slot_mapping[b]).
+#include <map>
 #include <mutex>
 
 #include "common.h"
@@ -167,14 +168,14 @@ __global__ __launch_bounds__(256) void paged_fuse_qkv_kernel(uint16_t *qkv, cons
     }
 }
 
-// grow-only scratch of the paged entry points (one process-wide set; calls on different streams race)
+// Scratch of the paged entry points, grow-only, one set per stream: the context splits and the fused q|k|v rows come
+// from stream_scratch, the FP16 scratch cache of the prefill from the table below.
+struct PrefillCache {
+    xfthip_kvcache_t cache = nullptr;
+    int heads = 0, seq = 0;
+};
 std::mutex g_mu;
-float *g_part = nullptr;
-size_t g_part_floats = 0;
-uint16_t *g_qkv = nullptr;
-size_t g_qkv_elems = 0;
-xfthip_kvcache_t g_cache = nullptr;
-int g_cache_heads = 0, g_cache_seq = 0;
+std::map<hipStream_t, PrefillCache> g_prefill_cache;
 
 int check_common(const void *out, const void *q, const void *k, const void *v, int q_heads, int kv_heads, int head_size, int q_stride,
         int kv_stride, int o_stride, const void *kc, const void *vc, int block_size) {
@@ -211,20 +212,12 @@ extern "C" int xfthip_paged_attention_decode(void *out, const void *q, const voi
     if (nsplit > cap) nsplit = cap;
     if (nsplit > 64) nsplit = 64;
     if (nsplit < 1) nsplit = 1;
-    std::lock_guard<std::mutex> lk(g_mu);
     const size_t need = (size_t)batch * q_heads * nsplit * 130;
-    if (need > g_part_floats) {
-        if (g_part) {
-            XFT_CHECK_HIP(hipDeviceSynchronize());
-            (void)hipFree(g_part);
-            g_part = nullptr, g_part_floats = 0;
-        }
-        XFT_CHECK_HIP(hipMalloc((void **)&g_part, need * sizeof(float)));
-        g_part_floats = need;
-    }
+    void *part = nullptr;
+    if (int rc = stream_scratch(kScratchPagedParts, st, need * sizeof(float), false, &part)) return rc;
     PagedParams p = {};
     p.out = (uint16_t *)out, p.q = (const uint16_t *)q, p.kc = (const uint16_t *)kcache, p.vc = (const uint16_t *)vcache;
-    p.tables = block_tables, p.ctx = context_lens, p.part = g_part;
+    p.tables = block_tables, p.ctx = context_lens, p.part = (float *)part;
     p.q_heads = q_heads, p.kv_heads = kv_heads, p.q_stride = q_stride, p.o_stride = o_stride, p.table_stride = table_stride;
     p.block_size = block_size, p.block_num = block_num, p.nsplit = nsplit, p.scale = scale;
     hipLaunchKernelGGL(paged_store_kernel, dim3(batch), dim3(256), 0, st, (uint16_t *)kcache, (uint16_t *)vcache, (const uint16_t *)k,
@@ -249,25 +242,24 @@ extern "C" int xfthip_paged_attention_prefill(void *out, const void *q, const vo
         if (token_lens_host[b] > longest) longest = token_lens_host[b];
     }
     const int q_elems = q_heads * 128, kv_elems = kv_heads * 128, fused = q_elems + 2 * kv_elems;
-    std::lock_guard<std::mutex> lk(g_mu);
-    if ((size_t)total * fused > g_qkv_elems) {
-        if (g_qkv) {
-            XFT_CHECK_HIP(hipDeviceSynchronize());
-            (void)hipFree(g_qkv);
-            g_qkv = nullptr, g_qkv_elems = 0;
+    void *fused_rows = nullptr;
+    if (int rc = stream_scratch(kScratchPagedQkv, st, (size_t)total * fused * 2, false, &fused_rows)) return rc;
+    uint16_t *g_qkv = (uint16_t *)fused_rows;
+    xfthip_kvcache_t g_cache = nullptr;
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        PrefillCache &pc = g_prefill_cache[st];
+        if (pc.cache == nullptr || pc.heads != kv_heads || pc.seq < longest) {
+            if (pc.cache) {
+                XFT_CHECK_HIP(hipDeviceSynchronize());
+                (void)xfthip_kvcache_destroy(pc.cache);
+                pc.cache = nullptr;
+            }
+            const int seq = ((longest + 255) / 256) * 256;
+            if (int rc = xfthip_kvcache_create(XFTHIP_FP16, 1, kv_heads, seq, 128, &pc.cache)) return rc;
+            pc.heads = kv_heads, pc.seq = seq;
         }
-        XFT_CHECK_HIP(hipMalloc((void **)&g_qkv, (size_t)total * fused * 2));
-        g_qkv_elems = (size_t)total * fused;
-    }
-    if (g_cache == nullptr || g_cache_heads != kv_heads || g_cache_seq < longest) {
-        if (g_cache) {
-            XFT_CHECK_HIP(hipDeviceSynchronize());
-            (void)xfthip_kvcache_destroy(g_cache);
-            g_cache = nullptr;
-        }
-        const int seq = ((longest + 255) / 256) * 256;
-        if (int rc = xfthip_kvcache_create(XFTHIP_FP16, 1, kv_heads, seq, 128, &g_cache)) return rc;
-        g_cache_heads = kv_heads, g_cache_seq = seq;
+        g_cache = pc.cache;
     }
     hipLaunchKernelGGL(paged_store_kernel, dim3(total), dim3(256), 0, st, (uint16_t *)kcache, (uint16_t *)vcache, (const uint16_t *)k,
             (const uint16_t *)v, slot_mapping, kv_stride, kv_elems, block_num * block_size);

@@ -66,7 +66,8 @@ struct SkinnyParams {
 int qgemm_skinny(const PackedWeight &pw, const SkinnyParams &p, hipStream_t stream); // M <= 32
 bool skinny_can_fuse_norm(const PackedWeight &pw, int M); // may SkinnyParams::norm_x be used
 int qgemm_mfma(const PackedWeight &pw, const SkinnyParams &p, hipStream_t stream); // any M, built for M > 32
-int qgemm_split_reserve(); // allocates the K-split workspace of qgemm_mfma now (before a stream capture, say)
+// the K-split workspace of qgemm_mfma launches on `stream` (allocated on the stream's first call: before a capture, say)
+int qgemm_split_reserve(hipStream_t stream, float **out = nullptr);
 // xfthip_gemm / xfthip_gemm_gateup_silu (by the weight's flag) with the row count in device memory: rows_dev =
 // {rows, first row of A, first row of C}, at most m_max rows, about m_hint expected; plain epilogue only
 int gemm_rows_dev(xfthip_weight_t w, int m_max, int m_hint, const int *rows_dev, const void *A, int lda, void *C, int ldc, int c_dtype,

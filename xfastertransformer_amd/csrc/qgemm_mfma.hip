@@ -94,22 +94,18 @@ __global__ __launch_bounds__(256) void qgemm_split_finish_kernel(SkinnyParams p)
     for (int v = 0; v < VEC; ++v) store_from_f32(p.C, p.c_dtype, ci + v, x[v]);
 }
 
-// Partial results of the K split: one buffer per process and device, allocated once at its upper bound (a
-// split launch has at most CUs / 2 tiles of 32 x 128 results in at most 16 parts: 33.5 MB on 256 CUs), so
-// nothing is allocated or freed once it exists.  Launches on one stream are ordered; split launches that
-// overlap on different streams race on it.
-std::mutex g_split_mu;
-float *g_split_part = nullptr;
-size_t g_split_floats = 0;
+// Partial results of the K split: one buffer per stream and device (stream_scratch), allocated once at its upper
+// bound (a split launch has at most CUs / 2 tiles of 32 x 128 results in at most 16 parts: 33.5 MB on 256 CUs), so
+// nothing is allocated or freed on a stream once its buffer exists.  Launches on one stream are ordered; launches
+// on different streams work in different buffers.
+size_t split_bound_floats() { return (size_t)16 * (device_cu_count() / 2 + 1) * 4096; }
 
 } // namespace
 
-int qgemm_split_reserve() {
-    std::lock_guard<std::mutex> lk(g_split_mu);
-    if (g_split_part) return 0;
-    const size_t floats = (size_t)16 * (device_cu_count() / 2 + 1) * 4096;
-    XFT_CHECK_HIP(hipMalloc((void **)&g_split_part, floats * sizeof(float)));
-    g_split_floats = floats;
+int qgemm_split_reserve(hipStream_t stream, float **out) {
+    void *p = nullptr;
+    if (int rc = stream_scratch(kScratchGemmSplit, stream, split_bound_floats() * sizeof(float), false, &p)) return rc;
+    if (out) *out = (float *)p;
     return 0;
 }
 
@@ -146,8 +142,7 @@ int qgemm_mfma(const PackedWeight &pw, const SkinnyParams &p0, hipStream_t strea
         long want = (8L * cus + tiles64 - 1) / tiles64;
         want = want < kt_n / 8 ? want : kt_n / 8;
         want = want < 16 ? want : 16;
-        if (int rc = qgemm_split_reserve()) return rc;
-        const long fit = (long)(g_split_floats / ((size_t)p.M * p.N));
+        const long fit = (long)(split_bound_floats() / ((size_t)p.M * p.N));
         want = want < fit ? want : fit;
         p.ksplit = 0;
         if (want >= 2) {
@@ -156,9 +151,8 @@ int qgemm_mfma(const PackedWeight &pw, const SkinnyParams &p0, hipStream_t strea
         }
     }
     if (p.ksplit > 1) {
-        if (int rc = qgemm_split_reserve()) return rc;
-        if ((size_t)p.ksplit * p.M * p.N > g_split_floats) p.ksplit = 0; // cannot happen within the bound; stay correct anyway
-        p.split_part = g_split_part;
+        if ((size_t)p.ksplit * p.M * p.N > split_bound_floats()) p.ksplit = 0; // cannot happen within the bound; stay correct anyway
+        else if (int rc = qgemm_split_reserve(stream, &p.split_part)) return rc;
     }
     if (p.ksplit <= 1) p.ksplit = 0;
     int rc;

@@ -2,9 +2,12 @@
 #include <stdarg.h>
 #include <string.h>
 
+#include <map>
 #include <mutex>
+#include <tuple>
 
 #include "common.h"
+#include "qgemm.h"
 
 namespace xfthip {
 
@@ -22,6 +25,47 @@ void set_error(const char *fmt, ...) {
 
 int device_cu_count() {
     return g_cus > 0 ? g_cus : 256;
+}
+
+namespace {
+struct ScratchEntry {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+};
+std::mutex g_scratch_registry_mu;
+std::map<std::tuple<int, int, hipStream_t>, ScratchEntry> g_scratch_registry;
+thread_local bool g_scratch_key_set = false;
+thread_local hipStream_t g_scratch_key = nullptr;
+} // namespace
+
+ScratchKeyScope::ScratchKeyScope(hipStream_t key) {
+    g_scratch_key_set = true;
+    g_scratch_key = key;
+}
+ScratchKeyScope::~ScratchKeyScope() {
+    g_scratch_key_set = false;
+}
+
+int stream_scratch(ScratchPurpose purpose, hipStream_t stream, size_t bytes, bool zero_new, void **out) {
+    int dev = 0;
+    XFT_CHECK_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lk(g_scratch_registry_mu);
+    ScratchEntry &e = g_scratch_registry[std::make_tuple((int)purpose, dev, g_scratch_key_set ? g_scratch_key : stream)];
+    if (e.bytes < bytes) {
+        if (e.ptr) {
+            XFT_CHECK_HIP(hipDeviceSynchronize()); // work already queued may still use the smaller buffer
+            (void)hipFree(e.ptr);
+            e.ptr = nullptr, e.bytes = 0;
+        }
+        XFT_CHECK_HIP(hipMalloc(&e.ptr, bytes));
+        if (zero_new) {
+            XFT_CHECK_HIP(hipMemset(e.ptr, 0, bytes));
+            XFT_CHECK_HIP(hipDeviceSynchronize());
+        }
+        e.bytes = bytes;
+    }
+    *out = e.ptr;
+    return 0;
 }
 
 } // namespace xfthip
@@ -180,6 +224,8 @@ int xfthip_device_synchronize(void) {
 
 int xfthip_graph_begin(xfthip_stream_t stream) {
     XFT_REQUIRE(stream != nullptr, "xfthip_graph_begin: capture needs a stream of its own, not the null stream");
+    // what the recordable entry points take from the per-stream scratch must exist before the capture starts
+    if (int rc = qgemm_split_reserve((hipStream_t)stream)) return rc;
     XFT_CHECK_HIP(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
     return 0;
 }

@@ -601,11 +601,6 @@ static int launch_w8a8_mfma(const W8A8Params &p, hipStream_t stream) {
     return 0;
 }
 
-// scratch for the quantised activations of xfthip_gemm on a W8A8 weight (grown on demand)
-static int8_t *g_qa = nullptr;
-static float *g_qstat = nullptr;
-static size_t g_qa_cap = 0, g_qstat_cap = 0;
-static std::mutex g_qa_mu;
 
 } // namespace xfthip
 
@@ -697,34 +692,21 @@ int xfthip_gemm_w8a8(xfthip_weight_t w, int M, const int8_t *qa, int ldq, const 
 
 namespace xfthip {
 
-// xfthip_gemm on a W8A8 weight: quantise the bf16 activations into a library-owned scratch, then
-// run the int8 GEMM.  The scratch grows with hipMalloc (after waiting for the whole device: launches on any
-// stream may still read the old one), so a first call of a given size is not for use under stream capture; calls
-// that overlap on different streams share the scratch and must be serialised by the caller.  The model driver
-// keeps a scratch of its own, sized when the weights are attached.
+// xfthip_gemm on a W8A8 weight: quantise the bf16 activations into the stream's scratch (stream_scratch: one buffer a
+// stream, grown on demand, so a first call of a given size is not for use under stream capture), then run the int8
+// GEMM.  The model driver keeps a scratch of its own, sized when the weights are attached.
 int gemm_w8a8_from_bf16(xfthip_weight_t w, int M, const void *A, int lda, void *C, int ldc, int c_dtype, int epilogue,
         const float *bias, const void *res, int ldres, int res_dtype, float gamma, hipStream_t stream) {
     const int K = w->pw.K;
     const int ldq = (K + 15) / 16 * 16;
     const size_t need = (size_t)M * ldq;
-    std::lock_guard<std::mutex> lk(g_qa_mu);
-    if (need > g_qa_cap) {
-        XFT_CHECK_HIP(hipDeviceSynchronize());
-        if (g_qa) (void)hipFree(g_qa);
-        g_qa = nullptr;
-        XFT_CHECK_HIP(hipMalloc((void **)&g_qa, need));
-        g_qa_cap = need;
-    }
-    if ((size_t)M * 3 > g_qstat_cap) {
-        XFT_CHECK_HIP(hipDeviceSynchronize());
-        if (g_qstat) (void)hipFree(g_qstat);
-        g_qstat = nullptr;
-        XFT_CHECK_HIP(hipMalloc((void **)&g_qstat, (size_t)M * 3 * sizeof(float)));
-        g_qstat_cap = (size_t)M * 3;
-    }
-    float *sA = g_qstat, *zA = g_qstat + M, *sumA = g_qstat + 2 * M;
-    if (int rc = xfthip_w8a8_quantize_rows(A, XFTHIP_BF16, M, K, lda, g_qa, ldq, sA, zA, sumA, stream)) return rc;
-    return xfthip_gemm_w8a8(w, M, g_qa, ldq, sA, zA, sumA, C, ldc, c_dtype, epilogue, bias, res, ldres, res_dtype, gamma, stream);
+    void *codes = nullptr, *stats = nullptr;
+    if (int rc = stream_scratch(kScratchW8a8Codes, stream, need, false, &codes)) return rc;
+    if (int rc = stream_scratch(kScratchW8a8Stats, stream, (size_t)M * 3 * sizeof(float), false, &stats)) return rc;
+    int8_t *qa = (int8_t *)codes;
+    float *sA = (float *)stats, *zA = sA + M, *sumA = sA + 2 * M;
+    if (int rc = xfthip_w8a8_quantize_rows(A, XFTHIP_BF16, M, K, lda, qa, ldq, sA, zA, sumA, stream)) return rc;
+    return xfthip_gemm_w8a8(w, M, qa, ldq, sA, zA, sumA, C, ldc, c_dtype, epilogue, bias, res, ldres, res_dtype, gamma, stream);
 }
 
 } // namespace xfthip

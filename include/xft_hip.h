@@ -415,6 +415,17 @@ int xfthip_model_mlp_forward(xfthip_model_t m, int idx, const float *x_in, int i
  */
 int xfthip_model_prefill(xfthip_model_t m, const int *ids_host, int B, int S, float *logits_host, xfthip_stream_t stream);
 /*
+ * Prefix sharing (CommonDecoder::setPrefix / prefixForward, src/models/common_decoder.h:695-768, and the step-0 branch
+ * of forward, :337-350, 440-443).  set_prefix runs the n prefix tokens once, as one sequence, into cache row 0.
+ * prefill_after_prefix is the prompt pass of B sequences whose first n tokens are that prefix: ids_host [B, S] holds
+ * only what follows the prefix; every sequence's cache row starts as a copy of the prefix's positions
+ * (KVCacheManager::expandPrefixCache) and the S new tokens run at positions n .. n + S - 1; decode steps follow as after
+ * xfthip_model_prefill.  The prefix stays usable for further prefill_after_prefix calls until a plain prompt pass writes
+ * row 0 again (xfthip_model_prefill, xfthip_model_seq_prefill into row 0).
+ */
+int xfthip_model_set_prefix(xfthip_model_t m, const int *ids_host, int n, xfthip_stream_t stream);
+int xfthip_model_prefill_after_prefix(xfthip_model_t m, const int *ids_host, int B, int S, float *logits_host, xfthip_stream_t stream);
+/*
  * `steps` greedy decode steps, each one replay of a captured HIP graph (embedding of the
  * previous ids, all layers, lm_head, argmax, position advance).  ids_out_host: int32
  * [steps, B] or NULL.  Must follow xfthip_model_prefill with the same B.

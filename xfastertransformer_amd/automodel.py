@@ -34,6 +34,8 @@ _lib.xft_automodel_max_seq_len.argtypes = [C.c_void_p]
 _lib.xft_automodel_set_input.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
                                          C.c_float, C.c_void_p]
 _lib.xft_automodel_free_seqs.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
+_lib.xft_automodel_set_prefix.restype = None
+_lib.xft_automodel_set_prefix.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
 _lib.xft_sample_candidates.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_float, C.c_void_p, C.c_void_p]
 _lib.xft_sample_pick.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_float]
 _lib.xft_beam_create.restype = C.c_void_p
@@ -194,6 +196,18 @@ class AutoModel:
     def forward_cb(self):
         """One step of the sequences chosen by set_input_cb: their next tokens, in that order."""
         return self.forward().ravel().tolist()
+
+    def prefix_sharing(self, input_ids=None, truncate_tail=0):
+        """The reference's AutoModel.prefix_sharing (automodel.py:180-184): input_ids [1, n] is run once; inputs that
+        follow carry it in front and only run what comes after it."""
+        ids = np.asarray(input_ids.tolist() if hasattr(input_ids, "tolist") else input_ids, np.int32)
+        if truncate_tail > 0:
+            ids = ids[..., :-truncate_tail]
+        ids = np.ascontiguousarray(ids.reshape(-1), np.int32)
+        _lib.xft_automodel_set_prefix(self._h, ids.ctypes.data, len(ids))
+
+    def disable_prefix_sharing(self):
+        _lib.xft_automodel_set_prefix(self._h, None, 0)
 
     def free_seqs(self, seq_ids):
         ids = np.ascontiguousarray(seq_ids.tolist() if hasattr(seq_ids, "tolist") else seq_ids, np.int32)

@@ -429,6 +429,18 @@ class Model:
         fn = np.ascontiguousarray(final_norm, np.float32)
         check(lib.xfthip_model_set_head(self.h, _hp(e), _hp(fn), lm_head.h))
 
+    def set_prefix(self, ids, stream=None):
+        ids = np.ascontiguousarray(ids, np.int32).reshape(-1)
+        check(lib.xfthip_model_set_prefix(self.h, _hp(ids), len(ids), stream))
+
+    def prefill_after_prefix(self, ids, want_logits=False, stream=None):
+        """ids [B, S]: what follows the shared prefix in each sequence."""
+        ids = np.ascontiguousarray(ids, np.int32)
+        B, S = ids.shape
+        logits = np.empty((B, self.cfg.vocab), np.float32) if want_logits else None
+        check(lib.xfthip_model_prefill_after_prefix(self.h, _hp(ids), B, S, _hp(logits), stream))
+        return self.last_ids(B), logits
+
     def layer_forward(self, idx, x_in_dev, x_out_dev, B, S, past, stride=None, stream=None):
         stride = stride or self.cfg.hidden
         check(lib.xfthip_model_layer_forward(self.h, idx, x_in_dev, stride, x_out_dev, stride, B, S, past, stream))

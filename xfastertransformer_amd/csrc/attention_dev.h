@@ -261,12 +261,13 @@ __device__ inline void attn_unit(const AttnParams &p, const int split, const int
         float pr[2][4];
         // INT8 values: the per-token scale is folded into the probability, normalised by the
         // block's largest scale so that the fp16 operand stays in [0, 1]
+        // (over the tokens this column sees: what lies behind them in the block may be left from an earlier sequence)
         float vmax = 0.0f;
         if constexpr (INT8) {
 #pragma unroll
             for (int a = 0; a < 2; ++a)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) vmax = fmaxf(vmax, vs[a][r]);
+                for (int r = 0; r < 4; ++r) vmax = fmaxf(vmax, vis[a][r] ? vs[a][r] : 0.0f);
             vmax = fmaxf(vmax, __shfl_xor(vmax, 16, 64));
             vmax = fmaxf(vmax, __shfl_xor(vmax, 32, 64));
         }

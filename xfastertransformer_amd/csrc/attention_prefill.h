@@ -89,7 +89,8 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
     const int lim_min = c0 + WC - 1 < ncols ? past + c0 / p.G + 1 : 0; // every column of the wave sees at least this many
     int wave_last = c0 + WC - 1;
     wave_last = wave_last < ncols ? wave_last : ncols - 1;
-    const int wave_nblk = c0 < ncols ? (past + wave_last / p.G + 1 + 31) >> 5 : 0;
+    const int wave_lim = c0 < ncols ? past + wave_last / p.G + 1 : 0; // no column of the wave sees a token from here on
+    const int wave_nblk = (wave_lim + 31) >> 5;
     int wg_last = (cgroup + 1) * NW * WC - 1;
     wg_last = wg_last < ncols ? wg_last : ncols - 1;
     const int nblk = (past + wg_last / p.G + 1 + 31) >> 5;
@@ -226,8 +227,9 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
             for (int q = 0; q < 4; ++q) {
                 ks[q] = *(const f32x4 *)(sl + 8 * q + 4 * h) * c1; // key scale and softmax scale in one factor
                 vs[q] = *(const f32x4 *)(sl + 32 + 8 * q + 4 * h);
+                // (tokens no column of the wave sees stay out: behind the sequence's end the cache may hold anything)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) vmax = fmaxf(vmax, vs[q][r]);
+                for (int r = 0; r < 4; ++r) vmax = fmaxf(vmax, t0 + 8 * q + 4 * h + r < wave_lim ? vs[q][r] : 0.0f);
             }
             vmax = fmaxf(vmax, swap32(vmax)); // the block's largest value scale, the same in every lane
             // value scales relative to vref; vref follows the blocks' largest scale lazily, like the maximum

@@ -442,6 +442,9 @@ struct ModelImpl {
         std::vector<float> router;
         std::vector<xfthip_weight_t> expertGateup, expertDown;
     };
+    // prefix sharing (Model::setPrefix): the prefix ids, and whether the device model's cache row 0 holds them
+    std::vector<int32_t> prefix;
+    bool prefixOnDevice = false;
     int experts = 0; // sparse_experts of a [mixtral] section, 0 for a dense model
     std::vector<xfthip_moe_t> moe; // one per layer, rebuilt with the device model (their buffers are sized by its token capacity)
     std::vector<Layer> L;
@@ -663,6 +666,7 @@ struct ModelImpl {
         if (!grow) return;
         if (model) CK(xfthip_model_destroy(model));
         model = nullptr;
+        prefixOnDevice = false;
         drop_moe();
         cfg.layers = layers, cfg.hidden = hidden, cfg.intermediate = inter;
         cfg.q_heads = heads, cfg.kv_heads = kvHeads, cfg.head_size = headSize;
@@ -696,6 +700,28 @@ struct ModelImpl {
             if (y.firstQkv) CK(xfthip_model_set_first_token_weights(model, l, y.firstQkv, y.firstO, y.firstGateup, y.firstDown));
         }
         CK(xfthip_model_set_head(model, embedding.data(), finalNorm.data(), lmHead));
+    }
+
+    // The prompt pass of a lockstep input.  With a prefix set, the first prefix.size() tokens of every sequence are
+    // taken to be the prefix (as the reference takes them, common_decoder.h:337-350) and only the rest runs.
+    void prompt_pass(const std::vector<int32_t> &ids, int B, int S, float *logits) {
+        if (prefix.empty()) {
+            prefixOnDevice = false;
+            CK(xfthip_model_prefill(model, ids.data(), B, S, logits, nullptr));
+            return;
+        }
+        const int n = (int)prefix.size(), rest = S - n;
+        if (rest <= 0) {
+            printf("[ERROR] The input (%d tokens) must be longer than the shared prefix (%d tokens).\n", S, n);
+            exit(-1);
+        }
+        if (!prefixOnDevice) {
+            CK(xfthip_model_set_prefix(model, prefix.data(), n, nullptr));
+            prefixOnDevice = true;
+        }
+        std::vector<int32_t> tail((size_t)B * rest);
+        for (int b = 0; b < B; ++b) std::copy(ids.begin() + (size_t)b * S + n, ids.begin() + (size_t)(b + 1) * S, tail.begin() + (size_t)b * rest);
+        CK(xfthip_model_prefill_after_prefix(model, tail.data(), B, rest, logits, nullptr));
     }
 
     // ---- searchers ------------------------------------------------------------------------------
@@ -995,13 +1021,15 @@ std::tuple<float *, int, int> Model::forward(bool logitsAll) {
     s.fit(batchSize, seqLen, std::max(seqLen + 1, s.maxLen));
     const size_t rows = logitsAll ? (size_t)batchSize * seqLen : (size_t)batchSize;
     s.logitsHost.resize(rows * s.vocab);
-    CK(xfthip_model_prefill(s.model, inputIds.data(), batchSize, seqLen, logitsAll ? nullptr : s.logitsHost.data(), nullptr));
+    if (logitsAll && !s.prefix.empty()) unsupported("Model::forward(logitsAll = true) with a shared prefix");
+    s.prompt_pass(inputIds, batchSize, seqLen, logitsAll ? nullptr : s.logitsHost.data());
     if (logitsAll) CK(xfthip_model_prompt_logits(s.model, 0, (int)rows, s.logitsHost.data(), nullptr));
     return std::make_tuple(s.logitsHost.data(), 0, s.vocab);
 }
 
 // models.cpp:847-903: one step of the working sequences, all prompts or all decodes
 static std::vector<int32_t> generate_cb(ModelImpl &s) {
+    s.prefixOnDevice = false; // sequences are started in any cache row
     if (s.working.empty()) {
         printf("Please set input tokens by model.set_input().\n");
         exit(-1);
@@ -1076,6 +1104,7 @@ static std::vector<int32_t> generate_cb(ModelImpl &s) {
 // row of its first beam; the other beams' rows are filled from it.  Later steps re-map the generated part of
 // the cache rows to the beams the scorer kept, feed every row its token and read all rows' logits.
 static std::vector<int32_t> generate_beam(ModelImpl &s, const std::vector<int32_t> &inputIds, int batchSize, int seqLen, bool first) {
+    s.prefixOnDevice = false; // the beams' prompts run into cache rows of their own
     const int nb = s.numBeams, rows = batchSize * nb;
     std::vector<int> all(rows);
     for (int i = 0; i < rows; ++i) all[i] = i;
@@ -1147,7 +1176,7 @@ std::vector<int32_t> Model::generate() {
             // nothing to generate: the reference still runs the prompt and emits one token
         }
         s.fit(batchSize, seqLen, std::max(seqLen + 1, s.maxLen));
-        CK(xfthip_model_prefill(s.model, inputIds.data(), batchSize, seqLen, nullptr, nullptr));
+        s.prompt_pass(inputIds, batchSize, seqLen, nullptr);
     } else {
         // feed back what the searcher chose where it differs from the device's own arg-max
         if (s.nextTokens != s.deviceIds) CK(xfthip_model_set_next_ids(s.model, s.nextTokens.data(), nullptr));
@@ -1207,11 +1236,20 @@ std::vector<int32_t> Model::finalize() {
     return result;
 }
 
-void Model::setPrefix(std::vector<int32_t> &) {
-    unsupported("Prefix sharing");
+// models.cpp:930-946: the prefix runs once; the inputs that follow carry it in front (greedy and sampling in lockstep
+// mode; the sequence-id and beam-search paths run whole prompts)
+void Model::setPrefix(std::vector<int32_t> &prefixIDs_) {
+    ModelImpl &s = *impl;
+    if (prefixIDs_.empty()) {
+        printf("[ERROR] Model::setPrefix needs at least one token.\n");
+        exit(-1);
+    }
+    s.prefix = prefixIDs_;
+    s.prefixOnDevice = false; // run before the next prompt pass (the device model may be rebuilt for it)
 }
 void Model::unsetPrefix() {
-    unsupported("Prefix sharing");
+    impl->prefix.clear();
+    impl->prefixOnDevice = false;
 }
 bool Model::freeSeqs(std::vector<int> &seqIDs) {
     ModelImpl &s = *impl;
@@ -1695,6 +1733,16 @@ int xft_automodel_set_input(void *h, const int *lens, const int *ids, int n, con
     std::vector<int> out = ((xft::AutoModel *)h)->set_input(prompts, given, cfg, {});
     memcpy(ids_out, out.data(), out.size() * 4);
     return (int)out.size();
+}
+
+// n > 0: Model::setPrefix with these ids; n == 0: Model::unsetPrefix
+void xft_automodel_set_prefix(void *h, const int *ids, int n) {
+    if (n <= 0) {
+        ((xft::AutoModel *)h)->unsetPrefix();
+        return;
+    }
+    std::vector<int32_t> v(ids, ids + n);
+    ((xft::AutoModel *)h)->setPrefix(v);
 }
 
 int xft_automodel_free_seqs(void *h, const int *seq_ids, int n) {

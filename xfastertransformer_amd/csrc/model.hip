@@ -187,6 +187,7 @@ struct xfthip_model {
     // decode state
     int cur_B = 0, cur_pos = 0;
     int prompt_rows = 0; // rows of `x` that hold the last layer's output of the most recent prompt pass (0 after a decode step)
+    int prefix_len = 0; // positions [0, prefix_len) of cache row 0 hold a shared prefix (xfthip_model_set_prefix)
     // continuous batching: sequences live in cache rows of their own, each at its own position
     int row0 = 0; // cache row of the first sequence of the forward call in flight
     bool ragged = false; // rows may differ in position or sit out a step (set by the xfthip_model_seq_* calls)
@@ -705,32 +706,64 @@ int xfthip_model_mlp_forward(xfthip_model_t m, int idx, const float *x_in, int i
     return mlp_block(m, idx, x_in, in_stride, x_out, out_stride, tokens, do_norm != 0, (hipStream_t)stream);
 }
 
-int xfthip_model_prefill(xfthip_model_t m, const int *ids_host, int B, int S, float *logits_host, xfthip_stream_t stream) {
-    XFT_REQUIRE(m && ids_host, "xfthip_model_prefill: null argument");
+// the prompt pass of B sequences of S tokens whose cache rows already hold `past` positions each
+static int prompt_pass(xfthip_model_t m, const char *who, const int *ids_host, int B, int S, int past, float *logits_host, hipStream_t st) {
     const xfthip_model_config &c = m->cfg;
-    XFT_REQUIRE(m->embedding && m->lm_head, "xfthip_model_prefill: embedding / lm_head not set");
-    XFT_REQUIRE(B > 0 && B <= c.max_batch && S > 0 && B * S <= c.max_tokens && S <= c.max_seq,
-            "xfthip_model_prefill: B=%d S=%d exceed the model limits", B, S);
-    hipStream_t st = (hipStream_t)stream;
+    XFT_REQUIRE(m->embedding && m->lm_head, "%s: embedding / lm_head not set", who);
+    XFT_REQUIRE(B > 0 && B <= c.max_batch && S > 0 && B * S <= c.max_tokens && past + S <= c.max_seq, "%s: B=%d S=%d past=%d exceed the model limits",
+            who, B, S, past);
     FirstTokenWeights first_token(m);
     m->row0 = 0;
     m->ragged = false;
     m->row_pos.assign(c.max_batch, -1);
-    for (int b = 0; b < B; ++b) m->row_pos[b] = S;
+    for (int b = 0; b < B; ++b) m->row_pos[b] = past + S;
     XFT_CHECK_HIP(hipMemcpyAsync(m->ids, ids_host, (size_t)B * S * 4, hipMemcpyHostToDevice, st));
     hipLaunchKernelGGL(embed_kernel, dim3(B * S), dim3(256), 0, st, m->embedding, m->ids, m->x, c.hidden, c.vocab);
     for (int l = 0; l < c.layers; ++l)
-        if (int rc = layer_forward(m, l, m->x, c.hidden, m->x, c.hidden, B, S, 0, nullptr, st)) return rc;
+        if (int rc = layer_forward(m, l, m->x, c.hidden, m->x, c.hidden, B, S, past, nullptr, st)) return rc;
     hipLaunchKernelGGL(gather_last_kernel, dim3(B), dim3(256), 0, st, m->x, m->xlast, S, c.hidden);
     if (int rc = head_forward(m, m->xlast, B, false, st)) return rc;
-    hipLaunchKernelGGL(fill_int_kernel, dim3((B + 63) / 64), dim3(64), 0, st, m->pos, B, S);
+    hipLaunchKernelGGL(fill_int_kernel, dim3((B + 63) / 64), dim3(64), 0, st, m->pos, B, past + S);
     hipLaunchKernelGGL(fill_int_kernel, dim3(1), dim3(64), 0, st, m->step, 1, 0);
     XFT_CHECK_HIP(hipGetLastError());
     XFT_CHECK_HIP(hipStreamSynchronize(st));
     if (logits_host) XFT_CHECK_HIP(hipMemcpy(logits_host, m->logits, (size_t)B * c.vocab * 4, hipMemcpyDeviceToHost));
     m->cur_B = B;
-    m->cur_pos = S;
+    m->cur_pos = past + S;
     m->prompt_rows = B * S;
+    return 0;
+}
+
+int xfthip_model_prefill(xfthip_model_t m, const int *ids_host, int B, int S, float *logits_host, xfthip_stream_t stream) {
+    XFT_REQUIRE(m && ids_host, "xfthip_model_prefill: null argument");
+    m->prefix_len = 0; // cache row 0 is written from position 0
+    return prompt_pass(m, "xfthip_model_prefill", ids_host, B, S, 0, logits_host, (hipStream_t)stream);
+}
+
+int xfthip_model_set_prefix(xfthip_model_t m, const int *ids_host, int n, xfthip_stream_t stream) {
+    XFT_REQUIRE(m && ids_host && n > 0, "xfthip_model_set_prefix: bad argument");
+    if (int rc = prompt_pass(m, "xfthip_model_set_prefix", ids_host, 1, n, 0, nullptr, (hipStream_t)stream)) return rc;
+    m->prefix_len = n;
+    return 0;
+}
+
+int xfthip_model_prefill_after_prefix(xfthip_model_t m, const int *ids_host, int B, int S, float *logits_host, xfthip_stream_t stream) {
+    XFT_REQUIRE(m && ids_host, "xfthip_model_prefill_after_prefix: null argument");
+    XFT_REQUIRE(m->prefix_len > 0, "xfthip_model_prefill_after_prefix: no prefix in the cache (xfthip_model_set_prefix, and no plain prompt pass since)");
+    const xfthip_model_config &c = m->cfg;
+    XFT_REQUIRE(B > 0 && B <= c.max_batch, "xfthip_model_prefill_after_prefix: batch %d exceeds the model's %d cache rows", B, c.max_batch);
+    hipStream_t st = (hipStream_t)stream;
+    if (B > 1) {
+        // KVCacheManager::expandPrefixCache: every sequence's row starts as a copy of the prefix's positions (whole
+        // 32-token blocks; what lies behind the prefix in the last block is overwritten by the pass below)
+        std::vector<int> dst(B - 1), src(B - 1, 0);
+        for (int b = 1; b < B; ++b) dst[b - 1] = b;
+        for (int l = 0; l < c.layers; ++l)
+            if (int rc = xfthip_kvcache_reorder(m->caches[l], dst.data(), src.data(), B - 1, 0, m->prefix_len, stream)) return rc;
+    }
+    const int keep = m->prefix_len;
+    if (int rc = prompt_pass(m, "xfthip_model_prefill_after_prefix", ids_host, B, S, keep, logits_host, st)) return rc;
+    m->prefix_len = keep;
     return 0;
 }
 
@@ -817,6 +850,7 @@ int xfthip_model_seq_prefill(xfthip_model_t m, int row, const int *ids_host, int
     XFT_REQUIRE(S > 0 && S <= c.max_tokens && S < c.max_seq, "xfthip_model_seq_prefill: %d tokens exceed max_tokens %d / max_seq %d", S,
             c.max_tokens, c.max_seq);
     hipStream_t st = (hipStream_t)stream;
+    if (row == 0) m->prefix_len = 0; // the row of a shared prefix is written from position 0
     if ((int)m->row_pos.size() != c.max_batch) m->row_pos.assign(c.max_batch, -1);
     if (!m->active) {
         XFT_CHECK_HIP(hipMalloc((void **)&m->active, (size_t)c.max_batch * 4));

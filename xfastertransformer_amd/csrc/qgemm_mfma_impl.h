@@ -57,19 +57,21 @@ struct StepTraits<XFTHIP_W_INT8> {
     // a lane of half h takes the whole 16-byte chunks of k groups h and 2 + h (one 128-bit load each):
     // the k index of an MFMA is only a summation index, so lane half h of micro-step (g, sb) stands for
     // k = 32 g + 16 h + 8 sb .. + 7 in both operands
-    static constexpr int KTILE = 64, GROUPS = 2, SUB = 2, WREGS = 4;
+    static constexpr int KTILE = 64, GROUPS = 2, SUB = 2, WREGS = 4, PACKED_K = 64;
 };
 template <>
 struct StepTraits<XFTHIP_W_UINT4> {
-    static constexpr int KTILE = 128, GROUPS = 4, SUB = 2, WREGS = 4; // 16 bytes per lane per k group, 2 MFMAs
+    // 16 bytes per lane per k group, 2 MFMAs.  A step covers half a packed tile (two of its four k groups): with the
+    // whole 128-deep tile a step the three activation buffers of a 128-row block take 104 KB of LDS, one workgroup a CU
+    static constexpr int KTILE = 64, GROUPS = 2, SUB = 2, WREGS = 4, PACKED_K = 128;
 };
 template <>
 struct StepTraits<XFTHIP_W_NF4> {
-    static constexpr int KTILE = 128, GROUPS = 4, SUB = 2, WREGS = 4;
+    static constexpr int KTILE = 64, GROUPS = 2, SUB = 2, WREGS = 4, PACKED_K = 128;
 };
 template <>
 struct StepTraits<XFTHIP_W_BF16> {
-    static constexpr int KTILE = 32, GROUPS = 2, SUB = 1, WREGS = 4;
+    static constexpr int KTILE = 32, GROUPS = 2, SUB = 1, WREGS = 4, PACKED_K = 32;
 };
 
 // DEVROWS: the row count (and, for a group of weights, the weight) comes from device memory (SkinnyParams::rows_dev /
@@ -78,6 +80,7 @@ template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL, bool DEVROWS = fa
 __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nblocks_n, int nblocks_m) {
     using T = StepTraits<KIND>;
     constexpr int KTILE = T::KTILE, GROUPS = T::GROUPS, SUB = T::SUB, WREGS = T::WREGS;
+    constexpr int PACKED_K = T::PACKED_K, STEPS_PER_TILE = PACKED_K / KTILE; // k of a packed 1-KiB tile; steps that share one
     constexpr int ROWS = 32 * WM;
     constexpr int ROWB = KTILE * 2 + 16; // padded LDS row pitch in bytes
     constexpr int CHUNKS_PER_ROW = KTILE / 8; // 16-byte chunks
@@ -147,9 +150,9 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     if (p.ksplit > 1) {
         // this workgroup owns a range of k tiles: shift the operands to it, the result goes to its part
         const int kt0 = part * p.split_ktiles;
-        const int k_left = p.K - kt0 * KTILE, k_span = p.split_ktiles * KTILE;
+        const int k_left = p.K - kt0 * PACKED_K, k_span = p.split_ktiles * PACKED_K; // (split_ktiles counts packed tiles)
         p.packed += (size_t)kt0 * 1024;
-        p.A += (size_t)kt0 * KTILE;
+        p.A += (size_t)kt0 * PACKED_K;
         p.K = k_left < k_span ? k_left : k_span;
         p.C = p.split_part + ((size_t)part * part_rows + part_row) * p.N;
         p.ldc = p.N;
@@ -240,7 +243,7 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
                 const u32x4 v = *(const u32x4 *)(wbase[t] + (size_t)kt * 1024 + (2 * gq + h) * 256);
                 wreg[buf][gq][t][0] = v[0]; wreg[buf][gq][t][1] = v[1]; wreg[buf][gq][t][2] = v[2]; wreg[buf][gq][t][3] = v[3];
             } else {
-                const u32x4 v = *(const u32x4 *)(wbase[t] + (size_t)kt * 1024 + gq * 256);
+                const u32x4 v = *(const u32x4 *)(wbase[t] + (size_t)(kt / STEPS_PER_TILE) * 1024 + ((kt % STEPS_PER_TILE) * GROUPS + gq) * 256);
                 wreg[buf][gq][t][0] = v[0]; wreg[buf][gq][t][1] = v[1]; wreg[buf][gq][t][2] = v[2]; wreg[buf][gq][t][3] = v[3];
             }
         }
@@ -265,13 +268,29 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
 #pragma unroll
         for (int i = 0; i < ALOADS; ++i) load_a_part(set, kt_, i);
     };
-    auto store_a_part = [&](int set, int buf, int i) {
+    // NEED_SUM: the row sums of A (zero-point term) are gathered where the rows are staged: the thread that moves a
+    // 16-byte chunk into LDS adds its 8 values to a partial of its own; the partials of a row's chunks are joined after
+    // the k loop.  (They used to come from one more MFMA a row tile and micro-step against a tile of ones: as many
+    // MFMAs again as the product itself with one column tile a wave, and 16 WM accumulator registers.)
+    float rs_part[ALOADS];
+#pragma unroll
+    for (int i = 0; i < ALOADS; ++i) rs_part[i] = 0.0f;
+    auto store_a_part = [&](int set, int buf, int i, bool real_tile) {
         unsigned char *dst = abuf_base + buf * (ROWS * ROWB);
         *(u32x4 *)(dst + (a_row0 + i * ROW_STEP) * ROWB + a_kc * 16) = areg[set][i];
-    };
-    auto store_a = [&](int set, int buf) {
+        if constexpr (NEED_SUM) {
+            if (real_tile) { // (uniform: tiles past the end of K are copies of the last one)
 #pragma unroll
-        for (int i = 0; i < ALOADS; ++i) store_a_part(set, buf, i);
+                for (int w = 0; w < 4; ++w) {
+                    const uint32_t u = areg[set][i][w];
+                    rs_part[i] += u2f(u << 16) + u2f(u & 0xFFFF0000u);
+                }
+            }
+        }
+    };
+    auto store_a = [&](int set, int buf, bool real_tile) {
+#pragma unroll
+        for (int i = 0; i < ALOADS; ++i) store_a_part(set, buf, i, real_tile);
     };
     // k offset (elements) of micro-step ms inside a tile: lane (row/col, h) holds k = koff .. koff + 7
     auto koff_of = [&](int ms) {
@@ -338,7 +357,7 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
             if (sb == 0) load_w_part(wnext, kt_cur + 2, gq);
             if (ms % A_EVERY == 0) {
                 load_a_part(ab_next, kt_cur + 4, ms / A_EVERY);
-                store_a_part(wnext, wnext, ms / A_EVERY);
+                store_a_part(wnext, wnext, ms / A_EVERY, kt_cur + 2 < kt_n);
             }
             if (ms + 1 < MICRO)
                 read_frags((ms + 1) & 1, ab, ms + 1);
@@ -359,12 +378,6 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
                     if constexpr (KIND == XFTHIP_W_NF4)
                         acc[t][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[m].v, wcur_lo.v, acc[t][m], 0, 0, 0);
                     acc[t][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[m].v, wcur_hi.v, acc[t][m], 0, 0, 0);
-                }
-                if constexpr (NEED_SUM) {
-                    if (t + 1 == WN) {
-#pragma unroll
-                        for (int m = 0; m < WM; ++m) accS[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[m].v, ones.v, accS[m], 0, 0, 0);
-                    }
                 }
                 wcur_hi = nhi;
                 if constexpr (KIND == XFTHIP_W_NF4) wcur_lo = nlo;
@@ -387,7 +400,6 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
                         if (t == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                         if (VPER > 0) __builtin_amdgcn_sched_group_barrier(0x002, VPER, 0);
                     }
-                    if (NEED_SUM && t + 1 == WN) __builtin_amdgcn_sched_group_barrier(0x008, WM, 0);
                 }
             }
         }
@@ -401,11 +413,11 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     load_a(1, 1);
     load_a(2, 2);
     XFT_FENCE();
-    store_a(0, 0);
+    store_a(0, 0, true);
     XFT_FENCE();
     load_a(0, 3);
     XFT_FENCE();
-    store_a(1, 1);
+    store_a(1, 1, kt_n > 1);
     __syncthreads();
     read_frags(0, 0, 0);
     widen(0, 0, 0, wcur_hi, wcur_lo);
@@ -437,6 +449,23 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     constexpr int OPITCH = 32 * WN * 4 + 32; // patch row pitch in bytes
     __syncthreads(); // every wave is past its last read of the activation tiles
     unsigned char *obuf = abuf_base + wave * (32 * OPITCH);
+    if constexpr (NEED_SUM) {
+        // join the partial sums of a row's chunks (adjacent lanes), hand them over through LDS behind the patches, and
+        // give every lane the sums of the 16 rows it holds results of
+        float *rowsum = (float *)(abuf_base + 4 * 32 * OPITCH);
+#pragma unroll
+        for (int i = 0; i < ALOADS; ++i) {
+            float v = rs_part[i];
+#pragma unroll
+            for (int off = 1; off < CHUNKS_PER_ROW; off <<= 1) v += __shfl_xor(v, off, 64);
+            if (a_kc == 0) rowsum[a_row0 + i * ROW_STEP] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < WM; ++m)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) accS[m][j] = rowsum[32 * m + 8 * (j >> 2) + 4 * h + (j & 3)];
+    }
     const bool c_wide = (((size_t)p.C | ((size_t)p.ldc * (p.c_dtype == XFTHIP_F32 ? 4 : 2))) & 15) == 0;
     const bool res_wide = (((size_t)p.res | ((size_t)p.ldres * (p.res_dtype == XFTHIP_F32 ? 4 : 2))) & 15) == 0;
     auto wave_sync = [&]() {
@@ -609,7 +638,8 @@ static int launch_big2(const SkinnyParams &p, hipStream_t stream) {
     const int nb8 = (nblocks_n + 7) / 8;
     const int blocks = nb8 * 8 * nblocks_m;
     // the three activation buffers, reused after the k loop by the four waves' output patches
-    const size_t pipe = 3 * ROWS * ROWB, patches = 4 * 32 * (32 * WN * 4 + 32);
+    // (the row sums of the zero-point term sit behind the patches)
+    const size_t pipe = 3 * ROWS * ROWB, patches = 4 * 32 * (32 * WN * 4 + 32) + (NEED_SUM ? ROWS * sizeof(float) : 0);
     const size_t smem = (pipe > patches ? pipe : patches) + (KIND == XFTHIP_W_NF4 ? 2048 : 0);
     if (smem > 64 * 1024) {
         // more dynamic LDS than the default limit: raise it once per instantiation
@@ -670,8 +700,10 @@ static int dispatch_big_tile(const SkinnyParams &p, hipStream_t stream) {
         // (one wave per SIMD, nothing to run while it waits) stays at 750-760 wherever it applies
         if (rows > 1024 && t_mid >= cus) return launch_big<KIND, 1, 4, NEED_SUM>(p, stream);
     } else {
-        // 4-bit kinds: the 128 x 128 tile holds half the accumulators of the 128 x 256 one at the
-        // same occupancy (LDS for the 128-deep k tile) and never won
+        // 4-bit kinds: 128 x 256 tiles, one workgroup a CU.  With 64-deep steps and the row sums gathered at the
+        // staging step the 128 x 128 tile fits two workgroups a CU like the INT8 one, but measured no better overall at
+        // 2048 rows (UINT4 751 / 766 / 813 TFLOP/s against 785 / 743 / 861 on 4096^2, 11008 x 4096, 4096 x 11008; NF4
+        // 515 / 512 / 551 against 495 / 483 / 540)
         if (rows > 512 && t_large >= cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
     }
     if constexpr (KIND != XFTHIP_W_BF16) {

@@ -192,8 +192,6 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     for (int m = 0; m < WM; ++m)
 #pragma unroll
         for (int j = 0; j < 16; ++j) accS[m][j] = 0.0f;
-    MFrag ones;
-    ones.u[0] = ones.u[1] = ones.u[2] = ones.u[3] = 0x3F803F80u;
 
     // weight source of this lane: 16-column packed tile (2 per 32-column MFMA tile), chunk of
     // its column inside the tile, and which 8-byte half (INT8) / dword pair (4-bit) it uses

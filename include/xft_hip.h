@@ -252,6 +252,11 @@ int xfthip_kvcache_reorder(xfthip_kvcache_t cache, const int *dst_rows_host, con
 int xfthip_kvcache_export(xfthip_kvcache_t c, int which, void *data_dev, float *scales_dev, xfthip_stream_t stream);
 int xfthip_kvcache_import(xfthip_kvcache_t c, int which, const void *data_dev, const float *scales_dev,
         xfthip_stream_t stream);
+/* the same with data_dev laid out [maxSeq][B][H][D], the reference's layout when ENABLE_KV_TRANS is off
+ * (src/common/kvcache_tensor.h:113-117); the scales stay [B][H][maxSeq] as there */
+int xfthip_kvcache_export_sbhd(xfthip_kvcache_t c, int which, void *data_dev, float *scales_dev, xfthip_stream_t stream);
+int xfthip_kvcache_import_sbhd(xfthip_kvcache_t c, int which, const void *data_dev, const float *scales_dev,
+        xfthip_stream_t stream);
 /*
  * RoPE on q and k, then append k and v of S new tokens per sequence to the cache at
  * positions past .. past+S-1.  Replaces the RoPE call of Attention::forward

@@ -155,6 +155,16 @@ def test_kv_import_export_roundtrip(xh, orc, int8):
         assert np.array_equal(d, data)
         if int8:
             assert np.array_equal(s, scales)
+        # the reference's other layout, [S][B][H][D] (ENABLE_KV_TRANS off, kvcache_tensor.h:113-117): out of the same cache,
+        # and into a fresh one
+        sbhd = np.ascontiguousarray(data.transpose(2, 0, 1, 3))
+        d2, s2 = cache.export(which, sbhd=True)
+        assert np.array_equal(d2, sbhd) and (not int8 or np.array_equal(s2, scales))
+        other = xh.KVCache(xh.INT8 if int8 else xh.FP16, B, H, S, D)
+        other.load(which, sbhd, scales, sbhd=True)
+        d3, s3 = other.export(which)
+        assert np.array_equal(d3, data) and (not int8 or np.array_equal(s3, scales))
+        other.free()
 
 
 # index vectors of the reference's own reorder test (tests/ut/kv_reorder_test.cpp:64-124): the fixed ones of

@@ -314,25 +314,27 @@ class KVCache:
     def _np_dtype(self):
         return np.int8 if self.dtype == INT8 else np.uint16
 
-    def export(self, which):
-        """Reference layout: data [B][H][maxSeq][D] (fp16 bits / int8), scales [B][H][maxSeq]."""
+    def export(self, which, sbhd=False):
+        """Reference layouts: data [B][H][maxSeq][D] (fp16 bits / int8), or [maxSeq][B][H][D] with sbhd; scales [B][H][maxSeq]."""
         n = self.B * self.H * self.S
         data = DeviceBuffer(n * self.D * (1 if self.dtype == INT8 else 2))
         scales = DeviceBuffer(n * 4)
         scales.zero()
-        check(lib.xfthip_kvcache_export(self.h, which, data.ptr, scales.ptr, None))
+        fn = lib.xfthip_kvcache_export_sbhd if sbhd else lib.xfthip_kvcache_export
+        check(fn(self.h, which, data.ptr, scales.ptr, None))
         synchronize()
-        return (data.to_numpy(self._np_dtype(), (self.B, self.H, self.S, self.D)),
-                scales.to_numpy(np.float32, (self.B, self.H, self.S)))
+        shape = (self.S, self.B, self.H, self.D) if sbhd else (self.B, self.H, self.S, self.D)
+        return (data.to_numpy(self._np_dtype(), shape), scales.to_numpy(np.float32, (self.B, self.H, self.S)))
 
-    def load(self, which, data, scales=None):
+    def load(self, which, data, scales=None, sbhd=False):
         data = np.ascontiguousarray(data, self._np_dtype())
-        assert data.shape == (self.B, self.H, self.S, self.D)
+        assert data.shape == ((self.S, self.B, self.H, self.D) if sbhd else (self.B, self.H, self.S, self.D))
         d = DeviceBuffer.from_numpy(data)
         s = None
         if self.dtype == INT8:
             s = DeviceBuffer.from_numpy(np.ascontiguousarray(scales, np.float32))
-        check(lib.xfthip_kvcache_import(self.h, which, d.ptr, None if s is None else s.ptr, None))
+        fn = lib.xfthip_kvcache_import_sbhd if sbhd else lib.xfthip_kvcache_import
+        check(fn(self.h, which, d.ptr, None if s is None else s.ptr, None))
         synchronize()
 
     def reorder(self, dst_rows, src_rows, pos0, pos1, stream=None):

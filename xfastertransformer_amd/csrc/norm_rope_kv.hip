@@ -294,8 +294,10 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(RopeKvParams p) {
     }
 }
 
-// ---- export / import between the private layout and [B][H][S][D] ----------------------------
-__global__ void kv_convert_kernel(KvView kv, int which, void *data, float *scales, int maxSeq, int to_private) {
+// ---- export / import between the private layout and the reference's two layouts -----------------
+// sbhd = 0: [B][H][S][D] (ENABLE_KV_TRANS, src/common/kvcache_tensor.h:108-112); 1: [S][B][H][D] (:113-117).  The
+// INT8 scales are [B][H][S] in both.
+__global__ void kv_convert_kernel(KvView kv, int which, void *data, float *scales, int maxSeq, int to_private, int sbhd) {
     const size_t total = (size_t)kv.B * kv.H * maxSeq * kv.D;
     const int esz = kv.int8 ? 1 : 2;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
@@ -312,7 +314,9 @@ __global__ void kv_convert_kernel(KvView kv, int which, void *data, float *scale
             priv = (char *)kv.v;
             poff = (bh * (kv.S / 32) + (t >> 5)) * (size_t)kv.D * 32 + (size_t)d * 32 + v_slot(t & 31);
         }
-        char *ext = (char *)data + i * esz;
+        const size_t b_of = bh / kv.H, h_of = bh % kv.H;
+        const size_t ei = sbhd ? (((size_t)t * kv.B + b_of) * kv.H + h_of) * kv.D + d : i;
+        char *ext = (char *)data + ei * esz;
         char *in = priv + poff * esz;
         if (to_private) {
             for (int bte = 0; bte < esz; ++bte) in[bte] = ext[bte];
@@ -520,13 +524,13 @@ int xfthip_kvcache_destroy(xfthip_kvcache_t c) {
     return 0;
 }
 
-static int kv_convert(xfthip_kvcache_t c, int which, void *data, float *scales, int to_private, hipStream_t stream) {
+static int kv_convert(xfthip_kvcache_t c, int which, void *data, float *scales, int to_private, hipStream_t stream, int sbhd = 0) {
     XFT_REQUIRE(c && data, "xfthip_kvcache_export/import: null argument");
     XFT_REQUIRE(which == 0 || which == 1, "xfthip_kvcache_export/import: which must be 0 (keys) or 1 (values)");
     const size_t total = (size_t)c->kv.B * c->kv.H * c->maxSeq * c->kv.D;
     int blocks = (int)((total + 255) / 256 > 1048576 ? 1048576 : (total + 255) / 256);
     hipLaunchKernelGGL(kv_convert_kernel, dim3(blocks), dim3(256), 0, stream, c->kv, which, data, scales, c->maxSeq,
-            to_private);
+            to_private, sbhd);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }
@@ -539,6 +543,16 @@ int xfthip_kvcache_import(xfthip_kvcache_t c, int which, const void *data_dev, c
         xfthip_stream_t stream) {
     XFT_REQUIRE(!(c && c->kv.int8) || scales_dev, "xfthip_kvcache_import: INT8 cache needs scales");
     return kv_convert(c, which, (void *)data_dev, (float *)scales_dev, 1, (hipStream_t)stream);
+}
+
+int xfthip_kvcache_export_sbhd(xfthip_kvcache_t c, int which, void *data_dev, float *scales_dev, xfthip_stream_t stream) {
+    return kv_convert(c, which, data_dev, scales_dev, 0, (hipStream_t)stream, 1);
+}
+
+int xfthip_kvcache_import_sbhd(xfthip_kvcache_t c, int which, const void *data_dev, const float *scales_dev,
+        xfthip_stream_t stream) {
+    XFT_REQUIRE(!(c && c->kv.int8) || scales_dev, "xfthip_kvcache_import_sbhd: INT8 cache needs scales");
+    return kv_convert(c, which, (void *)data_dev, (float *)scales_dev, 1, (hipStream_t)stream, 1);
 }
 
 int xfthip_rope_kvstore(xfthip_kvcache_t c, void *qkv, int dtype, int stride, int B, int S, int qHeads,

@@ -157,6 +157,27 @@ def test_chunked_prefill_over_cache(xh, orc, int8):
     assert _cos(got, exp) >= 0.9999
 
 
+@pytest.mark.parametrize("int8", [0, 1])
+def test_short_chunk_over_a_long_cache(xh, orc, int8):
+    """Three new tokens per sequence over 3000 cached ones, one sequence, 8 KV heads: 12 columns in one column group,
+    the sequence cut into 24 parts whose merge is a launch of its own over those 12 columns."""
+    rng = np.random.default_rng(35)
+    B, qh, kvh, past, S = 1, 32, 8, 3000, 3
+    kc, vc, dc = _filled(xh, orc, rng, int8, B, kvh, 3072, past)
+    stride = (qh + 2 * kvh) * D
+    qkv = orc.round_bf16(rng.standard_normal((B * S, stride)))
+    dev = xh.DeviceBuffer.from_numpy(orc.to_bf16(qkv))
+    xh.rope_kvstore(dc, dev.ptr, xh.BF16, stride, B, S, qh, None, past)
+    od = xh.DeviceBuffer(B * S * qh * D * 4)
+    xh.attention(dc, dev.ptr, stride, od.ptr, qh * D, xh.F32, B, S, qh, SCALE, past)
+    xh.synchronize()
+    got = od.to_numpy(np.float32, (B * S, qh * D))
+    exp = orc.cross_attn_by_head(qkv[:, :qh * D].copy(), qkv[:, qh * D:(qh + kvh) * D].copy(),
+                                 qkv[:, (qh + kvh) * D:].copy(), qh, kvh, D, [S] * B, [past] * B, SCALE, kc, vc)
+    assert np.abs(got - exp).max() < (2e-2 if int8 else 3e-3)
+    assert _cos(got, exp) >= 0.9999
+
+
 @pytest.mark.parametrize("n,S", [(900, 1024), (4000, 4096)])
 def test_split_count_independence(xh, orc, n, S):
     """The same query against the same rows gives the same answer whether the sequence is left whole (a large batch:

@@ -99,6 +99,35 @@ def test_forward_returns_the_logits_of_every_position(torch_class, model_dir):
     assert float((full[:, 1:] - full[:, :-1]).abs().max()) > 1e-2
 
 
+def test_prefix_sharing_through_the_class(torch_class, model_dir):
+    """set_prefix / unset_prefix (src/pytorch/auto_model.h: setPrefix / unsetPrefix): generation over a shared prefix
+    gives the ids of generation from the whole prompts (FP16 cache: the same keys and values bit for bit)."""
+    import torch
+    path, held = model_dir
+    V = held["cfg"]["vocab"]
+    B, n, tail, max_len = 2, 33, 5, 50
+    g = torch.Generator().manual_seed(12)
+    prefix = torch.randint(0, V, (1, n), generator=g)
+    ids = torch.cat([prefix.repeat(B, 1), torch.randint(0, V, (B, tail), generator=g)], 1)
+
+    def run(m):
+        m.config(max_len, 1, 1, 1.0, False, V + 1, None, False, 1.0, 50, 1.0, 1.0, None)
+        m.input(ids)
+        while not m.is_done():
+            m.generate()
+        return m.finalize()
+
+    m = torch_class(path, "int8", "fp16")
+    whole = run(m)
+    m.set_prefix(prefix)
+    shared = run(m)
+    m.unset_prefix()
+    again = run(m)
+    assert torch.equal(shared, whole) and torch.equal(again, whole)
+    with pytest.raises(Exception):
+        m.set_prefix(ids)  # one prompt only
+
+
 def test_sequence_id_interface(torch_class, am, model_dir):
     """set_input_cb with ragged prompts (1-D ids + lengths), forward_cb, tokens chosen by the caller fed back
     with set_input_cb(ids, None, seqIDs, None), a sequence that sits out, free_seqs: every sequence follows

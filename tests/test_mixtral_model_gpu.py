@@ -8,6 +8,7 @@ decoder_block.h:640-676 reads them).  The directory is written by tests/golden/m
     (LlamaLayerOracle with its MLP half replaced by mixtral_mlp), teacher-forced with the GPU's tokens;
   * decode steps replayed from the captured graph equal the eager ones, and a second, longer generation (which
     rebuilds the device model and with it the sparse MLPs' buffers) still equals the direct model's."""
+import ctypes as C
 import os
 import sys
 
@@ -126,3 +127,74 @@ def test_mixtral_directory_generates_what_the_directly_built_model_does(xh, orc,
     direct.free()
     for m in reversed(moes):
         m.free()
+
+
+def test_mixtral_8x7b_shape_layer_at_context_4096(xh, orc):
+    """The Mixtral-8x7B-shape layer at full size: GQA attention (32 query / 8 KV heads) at context 4096 followed by the
+    sparse MLP (hidden 4096, FFN 14336, 8 INT8 experts, top-2) over 256 tokens.  The device layer takes 3840 tokens
+    first and then the 256-token chunk over that past; the oracle follows three of the 256 tokens through the whole
+    layer (attention over their 3841 .. 4096 cached tokens, router, their two experts)."""
+    hidden, inter, E, qh, kvh, ctx, tokens = 4096, 14336, 8, 32, 8, 4096, 256
+    past = ctx - tokens
+    rng = np.random.default_rng(4)
+    wqkv = orc.quantize(0, (rng.standard_normal((hidden, (qh + 2 * kvh) * 128)) * 0.02).astype(np.float32))
+    wo = orc.quantize(0, (rng.standard_normal((qh * 128, hidden)) * 0.02).astype(np.float32))
+    # one expert's random codes shared by all experts keeps host time short; scales differ per expert
+    q_gu = rng.integers(-127, 128, (hidden, 2 * inter)).astype(np.int8)
+    q_dn = rng.integers(-127, 128, (inter, hidden)).astype(np.int8)
+    experts = []
+    for e in range(E):
+        s_gu = np.full(2 * inter, 0.02 * 1.7 / 127 * (1 + 0.05 * e), np.float32)
+        s_dn = np.full(hidden, 0.02 * 1.7 / 127 * (1 - 0.03 * e), np.float32)
+        experts.append((orc.QWeight(0, hidden, 2 * inter, q_gu, s_gu, np.zeros(2 * inter, np.float32)),
+                        orc.QWeight(0, inter, hidden, q_dn, s_dn, np.zeros(hidden, np.float32))))
+    router = (rng.standard_normal((hidden, E)) * 0.05).astype(np.float32)
+    ln1 = rng.uniform(0.9, 1.1, hidden).astype(np.float32)
+    ln2 = rng.uniform(0.9, 1.1, hidden).astype(np.float32)
+    x = orc.round_bf16(rng.standard_normal((ctx, hidden)))
+
+    model = xh.Model(1, hidden, inter, qh, kvh, 128, vocab=0, max_batch=1, max_seq=ctx, max_tokens=past)
+    dev = lambda w, flags=0: xh.Weight(0, w.K, w.N, w.q, w.scale, None, flags=flags)
+    moe = xh.MoE(hidden, inter, E, past, router, ln2)
+    for e, (gu, dn) in enumerate(experts):
+        moe.set_expert(e, dev(gu, xh.WF_GATEUP), dev(dn))
+    model.set_sparse_layer(0, dev(wqkv), dev(wo), moe, ln1)
+    xd = xh.DeviceBuffer.from_numpy(x)
+    od = xh.DeviceBuffer(x.nbytes)
+    model.layer_forward(0, xd.ptr, od.ptr, 1, past, 0)
+    off = past * hidden * 4
+    model.layer_forward(0, C.c_void_p(xd.ptr.value + off), C.c_void_p(od.ptr.value + off), 1, tokens, past)
+    xh.synchronize()
+    got = od.to_numpy(np.float32, x.shape)[past:]
+    assert np.isfinite(got).all()
+
+    # oracle: projections of all 4096 tokens through BLAS on the dequantised weight (compared with the scalar GEMM in the
+    # CPU tests), the cache filled with them, then three tokens of the chunk through attention and the sparse MLP
+    xn = orc.round_bf16(orc.rmsnorm(x, ln1, 1e-6))
+    qkv = orc.round_bf16(orc.blas_gemm(wqkv, xn))
+    layer = orc.LlamaLayerOracle(hidden, inter, qh, kvh, 128, wqkv, wo, None, None, ln1, ln2, batch=1, max_seq=ctx, max_pos=ctx,
+                                 rounding="bf16", gemm="blas", prefill_attention="cache", moe=(router, experts))
+    qcols, kvcols = qh * 128, kvh * 128
+    flat = qkv.reshape(-1)
+    orc.lib.orc_rope_apply(C.c_void_p(flat.ctypes.data), C.c_void_p(flat.ctypes.data + qcols * 4), qkv.shape[1], qkv.shape[1],
+                           orc.p(layer.cos), orc.p(layer.sin), 64, orc.p(orc.i32([1, ctx, qh, 128, kvh])), orc.p(orc.i32(np.arange(ctx))))
+    q = orc.round_bf16(np.ascontiguousarray(qkv[:, :qcols]))
+    k = np.ascontiguousarray(qkv[:, qcols:qcols + kvcols])
+    v = np.ascontiguousarray(qkv[:, qcols + kvcols:])
+    layer.kc.store(0, 0, k)
+    layer.vc.store(0, 0, v)
+    scale = 1.0 / np.sqrt(128.0)
+    worst = 0.0
+    for t in (past, past + 77, ctx - 1):
+        att = orc.cross_attn_by_head(q[t:t + 1].copy(), k[t:t + 1].copy(), v[t:t + 1].copy(), qh, kvh, 128, [1], [t], scale, layer.kc, layer.vc)
+        x1 = orc.blas_gemm(wo, orc.round_bf16(att), epi=orc.EPI_RESIDENTIAL, res=x[t:t + 1])
+        ref = orc.mixtral_mlp(x1, ln2, router, experts, rounding="bf16")[0]
+        err = float(np.abs(got[t - past] - ref[0]).max())
+        worst = max(worst, err)
+        assert err < 3e-2 * max(1.0, float(np.abs(ref).max())), (t, err)
+        assert float(got[t - past].astype(np.float64) @ ref[0].astype(np.float64)
+                     / np.sqrt((got[t - past].astype(np.float64) ** 2).sum() * (ref[0].astype(np.float64) ** 2).sum())) >= 0.9999
+    print(f"Mixtral-shape layer at context {ctx}: worst max-abs over three followed tokens {worst:.3e}", flush=True)
+    orc.clear_blas_cache()
+    model.free()
+    moe.free()

@@ -74,15 +74,38 @@ struct StepTraits<XFTHIP_W_BF16> {
     static constexpr int KTILE = 32, GROUPS = 2, SUB = 1, WREGS = 4, PACKED_K = 32;
 };
 
+// Row blocks a band: 8, or, with a device-side row count, only as many as the rows the host expects fill: the
+// workgroups that do work then come first in the launch order and spread over the CUs; the ones past the count (which
+// leave at once) follow them instead of sitting between them.  (Host and device: the grid is sized with it.)
+template <int ROWS, bool DEVROWS>
+__host__ __device__ inline int band_rows(const SkinnyParams &p) {
+    if constexpr (DEVROWS) {
+        if (!p.group) {
+            const int want = (p.m_hint + ROWS - 1) / ROWS;
+            return want < 1 ? 1 : want < 8 ? want : 8;
+        }
+    }
+    return 8;
+}
+
 // DEVROWS: the row count (and, for a group of weights, the weight) comes from device memory (SkinnyParams::rows_dev /
 // group); a form of its own, so that the plain kernels carry none of it
-template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL, bool DEVROWS = false>
-__global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nblocks_n, int nblocks_m) {
+//
+// DIRECT: the activation tiles go from global memory straight into LDS (global_load_lds_dwordx4: a wave instruction
+// fills 1 KiB of consecutive LDS, lane after lane, from 64 addresses of its choice) instead of through registers and
+// ds_write.  Rows are 128 bytes with no padding; the 16-byte chunk c of row r sits in slot c ^ ((r >> 1) & 7) of its
+// row, which a lane gets by choosing the global chunk it fetches, and which keeps the operand reads (32 rows, one
+// chunk index) free of bank conflicts.  Four LDS tiles: step k requests tile k + 3, and the barrier that ends a step
+// first waits until the wave's requests of the step before are in (vmcnt counts them in order with the weight
+// loads).  Without the staging registers the 128 x 256 tile fits two workgroups a CU.
+template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL, bool DEVROWS = false, bool DIRECT = false>
+__global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyParams p, int nblocks_n, int nblocks_m) {
     using T = StepTraits<KIND>;
     constexpr int KTILE = T::KTILE, GROUPS = T::GROUPS, SUB = T::SUB, WREGS = T::WREGS;
     constexpr int PACKED_K = T::PACKED_K, STEPS_PER_TILE = PACKED_K / KTILE; // k of a packed 1-KiB tile; steps that share one
     constexpr int ROWS = 32 * WM;
-    constexpr int ROWB = KTILE * 2 + 16; // padded LDS row pitch in bytes
+    constexpr int ROWB = DIRECT ? KTILE * 2 : KTILE * 2 + 16; // LDS row pitch in bytes (padded when staged through registers)
+    static_assert(!DIRECT || (KTILE == 64 && !KTAIL && !DEVROWS && ROWS % 32 == 0), "direct-to-LDS form: 64-deep steps, whole k tiles, host-side row count");
     constexpr int CHUNKS_PER_ROW = KTILE / 8; // 16-byte chunks
     constexpr int TOTAL_CHUNKS = ROWS * CHUNKS_PER_ROW;
     constexpr int ALOADS = TOTAL_CHUNKS / 256;
@@ -92,33 +115,27 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = lane >> 5, nl = lane & 31;
     const int part_rows = p.M; // rows of a K part: the host's bound, also when the device knows fewer
-    // workgroup -> (K part, column block, row block): workgroups that share a column block sit on the same XCD
-    // (workgroup ids round-robin over the 8 XCDs in launch order), so their weight reads hit that XCD's L2.  Row
-    // blocks are walked in bands of 8: all K parts and column blocks of a band before the next band, so that the
-    // band's activation rows stay cached while the weights stream past them.
+    // workgroup -> (K part, column block, row block).  Row blocks are walked in bands of 8; a unit of work is one
+    // (band, K part, column block): its 8 workgroups share the column block's weights.  Workgroup ids go round the 8
+    // XCDs in launch order, so the units are dealt out to the XCDs one by one - an XCD runs the 8 workgroups of a unit
+    // next to each other (the weights pass through its L2 once) and its units follow each other column block by column
+    // block inside a band (the band's activation rows stay in its L2 while the weights stream past them) - and the
+    // XCDs carry the same load whatever the number of column blocks (43 blocks of 256 columns dealt out block by block
+    // would give three XCDs 6 and five XCDs 5).
     int nb, mb, part;
     {
-        // With a device-side row count the band is only as tall as the rows the host expects: the workgroups
-        // that do work then come first in the launch order and spread over the CUs; the ones past the count
-        // (which leave at once) follow them instead of sitting between them.
-        int BAND = 8;
-        if constexpr (DEVROWS) {
-            if (!p.group) {
-                const int want = (p.m_hint + ROWS - 1) / ROWS;
-                BAND = want < 1 ? 1 : want < 8 ? want : 8;
-            }
-        }
+        const int BAND = band_rows<ROWS, DEVROWS>(p);
         const int parts = p.ksplit > 1 ? p.ksplit : 1;
-        const int id = blockIdx.y * gridDim.x + blockIdx.x, xcd = id & 7, slot = id >> 3; // gridDim.x is a multiple of 8
-        const int nb8 = (nblocks_n + 7) >> 3;
-        if (slot >= nb8 * nblocks_m * parts) return;
-        const int band = slot / (nb8 * BAND * parts), rem_band = slot - band * (nb8 * BAND * parts);
-        const int left = nblocks_m - band * BAND, rows_in_band = left < BAND ? left : BAND;
-        part = rem_band / (nb8 * rows_in_band);
-        const int rem = rem_band - part * (nb8 * rows_in_band);
-        nb = rem / rows_in_band + xcd * nb8;
-        mb = band * BAND + rem % rows_in_band;
-        if (nb >= nblocks_n) return;
+        const int id = blockIdx.x, xcd = id & 7, slot = id >> 3; // gridDim.x is a multiple of 8
+        const int nbands = (nblocks_m + BAND - 1) / BAND;
+        const int units = nbands * parts * nblocks_n;
+        const int unit = (slot / BAND) * 8 + xcd;
+        if (unit >= units) return;
+        const int band = unit / (parts * nblocks_n), rem = unit - band * (parts * nblocks_n);
+        part = rem / nblocks_n;
+        nb = rem - part * nblocks_n;
+        mb = band * BAND + slot % BAND;
+        if (mb >= nblocks_m) return;
     }
     int c_row = 0, part_row = 0; // first row of this GEMM in C and in a K part
     if constexpr (DEVROWS) {
@@ -168,8 +185,10 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     uint2 *lut = nullptr;
     unsigned char *abuf_base = lds;
     if constexpr (KIND == XFTHIP_W_NF4) {
-        lut = (uint2 *)lds;
-        abuf_base = lds + 2048;
+        // DIRECT: the table sits behind the tiles, which then start at LDS offset 0 of the workgroup and end below 64 KiB
+        // (the requests carry their LDS address in M0)
+        lut = (uint2 *)(DIRECT ? lds + 4 * ROWS * ROWB : lds);
+        abuf_base = DIRECT ? lds : lds + 2048;
         {
             const int i = threadIdx.x;
             const float c0 = c_nf4_big[i & 15], c1 = c_nf4_big[i >> 4];
@@ -208,9 +227,18 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     uint32_t a_off[ALOADS];
 #pragma unroll
     for (int i = 0; i < ALOADS; ++i) {
-        int row = m0 + a_row0 + i * ROW_STEP;
-        row = row < p.M ? row : p.M - 1;
-        a_off[i] = (uint32_t)row * (uint32_t)p.lda + a_kc * 8;
+        if constexpr (DIRECT) {
+            // request i of this wave fills LDS chunks 64 (ALOADS wave + i) ..+ 63 = rows 8 (ALOADS wave + i) ..+ 7;
+            // this lane's chunk is slot lane & 7 of row lane >> 3 of those, which holds global chunk slot ^ swizzle(row)
+            const int r = 8 * (ALOADS * (int)(threadIdx.x >> 6) + i) + (lane >> 3);
+            int row = m0 + r;
+            row = row < p.M ? row : p.M - 1;
+            a_off[i] = ((uint32_t)row * (uint32_t)p.lda + ((lane & 7) ^ ((r >> 1) & 7)) * 8) * 2; // in bytes
+        } else {
+            int row = m0 + a_row0 + i * ROW_STEP;
+            row = row < p.M ? row : p.M - 1;
+            a_off[i] = (uint32_t)row * (uint32_t)p.lda + a_kc * 8;
+        }
     }
 
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
@@ -266,6 +294,27 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
 #pragma unroll
         for (int i = 0; i < ALOADS; ++i) load_a_part(set, kt_, i);
     };
+    // DIRECT: request i of this wave's share of activation tile kt_ into LDS tile buf (wave-uniform)
+    // (Written as assembly: after the compiler's own builtin for this instruction it makes every later wait for a load
+    // or an LDS read a wait for all of them - an instruction of the flat family that touches both memories - which
+    // takes the two-tiles-ahead weight loads out of flight at every step.  Unaware of these requests, the compiler's
+    // counted waits for the weight loads come out a few requests early, never late: the counter retires in order.
+    // M0 carries the LDS address of the wave's first lane; one wait state between writing it and the request.)
+    const uint32_t lds_tiles = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)abuf_base +
+            ALOADS * 1024 * (uint32_t)__builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint64_t a_bits = (uint64_t)(uintptr_t)p.A; // the same in every lane; said so, for a scalar register pair
+    const uint16_t *a_uniform = (const uint16_t *)(uintptr_t)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(a_bits >> 32)) << 32) |
+            (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a_bits));
+    auto direct_a_part = [&](int buf, int kt_, int i) {
+        const int kt = __builtin_amdgcn_readfirstlane(kt_ < kt_n ? kt_ : kt_n - 1);
+        const uint32_t dst = lds_tiles + buf * (ROWS * ROWB) + i * 1024;
+        const uint16_t *src = a_uniform + (size_t)kt * KTILE;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(a_off[i]), "s"(src) : "memory");
+    };
+    auto direct_a = [&](int buf, int kt_) {
+#pragma unroll
+        for (int i = 0; i < ALOADS; ++i) direct_a_part(buf, kt_, i);
+    };
     // NEED_SUM: the row sums of A (zero-point term) are gathered where the rows are staged: the thread that moves a
     // 16-byte chunk into LDS adds its 8 values to a partial of its own; the partials of a row's chunks are joined after
     // the k loop.  (They used to come from one more MFMA a row tile and micro-step against a tile of ones: as many
@@ -295,11 +344,17 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
         const int gq = ms / SUB, sb = ms % SUB;
         return KIND == XFTHIP_W_INT8 ? 32 * gq + 16 * h + 8 * sb : KIND == XFTHIP_W_BF16 ? 16 * gq + 8 * h : 32 * gq + 16 * sb + 8 * h;
     };
+    // DIRECT + NEED_SUM: wave w walks the row tiles in the order w, w + 1, .. (mod WM), so that the operand it sums for
+    // the zero-point term (below) is always the first one it reads - no branch on the wave number inside the k loop
+    constexpr bool ROTATE = DIRECT && NEED_SUM;
+    const int wave_first = ROTATE ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
+    auto row_tile = [&](int m) { return ROTATE ? (m + wave_first) % WM : m; };
     MFrag afr[2][WM];
     auto read_frags = [&](int slot, int ab, int ms) {
-        const unsigned char *src = abuf_base + ab * (ROWS * ROWB) + nl * ROWB + koff_of(ms) * 2;
+        const unsigned char *src = abuf_base + ab * (ROWS * ROWB) + nl * ROWB +
+                (DIRECT ? (((koff_of(ms) >> 3) ^ ((nl >> 1) & 7)) << 4) : koff_of(ms) * 2);
 #pragma unroll
-        for (int m = 0; m < WM; ++m) afr[slot][m].q = *(const u32x4 *)(src + m * 32 * ROWB);
+        for (int m = 0; m < WM; ++m) afr[slot][m].q = *(const u32x4 *)(src + row_tile(m) * 32 * ROWB);
     };
     // one MFMA k step = 16 k.  Operands of micro-step ms sit in afr[ms & 1]; the next set (of the
     // next tile's buffer after the last micro-step) is read while this one's MFMAs run.
@@ -348,20 +403,35 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     // VALU instructions one widening takes (a hint for the instruction interleave below)
     constexpr int VW = KIND == XFTHIP_W_INT8 ? 12 : KIND == XFTHIP_W_UINT4 ? 9 : KIND == XFTHIP_W_NF4 ? 6 : 0;
     constexpr int VPER = (VW + WM - 1) / WM;
-    auto compute = [&](int wb, int ab, int ab_next, int wnext, int kt_cur) {
+    // DIRECT: lds_cur / lds_next / lds_req = LDS tiles of activation tile kt_cur, kt_cur + 1 and kt_cur + 3 (the one this
+    // step requests); staged form: the LDS tiles are numbered like the register sets (ab, ab_next, wnext)
+    float rs_direct = 0.0f; // DIRECT + NEED_SUM: wave w sums the rows of row tile w, the first operand it reads
+    auto compute = [&](int wb, int ab, int ab_next, int wnext, int kt_cur, int lds_cur, int lds_next, int lds_req) {
 #pragma unroll
         for (int ms = 0; ms < MICRO; ++ms) {
             const int gq = ms / SUB, sb = ms % SUB;
             if (sb == 0) load_w_part(wnext, kt_cur + 2, gq);
             if (ms % A_EVERY == 0) {
-                load_a_part(ab_next, kt_cur + 4, ms / A_EVERY);
-                store_a_part(wnext, wnext, ms / A_EVERY, kt_cur + 2 < kt_n);
+                if constexpr (DIRECT) {
+                    direct_a_part(lds_req, kt_cur + 3, ms / A_EVERY);
+                } else {
+                    load_a_part(ab_next, kt_cur + 4, ms / A_EVERY);
+                    store_a_part(wnext, wnext, ms / A_EVERY, kt_cur + 2 < kt_n);
+                }
             }
             if (ms + 1 < MICRO)
-                read_frags((ms + 1) & 1, ab, ms + 1);
+                read_frags((ms + 1) & 1, lds_cur, ms + 1);
             else
-                read_frags((ms + 1) & 1, ab_next, 0);
+                read_frags((ms + 1) & 1, lds_next, 0);
             const MFrag *a = afr[ms & 1];
+            if constexpr (DIRECT && NEED_SUM) {
+                static_assert(!(DIRECT && NEED_SUM) || WM == 4, "one row tile a wave");
+                typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+                const bf16x2_t ones2 = __builtin_bit_cast(bf16x2_t, 0x3F803F80u);
+#pragma unroll
+                for (int w = 0; w < 4; ++w)
+                    rs_direct = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a[0].u[w]), ones2, rs_direct, false);
+            }
 #pragma unroll
             for (int t = 0; t < WN; ++t) {
                 MFrag nhi, nlo;
@@ -404,6 +474,19 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     };
 
 #define XFT_FENCE() __builtin_amdgcn_sched_barrier(0)
+    // memory requests a wave sends per step (weight loads + activation requests), in program order
+    constexpr int REQS_PER_STEP = GROUPS * WN + ALOADS;
+    int kt = 0;
+    if constexpr (DIRECT) {
+        // prologue: activation tiles 0, 1 and 2 in LDS, weight tiles 0 and 1 under way
+        load_w(0, 0);
+        direct_a(0, 0);
+        load_w(1, 1);
+        direct_a(1, 1);
+        direct_a(2, 2);
+        XFT_FENCE();
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    } else {
     // prologue: tiles 0 and 1 in LDS, weight tiles 0 and 1 and activation tiles 2 and 3 under way
     load_w(0, 0);
     load_a(0, 0);
@@ -417,17 +500,25 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     XFT_FENCE();
     store_a(1, 1, kt_n > 1);
     __syncthreads();
+    }
     read_frags(0, 0, 0);
     widen(0, 0, 0, wcur_hi, wcur_lo);
     // step k with s = k % 3 (static): tile j lives in weight set, activation register set and LDS buffer j % 3
+    // (DIRECT: LDS tile j % 4; the barrier first waits for this wave's requests of the step before - everything but the
+    // REQS_PER_STEP youngest - and for its LDS reads, so the tile published is complete and the tile freed is read)
 #define XFT_STEP(s)                                        \
     {                                                      \
-        compute((s), (s), ((s) + 1) % 3, ((s) + 2) % 3, kt); \
-        XFT_FENCE();                                       \
-        __syncthreads();                                   \
+        if constexpr (DIRECT) {                            \
+            compute((s), (s), ((s) + 1) % 3, ((s) + 2) % 3, kt, kt & 3, (kt + 1) & 3, (kt + 3) & 3); \
+            XFT_FENCE();                                   \
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(REQS_PER_STEP) : "memory"); \
+        } else {                                           \
+            compute((s), (s), ((s) + 1) % 3, ((s) + 2) % 3, kt, (s), ((s) + 1) % 3, 0); \
+            XFT_FENCE();                                   \
+            __syncthreads();                               \
+        }                                                  \
         ++kt;                                              \
     }
-    int kt = 0;
     while (kt + 3 <= kt_n) {
         XFT_STEP(0) XFT_STEP(1) XFT_STEP(2)
     }
@@ -445,12 +536,18 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     // 8-column chunks, consecutive lanes along a row: residual, conversion and 16-byte stores run
     // in that short loop.
     constexpr int OPITCH = 32 * WN * 4 + 32; // patch row pitch in bytes
+    if constexpr (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the requests past the last tile have landed
     __syncthreads(); // every wave is past its last read of the activation tiles
     unsigned char *obuf = abuf_base + wave * (32 * OPITCH);
     if constexpr (NEED_SUM) {
         // join the partial sums of a row's chunks (adjacent lanes), hand them over through LDS behind the patches, and
         // give every lane the sums of the 16 rows it holds results of
         float *rowsum = (float *)(abuf_base + 4 * 32 * OPITCH);
+        if constexpr (DIRECT) {
+            // lane halves hold the two halves of a row's k range
+            const float v = rs_direct + __shfl_xor(rs_direct, 32, 64);
+            if (h == 0) rowsum[32 * wave + nl] = v;
+        } else {
 #pragma unroll
         for (int i = 0; i < ALOADS; ++i) {
             float v = rs_part[i];
@@ -458,11 +555,12 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
             for (int off = 1; off < CHUNKS_PER_ROW; off <<= 1) v += __shfl_xor(v, off, 64);
             if (a_kc == 0) rowsum[a_row0 + i * ROW_STEP] = v;
         }
+        }
         __syncthreads();
 #pragma unroll
         for (int m = 0; m < WM; ++m)
 #pragma unroll
-            for (int j = 0; j < 16; ++j) accS[m][j] = rowsum[32 * m + 8 * (j >> 2) + 4 * h + (j & 3)];
+            for (int j = 0; j < 16; ++j) accS[m][j] = rowsum[32 * row_tile(m) + 8 * (j >> 2) + 4 * h + (j & 3)];
     }
     const bool c_wide = (((size_t)p.C | ((size_t)p.ldc * (p.c_dtype == XFTHIP_F32 ? 4 : 2))) & 15) == 0;
     const bool res_wide = (((size_t)p.res | ((size_t)p.ldres * (p.res_dtype == XFTHIP_F32 ? 4 : 2))) & 15) == 0;
@@ -575,7 +673,7 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
                     put_at(put_base, 32 * t, j, x); // the residual operand joins in flush()
                 }
             }
-            flush(epi_tag, m, n32_0 * 32, 32 * WN, p.N);
+            flush(epi_tag, row_tile(m), n32_0 * 32, 32 * WN, p.N);
         }
     };
     if (p.gateup) {
@@ -610,7 +708,7 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
                     put_at(put_base, 16 * t, j, other * silu_big(x));
                 }
             }
-            flush(std::integral_constant<int, XFTHIP_EPI_NONE> {}, m, n32_0 * 16, 16 * WN, p.N / 2);
+            flush(std::integral_constant<int, XFTHIP_EPI_NONE> {}, row_tile(m), n32_0 * 16, 16 * WN, p.N / 2);
         }
         return;
     }
@@ -625,27 +723,34 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(SkinnyParams p, int nbl
     }
 }
 
-template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL, bool DEVROWS = false>
+template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL, bool DEVROWS = false, bool DIRECT = false>
 static int launch_big2(const SkinnyParams &p, hipStream_t stream) {
     using T = StepTraits<KIND>;
-    constexpr int ROWS = 32 * WM, ROWB = T::KTILE * 2 + 16;
+    constexpr int ROWS = 32 * WM, ROWB = DIRECT ? T::KTILE * 2 : T::KTILE * 2 + 16;
     const int n32 = (p.NTILES + 1) / 2;
     const int nblocks_n = (n32 + 4 * WN - 1) / (4 * WN);
     // a group's row blocks: every weight may end in a partly filled one
     const int nblocks_m = (p.M + ROWS - 1) / ROWS + (p.group ? p.group_n : 0);
-    const int nb8 = (nblocks_n + 7) / 8;
-    const int blocks = nb8 * 8 * nblocks_m;
+    // 8 workgroups a unit of (band of row blocks, K part, column block), the units dealt out to the 8 XCDs
+    const int band = band_rows<ROWS, DEVROWS>(p), parts = p.ksplit > 1 ? p.ksplit : 1;
+    const long units = (long)((nblocks_m + band - 1) / band) * parts * nblocks_n;
+    const long blocks_l = (units + 7) / 8 * 8 * band;
+    if (blocks_l > 0x7fffffffL) {
+        set_error("qgemm_mfma: too many workgroups");
+        return 2;
+    }
+    const int blocks = (int)blocks_l;
     // the three activation buffers, reused after the k loop by the four waves' output patches
     // (the row sums of the zero-point term sit behind the patches)
-    const size_t pipe = 3 * ROWS * ROWB, patches = 4 * 32 * (32 * WN * 4 + 32) + (NEED_SUM ? ROWS * sizeof(float) : 0);
+    const size_t pipe = (DIRECT ? 4 : 3) * ROWS * ROWB, patches = 4 * 32 * (32 * WN * 4 + 32) + (NEED_SUM ? ROWS * sizeof(float) : 0);
     const size_t smem = (pipe > patches ? pipe : patches) + (KIND == XFTHIP_W_NF4 ? 2048 : 0);
     if (smem > 64 * 1024) {
         // more dynamic LDS than the default limit: raise it once per instantiation
-        static const hipError_t attr = hipFuncSetAttribute((const void *)qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL, DEVROWS>,
+        static const hipError_t attr = hipFuncSetAttribute((const void *)qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL, DEVROWS, DIRECT>,
                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         XFT_CHECK_HIP(attr);
     }
-    hipLaunchKernelGGL((qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL, DEVROWS>), dim3(blocks, p.ksplit > 1 ? p.ksplit : 1), dim3(256), smem, stream,
+    hipLaunchKernelGGL((qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL, DEVROWS, DIRECT>), dim3(blocks), dim3(256), smem, stream,
             p, nblocks_n, nblocks_m);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
@@ -664,6 +769,12 @@ static int launch_big(const SkinnyParams &p, hipStream_t stream) {
         }
     }
     if (p.K % StepTraits<KIND>::KTILE != 0) return launch_big2<KIND, WN, WM, NEED_SUM, true>(p, stream);
+    if constexpr (WN == 2 && WM == 4 && KIND != XFTHIP_W_BF16) {
+        // whole k tiles: the 128 x 256 tile takes its activations straight into LDS, two workgroups a CU
+        // (the kernel keeps a lane's byte offset into the activations in 32 bits)
+        if ((size_t)p.M * (size_t)p.lda * 2 < ((size_t)1 << 32))
+            return launch_big2<KIND, WN, WM, NEED_SUM, false, false, true>(p, stream);
+    }
     return launch_big2<KIND, WN, WM, NEED_SUM, false>(p, stream);
 }
 
@@ -693,15 +804,18 @@ static int dispatch_big_tile(const SkinnyParams &p, hipStream_t stream) {
         if (t_mid >= cus) return launch_big<KIND, 1, 4, NEED_SUM>(p, stream);
         return launch_big<KIND, 1, 2, NEED_SUM>(p, stream);
     } else if constexpr (KIND == XFTHIP_W_INT8) {
-        // 128 x 128 tiles, two workgroups a CU: measured 745 / 888 / 821 / 786 / 814 TFLOP/s on N x K =
-        // 11008x4096 / 4096x4096 / 4096x11008 / 12288x4096 / 22016x4096 at 2048 rows; the 128 x 256 tile
-        // (one wave per SIMD, nothing to run while it waits) stays at 750-760 wherever it applies
+        // The 128 x 256 tile with the activations straight into LDS (two workgroups a CU) wherever it fills the
+        // device: 960 / 918 - 944 / 960 TFLOP/s on N x K = 4096x4096 / 11008x4096 / 4096x11008 at 2048 rows
+        // (1050 - 1110 at 4096 rows), against 921 / 777 / 856 on the 128 x 128 tile (two workgroups a CU, bound by the
+        // LDS port: 20 KB of operand reads and staging writes per 16 MFMAs and wave) and 750 - 760 on the 128 x 256
+        // tile staged through registers (one wave per SIMD, nothing to run while it waits).
+        if (rows > 512 && t_large >= cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
         if (rows > 1024 && t_mid >= cus) return launch_big<KIND, 1, 4, NEED_SUM>(p, stream);
     } else {
-        // 4-bit kinds: 128 x 256 tiles, one workgroup a CU.  With 64-deep steps and the row sums gathered at the
-        // staging step the 128 x 128 tile fits two workgroups a CU like the INT8 one, but measured no better overall at
-        // 2048 rows (UINT4 751 / 766 / 813 TFLOP/s against 785 / 743 / 861 on 4096^2, 11008 x 4096, 4096 x 11008; NF4
-        // 515 / 512 / 551 against 495 / 483 / 540)
+        // 4-bit kinds: the same 128 x 256 tile (UINT4 850 / 922 / 916 TFLOP/s at 2048 rows on 4096^2, 11008 x 4096,
+        // 4096 x 11008 against 785 / 743 / 861 staged through registers, one workgroup a CU; NF4 499 / 549 / 535
+        // against 495 / 483 / 540).  The 128 x 128 tile (two workgroups a CU) measured no better than the staged
+        // 128 x 256 one (UINT4 751 / 766 / 813, NF4 515 / 512 / 551).
         if (rows > 512 && t_large >= cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
     }
     if constexpr (KIND != XFTHIP_W_BF16) {

@@ -150,6 +150,24 @@ int qgemm_mfma(const PackedWeight &pw, const SkinnyParams &p0, hipStream_t strea
             p.ksplit = (kt_n + p.split_ktiles - 1) / p.split_ktiles;
         }
     }
+    if (p.ksplit <= 1 && !p.gateup && !p.group && !p.rows_dev && p.M >= 256 && pw.K >= 8192) {
+        // A few hundred rows against few columns and a very deep K (the down projection of a 512-token prompt, 4096
+        // columns x 11008): 64-row tiles give every CU at most one workgroup with a k loop of 172 steps, 32-row tiles
+        // (two a CU) widen every weight for a single row tile.  K is split until the 64-row tiles come two a CU:
+        // 65 us with the addition of the parts against 79 (512 x 4096 x 11008).  At K = 4096 the loops are too short
+        // for the split to pay (31 us either way).
+        const long tiles64 = (long)((n32 + 3) / 4) * ((p.M + 63) / 64);
+        if (tiles64 < 2 * cus) {
+            long want = (2L * cus + tiles64 - 1) / tiles64;
+            const long fit = (long)(split_bound_floats() / ((size_t)p.M * p.N));
+            want = want < fit ? want : fit;
+            want = want < pw.K / 2048 ? want : pw.K / 2048; // parts at least 2048 deep
+            if (want >= 2) {
+                p.split_ktiles = (kt_n + (int)want - 1) / (int)want;
+                p.ksplit = (kt_n + p.split_ktiles - 1) / p.split_ktiles;
+            }
+        }
+    }
     if (p.ksplit > 1) {
         if ((size_t)p.ksplit * p.M * p.N > split_bound_floats()) p.ksplit = 0; // cannot happen within the bound; stay correct anyway
         else if (int rc = qgemm_split_reserve(stream, &p.split_part)) return rc;

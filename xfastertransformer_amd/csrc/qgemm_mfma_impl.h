@@ -97,7 +97,10 @@ __host__ __device__ inline int band_rows(const SkinnyParams &p) {
 // row, which a lane gets by choosing the global chunk it fetches, and which keeps the operand reads (32 rows, one
 // chunk index) free of bank conflicts.  Four LDS tiles: step k requests tile k + 3, and the barrier that ends a step
 // first waits until the wave's requests of the step before are in (vmcnt counts them in order with the weight
-// loads).  Without the staging registers the 128 x 256 tile fits two workgroups a CU.
+// loads).  Without the staging registers the 128 x 256 tile fits two workgroups a CU.  (A deeper form for launches of
+// one workgroup a CU - weights four tiles ahead in five register sets, six LDS tiles requested five steps ahead - was
+// built and measured no faster, 921 / 919 against 953 / 956 TFLOP/s on 2048 x 4096 x 4096 and 2048 x 4096 x 11008:
+// a lone wave a SIMD is not waiting for memory there, it issues its widening and its MFMAs one after the other.)
 template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL, bool DEVROWS = false, bool DIRECT = false>
 __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyParams p, int nblocks_n, int nblocks_m) {
     using T = StepTraits<KIND>;
@@ -809,7 +812,8 @@ static int dispatch_big_tile(const SkinnyParams &p, hipStream_t stream) {
         // (1050 - 1110 at 4096 rows), against 921 / 777 / 856 on the 128 x 128 tile (two workgroups a CU, bound by the
         // LDS port: 20 KB of operand reads and staging writes per 16 MFMAs and wave) and 750 - 760 on the 128 x 256
         // tile staged through registers (one wave per SIMD, nothing to run while it waits).
-        if (rows > 512 && t_large >= cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
+        // (512 rows x 22016 columns, the gate / up projection of a 512-token prompt: 117 us against 133)
+        if (rows >= 512 && t_large >= cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
         if (rows > 1024 && t_mid >= cus) return launch_big<KIND, 1, 4, NEED_SUM>(p, stream);
     } else {
         // 4-bit kinds: the same 128 x 256 tile (UINT4 850 / 922 / 916 TFLOP/s at 2048 rows on 4096^2, 11008 x 4096,
@@ -822,7 +826,8 @@ static int dispatch_big_tile(const SkinnyParams &p, hipStream_t stream) {
         // Few rows against a deep K (512 tokens x 4096 columns): 64-row tiles would leave one
         // workgroup per CU, whose k loop is then a chain of load latencies; 32-row tiles put two
         // on a CU.
-        if (t_small < 2 * cus) return launch_big<KIND, 1, 1, NEED_SUM>(p, stream);
+        // (the K parts of a split GEMM count as workgroups of their own)
+        if (t_small * (p.ksplit > 1 ? p.ksplit : 1) < 2 * cus) return launch_big<KIND, 1, 1, NEED_SUM>(p, stream);
         return launch_big<KIND, 1, 2, NEED_SUM>(p, stream);
     }
 }

@@ -307,14 +307,26 @@ __device__ inline float w8a8_epilogue(int epi, float x, float bias, bool has_bia
 // A workgroup is 4 x WR waves: four side by side over 4 * WN * 32 columns, WR on top of each other over
 // WR * WM * 32 rows; a wave owns WN x WM accumulator tiles of 32 x 32.  (WR = 2, eight waves on 256 x 256, was
 // measured and is no better than 128 x 128 tiles at three workgroups a CU: every dispatch uses WR = 1.)
-template <int WN, int WM, int WR>
-__global__ __launch_bounds__(256 * WR) void w8a8_mfma_kernel(W8A8Params p, int nblocks_n, int nblocks_m) {
-    constexpr int ROWS = 32 * WM, BROWS = ROWS * WR, ROWB = 64 + 16; // rows of a wave / of the block, padded LDS row pitch in bytes
+//
+// DIRECT (the 128 x 256 block, K a multiple of 256): the quantised activation rows go from global memory straight into
+// LDS (global_load_lds_dwordx4: a wave instruction fills 1 KiB of consecutive LDS from 64 addresses of its choice), a
+// step covers 128 k.  Rows are 128 bytes without padding, the 16-byte chunk c of row r in slot c ^ ((r >> 1) & 7) of
+// its row (the lane picks the global chunk that belongs there), which keeps the operand reads free of bank conflicts.
+// Four LDS tiles of 16 KB, tile k + 3 requested in step k; the weights of a micro-step (32 k) are loaded two steps
+// ahead into the registers its MFMAs have just read; the barrier that ends a step first waits for the wave's requests
+// of the step before (s_waitcnt vmcnt: weights and requests retire in order).  Without staging registers and with
+// two instead of six weight tiles in registers the block fits two workgroups a CU; every operand read from LDS feeds
+// two MFMAs, where the 128 x 128 block (three workgroups a CU) needs one read per MFMA and is bound by the LDS port.
+template <int WN, int WM, int WR, bool DIRECT = false>
+__global__ __launch_bounds__(256 * WR, DIRECT ? 2 : 1) void w8a8_mfma_kernel(W8A8Params p, int nblocks_n, int nblocks_m) {
+    static_assert(!DIRECT || (WR == 1 && WM == 4), "direct-to-LDS form: four waves, 128 rows");
+    constexpr int ROWS = 32 * WM, BROWS = ROWS * WR, ROWB = DIRECT ? 128 : 64 + 16; // rows of a wave / of the block, LDS row pitch in bytes
     constexpr int CHUNKS = BROWS * 4; // 16-byte chunks of an activation tile
     constexpr int ALOADS = CHUNKS / (256 * WR);
     static_assert(CHUNKS % (256 * WR) == 0, "an activation tile must split evenly over the workgroup");
     constexpr int OPITCH = 32 * WN * 4 + 32; // row pitch in bytes of a wave's result patch
-    constexpr int STAT_OFF = 3 * BROWS * ROWB > 4 * WR * 32 * OPITCH ? 3 * BROWS * ROWB : 4 * WR * 32 * OPITCH;
+    constexpr int NTILE_LDS = DIRECT ? 4 : 3;
+    constexpr int STAT_OFF = NTILE_LDS * BROWS * ROWB > 4 * WR * 32 * OPITCH ? NTILE_LDS * BROWS * ROWB : 4 * WR * 32 * OPITCH;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_a[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = lane >> 5, nl = lane & 31;
@@ -351,6 +363,97 @@ __global__ __launch_bounds__(256 * WR) void w8a8_mfma_kernel(W8A8Params p, int n
         nt = nt < p.NTILES ? nt : p.NTILES - 1;
         wbase[t] = p.packed + (size_t)nt * p.KT * 1024 + h * 256 + (nl & 15) * 16;
     }
+    // per-row statistics of this row block, kept behind the tiles / result patches for the epilogue
+    float *rowstat = (float *)(lds_a + STAT_OFF);
+    if (threadIdx.x < BROWS) {
+        int row = m0 + threadIdx.x;
+        row = row < p.M ? row : p.M - 1;
+        rowstat[threadIdx.x] = p.sA[row];
+        rowstat[BROWS + threadIdx.x] = p.zA[row];
+        rowstat[2 * BROWS + threadIdx.x] = p.sumA[row];
+    }
+    if constexpr (DIRECT) {
+        constexpr int TILEB = BROWS * ROWB, MICRO = 4, REQS_PER_STEP = MICRO * WN + 4;
+        const int kt_n = p.K / 128; // (even: the launcher takes this form for K % 256 == 0 only)
+        const int wave_u = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        // request i of this wave fills LDS chunks 64 (4 wave + i) ..+ 63 = rows 8 (4 wave + i) ..+ 7 of a tile; this
+        // lane's chunk is slot lane & 7 of row lane >> 3 of those and holds global chunk slot ^ swizzle(row)
+        uint32_t a_off[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = 8 * (4 * wave_u + i) + (lane >> 3);
+            int row = m0 + r;
+            row = row < p.M ? row : p.M - 1;
+            a_off[i] = (uint32_t)row * (uint32_t)p.ldq + ((lane & 7) ^ ((r >> 1) & 7)) * 16;
+        }
+        const uint64_t a_bits = (uint64_t)(uintptr_t)p.qa; // the same in every lane; said so, for a scalar register pair
+        const int8_t *a_uniform = (const int8_t *)(uintptr_t)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(a_bits >> 32)) << 32) |
+                (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a_bits));
+        const uint32_t lds_tiles = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds_a + 4096 * (uint32_t)wave_u;
+        // (assembly, not the compiler's builtin: after that one every later counted wait becomes a wait for all loads.
+        // M0 carries the LDS address of the wave's first lane; one wait state between writing it and the request.)
+        auto request_a = [&](int buf, int kt_raw, int i) {
+            const int kt = __builtin_amdgcn_readfirstlane(kt_raw < kt_n ? kt_raw : kt_n - 1);
+            const uint32_t dst = lds_tiles + buf * TILEB + i * 1024;
+            const int8_t *src = a_uniform + (size_t)kt * 128;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(a_off[i]), "s"(src) : "memory");
+        };
+        // weights of micro-step ms (32 k) of step kt: half ms & 1 of packed tile 2 kt + ms / 2
+        i32x4 wreg[2][MICRO][WN];
+        auto load_w = [&](int slot, int kt_raw, int ms) {
+            const int kt = kt_raw < kt_n ? kt_raw : kt_n - 1;
+#pragma unroll
+            for (int t = 0; t < WN; ++t) wreg[slot][ms][t] = *(const i32x4 *)(wbase[t] + (size_t)(2 * kt + (ms >> 1)) * 1024 + (ms & 1) * 512);
+        };
+        // operand of micro-step ms: bytes 32 ms + 16 h ..+ 15 of a row = chunk 2 ms + h
+        i32x4 afr[2][WM];
+        auto read_frags = [&](int slot, int buf, int ms) {
+            const unsigned char *src = lds_a + buf * TILEB + (mw + nl) * ROWB + (((2 * ms + h) ^ ((nl >> 1) & 7)) << 4);
+#pragma unroll
+            for (int m = 0; m < WM; ++m) afr[slot][m] = *(const i32x4 *)(src + m * 32 * ROWB);
+        };
+#pragma unroll
+        for (int d = 0; d < 3; ++d) {
+            if (d < 2) {
+#pragma unroll
+                for (int ms = 0; ms < MICRO; ++ms) load_w(d, d, ms);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) request_a(d, d, i);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        read_frags(0, 0, 0);
+        int lds_cur = 0;
+        auto step = [&](auto slot_tag, int kt) {
+            constexpr int SLOT = decltype(slot_tag)::value;
+            const int lds_next = (lds_cur + 1) & 3, lds_req = (lds_cur + 3) & 3;
+#pragma unroll
+            for (int ms = 0; ms < MICRO; ++ms) {
+                request_a(lds_req, kt + 3, ms);
+                if (ms + 1 < MICRO)
+                    read_frags((ms + 1) & 1, lds_cur, ms + 1);
+                else
+                    read_frags((ms + 1) & 1, lds_next, 0);
+#pragma unroll
+                for (int t = 0; t < WN; ++t)
+#pragma unroll
+                    for (int m = 0; m < WM; ++m)
+                        acc[t][m] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afr[ms & 1][m], wreg[SLOT][ms][t], acc[t][m], 0, 0, 0);
+                load_w(SLOT, kt + 2, ms);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // everything but this step's requests is in: the tile the next step reads its last operands from
+            // (requested in the step before) is complete, and this wave's reads of the tile freed are done
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(REQS_PER_STEP) : "memory");
+            lds_cur = lds_next;
+        };
+        for (int kt = 0; kt < kt_n; kt += 2) {
+            step(std::integral_constant<int, 0> {}, kt);
+            step(std::integral_constant<int, 1> {}, kt + 1);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the requests past the last tile have landed
+    } else {
     const int a_kc = threadIdx.x & 3, a_row0 = threadIdx.x >> 2;
     const int8_t *a_src[ALOADS];
 #pragma unroll
@@ -405,15 +508,6 @@ __global__ __launch_bounds__(256 * WR) void w8a8_mfma_kernel(W8A8Params p, int n
 #pragma unroll
             for (int m = 0; m < WM; ++m) acc[t][m] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[m], wreg[slot][s][t], acc[t][m], 0, 0, 0);
     };
-    // per-row statistics of this row block, kept behind the tiles / result patches for the epilogue
-    float *rowstat = (float *)(lds_a + STAT_OFF);
-    if (threadIdx.x < BROWS) {
-        int row = m0 + threadIdx.x;
-        row = row < p.M ? row : p.M - 1;
-        rowstat[threadIdx.x] = p.sA[row];
-        rowstat[BROWS + threadIdx.x] = p.zA[row];
-        rowstat[2 * BROWS + threadIdx.x] = p.sumA[row];
-    }
 #pragma unroll
     for (int d = 0; d < SLOTS; ++d) {
         load_w(d, d);
@@ -452,6 +546,7 @@ __global__ __launch_bounds__(256 * WR) void w8a8_mfma_kernel(W8A8Params p, int n
     }
 #undef XFT_W8_STEP
 #undef XFT_FENCE
+    }
 
     // ---- epilogue: lane holds C[m0 + 32 m + 8 (j / 4) + 4 h + j % 4][32 (n32_0 + t) + nl] ----------
     // Each wave drops one 32-row block of its int32 sums at a time into an LDS patch of its own (constant
@@ -581,22 +676,22 @@ __global__ __launch_bounds__(256 * WR) void w8a8_mfma_kernel(W8A8Params p, int n
     }
 }
 
-template <int WN, int WM, int WR>
+template <int WN, int WM, int WR, bool DIRECT = false>
 static int launch_w8a8_mfma(const W8A8Params &p, hipStream_t stream) {
     const int n32 = (p.NTILES + 1) / 2;
     const int brows = 32 * WM * WR;
     const int nblocks_n = (n32 + 4 * WN - 1) / (4 * WN);
     const int nblocks_m = (p.M + brows - 1) / brows;
     const int blocks = ((nblocks_n + 7) / 8) * 8 * nblocks_m;
-    const size_t tiles = 3 * (size_t)brows * (64 + 16), patches = 4 * WR * 32 * (size_t)(32 * WN * 4 + 32);
+    const size_t tiles = DIRECT ? 4 * (size_t)brows * 128 : 3 * (size_t)brows * (64 + 16), patches = 4 * WR * 32 * (size_t)(32 * WN * 4 + 32);
     // the result patches reuse the activation tiles; the per-row statistics sit behind both
     const size_t smem = (tiles > patches ? tiles : patches) + 3 * (size_t)brows * sizeof(float);
     if (smem > 64 * 1024) {
-        static const hipError_t attr = hipFuncSetAttribute((const void *)w8a8_mfma_kernel<WN, WM, WR>,
+        static const hipError_t attr = hipFuncSetAttribute((const void *)w8a8_mfma_kernel<WN, WM, WR, DIRECT>,
                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         XFT_CHECK_HIP(attr);
     }
-    hipLaunchKernelGGL((w8a8_mfma_kernel<WN, WM, WR>), dim3(blocks), dim3(256 * WR), smem, stream, p, nblocks_n, nblocks_m);
+    hipLaunchKernelGGL((w8a8_mfma_kernel<WN, WM, WR, DIRECT>), dim3(blocks), dim3(256 * WR), smem, stream, p, nblocks_n, nblocks_m);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
 }
@@ -643,11 +738,17 @@ int xfthip_gemm_w8a8(xfthip_weight_t w, int M, const int8_t *qa, int ldq, const 
         p.C = C, p.ldc = ldc, p.c_dtype = c_dtype, p.epi = epilogue, p.bias = bias;
         p.res = res, p.ldres = ldres, p.res_dtype = res_dtype, p.gamma = gamma;
         const int n32 = (pw.NTILES + 1) / 2;
-        // 128 x 128 tiles once they give every CU its three resident workgroups (registers allow three), else
-        // 128 x 256 with one (measured at 2048 / 8192 rows: 64 / 165 / 148 us and 225 / 554 / 510 us on
-        // 4096x4096 / 11008x4096 / 4096x11008; eight-wave 256 x 256 blocks were no better anywhere)
+        // Staged through registers (other K): 128 x 128 tiles once they give every CU its three resident workgroups
+        // (registers allow three), else 128 x 256 with one (eight-wave 256 x 256 blocks were no better anywhere)
         const long t_large = (long)((n32 + 7) / 8) * ((M + 127) / 128);
         const long t_mid = (long)((n32 + 3) / 4) * ((M + 127) / 128);
+        // 128 x 256 blocks with the activation rows straight into LDS, two workgroups a CU, wherever they give every
+        // CU a block and K is a whole number of step pairs (the kernel keeps a lane's byte offset into the rows in 32
+        // bits).  With the quantisation of the rows, 2048 / 4096 / 8192 rows on 4096x4096 / 11008x4096 / 4096x11008:
+        // 58 / 130 / 129, 94 / 251 / 226 and 184 / 488 / 483 us against 64 / 163 / 148, 112 / 309 / 317 and
+        // 231 / 583 / 604 us for the forms below.
+        if (t_large >= cus && pw.K % 256 == 0 && (size_t)M * (size_t)ldq < ((size_t)1 << 32))
+            return launch_w8a8_mfma<2, 4, 1, true>(p, (hipStream_t)stream);
         if (t_mid >= 3 * cus) return launch_w8a8_mfma<1, 4, 1>(p, (hipStream_t)stream);
         if (t_large >= cus) return launch_w8a8_mfma<2, 4, 1>(p, (hipStream_t)stream);
         return launch_w8a8_mfma<1, 2, 1>(p, (hipStream_t)stream);

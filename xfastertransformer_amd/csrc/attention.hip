@@ -54,7 +54,8 @@ __global__ __launch_bounds__(128) void attn_merge_kernel(AttnParams p) {
 // two pairs' keys and values in its L2 instead of all of them.
 template <bool INT8, int CT>
 __global__ __launch_bounds__(256, (CT == 1 ? 2 : 1)) void attn_prefill32_kernel(AttnParams p, int ncg, int npairs) {
-    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kP32BufBytes];
+    // INT8 cache: two buffers of widened blocks; FP16 cache: three 16 KB buffers the blocks are loaded into directly
+    __shared__ __attribute__((aligned(16))) unsigned char lds[INT8 ? 2 * kP32BufBytes : 3 * 16384];
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int pair = (slot / ncg) * 8 + xcd;
     if (pair >= npairs) return;

@@ -60,7 +60,8 @@ union HFrag32 {
 // operands straight from the cache instead (they are laid out as the MFMA wants them; one block ahead, into the
 // registers the products have just read: 209 registers) to share the bytes between the LDS port and the vector
 // memory pipeline ran 262 us: a lane's 16 bytes lie 64 bytes from its neighbour's, and the memory pipeline serves
-// such a load line by line.
+// such a load line by line.  What did pay for the FP16 cache: sending the blocks global -> LDS directly (below) instead
+// of through registers and ds_write - 4 of a wave's 20 LDS instructions a block gone, 16 registers free: 213 -> 202 us.
 template <int NW, int CT, bool INT8>
 __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, const int cgroup, const int b, unsigned char *lds) {
     constexpr int D = 128, NT = NW * 64, WC = 32 * CT;
@@ -102,7 +103,47 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
     const ATTN_GLOBAL float *ksc = INT8 ? (const ATTN_GLOBAL float *)p.kv.kscale + bh * p.kv.S : nullptr;
     const ATTN_GLOBAL float *vsc = INT8 ? (const ATTN_GLOBAL float *)p.kv.vscale + bh * p.kv.S : nullptr;
 
-    // ---- the block copy global -> registers -> LDS: 512 + 512 chunks of 16 bytes (FP16) or 256 + 256 (INT8) ----
+    // ---- FP16 cache: the block copy global -> LDS without a stop in registers (global_load_lds_dwordx4: a wave
+    // instruction fills 1 KiB of consecutive LDS, lane after lane, from 64 addresses of its choice).  Rows carry no
+    // padding; the 16-byte chunk c of a key row (token r, 256 bytes) sits in slot c ^ (r & 15), of a value row (dim
+    // r, 64 bytes) in slot c ^ ((r >> 2) & 3) - the lane fetches the global chunk that belongs in its slot - which
+    // keeps the operand reads (32 rows, one chunk index) free of bank conflicts.  Three buffers of 16 KB: block
+    // k + 2 is requested before block k is computed, and the barrier that ends a block first waits (vmcnt: the
+    // requests retire in order) for the requests of the block before.  A wave sends requests 2 w, 2 w + 1 of the
+    // keys' eight and of the values' eight.
+    constexpr bool DIRECT = !INT8;
+    constexpr int BUFB = DIRECT ? 16384 : kP32BufBytes, KPITCH = DIRECT ? 256 : kPfKPitch, VPITCH = DIRECT ? 64 : kPfVPitch;
+    uint32_t rq_koff[2], rq_voff[2];
+    const int wave_u = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int j = 2 * wave_u + i;
+        const int kr = 4 * j + (lane >> 4), vr = 16 * j + (lane >> 2);
+        rq_koff[i] = kr * 256 + (((lane & 15) ^ (kr & 15)) << 4);
+        rq_voff[i] = vr * 64 + (((lane & 3) ^ ((vr >> 2) & 3)) << 4);
+    }
+    const uint32_t lds_rq = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds + 2048 * (uint32_t)wave_u;
+    auto sgpr_ptr = [](const ATTN_GLOBAL char *ptr) { // the same in every lane; said so, for a scalar register pair
+        const uint64_t bits = (uint64_t)(uintptr_t)ptr;
+        return (const char *)(uintptr_t)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(bits >> 32)) << 32) |
+                (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)bits));
+    };
+    const char *k_uniform = sgpr_ptr(kbase), *v_uniform = sgpr_ptr(vbase);
+    // (assembly, not the compiler's builtin for the instruction: after that one every later counted wait becomes a wait
+    // for everything.  M0 carries the LDS address of the wave's first lane; one wait state between writing it and the
+    // request.)
+    auto request = [&](const int buf, const int blk_raw) {
+        const int blk = __builtin_amdgcn_readfirstlane(blk_raw);
+        const char *ks = k_uniform + (size_t)blk * (32 * D * 2), *vs = v_uniform + (size_t)blk * (32 * D * 2);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const uint32_t kd = lds_rq + buf * BUFB + i * 1024, vd = kd + 8192;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(kd), "v"(rq_koff[i]), "s"(ks) : "memory");
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(vd), "v"(rq_voff[i]), "s"(vs) : "memory");
+        }
+    };
+
+    // ---- INT8 cache: the block copy global -> registers -> LDS (widened on the way): 256 + 256 chunks of 16 bytes ----
     constexpr int CHUNKS = INT8 ? 256 : 512, PER = (CHUNKS + NT - 1) / NT;
     u32x4 kstage[PER], vstage[PER];
     f32x4 sstage; // INT8: threads 0..7 carry 4 key scales each, threads 8..15 4 value scales
@@ -190,11 +231,11 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
 
     auto compute = [&](const int buf, const int blk) {
         const int t0 = blk << 5;
-        const unsigned char *kb = lds + buf * kP32BufBytes, *vb = kb + 32 * kPfKPitch;
-        const unsigned char *krow = kb + cl * kPfKPitch + 16 * h;
+        const unsigned char *kb = lds + buf * BUFB, *vb = kb + 32 * KPITCH;
+        const unsigned char *krow = kb + cl * KPITCH + (DIRECT ? 0 : 16 * h);
         HFrag32 kf[8];
 #pragma unroll
-        for (int s = 0; s < 8; ++s) kf[s].q = *(const u32x4 *)(krow + 32 * s);
+        for (int s = 0; s < 8; ++s) kf[s].q = *(const u32x4 *)(krow + (DIRECT ? (((2 * s + h) ^ (cl & 15)) << 4) : 32 * s));
         f32x16 sc[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
@@ -216,7 +257,8 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt) vf[t][dt].q = *(const u32x4 *)(vb + (32 * dt + cl) * kPfVPitch + 16 * (2 * t + h));
+            for (int dt = 0; dt < 4; ++dt)
+                vf[t][dt].q = *(const u32x4 *)(vb + (32 * dt + cl) * VPITCH + (DIRECT ? (((2 * t + h) ^ ((cl >> 2) & 3)) << 4) : 16 * (2 * t + h)));
         const bool masked = t0 + 32 > lim_min; // wave-uniform
         // INT8: scales of this lane's 16 tokens (8 q + 4 h ..)
         f32x4 ks[4], vs[4];
@@ -336,6 +378,24 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
         }
     };
 
+    if constexpr (DIRECT) {
+        if (nblk > 0) request(0, 0);
+        if (nblk > 1) request(1, 1);
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        int cur = 0;
+        for (int blk = 0; blk < nblk; ++blk) {
+            const bool more = blk + 2 < nblk; // uniform over the workgroup
+            // (the buffer it goes to held block blk - 1, which every wave has left behind at the last barrier)
+            if (more) request(cur == 0 ? 2 : cur - 1, blk + 2);
+            if (blk < wave_nblk) compute(cur, blk);
+            __builtin_amdgcn_sched_barrier(0);
+            // block blk + 1 (requested an iteration ago: everything but this iteration's four requests) is in, and
+            // this wave's reads of block blk are done
+            if (more) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            cur = cur == 2 ? 0 : cur + 1;
+        }
+    } else {
     if (nblk > 0) {
         fetch(0);
         stash(0);
@@ -347,6 +407,7 @@ __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, c
         if (blk < wave_nblk) compute(blk & 1, blk);
         if (more) stash((blk + 1) & 1);
         __syncthreads();
+    }
     }
 
 #pragma unroll

@@ -75,9 +75,12 @@ def _sample_rows(M, n=48):
 # ------------------------------------------------------------------ config 2: GEMM sweep
 @pytest.mark.parametrize("kind", ["int8", "uint4", "nf4"])
 @pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 11008), (11008, 4096)])
-@pytest.mark.parametrize("M", [256, 512, 1024, 2011, 2048])
+@pytest.mark.parametrize("M", [256, 512, 768, 1024, 2011, 2048])
 def test_gemm_sweep_large_m(xh, orc, kind, K, N, M):
-    if M in (512, 1024, 2011) and kind == "nf4" and (K, N) != (4096, 4096):
+    # (the row counts cross every tile choice: 32- and 64-row tiles, K split over 64-row tiles at K = 11008 up to 768
+    # rows, the 128 x 256 tile with the activations loaded straight into LDS from 512 rows on where it fills the CUs,
+    # a ragged last row block at 2011)
+    if M in (512, 768, 1024, 2011) and kind == "nf4" and (K, N) != (4096, 4096):
         pytest.skip("NF4 shares every tile shape with UINT4; covered at M = 256 / 2048")
     print(f"case kind={kind} M={M} K={K} N={N}", flush=True)
     w, dw, Wd = _weight(xh, orc, kind, K, N)

@@ -104,9 +104,12 @@ def test_rotary_embedding_golden_and_bit_exact(xh, orc):
 
 @pytest.mark.parametrize("int8", [0, 1])
 @pytest.mark.parametrize("rope", [0, 1])
-def test_kv_append_bit_exact(xh, orc, int8, rope):
-    rng = np.random.default_rng(11 + int8)
-    B, S, qh, kh, D, max_seq, past = 2, 5, 8, 2, 128, 70, 33
+@pytest.mark.parametrize("S,past,max_seq", [(5, 33, 70), (75, 13, 128), (64, 32, 96), (16, 0, 40)])
+def test_kv_append_bit_exact(xh, orc, int8, rope, S, past, max_seq):
+    """(From 16 tokens on a rotating append takes the kernel that works by 32-token cache blocks: 75 tokens behind 13
+    fill their first and last block partly, 64 behind 32 fill two blocks exactly, 16 from 0 half of one.)"""
+    rng = np.random.default_rng(11 + int8 + S)
+    B, qh, kh, D = 2, 8, 2, 128
     stride = (qh + 2 * kh) * D
     qkv = orc.round_bf16(rng.standard_normal((B * S, stride)) * 3.0)
     qkv[1, qh * D:(qh + 1) * D] = 0.0  # an all-zero key row: scale 0, codes 0

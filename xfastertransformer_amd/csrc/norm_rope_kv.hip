@@ -294,6 +294,169 @@ __global__ __launch_bounds__(64) void rope_kv_kernel(RopeKvParams p) {
     }
 }
 
+// ---- RoPE + KV append for many tokens: one workgroup per (head, sequence, 32-token cache block) ------------------
+// The per-token kernel above moves 2 bytes a lane and scatters a token's value row over 128 cache rows; with a whole
+// prompt to append that is 49152 one-wave workgroups a layer at 512 tokens.  Here thread (token tid / 8, chunk tid % 8)
+// moves the 8 + 8 values of a rotation pair's two halves with 16-byte accesses, the key rows leave as 16-byte (FP16) or
+// 8-byte (INT8) stores, and the value rows of a block are turned through LDS into the cache's [dim][32 slots] tile and
+// leave as 16-byte runs.  Blocks the new tokens only partly fill (the first and the last of an append) fall back to
+// element stores for the values: the other slots of the tile belong to tokens already there.  Same arithmetic and the
+// same rounding points as the per-token kernel.  D = 128, bf16 rows, [maxPos, 64] tables, fused q | k | v rows.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <bool INT8>
+__global__ __launch_bounds__(256) void rope_kv_block_kernel(RopeKvParams p, int nblk) {
+    __shared__ __attribute__((aligned(16))) unsigned char tile[128 * 32 * 2];
+    const int head = blockIdx.x;
+    const int b = blockIdx.y / nblk, wb = blockIdx.y % nblk;
+    int past = p.past;
+    if (p.past_dev) {
+        past = p.past_dev[b];
+        past = past < 0 ? 0 : past;
+        if (past > p.kv.S - p.S) past = p.kv.S - p.S;
+    }
+    const int cb = (past >> 5) + wb; // cache block of this workgroup
+    const int t_lo = past > 32 * cb ? past : 32 * cb;
+    int t_hi = past + p.S < 32 * cb + 32 ? past + p.S : 32 * cb + 32;
+    t_hi = t_hi < p.kv.S ? t_hi : p.kv.S; // (the host checks the append fits; never write outside the cache)
+    if (t_lo >= t_hi) return; // (the whole workgroup)
+    const bool isq = head < p.qHeads;
+    if (isq && p.skip_q) return;
+    const int kvh = head - p.qHeads;
+    const int tl = threadIdx.x >> 3, c = threadIdx.x & 7;
+    const int t = 32 * cb + tl;
+    const bool live = t >= t_lo && t < t_hi;
+    const size_t tok = (size_t)b * p.S + (live ? t - past : t_lo - past);
+    const uint16_t *row = (const uint16_t *)p.qkv + tok * p.stride + (size_t)head * 128;
+    const u32x4 rlo = *(const u32x4 *)(row + 8 * c), rhi = *(const u32x4 *)(row + 64 + 8 * c);
+    const float *ct = p.cosT + (size_t)(live ? t : t_lo) * 64 + 8 * c, *st = p.sinT + (size_t)(live ? t : t_lo) * 64 + 8 * c;
+    const f32x4 c0 = *(const f32x4 *)ct, c1 = *(const f32x4 *)(ct + 4), s0 = *(const f32x4 *)st, s1 = *(const f32x4 *)(st + 4);
+    float lo[8], hi[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const uint32_t wl = rlo[e >> 1], wh = rhi[e >> 1];
+        const float a = bf16_to_f32((uint16_t)(e & 1 ? wl >> 16 : wl)), bb = bf16_to_f32((uint16_t)(e & 1 ? wh >> 16 : wh));
+        const float cs = e < 4 ? c0[e & 3] : c1[e & 3], sn = e < 4 ? s0[e & 3] : s1[e & 3];
+        // reference: fmsub(q, cos, qHalf*sin) ; fmadd(qHalf, cos, q*sin)
+        lo[e] = fmaf(a, cs, -(bb * sn));
+        hi[e] = fmaf(bb, cs, a * sn);
+    }
+    if (isq) {
+        if (live) {
+            u32x4 olo, ohi;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                olo[e] = (uint32_t)f32_to_bf16_ref(lo[2 * e]) | ((uint32_t)f32_to_bf16_ref(lo[2 * e + 1]) << 16);
+                ohi[e] = (uint32_t)f32_to_bf16_ref(hi[2 * e]) | ((uint32_t)f32_to_bf16_ref(hi[2 * e + 1]) << 16);
+            }
+            uint16_t *dst = (uint16_t *)p.qkv + tok * p.stride + (size_t)head * 128;
+            *(u32x4 *)(dst + 8 * c) = olo;
+            *(u32x4 *)(dst + 64 + 8 * c) = ohi;
+        }
+        return;
+    }
+    // ---- key row into the cache, value row into the tile ----
+    const size_t bh = (size_t)b * p.kv.H + kvh;
+    const uint16_t *vrow = (const uint16_t *)p.qkv + tok * p.stride + (size_t)(p.qHeads + p.kvHeads + kvh) * 128;
+    const u32x4 vl = *(const u32x4 *)(vrow + 8 * c), vh = *(const u32x4 *)(vrow + 64 + 8 * c);
+    float vlo[8], vhi[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const uint32_t wl = vl[e >> 1], wh = vh[e >> 1];
+        vlo[e] = bf16_to_f32((uint16_t)(e & 1 ? wl >> 16 : wl));
+        vhi[e] = bf16_to_f32((uint16_t)(e & 1 ? wh >> 16 : wh));
+    }
+    const int slot = v_slot(tl);
+    const bool full = t_lo == 32 * cb && t_hi == 32 * cb + 32; // (the whole workgroup)
+    const size_t vblk = (bh * (p.kv.S / 32) + cb) * (size_t)128 * 32; // elements
+    if constexpr (INT8) {
+        // xft::quantize: max = absmax, factor = max == 0 ? 1 : 127/max, scale = max/127, q = rne(x*factor)
+        float km = 0.0f, vm = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            km = fmaxf(km, fmaxf(fabsf(lo[e]), fabsf(hi[e])));
+            vm = fmaxf(vm, fmaxf(fabsf(vlo[e]), fabsf(vhi[e])));
+        }
+#pragma unroll
+        for (int off = 1; off < 8; off <<= 1) { // the 8 threads of a token are neighbours
+            km = fmaxf(km, __shfl_xor(km, off, 64));
+            vm = fmaxf(vm, __shfl_xor(vm, off, 64));
+        }
+        const float kf = (km == 0.0f) ? 1.0f : 127.0f / km;
+        const float vf = (vm == 0.0f) ? 1.0f : 127.0f / vm;
+        uint32_t klo[2], khi[2];
+        int8_t vql[8], vqh[8];
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+            klo[w] = khi[w] = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                klo[w] |= (uint32_t)(uint8_t)(int8_t)__float2int_rn(lo[4 * w + e] * kf) << (8 * e);
+                khi[w] |= (uint32_t)(uint8_t)(int8_t)__float2int_rn(hi[4 * w + e] * kf) << (8 * e);
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            vql[e] = (int8_t)__float2int_rn(vlo[e] * vf);
+            vqh[e] = (int8_t)__float2int_rn(vhi[e] * vf);
+        }
+        if (live) {
+            if (c == 0) {
+                p.kv.kscale[bh * p.kv.S + t] = km / 127.0f;
+                p.kv.vscale[bh * p.kv.S + t] = vm / 127.0f;
+            }
+            int8_t *kd = (int8_t *)p.kv.k + (bh * p.kv.S + t) * (size_t)128;
+            *(uint2 *)(kd + 8 * c) = make_uint2(klo[0], klo[1]);
+            *(uint2 *)(kd + 64 + 8 * c) = make_uint2(khi[0], khi[1]);
+        }
+        int8_t *vd = (int8_t *)p.kv.v + vblk;
+        if (full) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                ((int8_t *)tile)[(8 * c + e) * 32 + slot] = vql[e];
+                ((int8_t *)tile)[(64 + 8 * c + e) * 32 + slot] = vqh[e];
+            }
+            __syncthreads();
+            *(u32x4 *)(vd + (size_t)threadIdx.x * 16) = *(const u32x4 *)(tile + threadIdx.x * 16); // 128 rows of 32 bytes
+        } else if (live) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                vd[(size_t)(8 * c + e) * 32 + slot] = vql[e];
+                vd[(size_t)(64 + 8 * c + e) * 32 + slot] = vqh[e];
+            }
+        }
+    } else {
+        if (live) {
+            u32x4 klo, khi;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                klo[e] = (uint32_t)f32_to_fp16_bits(lo[2 * e]) | ((uint32_t)f32_to_fp16_bits(lo[2 * e + 1]) << 16);
+                khi[e] = (uint32_t)f32_to_fp16_bits(hi[2 * e]) | ((uint32_t)f32_to_fp16_bits(hi[2 * e + 1]) << 16);
+            }
+            uint16_t *kd = (uint16_t *)p.kv.k + (bh * p.kv.S + t) * (size_t)128;
+            *(u32x4 *)(kd + 8 * c) = klo;
+            *(u32x4 *)(kd + 64 + 8 * c) = khi;
+        }
+        uint16_t *vd = (uint16_t *)p.kv.v + vblk;
+        if (full) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                ((uint16_t *)tile)[(8 * c + e) * 32 + slot] = f32_to_fp16_bits(vlo[e]);
+                ((uint16_t *)tile)[(64 + 8 * c + e) * 32 + slot] = f32_to_fp16_bits(vhi[e]);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < 2; ++i) // 128 rows of 64 bytes
+                *(u32x4 *)((char *)vd + (size_t)(threadIdx.x + 256 * i) * 16) = *(const u32x4 *)(tile + (threadIdx.x + 256 * i) * 16);
+        } else if (live) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                vd[(size_t)(8 * c + e) * 32 + slot] = f32_to_fp16_bits(vlo[e]);
+                vd[(size_t)(64 + 8 * c + e) * 32 + slot] = f32_to_fp16_bits(vhi[e]);
+            }
+        }
+    }
+}
+
 // ---- export / import between the private layout and the reference's two layouts -----------------
 // sbhd = 0: [B][H][S][D] (ENABLE_KV_TRANS, src/common/kvcache_tensor.h:108-112); 1: [S][B][H][D] (:113-117).  The
 // INT8 scales are [B][H][S] in both.
@@ -422,6 +585,16 @@ int xfthip_rope_tables_create(int dim, int maxPos, int base, float scalingFactor
 
 static int launch_rope(const RopeKvParams &p, int tokens, hipStream_t stream) {
     const int half = p.D / 2;
+    // many tokens of fused bf16 rows into a cache: the block form (see rope_kv_block_kernel for what it assumes)
+    if (p.kv.k && p.S >= 16 && p.D == 128 && p.dtype == XFTHIP_BF16 && p.cosT && !p.table_full && !p.positions && !p.key &&
+            p.stride % 8 == 0 && ((uintptr_t)p.qkv & 15) == 0 && ((uintptr_t)p.cosT & 15) == 0 && ((uintptr_t)p.sinT & 15) == 0) {
+        const int nblk = (p.S + 31) / 32 + 1; // cache blocks an append of S tokens can touch
+        dim3 grid(p.qHeads + p.kvHeads, p.B * nblk);
+        if (p.kv.int8) hipLaunchKernelGGL(rope_kv_block_kernel<true>, grid, dim3(256), 0, stream, p, nblk);
+        else hipLaunchKernelGGL(rope_kv_block_kernel<false>, grid, dim3(256), 0, stream, p, nblk);
+        XFT_CHECK_HIP(hipGetLastError());
+        return 0;
+    }
     dim3 grid(p.qHeads + p.kvHeads, tokens);
     if (half <= 64)
         hipLaunchKernelGGL(rope_kv_kernel<1>, grid, dim3(64), 0, stream, p);

@@ -101,7 +101,7 @@ __host__ __device__ inline int band_rows(const SkinnyParams &p) {
 // one workgroup a CU - weights four tiles ahead in five register sets, six LDS tiles requested five steps ahead - was
 // built and measured no faster, 921 / 919 against 953 / 956 TFLOP/s on 2048 x 4096 x 4096 and 2048 x 4096 x 11008:
 // a lone wave a SIMD is not waiting for memory there, it issues its widening and its MFMAs one after the other.)
-template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL, bool DEVROWS = false, bool DIRECT = false>
+template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL, bool DEVROWS = false, bool DIRECT = false, int WSETS = 3>
 __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyParams p, int nblocks_n, int nblocks_m) {
     using T = StepTraits<KIND>;
     constexpr int KTILE = T::KTILE, GROUPS = T::GROUPS, SUB = T::SUB, WREGS = T::WREGS;
@@ -255,7 +255,12 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
     // buffer (k + 2) % 3.  Every wait is for loads at least one full step old, and the MFMAs after a
     // barrier never wait for an LDS read.
     constexpr int MICRO = GROUPS * SUB;
-    uint32_t wreg[3][GROUPS][WN][WREGS];
+    // weight register sets: tile j in set j % WSETS, loaded WSETS - 1 steps ahead.  Three for the large tiles (MFMA
+    // bound; the registers are the accumulators'); six for the 32- and 64-row tiles, whose launches are bound by
+    // the weights' trip from HBM - with two tiles in flight a step of such a workgroup waited most of a round trip
+    static_assert(WSETS % 3 == 0 && (!DIRECT || WSETS == 3), "the activation side of the pipeline walks three buffers");
+    constexpr int WD = WSETS - 1;
+    uint32_t wreg[WSETS][GROUPS][WN][WREGS];
     u32x4 areg[3][ALOADS];
     const int kt_n = (p.K + KTILE - 1) / KTILE;
 
@@ -409,11 +414,11 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
     // DIRECT: lds_cur / lds_next / lds_req = LDS tiles of activation tile kt_cur, kt_cur + 1 and kt_cur + 3 (the one this
     // step requests); staged form: the LDS tiles are numbered like the register sets (ab, ab_next, wnext)
     float rs_direct = 0.0f; // DIRECT + NEED_SUM: wave w sums the rows of row tile w, the first operand it reads
-    auto compute = [&](int wb, int ab, int ab_next, int wnext, int kt_cur, int lds_cur, int lds_next, int lds_req) {
+    auto compute = [&](int wb, int w_next, int w_load, int ab_next, int wnext, int kt_cur, int lds_cur, int lds_next, int lds_req) {
 #pragma unroll
         for (int ms = 0; ms < MICRO; ++ms) {
             const int gq = ms / SUB, sb = ms % SUB;
-            if (sb == 0) load_w_part(wnext, kt_cur + 2, gq);
+            if (sb == 0) load_w_part(w_load, kt_cur + WD, gq);
             if (ms % A_EVERY == 0) {
                 if constexpr (DIRECT) {
                     direct_a_part(lds_req, kt_cur + 3, ms / A_EVERY);
@@ -443,7 +448,7 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
                 else if (ms + 1 < MICRO)
                     widen(wb, ms + 1, 0, nhi, nlo);
                 else
-                    widen(ab_next, 0, 0, nhi, nlo); // the next tile's set: loaded during the step before this one
+                    widen(w_next, 0, 0, nhi, nlo); // the next tile's set: loaded in an earlier step
 #pragma unroll
                 for (int m = 0; m < WM; ++m) {
                     if constexpr (KIND == XFTHIP_W_NF4)
@@ -496,6 +501,8 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
     load_w(1, 1);
     load_a(1, 1);
     load_a(2, 2);
+#pragma unroll
+    for (int i = 2; i < WD; ++i) load_w(i, i);
     XFT_FENCE();
     store_a(0, 0, true);
     XFT_FENCE();
@@ -512,21 +519,32 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
 #define XFT_STEP(s)                                        \
     {                                                      \
         if constexpr (DIRECT) {                            \
-            compute((s), (s), ((s) + 1) % 3, ((s) + 2) % 3, kt, kt & 3, (kt + 1) & 3, (kt + 3) & 3); \
+            compute((s), ((s) + 1) % 3, ((s) + 2) % 3, 0, 0, kt, kt & 3, (kt + 1) & 3, (kt + 3) & 3); \
             XFT_FENCE();                                   \
             asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(REQS_PER_STEP) : "memory"); \
         } else {                                           \
-            compute((s), (s), ((s) + 1) % 3, ((s) + 2) % 3, kt, (s), ((s) + 1) % 3, 0); \
+            compute((s), ((s) + 1) % WSETS, ((s) + WD) % WSETS, ((s) + 1) % 3, ((s) + 2) % 3, kt, (s) % 3, ((s) + 1) % 3, 0); \
             XFT_FENCE();                                   \
             __syncthreads();                               \
         }                                                  \
         ++kt;                                              \
     }
-    while (kt + 3 <= kt_n) {
-        XFT_STEP(0) XFT_STEP(1) XFT_STEP(2)
+    if constexpr (WSETS == 6) {
+        while (kt + 6 <= kt_n) {
+            XFT_STEP(0) XFT_STEP(1) XFT_STEP(2) XFT_STEP(3) XFT_STEP(4) XFT_STEP(5)
+        }
+        if (kt < kt_n) XFT_STEP(0)
+        if (kt < kt_n) XFT_STEP(1)
+        if (kt < kt_n) XFT_STEP(2)
+        if (kt < kt_n) XFT_STEP(3)
+        if (kt < kt_n) XFT_STEP(4)
+    } else {
+        while (kt + 3 <= kt_n) {
+            XFT_STEP(0) XFT_STEP(1) XFT_STEP(2)
+        }
+        if (kt < kt_n) XFT_STEP(0)
+        if (kt < kt_n) XFT_STEP(1)
     }
-    if (kt < kt_n) XFT_STEP(0)
-    if (kt < kt_n) XFT_STEP(1)
 #undef XFT_STEP
 #undef XFT_FENCE
 
@@ -728,6 +746,8 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
 
 template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL, bool DEVROWS = false, bool DIRECT = false>
 static int launch_big2(const SkinnyParams &p, hipStream_t stream) {
+    // six weight tiles in flight for the 32- and 64-row tiles (see the kernel), three for the others
+    constexpr int WSETS = (!DIRECT && WN == 1 && WM <= 2) ? 6 : 3;
     using T = StepTraits<KIND>;
     constexpr int ROWS = 32 * WM, ROWB = DIRECT ? T::KTILE * 2 : T::KTILE * 2 + 16;
     const int n32 = (p.NTILES + 1) / 2;
@@ -749,11 +769,11 @@ static int launch_big2(const SkinnyParams &p, hipStream_t stream) {
     const size_t smem = (pipe > patches ? pipe : patches) + (KIND == XFTHIP_W_NF4 ? 2048 : 0);
     if (smem > 64 * 1024) {
         // more dynamic LDS than the default limit: raise it once per instantiation
-        static const hipError_t attr = hipFuncSetAttribute((const void *)qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL, DEVROWS, DIRECT>,
+        static const hipError_t attr = hipFuncSetAttribute((const void *)qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL, DEVROWS, DIRECT, WSETS>,
                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         XFT_CHECK_HIP(attr);
     }
-    hipLaunchKernelGGL((qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL, DEVROWS, DIRECT>), dim3(blocks), dim3(256), smem, stream,
+    hipLaunchKernelGGL((qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL, DEVROWS, DIRECT, WSETS>), dim3(blocks), dim3(256), smem, stream,
             p, nblocks_n, nblocks_m);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;

@@ -246,10 +246,10 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
 
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
     // Three-stage pipeline over k tiles.  At the start of step k: LDS buffers k % 3 and (k + 1) % 3 hold the
-    // activation tiles k and k + 1 (published by earlier barriers), the weight registers of sets k % 3
-    // and (k + 1) % 3 hold or await tiles k and k + 1, the activation registers await tile k + 2, and
-    // the first MFMA operands of tile k are already in registers.  Step k sends the loads of weight
-    // tile k + 2 and activation tile k + 3, moves activation tile k + 2 from registers into LDS buffer
+    // activation tiles k and k + 1 (published by earlier barriers), the weight registers of sets k % WSETS
+    // .. (k + WSETS - 2) % WSETS hold or await tiles k .. k + WSETS - 2, the activation registers await tile k + 2,
+    // and the first MFMA operands of tile k are already in registers.  Step k sends the loads of weight
+    // tile k + WSETS - 1 and activation tile k + 4, moves activation tile k + 2 from registers into LDS buffer
     // (k + 2) % 3 (last read two steps ago), computes tile k while reading each next operand set a
     // micro-step ahead (the last one from tile k + 1's buffer), and ends in the barrier that publishes
     // buffer (k + 2) % 3.  Every wait is for loads at least one full step old, and the MFMAs after a
@@ -366,10 +366,10 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
     };
     // one MFMA k step = 16 k.  Operands of micro-step ms sit in afr[ms & 1]; the next set (of the
     // next tile's buffer after the last micro-step) is read while this one's MFMAs run.
-    // Besides the MFMAs of tile kt (weight set wb, LDS buffer ab), a step sends the loads of weight
-    // tile kt + 2 (into set wnext) and activation tile kt + 4 (into register set ab_next) and moves
-    // activation tile kt + 2 (register set wnext, loaded two steps ago) into LDS buffer
-    // wnext: one slice of each per micro-step, so that no wave ever queues a burst of memory
+    // Besides the MFMAs of tile kt (weight set w_cur, LDS buffer lds_cur), a step sends the loads of weight
+    // tile kt + WD (into set w_load) and activation tile kt + 4 (into register set a_load) and moves
+    // activation tile kt + 2 (register set a_stage, loaded two steps ago) into LDS buffer
+    // a_stage: one slice of each per micro-step, so that no wave ever queues a burst of memory
     // instructions in front of its MFMAs (a wave issues in order; 4 waves sending 12 loads each right
     // after a barrier kept the MFMA pipes waiting for the address path).
     constexpr int A_EVERY = MICRO / ALOADS;
@@ -411,10 +411,12 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
     // VALU instructions one widening takes (a hint for the instruction interleave below)
     constexpr int VW = KIND == XFTHIP_W_INT8 ? 12 : KIND == XFTHIP_W_UINT4 ? 9 : KIND == XFTHIP_W_NF4 ? 6 : 0;
     constexpr int VPER = (VW + WM - 1) / WM;
-    // DIRECT: lds_cur / lds_next / lds_req = LDS tiles of activation tile kt_cur, kt_cur + 1 and kt_cur + 3 (the one this
-    // step requests); staged form: the LDS tiles are numbered like the register sets (ab, ab_next, wnext)
+    // w_cur / w_next / w_load: weight register sets of tiles kt_cur, kt_cur + 1 and kt_cur + WD (the one this step loads).
+    // lds_cur / lds_next: LDS tiles of activation tiles kt_cur and kt_cur + 1.  DIRECT: lds_req, the LDS tile this step
+    // requests activation tile kt_cur + 3 into; staged form: a_load, the register set tile kt_cur + 4 is loaded into,
+    // and a_stage, the register set (and LDS tile of the same number) tile kt_cur + 2 moves from (to)
     float rs_direct = 0.0f; // DIRECT + NEED_SUM: wave w sums the rows of row tile w, the first operand it reads
-    auto compute = [&](int wb, int w_next, int w_load, int ab_next, int wnext, int kt_cur, int lds_cur, int lds_next, int lds_req) {
+    auto compute = [&](int w_cur, int w_next, int w_load, int a_load, int a_stage, int kt_cur, int lds_cur, int lds_next, int lds_req) {
 #pragma unroll
         for (int ms = 0; ms < MICRO; ++ms) {
             const int gq = ms / SUB, sb = ms % SUB;
@@ -423,8 +425,8 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
                 if constexpr (DIRECT) {
                     direct_a_part(lds_req, kt_cur + 3, ms / A_EVERY);
                 } else {
-                    load_a_part(ab_next, kt_cur + 4, ms / A_EVERY);
-                    store_a_part(wnext, wnext, ms / A_EVERY, kt_cur + 2 < kt_n);
+                    load_a_part(a_load, kt_cur + 4, ms / A_EVERY);
+                    store_a_part(a_stage, a_stage, ms / A_EVERY, kt_cur + 2 < kt_n);
                 }
             }
             if (ms + 1 < MICRO)
@@ -444,9 +446,9 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
             for (int t = 0; t < WN; ++t) {
                 MFrag nhi, nlo;
                 if (t + 1 < WN)
-                    widen(wb, ms, t + 1, nhi, nlo);
+                    widen(w_cur, ms, t + 1, nhi, nlo);
                 else if (ms + 1 < MICRO)
-                    widen(wb, ms + 1, 0, nhi, nlo);
+                    widen(w_cur, ms + 1, 0, nhi, nlo);
                 else
                     widen(w_next, 0, 0, nhi, nlo); // the next tile's set: loaded in an earlier step
 #pragma unroll

@@ -101,8 +101,14 @@ __host__ __device__ inline int band_rows(const SkinnyParams &p) {
 // one workgroup a CU - weights four tiles ahead in five register sets, six LDS tiles requested five steps ahead - was
 // built and measured no faster, 921 / 919 against 953 / 956 TFLOP/s on 2048 x 4096 x 4096 and 2048 x 4096 x 11008:
 // a lone wave a SIMD is not waiting for memory there, it issues its widening and its MFMAs one after the other.)
-template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL, bool DEVROWS = false, bool DIRECT = false, int WSETS = 3>
-__global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyParams p, int nblocks_n, int nblocks_m) {
+//
+// KG = 2 (DIRECT only): the form for launches of at most one block a CU.  Eight waves a workgroup: waves 0..3 take the
+// first half of K, waves 4..7 the second, each group with LDS tiles and a pipeline of its own (the step barriers are
+// the workgroup's, both groups take the same number of steps), so that a SIMD has two waves to issue from as it has
+// with two blocks a CU.  After the k loop the second group hands its accumulators (and row sums) to the first
+// through LDS, which runs the epilogue.
+template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL, bool DEVROWS = false, bool DIRECT = false, int WSETS = 3, int KG = 1>
+__global__ __launch_bounds__(256 * KG, (DIRECT && KG == 1) ? 2 : 1) void qgemm_mfma_kernel(SkinnyParams p, int nblocks_n, int nblocks_m) {
     using T = StepTraits<KIND>;
     constexpr int KTILE = T::KTILE, GROUPS = T::GROUPS, SUB = T::SUB, WREGS = T::WREGS;
     constexpr int PACKED_K = T::PACKED_K, STEPS_PER_TILE = PACKED_K / KTILE; // k of a packed 1-KiB tile; steps that share one
@@ -115,7 +121,9 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
     static_assert(TOTAL_CHUNKS % 256 == 0, "activation tile must split evenly over the block");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    static_assert(KG == 1 || (KG == 2 && DIRECT), "K groups: the direct-to-LDS form only");
+    const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) & 3; // wave: position among the 4 waves that split the columns
+    const int kgroup = KG == 2 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 8) : 0;
     const int h = lane >> 5, nl = lane & 31;
     const int part_rows = p.M; // rows of a K part: the host's bound, also when the device knows fewer
     // workgroup -> (K part, column block, row block).  Row blocks are walked in bands of 8; a unit of work is one
@@ -179,6 +187,13 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
         p.c_dtype = XFTHIP_F32;
         p.epi = XFTHIP_EPI_NONE;
     }
+    if constexpr (KG == 2) {
+        // (the launcher takes this form only for a K of a whole number of packed tiles per group)
+        const int half_k = p.K / 2;
+        p.packed += (size_t)kgroup * (half_k / PACKED_K) * 1024;
+        p.A += (size_t)kgroup * half_k;
+        p.K = half_k;
+    }
     const int n32_0 = (nb * 4 + wave) * WN; // first 32-column tile of this wave
     const int m0 = mb * ROWS;
     if constexpr (DEVROWS) {
@@ -190,9 +205,9 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
     if constexpr (KIND == XFTHIP_W_NF4) {
         // DIRECT: the table sits behind the tiles, which then start at LDS offset 0 of the workgroup and end below 64 KiB
         // (the requests carry their LDS address in M0)
-        lut = (uint2 *)(DIRECT ? lds + 4 * ROWS * ROWB : lds);
+        lut = (uint2 *)(DIRECT ? lds + KG * 4 * ROWS * ROWB + (KG == 2 ? 1024 : 0) : lds);
         abuf_base = DIRECT ? lds : lds + 2048;
-        {
+        if (threadIdx.x < 256) {
             const int i = threadIdx.x;
             const float c0 = c_nf4_big[i & 15], c1 = c_nf4_big[i >> 4];
             const uint32_t h0 = f32_to_bf16_ref(c0), h1 = f32_to_bf16_ref(c1);
@@ -202,6 +217,7 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
         }
     }
 
+    if constexpr (KG == 2) abuf_base += kgroup * (4 * ROWS * ROWB); // this group's LDS tiles
     f32x16 acc[WN][WM];
     f32x16 accS[WM];
 #pragma unroll
@@ -233,7 +249,7 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
         if constexpr (DIRECT) {
             // request i of this wave fills LDS chunks 64 (ALOADS wave + i) ..+ 63 = rows 8 (ALOADS wave + i) ..+ 7;
             // this lane's chunk is slot lane & 7 of row lane >> 3 of those, which holds global chunk slot ^ swizzle(row)
-            const int r = 8 * (ALOADS * (int)(threadIdx.x >> 6) + i) + (lane >> 3);
+            const int r = 8 * (ALOADS * wave + i) + (lane >> 3);
             int row = m0 + r;
             row = row < p.M ? row : p.M - 1;
             a_off[i] = ((uint32_t)row * (uint32_t)p.lda + ((lane & 7) ^ ((r >> 1) & 7)) * 8) * 2; // in bytes
@@ -309,7 +325,7 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
     // counted waits for the weight loads come out a few requests early, never late: the counter retires in order.
     // M0 carries the LDS address of the wave's first lane; one wait state between writing it and the request.)
     const uint32_t lds_tiles = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)abuf_base +
-            ALOADS * 1024 * (uint32_t)__builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+            ALOADS * 1024 * (uint32_t)__builtin_amdgcn_readfirstlane(wave);
     const uint64_t a_bits = (uint64_t)(uintptr_t)p.A; // the same in every lane; said so, for a scalar register pair
     const uint16_t *a_uniform = (const uint16_t *)(uintptr_t)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(a_bits >> 32)) << 32) |
             (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a_bits));
@@ -355,7 +371,7 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
     // DIRECT + NEED_SUM: wave w walks the row tiles in the order w, w + 1, .. (mod WM), so that the operand it sums for
     // the zero-point term (below) is always the first one it reads - no branch on the wave number inside the k loop
     constexpr bool ROTATE = DIRECT && NEED_SUM;
-    const int wave_first = ROTATE ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
+    const int wave_first = ROTATE ? __builtin_amdgcn_readfirstlane(wave) : 0;
     auto row_tile = [&](int m) { return ROTATE ? (m + wave_first) % WM : m; };
     MFrag afr[2][WM];
     auto read_frags = [&](int slot, int ab, int ms) {
@@ -561,6 +577,33 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
     constexpr int OPITCH = 32 * WN * 4 + 32; // patch row pitch in bytes
     if constexpr (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the requests past the last tile have landed
     __syncthreads(); // every wave is past its last read of the activation tiles
+    if constexpr (KG == 2) {
+        // the second K group hands its accumulators over, [wave][register][lane] floats from the start of LDS (exactly
+        // the two groups' tiles), its row sums behind them
+        float *hand = (float *)lds + (size_t)wave * (WN * WM * 16) * 64 + lane;
+        float *hand_rs = (float *)(lds + 2 * 4 * ROWS * ROWB) + wave * 64 + lane;
+        if (kgroup == 1) {
+#pragma unroll
+            for (int t = 0; t < WN; ++t)
+#pragma unroll
+                for (int m = 0; m < WM; ++m)
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) hand[((t * WM + m) * 16 + j) * 64] = acc[t][m][j];
+            if constexpr (NEED_SUM) *hand_rs = rs_direct;
+        }
+        __syncthreads();
+        if (kgroup == 0) {
+#pragma unroll
+            for (int t = 0; t < WN; ++t)
+#pragma unroll
+                for (int m = 0; m < WM; ++m)
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) acc[t][m][j] += hand[((t * WM + m) * 16 + j) * 64];
+            if constexpr (NEED_SUM) rs_direct += *hand_rs;
+        }
+        __syncthreads(); // (the result patches below overwrite what was handed over)
+        abuf_base = lds;
+    }
     unsigned char *obuf = abuf_base + wave * (32 * OPITCH);
     if constexpr (NEED_SUM) {
         // join the partial sums of a row's chunks (adjacent lanes), hand them over through LDS behind the patches, and
@@ -569,7 +612,7 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
         if constexpr (DIRECT) {
             // lane halves hold the two halves of a row's k range
             const float v = rs_direct + __shfl_xor(rs_direct, 32, 64);
-            if (h == 0) rowsum[32 * wave + nl] = v;
+            if (h == 0 && kgroup == 0) rowsum[32 * wave + nl] = v;
         } else {
 #pragma unroll
         for (int i = 0; i < ALOADS; ++i) {
@@ -585,6 +628,7 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
 #pragma unroll
             for (int j = 0; j < 16; ++j) accS[m][j] = rowsum[32 * row_tile(m) + 8 * (j >> 2) + 4 * h + (j & 3)];
     }
+    if (KG == 2 && kgroup == 1) return; // (no workgroup barrier from here on)
     const bool c_wide = (((size_t)p.C | ((size_t)p.ldc * (p.c_dtype == XFTHIP_F32 ? 4 : 2))) & 15) == 0;
     const bool res_wide = (((size_t)p.res | ((size_t)p.ldres * (p.res_dtype == XFTHIP_F32 ? 4 : 2))) & 15) == 0;
     auto wave_sync = [&]() {
@@ -746,7 +790,7 @@ __global__ __launch_bounds__(256, DIRECT ? 2 : 1) void qgemm_mfma_kernel(SkinnyP
     }
 }
 
-template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL, bool DEVROWS = false, bool DIRECT = false>
+template <int KIND, int WN, int WM, bool NEED_SUM, bool KTAIL, bool DEVROWS = false, bool DIRECT = false, int KG = 1>
 static int launch_big2(const SkinnyParams &p, hipStream_t stream) {
     // six weight tiles in flight for the 32- and 64-row tiles (see the kernel), three for the others
     constexpr int WSETS = (!DIRECT && WN == 1 && WM <= 2) ? 6 : 3;
@@ -767,15 +811,15 @@ static int launch_big2(const SkinnyParams &p, hipStream_t stream) {
     const int blocks = (int)blocks_l;
     // the three activation buffers, reused after the k loop by the four waves' output patches
     // (the row sums of the zero-point term sit behind the patches)
-    const size_t pipe = (DIRECT ? 4 : 3) * ROWS * ROWB, patches = 4 * 32 * (32 * WN * 4 + 32) + (NEED_SUM ? ROWS * sizeof(float) : 0);
+    const size_t pipe = (DIRECT ? 4 : 3) * ROWS * ROWB * KG + (KG == 2 ? 1024 : 0), patches = 4 * 32 * (32 * WN * 4 + 32) + (NEED_SUM ? ROWS * sizeof(float) : 0);
     const size_t smem = (pipe > patches ? pipe : patches) + (KIND == XFTHIP_W_NF4 ? 2048 : 0);
     if (smem > 64 * 1024) {
         // more dynamic LDS than the default limit: raise it once per instantiation
-        static const hipError_t attr = hipFuncSetAttribute((const void *)qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL, DEVROWS, DIRECT, WSETS>,
+        static const hipError_t attr = hipFuncSetAttribute((const void *)qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL, DEVROWS, DIRECT, WSETS, KG>,
                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         XFT_CHECK_HIP(attr);
     }
-    hipLaunchKernelGGL((qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL, DEVROWS, DIRECT, WSETS>), dim3(blocks), dim3(256), smem, stream,
+    hipLaunchKernelGGL((qgemm_mfma_kernel<KIND, WN, WM, NEED_SUM, KTAIL, DEVROWS, DIRECT, WSETS, KG>), dim3(blocks), dim3(256 * KG), smem, stream,
             p, nblocks_n, nblocks_m);
     XFT_CHECK_HIP(hipGetLastError());
     return 0;
@@ -797,8 +841,15 @@ static int launch_big(const SkinnyParams &p, hipStream_t stream) {
     if constexpr (WN == 2 && WM == 4 && KIND != XFTHIP_W_BF16) {
         // whole k tiles: the 128 x 256 tile takes its activations straight into LDS, two workgroups a CU
         // (the kernel keeps a lane's byte offset into the activations in 32 bits)
-        if ((size_t)p.M * (size_t)p.lda * 2 < ((size_t)1 << 32))
+        if ((size_t)p.M * (size_t)p.lda * 2 < ((size_t)1 << 32)) {
+            // at most one block a CU: two K groups a workgroup give every SIMD a second wave (see the kernel)
+            const long wgs = (long)(((p.NTILES + 1) / 2 + 4 * WN - 1) / (4 * WN)) * ((p.M + 32 * WM - 1) / (32 * WM));
+            // (2048 rows x 4096 columns, K = 4096 / 11008: INT8 963 / 993 against 926 / 934 TFLOP/s on the same box, UINT4
+            // 859 / 954 against 812 / 926, NF4 519 / 569 against 492 / 532)
+            if (wgs <= device_cu_count() && p.ksplit <= 1 && p.K % (2 * StepTraits<KIND>::PACKED_K) == 0)
+                return launch_big2<KIND, WN, WM, NEED_SUM, false, false, true, 2>(p, stream);
             return launch_big2<KIND, WN, WM, NEED_SUM, false, false, true>(p, stream);
+        }
     }
     return launch_big2<KIND, WN, WM, NEED_SUM, false>(p, stream);
 }

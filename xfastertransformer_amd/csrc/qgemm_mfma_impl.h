@@ -323,7 +323,9 @@ __global__ __launch_bounds__(256 * KG, (DIRECT && KG == 1) ? 2 : 1) void qgemm_m
     // or an LDS read a wait for all of them - an instruction of the flat family that touches both memories - which
     // takes the two-tiles-ahead weight loads out of flight at every step.  Unaware of these requests, the compiler's
     // counted waits for the weight loads come out a few requests early, never late: the counter retires in order.
-    // M0 carries the LDS address of the wave's first lane; one wait state between writing it and the request.)
+    // M0 carries the LDS address of the wave's first lane; one wait state between writing it and the request.  The
+    // compiler holds nothing in M0 across statements - it is a reserved register that it writes right in front of each
+    // instruction of its own that reads it - so the statement may overwrite it.)
     const uint32_t lds_tiles = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)abuf_base +
             ALOADS * 1024 * (uint32_t)__builtin_amdgcn_readfirstlane(wave);
     const uint64_t a_bits = (uint64_t)(uintptr_t)p.A; // the same in every lane; said so, for a scalar register pair

@@ -120,6 +120,27 @@ def test_gateup_silu_large_m(xh, orc, kind, M):
     assert np.abs(got[rows] - exp).max() < 2e-3 + 2e-4 * np.abs(exp).max()
 
 
+@pytest.mark.parametrize("kind", ["int8", "uint4", "nf4"])
+def test_gateup_silu_one_block_a_cu(xh, orc, kind):
+    """The SwiGLU pairing on a launch of exactly one 128 x 256 block a CU (2048 rows x 2 x 2048 columns on 256 CUs): the
+    form whose eight waves split K in two groups and hand the second group's sums over before the epilogue."""
+    M, K, I = 2048, 1024, 2048
+    w, dw, Wd = _weight(xh, orc, kind, K, 2 * I, gateup=True)
+    A = orc.round_bf16(np.random.default_rng(5).standard_normal((M, K)))
+    a_dev = xh.DeviceBuffer.from_numpy(orc.to_bf16(A))
+    o_dev = xh.DeviceBuffer(M * I * 4)
+    xh.gemm_gateup_silu(dw, a_dev.ptr, M, K, o_dev.ptr, I, xh.F32)
+    xh.synchronize()
+    got = o_dev.to_numpy(np.float32, (M, I))
+    cat = A @ Wd
+    blas = cat[:, :I] / (1.0 + np.exp(-cat[:, :I])) * cat[:, I:]
+    assert np.abs(got - blas).max() < 2e-3 + 2e-4 * np.abs(blas).max()
+    assert _cos(got, blas) >= 0.9999
+    rows = _sample_rows(M, 16)
+    exp = orc.silu_sum(orc.qgemm(w, A[rows]))
+    assert np.abs(got[rows] - exp).max() < 2e-3 + 2e-4 * np.abs(exp).max()
+
+
 EPILOGUES = ["none", "bias", "silu", "gelu", "resmul", "residential", "residential_bias", "resext", "resext_bias"]
 
 

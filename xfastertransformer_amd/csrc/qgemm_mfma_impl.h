@@ -897,7 +897,8 @@ static int dispatch_big_tile(const SkinnyParams &p, hipStream_t stream) {
         // 4096 x 11008 against 785 / 743 / 861 staged through registers, one workgroup a CU; NF4 499 / 549 / 535
         // against 495 / 483 / 540).  The 128 x 128 tile (two workgroups a CU) measured no better than the staged
         // 128 x 256 one (UINT4 751 / 766 / 813, NF4 515 / 512 / 551).
-        if (rows > 512 && t_large >= cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
+        // (512 rows x 22016 columns: UINT4 119 us against 138, NF4 203 against 210)
+        if (rows >= 512 && t_large >= cus) return launch_big<KIND, 2, 4, NEED_SUM>(p, stream);
     }
     if constexpr (KIND != XFTHIP_W_BF16) {
         // Few rows against a deep K (512 tokens x 4096 columns): 64-row tiles would leave one

@@ -141,6 +141,29 @@ def test_gateup_silu_one_block_a_cu(xh, orc, kind):
     assert np.abs(got[rows] - exp).max() < 2e-3 + 2e-4 * np.abs(exp).max()
 
 
+@pytest.mark.parametrize("kind", ["int8", "uint4", "nf4"])
+@pytest.mark.parametrize("M,K,N", [(2048, 512, 4096), (1000, 1024, 11008)])
+def test_large_m_activation_row_pitch(xh, orc, kind, M, K, N):
+    """Activation rows with a pitch wider than K (NaN behind every row) through the tiles whose activations are loaded
+    straight into LDS: one block a CU in two K groups (2048 x 4096) and several blocks a CU with a ragged last row block
+    (1000 x 11008)."""
+    w, dw, Wd = _weight(xh, orc, kind, K, N)
+    lda = K + 64
+    A = orc.round_bf16(np.random.default_rng(3 * M + K).standard_normal((M, K)))
+    padded = np.full((M, lda), 0x7FC0, np.uint16)  # bf16 NaN
+    padded[:, :K] = orc.to_bf16(A)
+    a_dev = xh.DeviceBuffer.from_numpy(padded)
+    c_dev = xh.DeviceBuffer(M * N * 4)
+    xh.gemm(dw, a_dev.ptr, M, lda, c_dev.ptr, N, xh.F32)
+    xh.synchronize()
+    got = c_dev.to_numpy(np.float32, (M, N))
+    assert np.isfinite(got).all()
+    blas = A @ Wd
+    assert np.abs(got - blas).max() < 2e-3, np.abs(got - blas).max()
+    rows = _sample_rows(M, 8)
+    assert np.abs(got[rows] - orc.qgemm(w, A[rows])).max() < 2e-3
+
+
 EPILOGUES = ["none", "bias", "silu", "gelu", "resmul", "residential", "residential_bias", "resext", "resext_bias"]
 
 

@@ -232,6 +232,73 @@ def pmc_summary(fetch_csv, write_csv):
         print("traffic_bytes %s=%d" % (key, round(fb + wb)))
 
 
+def traffic_from_counters(fetch_csv, write_csv):
+    """HBM bytes per launch of the three decode GEMV forms ({'qkv' | 'narrow' | 'wide': bytes}) from the counter CSVs of two
+    `rocprofv3 --pmc FETCH_SIZE | WRITE_SIZE -- python3 bench.py --pmc-workload` runs, each counter scaled by what it reads
+    for the plain copy kernel of known size in the same run."""
+    import csv
+
+    def per_kernel(path, counter):
+        acc = {}
+        with open(path, newline="") as f:
+            for r in csv.DictReader(f):
+                if r["Counter_Name"] != counter:
+                    continue
+                name = r["Kernel_Name"]
+                if "stream_copy_kernel" in name:
+                    key = "copy"
+                elif "qgemm_skinny_kernel<" in name:
+                    targs = name.split("qgemm_skinny_kernel<")[1].split(">")[0].replace(" ", "").split(",")
+                    key = "qkv" if targs[7] in ("true", "1") else ("wide" if targs[1] == "2" else "narrow")
+                else:
+                    continue
+                acc.setdefault(key, []).append(float(r["Counter_Value"]))
+        return {k: sum(v) / len(v) for k, v in acc.items()}
+
+    fetch, write = per_kernel(fetch_csv, "FETCH_SIZE"), per_kernel(write_csv, "WRITE_SIZE")
+    copy_kib = PMC_COPY_BYTES / 1024.0
+    sf, sw = copy_kib / fetch["copy"], copy_kib / write["copy"]
+    return {k: int(round((fetch[k] * sf + write[k] * sw) * 1024.0)) for k in ("qkv", "narrow", "wide")}
+
+
+def live_traffic(timeout_s=150):
+    """Runs the two counter passes as child processes of this run (rocprofv3 with this file's --pmc-workload after `--`,
+    one counter a pass, each under a time limit and in a process group of its own) and returns traffic_from_counters() of
+    them, or None when the profiler is missing, a pass fails or runs out of time.  Called before this process touches
+    the GPU."""
+    import glob
+    import shutil
+    import signal
+    import subprocess
+    import tempfile
+    if shutil.which("rocprofv3") is None:
+        return None
+    me = os.path.abspath(__file__)
+    out = tempfile.mkdtemp(prefix="xft_pmc_", dir="/tmp")
+    env = dict(os.environ, TMPDIR="/tmp")
+    csvs = []
+    try:
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            d = os.path.join(out, counter)
+            cmd = ["rocprofv3", "--pmc", counter, "--output-format", "csv", "-d", d, "--", sys.executable, me, "--pmc-workload"]
+            pr = subprocess.Popen(cmd, cwd="/tmp", env=env, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL, start_new_session=True)
+            try:
+                rc = pr.wait(timeout=timeout_s)
+            except subprocess.TimeoutExpired:
+                os.killpg(pr.pid, signal.SIGKILL)
+                pr.wait()
+                return None
+            found = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)
+            if rc != 0 or not found:
+                return None
+            csvs.append(found[0])
+        return traffic_from_counters(csvs[0], csvs[1])
+    except Exception:
+        return None
+    finally:
+        shutil.rmtree(out, ignore_errors=True)
+
+
 def measured_traffic(key):
     """HBM bytes per launch recorded by the last counter run (see pmc_summary), or None."""
     try:
@@ -522,6 +589,7 @@ def main():
     ap.add_argument("--prefill-gemm", action="store_true", help="only the weight-only GEMM sweep at M = 1, 8, 32, 256, 2048 (one JSON line)")
     ap.add_argument("--attention", action="store_true", help="only the GQA attention sweep (one JSON line)")
     ap.add_argument("--moe", action="store_true", help="only the sparse-MLP layer (one JSON line)")
+    ap.add_argument("--no-live-traffic", action="store_true", help="do not run the two rocprofv3 counter passes for roofline.traffic (the recorded figure under profiles/ is reported instead)")
     ap.add_argument("--stream-floor", action="store_true", help="only the read-only streaming floor at the decode GEMVs' byte counts (one JSON line)")
     args = ap.parse_args()
     if args.pmc_summary:
@@ -530,6 +598,13 @@ def main():
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (no collectives are part of it)", file=sys.stderr)
         sys.exit(2)
+
+    # HBM counters of the dominant kernel, measured by two profiler passes over child runs of this file: only in the
+    # full default run (the headline configuration), and first, while this process has not touched the GPU
+    single = args.prefill_gemm or args.attention or args.moe or args.stream_floor or args.pmc_workload or args.eager or args.no_extras
+    live = None
+    if not single and not args.no_live_traffic and args.weights == "int8" and args.batch == 1 and args.kv == "fp16":
+        live = live_traffic()
 
     from xfastertransformer_amd import capi as xh
     xh.init(0)
@@ -599,6 +674,11 @@ def main():
     achieved = dom["bytes"] / dom["us"] / 1e3
     # counter-measured HBM bytes per launch exist for the configuration the counters were run on
     traffic = measured_traffic(dom["key"]) if (args.weights == "int8" and B == 1) else None
+    traffic_source = "recorded counter run, profiles/qgemm_skinny_int8_bs1_hbm_traffic.txt (not measured in this run)"
+    if live is not None:
+        traffic = live[dom["key"]]
+        traffic_source = ("two rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE) over child runs of `bench.py --pmc-workload` started by "
+                          "this run, each scaled by the same counter over the library's 256 MiB copy kernel")
 
     result = {
         "metric": "decode tok/s (7B-shape, INT8/INT4 wts, bs1/32); qGEMM % HBM roofline",
@@ -622,7 +702,7 @@ def main():
         "step_hbm_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         "roofline": {"bound": "hbm", "kernel": dom["name"], "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "traffic_source": "recorded counter run, profiles/qgemm_skinny_int8_bs1_hbm_traffic.txt (not measured in this run)",
+                     "traffic_source": traffic_source,
                      "avg_launch_us": round(dom["us"], 3), "bytes_per_launch": int(dom["bytes"])},
         "other_kernels": [{"kernel": g["name"], "launches_per_layer": g["launches"], "avg_launch_us": round(g["us"], 3),
                            "bytes_per_launch": int(g["bytes"]),

@@ -62,6 +62,10 @@ union HFrag32 {
 // memory pipeline ran 262 us: a lane's 16 bytes lie 64 bytes from its neighbour's, and the memory pipeline serves
 // such a load line by line.  What did pay for the FP16 cache: sending the blocks global -> LDS directly (below) instead
 // of through registers and ds_write - 4 of a wave's 20 LDS instructions a block gone, 16 registers free: 213 -> 202 us.
+// INT8 cache, measured and not kept: the block kept in LDS as codes (8 KB instead of 16), a lane's 128-bit read serving
+// two k-steps (the queries' dims and, through a lane-half exchange, the probabilities' tokens permuted to match) -
+// 8 operand reads a block and wave instead of 16, widened by every wave in registers: correct, and 354 us against
+// 292: the 160 widening instructions a wave and block cost more than the LDS port had.
 template <int NW, int CT, bool INT8>
 __device__ inline void attn_prefill32_unit(const AttnParams &p, const int kvh, const int cgroup, const int b, unsigned char *lds) {
     constexpr int D = 128, NT = NW * 64, WC = 32 * CT;

@@ -479,6 +479,41 @@ def prefill_gemm_sweep(xh, M=2048, nweights=8, iters=3):
     return res
 
 
+def gemm_few_rows_sweep(xh, Ms=(1, 8, 32), iters=4):
+    """The few-row cells of the weight-only GEMM sweep (bf16 in, bf16 out, plain epilogue): every (N, K) x kind at M rows
+    over enough distinct weights to exceed the Infinity Cache, HIP events on the launch stream; these launches are bound
+    by the weight bytes, so the figure is GB/s over packed weight + activation rows + result rows against the HBM peak."""
+    rng = np.random.default_rng(1)
+    res = []
+    for (N, K) in ((4096, 4096), (11008, 4096), (4096, 11008)):
+        for kind, name in ((xh.W_INT8, "int8"), (xh.W_UINT4, "uint4"), (xh.W_NF4, "nf4")):
+            q, sc, z = synth_codes(rng, 0 if kind == xh.W_INT8 else 1, K, N)
+            if kind == xh.W_NF4:
+                z = None
+            nw = 24 if kind == xh.W_INT8 else 40
+            ws = [xh.Weight(kind, K, N, q, sc, z) for _ in range(nw)]
+            for M in Ms:
+                A = xh.DeviceBuffer.from_numpy(xh.f32_to_bf16_bits(rng.standard_normal((M, K), dtype=np.float32)))
+                Cd = xh.DeviceBuffer(M * N * 2)
+                for w in ws:
+                    xh.gemm(w, A.ptr, M, K, Cd.ptr, N, xh.BF16)
+                xh.synchronize()
+                t = xh.Timer()
+                t.start()
+                for _ in range(iters):
+                    for w in ws:
+                        xh.gemm(w, A.ptr, M, K, Cd.ptr, N, xh.BF16)
+                us = t.stop() * 1e3 / (iters * nw)
+                byts = ws[0].bytes() + 2 * M * K + 2 * M * N
+                res.append(dict(kind=name, M=M, N=N, K=K, avg_launch_us=round(us, 2), gbs=round(byts / us / 1e3, 1),
+                                frac_of_hbm_peak=round(byts / us / 1e3 / HBM_PEAK_GBS, 4)))
+                A.free()
+                Cd.free()
+            for w in ws:
+                w.free()
+    return res
+
+
 def attention_sweep(xh, iters=10):
     """GQA attention, 32 query / 8 KV heads, head size 128: decode at batch 1 / 16 / 64 and context
     1024 / 4096 / 16384 over FP16 and INT8 caches (achieved GB/s against B ctx 8 128 2 e bytes, e = 2
@@ -586,7 +621,7 @@ def main():
     ap.add_argument("--pmc-summary", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"), help="summarise the two counter CSVs of the --pmc-workload runs (CPU only)")
     ap.add_argument("--eager", action="store_true", help="launch decode kernels one by one instead of replaying the captured graph (for per-kernel profiling)")
     ap.add_argument("--no-extras", action="store_true", help="skip the extra measurements (batch 32 / UINT4 decode, GEMM sweep, attention sweep, sparse MLP)")
-    ap.add_argument("--prefill-gemm", action="store_true", help="only the weight-only GEMM sweep at M = 1, 8, 32, 256, 2048 (one JSON line)")
+    ap.add_argument("--prefill-gemm", action="store_true", help="only the weight-only GEMM sweep: M = 256, 2048 against the MFMA peak, M = 1, 8, 32 against the HBM peak (one JSON line)")
     ap.add_argument("--attention", action="store_true", help="only the GQA attention sweep (one JSON line)")
     ap.add_argument("--moe", action="store_true", help="only the sparse-MLP layer (one JSON line)")
     ap.add_argument("--no-live-traffic", action="store_true", help="do not run the two rocprofv3 counter passes for roofline.traffic (the recorded figure under profiles/ is reported instead)")
@@ -609,7 +644,8 @@ def main():
     from xfastertransformer_amd import capi as xh
     xh.init(0)
     if args.prefill_gemm:
-        print(json.dumps({"prefill_gemm": [r for M in (256, 2048) for r in prefill_gemm_sweep(xh, M)], "peak_tflops": MFMA_BF16_PEAK_TFLOPS}))
+        print(json.dumps({"prefill_gemm": [r for M in (256, 2048) for r in prefill_gemm_sweep(xh, M)], "peak_tflops": MFMA_BF16_PEAK_TFLOPS,
+                          "gemm_few_rows": gemm_few_rows_sweep(xh), "hbm_peak_gbs": HBM_PEAK_GBS}))
         return
     if args.attention:
         print(json.dumps({"attention": attention_sweep(xh), "hbm_peak_gbs": HBM_PEAK_GBS, "peak_tflops": MFMA_BF16_PEAK_TFLOPS}))
@@ -722,6 +758,7 @@ def main():
         # the INT8 KV cache at the batch where the cache is most of the step's bytes
         extra["decode"].append(decode_run(xh, 0, 32, args.prompt, 64, 8, kv_int8=True))
         extra["prefill_gemm"] = prefill_gemm_sweep(xh, 2048)
+        extra["gemm_few_rows"] = gemm_few_rows_sweep(xh)
         extra["attention"] = attention_sweep(xh)
         extra["moe"] = moe_layer(xh)
         # what the bytes of a decode layer's four GEMVs cost as a pure read (out-proj, down, QKV, gate/up)

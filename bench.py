@@ -261,7 +261,7 @@ def traffic_from_counters(fetch_csv, write_csv):
     return {k: int(round((fetch[k] * sf + write[k] * sw) * 1024.0)) for k in ("qkv", "narrow", "wide")}
 
 
-def live_traffic(timeout_s=150):
+def live_traffic(timeout_s=100):
     """Runs the two counter passes as child processes of this run (rocprofv3 with this file's --pmc-workload after `--`,
     one counter a pass, each under a time limit and in a process group of its own) and returns traffic_from_counters() of
     them, or None when the profiler is missing, a pass fails or runs out of time.  Called before this process touches

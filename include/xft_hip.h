@@ -76,6 +76,9 @@ int xfthip_copy_kernel(void *dst, const void *src, size_t bytes, xfthip_stream_t
  * kernels.  A measurement aid with no counterpart in the reference. */
 int xfthip_read_kernel(const void *src, size_t bytes, int blocks, xfthip_stream_t stream);
 int xfthip_memset(void *dst, int value, size_t bytes, xfthip_stream_t stream);
+/* Free and total device memory of the current device in bytes (either pointer may be null).  The host layer sizes
+ * the cache rows of its sequence pool with it; no counterpart in the reference, whose caches live in host memory. */
+int xfthip_device_memory(size_t *free_bytes, size_t *total_bytes);
 int xfthip_stream_create(xfthip_stream_t *stream);
 int xfthip_stream_destroy(xfthip_stream_t stream);
 int xfthip_stream_synchronize(xfthip_stream_t stream);

@@ -500,8 +500,21 @@ struct ModelImpl {
     // is rebuilt when it has to grow, which is only possible while no sequence is alive.
     void fit_rows(int add, int maxLen, int longestPrompt) {
         const int live = (int)pool.size();
+        // Cache rows the pool starts with: XFT_CB_ROWS, or as many rows of maxLen + 1 positions as fit 40 % of the free
+        // device memory, between 8 and 64 (a row is layers x 2 x kv heads x positions x head size values of the cache's
+        // type; the weights are already on the device when the pool is sized)
         int rows = 8;
-        if (const char *e = getenv("XFT_CB_ROWS")) rows = atoi(e) > 0 ? atoi(e) : rows;
+        if (const char *e = getenv("XFT_CB_ROWS")) {
+            rows = atoi(e) > 0 ? atoi(e) : rows;
+        } else {
+            size_t free_b = 0;
+            if (xfthip_device_memory(&free_b, nullptr) == 0 && free_b > 0) {
+                const double per_value = cfg.kv_dtype == XFTHIP_INT8 ? 1.0 + 4.0 / cfg.head_size : 2.0;
+                const double row_b = (double)cfg.layers * 2.0 * cfg.kv_heads * ((maxLen + 1 + 31) / 32 * 32) * cfg.head_size * per_value;
+                const double fit_rows_d = 0.4 * (double)free_b / (row_b > 1.0 ? row_b : 1.0);
+                rows = fit_rows_d >= 64.0 ? 64 : (fit_rows_d <= 8.0 ? 8 : (int)fit_rows_d);
+            }
+        }
         const bool grow = model == nullptr || live + add > cfg.max_batch || maxLen + 1 > cfg.max_seq || longestPrompt > cfg.max_tokens;
         if (!grow) return;
         if (live > 0) {

@@ -194,6 +194,14 @@ int xfthip_read_kernel(const void *src, size_t bytes, int blocks, xfthip_stream_
     return 0;
 }
 
+int xfthip_device_memory(size_t *free_bytes, size_t *total_bytes) {
+    size_t f = 0, t = 0;
+    XFT_CHECK_HIP(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
+    return 0;
+}
+
 int xfthip_memset(void *dst, int value, size_t bytes, xfthip_stream_t stream) {
     if (bytes == 0) return 0;
     XFT_CHECK_HIP(hipMemsetAsync(dst, value, bytes, (hipStream_t)stream));
